@@ -1,0 +1,603 @@
+/*
+ * hyle_oracle.c -- CPU restatement of the reference's scalar semantics for the
+ * tensor hot path.  TEST INFRASTRUCTURE ONLY (see hyle_oracle.h): the shipped
+ * library never links, loads or calls this file.
+ *
+ * Build: gcc -O2 -ffp-contract=off -fno-fast-math (see oracle/Makefile).
+ */
+#include "hyle_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------------ */
+/* bit helpers                                                              */
+/* ------------------------------------------------------------------------ */
+static inline float bits_to_f32(uint32_t b) {
+  float f;
+  memcpy(&f, &b, sizeof f);
+  return f;
+}
+static inline uint32_t f32_to_bits(float f) {
+  uint32_t b;
+  memcpy(&b, &f, sizeof b);
+  return b;
+}
+
+/* ------------------------------------------------------------------------ */
+/* codecs: include/hyle/simd/dtype.h:55-121                                 */
+/* ------------------------------------------------------------------------ */
+
+/* include/hyle/simd/dtype.h:55-67.  Subnormals: mantissa * 2^-24 (exact). */
+float hyle_oracle_f16_to_f32(uint16_t h) {
+  const uint32_t sign = (uint32_t)h >> 15;
+  const uint32_t exp5 = ((uint32_t)h >> 10) & 0x1Fu;
+  const uint32_t man = (uint32_t)h & 0x3FFu;
+  if (exp5 == 0) {
+    const float sub = (1.0f / 16384) * ((float)man * (1.0f / 1024));
+    return sign ? -sub : sub;
+  }
+  const uint32_t exp8 = (exp5 == 31) ? 0xFFu : exp5 + (127 - 15);
+  return bits_to_f32((sign << 31) | (exp8 << 23) | (man << 13));
+}
+
+/* include/hyle/simd/dtype.h:72-101.  RN-even through an odd-bit + (half-ulp-1)
+ * bias; overflow -> inf; NaN -> mantissa 0x3FF. */
+uint16_t hyle_oracle_f32_to_f16(float f) {
+  const uint32_t u = f32_to_bits(f);
+  const uint32_t sign = u >> 31;
+  const uint32_t exp8 = (u >> 23) & 0xFFu;
+  const uint32_t man = u & 0x7FFFFFu;
+
+  int idx = 126 - (int)exp8;
+  if (idx < 13) idx = 13;
+  if (idx > 24) idx = 24;
+  const uint32_t odd = ((man | 0x800000u) >> idx) & 1u;
+  const uint32_t rounded = man + odd + (1u << (idx - 1)) - 1u;
+  const int carry = rounded >= (1u << 23);
+  const int exp = (int)exp8 - 127 + (carry ? 1 : 0);
+
+  if (exp < -24) return (uint16_t)(sign << 15);
+
+  const int is_nan = (exp8 == 255) && (man != 0);
+  const int overflowed = exp >= 16;
+  int be16 = exp + 15;
+  if (be16 < 0) be16 = 0;
+  if (be16 > 31) be16 = 31;
+  const int sub_exp = (-14 - exp) > 0 ? (-14 - exp) : 0;
+  const uint32_t shifted = (rounded & 0x7FFFFFu) >> (13 + sub_exp);
+  const uint32_t leading = (sub_exp == 0) ? 0u : (1024u >> sub_exp);
+  const uint32_t man16 = is_nan ? 0x3FFu : (overflowed ? 0u : leading + shifted);
+  return (uint16_t)((sign << 15) | ((uint32_t)be16 << 10) | man16);
+}
+
+/* include/hyle/simd/dtype.h:107-109 */
+float hyle_oracle_bf16_to_f32(uint16_t b) {
+  return bits_to_f32((uint32_t)b << 16);
+}
+
+/* include/hyle/simd/dtype.h:114-121.  RN-even for finite input, truncation for
+ * inf/NaN, NaN keeps its upper payload and gets bit 6 set. */
+uint16_t hyle_oracle_f32_to_bf16(float f) {
+  const uint32_t u = f32_to_bits(f);
+  const uint32_t mag = u & 0x7FFFFFFFu;
+  const uint32_t incr = (mag < 0x7F800000u) ? (0x7FFFu + ((u >> 16) & 1u)) : 0u;
+  const uint32_t quiet = (mag > 0x7F800000u) ? (1u << 6) : 0u;
+  return (uint16_t)(quiet | ((u + incr) >> 16));
+}
+
+static inline size_t type_size(int type) {
+  return type == HYLE_ORACLE_F32 ? 4u : 2u;
+}
+
+/* src/compute_provider_native/numeric.h:13-47 (decode / encode / load / store) */
+static inline float load_as_f32(int type, const void *p) {
+  if (type == HYLE_ORACLE_F32) {
+    float v;
+    memcpy(&v, p, 4);
+    return v;
+  }
+  uint16_t h;
+  memcpy(&h, p, 2);
+  return type == HYLE_ORACLE_F16 ? hyle_oracle_f16_to_f32(h)
+                                 : hyle_oracle_bf16_to_f32(h);
+}
+static inline void store_from_f32(int type, void *p, float v) {
+  if (type == HYLE_ORACLE_F32) {
+    memcpy(p, &v, 4);
+    return;
+  }
+  const uint16_t h = type == HYLE_ORACLE_F16 ? hyle_oracle_f32_to_f16(v)
+                                             : hyle_oracle_f32_to_bf16(v);
+  memcpy(p, &h, 2);
+}
+
+void hyle_oracle_convert_to_f32(int type, const void *src, float *dst,
+                                size_t n) {
+  const unsigned char *s = (const unsigned char *)src;
+  const size_t w = type_size(type);
+  for (size_t i = 0; i < n; ++i) dst[i] = load_as_f32(type, s + i * w);
+}
+void hyle_oracle_convert_from_f32(int type, const float *src, void *dst,
+                                  size_t n) {
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  for (size_t i = 0; i < n; ++i) store_from_f32(type, d + i * w, src[i]);
+}
+
+/* ------------------------------------------------------------------------ */
+/* shapes                                                                   */
+/* ------------------------------------------------------------------------ */
+
+/* src/compute_ops/operation.cc:249-278: NumPy right-aligned broadcasting. */
+int hyle_oracle_broadcast_shape(const int64_t *left, int left_rank,
+                                const int64_t *right, int right_rank,
+                                int64_t *out) {
+  const int rank = left_rank > right_rank ? left_rank : right_rank;
+  if (rank > HYLE_ORACLE_MAX_RANK) return -1;
+  for (int reverse = 0; reverse < rank; ++reverse) {
+    const int64_t l = reverse < left_rank ? left[left_rank - 1 - reverse] : 1;
+    const int64_t r = reverse < right_rank ? right[right_rank - 1 - reverse] : 1;
+    int64_t extent;
+    if (l == r)
+      extent = l;
+    else if (l == 1)
+      extent = r;
+    else if (r == 1)
+      extent = l;
+    else
+      return -1;
+    out[rank - 1 - reverse] = extent;
+  }
+  return rank;
+}
+
+/* src/compute_provider_native/native_plan.h:152-174: walk the dense output
+ * coordinate from the innermost axis; an input axis of extent 1 (or a missing
+ * leading axis) contributes nothing. */
+size_t hyle_oracle_broadcast_byte_offset(const int64_t *in_dims,
+                                         const int64_t *in_strides, int in_rank,
+                                         const int64_t *out_dims, int out_rank,
+                                         size_t linear) {
+  size_t offset = 0;
+  for (int reverse = 0; reverse < out_rank; ++reverse) {
+    const int out_axis = out_rank - 1 - reverse;
+    const size_t extent = (size_t)out_dims[out_axis];
+    const size_t coordinate = linear % extent;
+    linear /= extent;
+    if (reverse >= in_rank) continue;
+    const int in_axis = in_rank - 1 - reverse;
+    if (in_dims[in_axis] != 1) offset += coordinate * (size_t)in_strides[in_axis];
+  }
+  return offset;
+}
+
+/* src/compute_provider_native/native_plan.h:135-147 */
+size_t hyle_oracle_logical_byte_offset(const int64_t *dims,
+                                       const int64_t *strides, int rank,
+                                       size_t linear) {
+  size_t offset = 0;
+  for (int reverse = 0; reverse < rank; ++reverse) {
+    const int axis = rank - 1 - reverse;
+    const size_t extent = (size_t)dims[axis];
+    offset += (linear % extent) * (size_t)strides[axis];
+    linear /= extent;
+  }
+  return offset;
+}
+
+static size_t element_count(const int64_t *dims, int rank) {
+  size_t n = 1;
+  for (int i = 0; i < rank; ++i) n *= (size_t)dims[i];
+  return n;
+}
+
+/* ------------------------------------------------------------------------ */
+/* elementwise                                                              */
+/* ------------------------------------------------------------------------ */
+
+/* src/compute_provider_native/elementwise.cc:102-114 gives Add / Subtract /
+ * Divide / Minimum; Multiply and Maximum follow the reference's own test
+ * oracle (tests/compute_provider_native/elementwise_test.cc:84-101) and the
+ * CUDA tensor kernel (src/compute_provider_cuda/tensor_kernel.cu:150-165). */
+float hyle_oracle_binary_scalar(int kind, float l, float r) {
+  switch (kind) {
+    case HYLE_ORACLE_ADD: return l + r;
+    case HYLE_ORACLE_SUBTRACT: return l - r;
+    case HYLE_ORACLE_MULTIPLY: return l * r;
+    case HYLE_ORACLE_DIVIDE: return l / r;
+    case HYLE_ORACLE_MINIMUM: return fminf(l, r);
+    case HYLE_ORACLE_MAXIMUM: return fmaxf(l, r);
+    default: return NAN;
+  }
+}
+
+/* src/compute_provider_native/elementwise.cc:349-366 (per-element route; the
+ * linear and chunked routes compute the same values). */
+void hyle_oracle_binary(int kind, int type, const void *left,
+                        const int64_t *ld, const int64_t *ls, int lr,
+                        const void *right, const int64_t *rd, const int64_t *rs,
+                        int rr, void *out, const int64_t *od, int orank) {
+  const size_t n = element_count(od, orank);
+  const size_t w = type_size(type);
+  const unsigned char *a = (const unsigned char *)left;
+  const unsigned char *b = (const unsigned char *)right;
+  unsigned char *o = (unsigned char *)out;
+  for (size_t i = 0; i < n; ++i) {
+    const float x = load_as_f32(
+        type, a + hyle_oracle_broadcast_byte_offset(ld, ls, lr, od, orank, i));
+    const float y = load_as_f32(
+        type, b + hyle_oracle_broadcast_byte_offset(rd, rs, rr, od, orank, i));
+    store_from_f32(type, o + i * w, hyle_oracle_binary_scalar(kind, x, y));
+  }
+}
+
+void hyle_oracle_binary_chain(int kind0, int kind1, int type, const void *a,
+                              const int64_t *ad, const int64_t *as, int ar,
+                              const void *b, const int64_t *bd,
+                              const int64_t *bs, int br, const void *c,
+                              const int64_t *cd, const int64_t *cs, int cr,
+                              void *out, const int64_t *od, int orank) {
+  const size_t n = element_count(od, orank);
+  const size_t w = type_size(type);
+  const unsigned char *pa = (const unsigned char *)a;
+  const unsigned char *pb = (const unsigned char *)b;
+  const unsigned char *pc = (const unsigned char *)c;
+  unsigned char *o = (unsigned char *)out;
+  for (size_t i = 0; i < n; ++i) {
+    const float x = load_as_f32(
+        type, pa + hyle_oracle_broadcast_byte_offset(ad, as, ar, od, orank, i));
+    const float y = load_as_f32(
+        type, pb + hyle_oracle_broadcast_byte_offset(bd, bs, br, od, orank, i));
+    const float z = load_as_f32(
+        type, pc + hyle_oracle_broadcast_byte_offset(cd, cs, cr, od, orank, i));
+    /* the intermediate passes through the storage type, exactly as two
+     * separately submitted Binary operations would leave it */
+    unsigned char tmp[4];
+    store_from_f32(type, tmp, hyle_oracle_binary_scalar(kind0, x, y));
+    const float t = load_as_f32(type, tmp);
+    store_from_f32(type, o + i * w, hyle_oracle_binary_scalar(kind1, t, z));
+  }
+}
+
+/* src/simd/math/activations.cc:21-25 */
+float hyle_oracle_sigmoid(float x) {
+  if (isnan(x)) return x;
+  const float e = expf(-fabsf(x));
+  return x < 0.0f ? e / (1.0f + e) : 1.0f / (1.0f + e);
+}
+
+/* src/simd/math/activations.cc:44-47 */
+float hyle_oracle_silu(float x) {
+  if (x == -INFINITY) return 0.0f;
+  return x * hyle_oracle_sigmoid(x);
+}
+
+/* src/simd/math/activations.cc:106-112 */
+void hyle_oracle_silu_rows(int type, const void *src, void *dst, size_t n) {
+  const unsigned char *s = (const unsigned char *)src;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  for (size_t i = 0; i < n; ++i)
+    store_from_f32(type, d + i * w, hyle_oracle_silu(load_as_f32(type, s + i * w)));
+}
+
+/* src/simd/math/activations.cc:114-122 */
+void hyle_oracle_swiglu(int type, const void *gate, const void *value,
+                        void *dst, size_t n) {
+  const unsigned char *g = (const unsigned char *)gate;
+  const unsigned char *v = (const unsigned char *)value;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  for (size_t i = 0; i < n; ++i) {
+    const float gv = load_as_f32(type, g + i * w);
+    const float lv = load_as_f32(type, v + i * w);
+    store_from_f32(type, d + i * w, hyle_oracle_silu(gv) * lv);
+  }
+}
+
+/* src/compute_provider_native/elementwise.cc:192-208: value = gate + hidden */
+void hyle_oracle_swiglu_packed(int type, const void *packed, void *dst,
+                               size_t rows, size_t hidden) {
+  const unsigned char *p = (const unsigned char *)packed;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  for (size_t r = 0; r < rows; ++r) {
+    const unsigned char *gate = p + r * 2 * hidden * w;
+    hyle_oracle_swiglu(type, gate, gate + hidden * w, d + r * hidden * w, hidden);
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* RMSNorm                                                                  */
+/* ------------------------------------------------------------------------ */
+
+/* src/simd/math/activations.cc:124-146 */
+void hyle_oracle_rms_norm_row(int type, int weight_type, const void *src,
+                              const void *weight, void *dst, size_t n,
+                              float epsilon) {
+  if (n == 0) return;
+  const unsigned char *s = (const unsigned char *)src;
+  const unsigned char *wp = (const unsigned char *)weight;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  const size_t ww = type_size(weight_type);
+  float sum_squares = 0.0f;
+  for (size_t i = 0; i < n; ++i) {
+    const float v = load_as_f32(type, s + i * w);
+    sum_squares = fmaf(v, v, sum_squares);
+  }
+  const float inverse_rms = 1.0f / sqrtf(sum_squares / (float)n + epsilon);
+  if (weight == NULL) {
+    for (size_t i = 0; i < n; ++i)
+      store_from_f32(type, d + i * w, load_as_f32(type, s + i * w) * inverse_rms);
+  } else {
+    for (size_t i = 0; i < n; ++i) {
+      const float v = load_as_f32(type, s + i * w);
+      const float scale = load_as_f32(weight_type, wp + i * ww);
+      store_from_f32(type, d + i * w, v * inverse_rms * scale);
+    }
+  }
+}
+
+void hyle_oracle_rms_norm(int type, int weight_type, const void *src,
+                          const void *weight, void *dst, size_t rows,
+                          size_t hidden, float epsilon) {
+  const unsigned char *s = (const unsigned char *)src;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  for (size_t r = 0; r < rows; ++r)
+    hyle_oracle_rms_norm_row(type, weight_type, s + r * hidden * w, weight,
+                             d + r * hidden * w, hidden, epsilon);
+}
+
+/* src/compute_provider_native/normalization.cc:41-80.  The reference sums each
+ * tile with simd::dot (a Highway vector dot: lane order is target-dependent),
+ * here each tile is summed in index order without fusing; the row total adds
+ * tile sums in tile order as the reference does.  Parity of the tile-internal
+ * order is unpinned at the bit level. */
+void hyle_oracle_rms_norm_native(int type, int weight_type, const void *src,
+                                 const void *weight, void *dst, size_t rows,
+                                 size_t hidden, float epsilon) {
+  const unsigned char *s = (const unsigned char *)src;
+  const unsigned char *wp = (const unsigned char *)weight;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  const size_t ww = type_size(weight_type);
+  float values[128];
+  if (hidden == 0) return;
+  for (size_t r = 0; r < rows; ++r) {
+    const unsigned char *row = s + r * hidden * w;
+    unsigned char *out = d + r * hidden * w;
+    float squares = 0.0f;
+    for (size_t c = 0; c < hidden; c += 128) {
+      const size_t size = hidden - c < 128 ? hidden - c : 128;
+      float tile = 0.0f;
+      for (size_t i = 0; i < size; ++i) {
+        const float v = load_as_f32(type, row + (c + i) * w);
+        tile += v * v;
+      }
+      squares += tile;
+    }
+    const float inverse = 1.0f / sqrtf(squares / (float)hidden + epsilon);
+    for (size_t c = 0; c < hidden; c += 128) {
+      const size_t size = hidden - c < 128 ? hidden - c : 128;
+      for (size_t i = 0; i < size; ++i)
+        values[i] = (load_as_f32(type, row + (c + i) * w) - 0.0f) * inverse;
+      if (weight != NULL) {
+        for (size_t i = 0; i < size; ++i)
+          values[i] = values[i] * load_as_f32(weight_type, wp + (c + i) * ww);
+      }
+      for (size_t i = 0; i < size; ++i)
+        store_from_f32(type, out + (c + i) * w, values[i]);
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* softmax                                                                  */
+/* ------------------------------------------------------------------------ */
+
+/* src/simd/math/activations.cc:177-192 */
+static int finite_row_max(const float *src, size_t n, float *maximum) {
+  float m = -INFINITY;
+  for (size_t i = 0; i < n; ++i) {
+    const float x = src[i];
+    if (isnan(x) || x == INFINITY) {
+      *maximum = m;
+      return 0;
+    }
+    if (x > m) m = x;
+  }
+  *maximum = m;
+  return isfinite(m);
+}
+
+/* src/simd/math/activations.cc:301-317: invalid row (any NaN, any +inf, or no
+ * finite maximum) becomes all quiet NaN; the exp sum is accumulated in double
+ * and the row scaled by float(1/sum). */
+void hyle_oracle_softmax_f32_row(const float *src, float *dst, size_t n) {
+  if (n == 0) return;
+  float maximum = 0.0f;
+  if (!finite_row_max(src, n, &maximum)) {
+    for (size_t i = 0; i < n; ++i) dst[i] = NAN;
+    return;
+  }
+  double sum = 0.0;
+  for (size_t i = 0; i < n; ++i) {
+    const float value = expf(src[i] - maximum);
+    dst[i] = value;
+    sum += (double)value;
+  }
+  const float inverse = (float)(1.0 / sum);
+  for (size_t i = 0; i < n; ++i) dst[i] *= inverse;
+}
+
+/* src/compute_provider_native/transformer.cc:44-57 (bool mask) and 165-191 (row
+ * loop over a dense last axis); additive mask per
+ * src/compute_provider_cuda/reduction_kernel.cu:130-146. */
+void hyle_oracle_softmax(int type, const void *src, void *dst,
+                         const int64_t *in_dims, int in_rank, float scale,
+                         int mask_kind, const void *mask,
+                         const int64_t *mask_dims, const int64_t *mask_strides,
+                         int mask_rank) {
+  if (in_rank <= 0) return;
+  const size_t width = (size_t)in_dims[in_rank - 1];
+  const size_t total = element_count(in_dims, in_rank);
+  if (total == 0 || width == 0) return;
+  const size_t rows = total / width;
+  const size_t w = type_size(type);
+  const unsigned char *s = (const unsigned char *)src;
+  const unsigned char *m = (const unsigned char *)mask;
+  unsigned char *d = (unsigned char *)dst;
+  float *scratch = (float *)malloc(width * sizeof(float));
+  if (scratch == NULL) return;
+  for (size_t r = 0; r < rows; ++r) {
+    for (size_t lane = 0; lane < width; ++lane) {
+      const size_t logical = r * width + lane;
+      float value = load_as_f32(type, s + logical * w);
+      value *= scale;
+      if (mask_kind == HYLE_ORACLE_MASK_BOOLEAN) {
+        const size_t off = hyle_oracle_broadcast_byte_offset(
+            mask_dims, mask_strides, mask_rank, in_dims, in_rank, logical);
+        if (m[off] == 0) value = -INFINITY;
+      } else if (mask_kind == HYLE_ORACLE_MASK_ADDITIVE) {
+        const size_t off = hyle_oracle_broadcast_byte_offset(
+            mask_dims, mask_strides, mask_rank, in_dims, in_rank, logical);
+        value = value + load_as_f32(type, m + off);
+      }
+      scratch[lane] = value;
+    }
+    hyle_oracle_softmax_f32_row(scratch, scratch, width);
+    for (size_t lane = 0; lane < width; ++lane)
+      store_from_f32(type, d + (r * width + lane) * w, scratch[lane]);
+  }
+  free(scratch);
+}
+
+/* ------------------------------------------------------------------------ */
+/* reductions                                                               */
+/* ------------------------------------------------------------------------ */
+
+/* src/compute_provider_native/reduction.cc:24-47: once the running extremum is
+ * NaN it stays NaN; a NaN input replaces a non-NaN running value. */
+static void accumulate_extremum(int maximum, float value, float *result) {
+  if (isnan(*result)) return;
+  if (isnan(value)) {
+    *result = value;
+    return;
+  }
+  *result = maximum ? fmaxf(*result, value) : fminf(*result, value);
+}
+
+void hyle_oracle_reduce_last_axis(int kind, int type, const void *src,
+                                  void *dst, size_t rows, size_t width) {
+  const unsigned char *s = (const unsigned char *)src;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  for (size_t r = 0; r < rows; ++r) {
+    const unsigned char *row = s + r * width * w;
+    float result;
+    if (kind == HYLE_ORACLE_MIN || kind == HYLE_ORACLE_MAX) {
+      const int maximum = kind == HYLE_ORACLE_MAX;
+      result = maximum ? -INFINITY : INFINITY;
+      for (size_t i = 0; i < width; ++i)
+        accumulate_extremum(maximum, load_as_f32(type, row + i * w), &result);
+    } else {
+      /* src/compute_provider_cuda/reduction_kernel.cu:92-116: f32 accumulate;
+       * the summation order is unspecified there (tolerance-compared). */
+      float sum = 0.0f;
+      for (size_t i = 0; i < width; ++i) sum += load_as_f32(type, row + i * w);
+      result = sum;
+      if (kind == HYLE_ORACLE_MEAN)
+        result = width == 0 ? NAN : sum / (float)width;
+    }
+    store_from_f32(type, d + r * w, result);
+  }
+}
+
+/* include/hyle/simd/search.h:11-19 */
+size_t hyle_oracle_index_of_max_f32(const float *data, size_t n) {
+  if (n == 0) return 0;
+  size_t best = 0;
+  for (size_t i = 0; i < n; ++i) {
+    if (isnan(data[i])) return i;
+    if (data[i] > data[best]) best = i;
+  }
+  return best;
+}
+
+/* src/compute_provider_cuda/collectives.cu:478-495 (ArgBest, largest=true):
+ * a NaN never beats a number; equal values (including -0 == +0) and NaN pairs
+ * resolve to the lower index. */
+void hyle_oracle_topk1_f32(const float *data, size_t rows, size_t width,
+                           float *values, int32_t *indices) {
+  for (size_t r = 0; r < rows; ++r) {
+    const float *row = data + r * width;
+    size_t best = 0;
+    for (size_t i = 1; i < width; ++i) {
+      const int best_nan = isnan(row[best]);
+      const int cand_nan = isnan(row[i]);
+      if (best_nan != cand_nan) {
+        if (best_nan) best = i;
+        continue;
+      }
+      if (!best_nan && row[i] > row[best]) best = i;
+    }
+    if (width != 0) {
+      if (values) values[r] = row[best];
+      if (indices) indices[r] = (int32_t)best;
+    }
+  }
+}
+
+/* ------------------------------------------------------------------------ */
+/* Q8_0                                                                     */
+/* ------------------------------------------------------------------------ */
+
+/* Format constants: src/compute_ops/low_precision.cc:28-29 (32 elements, 34
+ * bytes).  Decode restated from ggml dequantize_row_q8_0: y[j] = qs[j] * d
+ * with d = fp16 -> f32.  |qs| <= 128 has at most 8 significant bits and d has
+ * 11, so the f32 product is exact; the bf16 store is then a single RN-even. */
+void hyle_oracle_q8_0_dequant_bf16(const void *blocks, size_t rows, size_t k,
+                                   size_t row_stride_bytes, uint16_t *out,
+                                   float *sumsq, float *sumsq_rounded) {
+  const unsigned char *base = (const unsigned char *)blocks;
+  const size_t nb = k / 32;
+  for (size_t r = 0; r < rows; ++r) {
+    const unsigned char *row = base + r * row_stride_bytes;
+    float acc = 0.0f, acc_rounded = 0.0f;
+    for (size_t b = 0; b < nb; ++b) {
+      const unsigned char *blk = row + b * 34;
+      const uint16_t dbits = (uint16_t)(blk[0] | ((uint16_t)blk[1] << 8));
+      const float d = hyle_oracle_f16_to_f32(dbits);
+      for (size_t j = 0; j < 32; ++j) {
+        const float y = (float)(int8_t)blk[2 + j] * d;
+        const uint16_t h = hyle_oracle_f32_to_bf16(y);
+        out[r * k + b * 32 + j] = h;
+        acc += y * y;
+        const float yr = hyle_oracle_bf16_to_f32(h);
+        acc_rounded += yr * yr;
+      }
+    }
+    if (sumsq) sumsq[r] = acc;
+    if (sumsq_rounded) sumsq_rounded[r] = acc_rounded;
+  }
+}
+
+void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
+                                  size_t row_stride_bytes, float *out) {
+  const unsigned char *base = (const unsigned char *)blocks;
+  const size_t nb = k / 32;
+  for (size_t r = 0; r < rows; ++r) {
+    const unsigned char *row = base + r * row_stride_bytes;
+    for (size_t b = 0; b < nb; ++b) {
+      const unsigned char *blk = row + b * 34;
+      const uint16_t dbits = (uint16_t)(blk[0] | ((uint16_t)blk[1] << 8));
+      const float d = hyle_oracle_f16_to_f32(dbits);
+      for (size_t j = 0; j < 32; ++j)
+        out[r * k + b * 32 + j] = (float)(int8_t)blk[2 + j] * d;
+    }
+  }
+}

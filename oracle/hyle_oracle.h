@@ -1,0 +1,204 @@
+/*
+ * hyle_oracle.h -- CPU restatement of the reference's scalar semantics for the
+ * tensor hot path (broadcast add/mul, SiLU, SwiGLU, RMSNorm, row softmax, row
+ * max/sum, argmax, Q8_0 block decode).
+ *
+ * THIS IS TEST INFRASTRUCTURE.  It is the checker the HIP kernels are compared
+ * against and the "port" CPU baseline that bench.py times beside the GPU; it
+ * is never linked into, loaded by, or called from the shipped library.
+ *
+ * Every function cites the reference file:line it follows (paths relative to
+ * the reference tree).  Storage types f16/bf16 are carried as uint16_t bit
+ * patterns.  Built with -ffp-contract=off: a fused multiply-add happens only
+ * where the reference itself writes std::fma.
+ *
+ * Parity status (what pins each function is listed in oracle/README.md):
+ *   - codecs, silu, swiglu, rms_norm (scalar floor), softmax: pinned bit-exact
+ *     against the reference's own scalar floor compiled from its sources
+ *     (oracle/_ref), plus the reference tests' known-answer vectors.
+ *   - binary add/mul, broadcast offsets, reduce, index_of_max, topk1: pinned by
+ *     IEEE closed forms, brute force and the reference tests' known answers.
+ *   - q8_0 decode: the arithmetic lives in ggml (not in the reference tree);
+ *     restated from the published block format, pinned by an exactness proof
+ *     and exhaustive scale x quant enumeration against an independent
+ *     integer/double evaluation.
+ *   - rms_norm_bf16_native tile order: "parity unpinned" at the bit level (the
+ *     reference sums each 128-wide tile with a Highway vector dot whose lane
+ *     order is target-dependent); pinned only to tolerance.
+ */
+#ifndef HYLE_ORACLE_H_
+#define HYLE_ORACLE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HYLE_ORACLE_MAX_RANK 8
+
+/* element types understood by the typed entry points */
+enum {
+  HYLE_ORACLE_F32 = 0,
+  HYLE_ORACLE_F16 = 1,
+  HYLE_ORACLE_BF16 = 2,
+};
+
+/* include/hyle/compute/operation.h:75-82 */
+enum {
+  HYLE_ORACLE_ADD = 0,
+  HYLE_ORACLE_SUBTRACT = 1,
+  HYLE_ORACLE_MULTIPLY = 2,
+  HYLE_ORACLE_DIVIDE = 3,
+  HYLE_ORACLE_MINIMUM = 4,
+  HYLE_ORACLE_MAXIMUM = 5,
+};
+
+/* include/hyle/compute/operation.h:84-89 */
+enum {
+  HYLE_ORACLE_SUM = 0,
+  HYLE_ORACLE_MEAN = 1,
+  HYLE_ORACLE_MIN = 2,
+  HYLE_ORACLE_MAX = 3,
+};
+
+/* include/hyle/compute/operation.h:122-126 */
+enum {
+  HYLE_ORACLE_MASK_NONE = 0,
+  HYLE_ORACLE_MASK_ADDITIVE = 1,
+  HYLE_ORACLE_MASK_BOOLEAN = 2,
+};
+
+/* ---- codecs: include/hyle/simd/dtype.h:55-121 --------------------------- */
+float hyle_oracle_f16_to_f32(uint16_t bits);
+uint16_t hyle_oracle_f32_to_f16(float value);
+float hyle_oracle_bf16_to_f32(uint16_t bits);
+uint16_t hyle_oracle_f32_to_bf16(float value);
+void hyle_oracle_convert_to_f32(int type, const void *src, float *dst, size_t n);
+void hyle_oracle_convert_from_f32(int type, const float *src, void *dst, size_t n);
+
+/* ---- shape helpers ------------------------------------------------------ */
+/* src/compute_ops/operation.cc:249-278.  Returns the result rank, or -1 when
+ * the shapes cannot be broadcast / the rank exceeds 8. */
+int hyle_oracle_broadcast_shape(const int64_t *left, int left_rank,
+                                const int64_t *right, int right_rank,
+                                int64_t *out);
+/* src/compute_provider_native/native_plan.h:152-174 */
+size_t hyle_oracle_broadcast_byte_offset(const int64_t *in_dims,
+                                         const int64_t *in_strides, int in_rank,
+                                         const int64_t *out_dims, int out_rank,
+                                         size_t linear_index);
+/* src/compute_provider_native/native_plan.h:135-147 */
+size_t hyle_oracle_logical_byte_offset(const int64_t *dims,
+                                       const int64_t *strides, int rank,
+                                       size_t linear_index);
+
+/* ---- elementwise -------------------------------------------------------- */
+/* Scalar semantic of one Binary kind on f32 operands
+ * (src/compute_provider_native/elementwise.cc:102-114; Multiply and Maximum
+ * from tests/compute_provider_native/elementwise_test.cc:84-101). */
+float hyle_oracle_binary_scalar(int kind, float left, float right);
+
+/* Broadcasting Binary: dense output of out_rank dims, inputs described by
+ * dims + byte strides (zero stride on a broadcast axis is honoured through
+ * the "input dimension == 1" rule of the reference).  Storage type `type`;
+ * narrow types decode -> f32 op -> one RN-even store
+ * (src/compute_provider_native/elementwise.cc:135-157, 333-366). */
+void hyle_oracle_binary(int kind, int type, const void *left,
+                        const int64_t *left_dims, const int64_t *left_strides,
+                        int left_rank, const void *right,
+                        const int64_t *right_dims,
+                        const int64_t *right_strides, int right_rank, void *out,
+                        const int64_t *out_dims, int out_rank);
+
+/* Two chained Binary ops with the intermediate rounded to the storage type:
+ * out = (a kind0 b) kind1 c.  All three inputs broadcast to out. This equals
+ * running hyle_oracle_binary twice through a temporary. */
+void hyle_oracle_binary_chain(int kind0, int kind1, int type, const void *a,
+                              const int64_t *a_dims, const int64_t *a_strides,
+                              int a_rank, const void *b, const int64_t *b_dims,
+                              const int64_t *b_strides, int b_rank,
+                              const void *c, const int64_t *c_dims,
+                              const int64_t *c_strides, int c_rank, void *out,
+                              const int64_t *out_dims, int out_rank);
+
+/* src/simd/math/activations.cc:21-25,44-47 */
+float hyle_oracle_sigmoid(float x);
+float hyle_oracle_silu(float x);
+/* src/simd/math/activations.cc:106-112 (unary_storage) */
+void hyle_oracle_silu_rows(int type, const void *src, void *dst, size_t n);
+/* src/simd/math/activations.cc:114-122 (gated_storage, activation = silu) */
+void hyle_oracle_swiglu(int type, const void *gate, const void *value,
+                        void *dst, size_t n);
+/* GatedInputKind::kPackedHalves: row = [gate half | value half]
+ * (src/compute_provider_native/elementwise.cc:192-208). */
+void hyle_oracle_swiglu_packed(int type, const void *packed, void *dst,
+                               size_t rows, size_t hidden);
+
+/* ---- normalisation ------------------------------------------------------ */
+/* src/simd/math/activations.cc:124-146 (fma chain, x*inv*w).  weight may be
+ * NULL.  weight_type may be HYLE_ORACLE_F32 for a narrow input
+ * (src/compute_ops/operation.cc:492-505). */
+void hyle_oracle_rms_norm_row(int type, int weight_type, const void *src,
+                              const void *weight, void *dst, size_t n,
+                              float epsilon);
+void hyle_oracle_rms_norm(int type, int weight_type, const void *src,
+                          const void *weight, void *dst, size_t rows,
+                          size_t hidden, float epsilon);
+/* src/compute_provider_native/normalization.cc:41-80: 128-wide f32 tiles,
+ * squares += dot(tile, tile); (x * inv) then * w; one RN-even store. */
+void hyle_oracle_rms_norm_native(int type, int weight_type, const void *src,
+                                 const void *weight, void *dst, size_t rows,
+                                 size_t hidden, float epsilon);
+
+/* ---- softmax / reductions ---------------------------------------------- */
+/* src/simd/math/activations.cc:177-192,301-317.  In place allowed. */
+void hyle_oracle_softmax_f32_row(const float *src, float *dst, size_t n);
+/* Row softmax over the last axis of a dense [rows, width] tensor of storage
+ * type `type` with `scale` and an optional broadcast mask
+ * (src/compute_provider_native/transformer.cc:44-57,165-191).  The mask is
+ * described by dims/byte strides and broadcast against in_dims
+ * (rank in_rank, last axis = width).  mask_kind BOOLEAN: uint8 0 => -inf;
+ * ADDITIVE: same storage type, v + mask
+ * (src/compute_provider_cuda/reduction_kernel.cu:130-146). */
+void hyle_oracle_softmax(int type, const void *src, void *dst,
+                         const int64_t *in_dims, int in_rank, float scale,
+                         int mask_kind, const void *mask,
+                         const int64_t *mask_dims, const int64_t *mask_strides,
+                         int mask_rank);
+
+/* src/compute_provider_native/reduction.cc:24-47 (NaN-propagating extrema,
+ * identities +-inf) and src/compute_provider_cuda/reduction_kernel.cu:92-116
+ * (sum / mean, f32 accumulate, mean of an empty row is NaN).  Reduces the
+ * last axis of dense [rows, width]. */
+void hyle_oracle_reduce_last_axis(int kind, int type, const void *src,
+                                  void *dst, size_t rows, size_t width);
+
+/* include/hyle/simd/search.h:11-19: first index of the maximum; first NaN
+ * index when any NaN is present; n for an empty range. */
+size_t hyle_oracle_index_of_max_f32(const float *data, size_t n);
+/* TopK{count=1, largest} rule: src/compute_provider_cuda/collectives.cu:478-495
+ * (non-NaN beats NaN, ties -> lower index; an all-NaN row returns index 0). */
+void hyle_oracle_topk1_f32(const float *data, size_t rows, size_t width,
+                           float *values, int32_t *indices);
+
+/* ---- Q8_0 --------------------------------------------------------------- */
+/* Block = { fp16 d; int8 qs[32] }, 34 bytes, little-endian
+ * (src/compute_ops/low_precision.cc:28-29; ggml block_q8_0, module ggml pinned
+ * at ffa4e8b80930029a35991f94e7c8a93cd67730ab in cmake/HyleDependencyLock.json).
+ * y = (float)qs[j] * f16_to_f32(d), stored as bf16 RN-even.  sumsq[row] is the
+ * f32 sum over the exact f32 products (before bf16 rounding), accumulated in
+ * index order; sumsq_rounded (optional, may be NULL) sums the squares of the
+ * bf16-rounded outputs instead. */
+void hyle_oracle_q8_0_dequant_bf16(const void *blocks, size_t rows, size_t k,
+                                   size_t row_stride_bytes, uint16_t *out,
+                                   float *sumsq, float *sumsq_rounded);
+/* ggml dequantize_row_q8_0 to f32 */
+void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
+                                  size_t row_stride_bytes, float *out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HYLE_ORACLE_H_ */

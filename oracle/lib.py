@@ -1,0 +1,320 @@
+"""ctypes binding of oracle/libhyle_oracle.so over numpy arrays.
+
+Test infrastructure only.  Narrow floats travel as uint16 bit patterns.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libhyle_oracle.so")
+
+F32, F16, BF16 = 0, 1, 2
+ADD, SUBTRACT, MULTIPLY, DIVIDE, MINIMUM, MAXIMUM = range(6)
+SUM, MEAN, MIN, MAX = range(4)
+MASK_NONE, MASK_ADDITIVE, MASK_BOOLEAN = range(3)
+
+_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16}
+
+
+def build() -> None:
+    """Compile the checker (and oracle/_ref when the reference tree exists)."""
+    subprocess.run(["make", "-C", _HERE, "--no-print-directory"], check=True)
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(_SO):
+        build()
+    return C.CDLL(_SO)
+
+
+_lib = _load()
+
+_vp = C.c_void_p
+_sz = C.c_size_t
+_i64p = C.POINTER(C.c_int64)
+
+
+def _sig(name, restype, *argtypes):
+    fn = getattr(_lib, name)
+    fn.restype = restype
+    fn.argtypes = list(argtypes)
+    return fn
+
+
+_f16_to_f32 = _sig("hyle_oracle_f16_to_f32", C.c_float, C.c_uint16)
+_f32_to_f16 = _sig("hyle_oracle_f32_to_f16", C.c_uint16, C.c_float)
+_bf16_to_f32 = _sig("hyle_oracle_bf16_to_f32", C.c_float, C.c_uint16)
+_f32_to_bf16 = _sig("hyle_oracle_f32_to_bf16", C.c_uint16, C.c_float)
+_to_f32 = _sig("hyle_oracle_convert_to_f32", None, C.c_int, _vp, _vp, _sz)
+_from_f32 = _sig("hyle_oracle_convert_from_f32", None, C.c_int, _vp, _vp, _sz)
+_bshape = _sig("hyle_oracle_broadcast_shape", C.c_int, _i64p, C.c_int, _i64p, C.c_int, _i64p)
+_boff = _sig("hyle_oracle_broadcast_byte_offset", _sz, _i64p, _i64p, C.c_int, _i64p, C.c_int, _sz)
+_loff = _sig("hyle_oracle_logical_byte_offset", _sz, _i64p, _i64p, C.c_int, _sz)
+_bscalar = _sig("hyle_oracle_binary_scalar", C.c_float, C.c_int, C.c_float, C.c_float)
+_binary = _sig("hyle_oracle_binary", None, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int,
+               _vp, _i64p, _i64p, C.c_int, _vp, _i64p, C.c_int)
+_chain = _sig("hyle_oracle_binary_chain", None, C.c_int, C.c_int, C.c_int,
+              _vp, _i64p, _i64p, C.c_int, _vp, _i64p, _i64p, C.c_int,
+              _vp, _i64p, _i64p, C.c_int, _vp, _i64p, C.c_int)
+_sigmoid = _sig("hyle_oracle_sigmoid", C.c_float, C.c_float)
+_silu1 = _sig("hyle_oracle_silu", C.c_float, C.c_float)
+_silu = _sig("hyle_oracle_silu_rows", None, C.c_int, _vp, _vp, _sz)
+_swiglu = _sig("hyle_oracle_swiglu", None, C.c_int, _vp, _vp, _vp, _sz)
+_swiglu_packed = _sig("hyle_oracle_swiglu_packed", None, C.c_int, _vp, _vp, _sz, _sz)
+_rms = _sig("hyle_oracle_rms_norm", None, C.c_int, C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_float)
+_rms_native = _sig("hyle_oracle_rms_norm_native", None, C.c_int, C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_float)
+_softmax_row = _sig("hyle_oracle_softmax_f32_row", None, _vp, _vp, _sz)
+_softmax = _sig("hyle_oracle_softmax", None, C.c_int, _vp, _vp, _i64p, C.c_int, C.c_float,
+                C.c_int, _vp, _i64p, _i64p, C.c_int)
+_reduce = _sig("hyle_oracle_reduce_last_axis", None, C.c_int, C.c_int, _vp, _vp, _sz, _sz)
+_iom = _sig("hyle_oracle_index_of_max_f32", _sz, _vp, _sz)
+_topk1 = _sig("hyle_oracle_topk1_f32", None, _vp, _sz, _sz, _vp, _vp)
+_q8_bf16 = _sig("hyle_oracle_q8_0_dequant_bf16", None, _vp, _sz, _sz, _sz, _vp, _vp, _vp)
+_q8_f32 = _sig("hyle_oracle_q8_0_dequant_f32", None, _vp, _sz, _sz, _sz, _vp)
+
+
+def _ptr(a: np.ndarray | None):
+    return None if a is None else a.ctypes.data_as(_vp)
+
+
+def _i64(values):
+    arr = (C.c_int64 * max(len(values), 1))(*[int(v) for v in values])
+    return arr
+
+
+def _c(a: np.ndarray, dtype=None) -> np.ndarray:
+    a = np.ascontiguousarray(a)
+    if dtype is not None and a.dtype != np.dtype(dtype):
+        raise TypeError(f"expected {np.dtype(dtype)}, got {a.dtype}")
+    return a
+
+
+def np_dtype(type_id: int):
+    return _NP[type_id]
+
+
+def itemsize(type_id: int) -> int:
+    return 4 if type_id == F32 else 2
+
+
+def dense_strides(dims, type_id) -> list[int]:
+    strides, step = [], itemsize(type_id)
+    for d in reversed(list(dims)):
+        strides.append(step)
+        step *= int(d)
+    return list(reversed(strides))
+
+
+# ---- codecs ---------------------------------------------------------------
+def f16_to_f32(bits: int) -> float:
+    return _f16_to_f32(int(bits))
+
+
+def f32_to_f16(x: float) -> int:
+    return _f32_to_f16(np.float32(x).item() if not isinstance(x, float) else x)
+
+
+def bf16_to_f32(bits: int) -> float:
+    return _bf16_to_f32(int(bits))
+
+
+def f32_bits_to_bf16(bits32: int) -> int:
+    """Round one f32 given as its bit pattern (keeps NaN payloads intact)."""
+    src = np.array([bits32], dtype=np.uint32).view(np.float32)
+    return int(from_f32(BF16, src)[0])
+
+
+def to_f32(type_id: int, a: np.ndarray) -> np.ndarray:
+    a = _c(a, _NP[type_id])
+    out = np.empty(a.shape, np.float32)
+    _to_f32(type_id, _ptr(a), _ptr(out), a.size)
+    return out
+
+
+def from_f32(type_id: int, a: np.ndarray) -> np.ndarray:
+    a = _c(a, np.float32)
+    out = np.empty(a.shape, _NP[type_id])
+    _from_f32(type_id, _ptr(a), _ptr(out), a.size)
+    return out
+
+
+# ---- shapes ---------------------------------------------------------------
+def broadcast_shape(left, right):
+    out = (C.c_int64 * 8)()
+    rank = _bshape(_i64(left), len(left), _i64(right), len(right), out)
+    if rank < 0:
+        return None
+    return [int(out[i]) for i in range(rank)]
+
+
+def broadcast_byte_offset(in_dims, in_strides, out_dims, linear: int) -> int:
+    return _boff(_i64(in_dims), _i64(in_strides), len(in_dims), _i64(out_dims), len(out_dims), linear)
+
+
+def logical_byte_offset(dims, strides, linear: int) -> int:
+    return _loff(_i64(dims), _i64(strides), len(dims), linear)
+
+
+# ---- elementwise ----------------------------------------------------------
+def binary_scalar(kind: int, left: float, right: float) -> float:
+    return _bscalar(kind, left, right)
+
+
+def binary(kind, type_id, left, right, left_strides=None, right_strides=None):
+    """Broadcasting Binary.  Arrays carry the logical dims; strides default to
+    dense.  A custom stride list (bytes) reads `left`/`right` as raw storage."""
+    left, right = _c(left, _NP[type_id]), _c(right, _NP[type_id])
+    ld, rd = list(left.shape), list(right.shape)
+    od = broadcast_shape(ld, rd)
+    if od is None:
+        raise ValueError("shapes do not broadcast")
+    ls = left_strides or dense_strides(ld, type_id)
+    rs = right_strides or dense_strides(rd, type_id)
+    out = np.empty(od, _NP[type_id])
+    _binary(kind, type_id, _ptr(left), _i64(ld), _i64(ls), len(ld), _ptr(right), _i64(rd),
+            _i64(rs), len(rd), _ptr(out), _i64(od), len(od))
+    return out
+
+
+def binary_raw(kind, type_id, left, ld, ls, right, rd, rs, od):
+    """Binary over raw storage buffers with explicit dims / byte strides."""
+    out = np.empty(od, _NP[type_id])
+    _binary(kind, type_id, _ptr(left), _i64(ld), _i64(ls), len(ld), _ptr(right), _i64(rd),
+            _i64(rs), len(rd), _ptr(out), _i64(od), len(od))
+    return out
+
+
+def binary_chain(kind0, kind1, type_id, a, b, c):
+    a, b, c = (_c(x, _NP[type_id]) for x in (a, b, c))
+    ad, bd, cd = list(a.shape), list(b.shape), list(c.shape)
+    od = broadcast_shape(broadcast_shape(ad, bd), cd)
+    out = np.empty(od, _NP[type_id])
+    _chain(kind0, kind1, type_id,
+           _ptr(a), _i64(ad), _i64(dense_strides(ad, type_id)), len(ad),
+           _ptr(b), _i64(bd), _i64(dense_strides(bd, type_id)), len(bd),
+           _ptr(c), _i64(cd), _i64(dense_strides(cd, type_id)), len(cd),
+           _ptr(out), _i64(od), len(od))
+    return out
+
+
+def sigmoid(x: float) -> float:
+    return _sigmoid(x)
+
+
+def silu_scalar(x: float) -> float:
+    return _silu1(x)
+
+
+def silu(type_id, src):
+    src = _c(src, _NP[type_id])
+    out = np.empty_like(src)
+    _silu(type_id, _ptr(src), _ptr(out), src.size)
+    return out
+
+
+def swiglu(type_id, gate, value):
+    gate, value = _c(gate, _NP[type_id]), _c(value, _NP[type_id])
+    assert gate.shape == value.shape
+    out = np.empty_like(gate)
+    _swiglu(type_id, _ptr(gate), _ptr(value), _ptr(out), gate.size)
+    return out
+
+
+def swiglu_packed(type_id, packed):
+    packed = _c(packed, _NP[type_id])
+    hidden = packed.shape[-1] // 2
+    rows = packed.size // (2 * hidden) if hidden else 0
+    out = np.empty(packed.shape[:-1] + (hidden,), _NP[type_id])
+    _swiglu_packed(type_id, _ptr(packed), _ptr(out), rows, hidden)
+    return out
+
+
+# ---- normalisation --------------------------------------------------------
+def rms_norm(type_id, src, weight, epsilon, weight_type=None, native=False):
+    src = _c(src, _NP[type_id])
+    weight_type = type_id if weight_type is None else weight_type
+    if weight is not None:
+        weight = _c(weight, _NP[weight_type])
+    hidden = src.shape[-1]
+    rows = src.size // hidden if hidden else 0
+    out = np.empty_like(src)
+    fn = _rms_native if native else _rms
+    fn(type_id, weight_type, _ptr(src), _ptr(weight), _ptr(out), rows, hidden, float(epsilon))
+    return out
+
+
+# ---- softmax / reductions -------------------------------------------------
+def softmax_f32_row(src):
+    src = _c(src, np.float32)
+    out = np.empty_like(src)
+    _softmax_row(_ptr(src), _ptr(out), src.size)
+    return out
+
+
+def softmax(type_id, src, scale=1.0, mask_kind=MASK_NONE, mask=None, mask_strides=None):
+    src = _c(src, _NP[type_id])
+    out = np.empty_like(src)
+    md, ms = [], []
+    if mask_kind != MASK_NONE:
+        mask = np.ascontiguousarray(mask)
+        md = list(mask.shape)
+        ms = mask_strides or _byte_strides(md, mask.itemsize)
+    _softmax(type_id, _ptr(src), _ptr(out), _i64(src.shape), src.ndim, float(scale),
+             mask_kind, _ptr(mask), _i64(md), _i64(ms), len(md))
+    return out
+
+
+def _byte_strides(dims, width):
+    strides, step = [], width
+    for d in reversed(list(dims)):
+        strides.append(step)
+        step *= int(d)
+    return list(reversed(strides))
+
+
+def reduce_last_axis(kind, type_id, src):
+    src = _c(src, _NP[type_id])
+    width = src.shape[-1]
+    rows = int(np.prod(src.shape[:-1], dtype=np.int64))
+    out = np.empty(src.shape[:-1], _NP[type_id])
+    _reduce(kind, type_id, _ptr(src), _ptr(out), rows, width)
+    return out
+
+
+def index_of_max(data) -> int:
+    data = _c(data, np.float32)
+    return int(_iom(_ptr(data), data.size))
+
+
+def topk1(data):
+    data = _c(data, np.float32)
+    width = data.shape[-1]
+    rows = int(np.prod(data.shape[:-1], dtype=np.int64))
+    values = np.empty(data.shape[:-1], np.float32)
+    indices = np.empty(data.shape[:-1], np.int32)
+    _topk1(_ptr(data), rows, width, _ptr(values), _ptr(indices))
+    return values, indices
+
+
+# ---- Q8_0 -----------------------------------------------------------------
+def q8_0_dequant_bf16(blocks: np.ndarray, rows: int, k: int, row_stride: int | None = None):
+    blocks = _c(blocks, np.uint8)
+    row_stride = (k // 32) * 34 if row_stride is None else row_stride
+    out = np.empty((rows, k), np.uint16)
+    sumsq = np.empty(rows, np.float32)
+    sumsq_rounded = np.empty(rows, np.float32)
+    _q8_bf16(_ptr(blocks), rows, k, row_stride, _ptr(out), _ptr(sumsq), _ptr(sumsq_rounded))
+    return out, sumsq, sumsq_rounded
+
+
+def q8_0_dequant_f32(blocks: np.ndarray, rows: int, k: int, row_stride: int | None = None):
+    blocks = _c(blocks, np.uint8)
+    row_stride = (k // 32) * 34 if row_stride is None else row_stride
+    out = np.empty((rows, k), np.float32)
+    _q8_f32(_ptr(blocks), rows, k, row_stride, _ptr(out))
+    return out
