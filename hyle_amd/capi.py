@@ -1,0 +1,87 @@
+"""ctypes view of include/hyle_hip.h (the C ABI of libhyle_hip.so).
+
+The structures mirror the header field for field.  The library is loaded once; if it has
+not been built the import fails loudly rather than falling back to any CPU path.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libhyle_hip.so")
+
+MAX_RANK, MAX_INPUTS, MAX_OUTPUTS, ABI_VERSION = 8, 4, 2, 1
+
+# hyle_hip_status
+OK, INVALID_ARGUMENT, RESOURCE_EXHAUSTED, FAILED_PRECONDITION = 0, 3, 8, 9
+OUT_OF_RANGE, UNIMPLEMENTED, INTERNAL, UNAVAILABLE = 11, 12, 13, 14
+
+
+class TensorDescC(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_uint8), ("rank", C.c_uint8), ("storage", C.c_uint8), ("block_axis", C.c_uint8),
+        ("elements_per_block", C.c_uint32), ("bytes_per_block", C.c_uint32), ("reserved", C.c_uint32),
+        ("dims", C.c_int64 * MAX_RANK), ("byte_strides", C.c_int64 * MAX_RANK),
+    ]
+
+
+class OpDescC(C.Structure):
+    _fields_ = [
+        ("abi_version", C.c_uint32), ("op", C.c_uint32), ("kind", C.c_uint32), ("kind2", C.c_uint32),
+        ("axis", C.c_int32), ("mask", C.c_uint32), ("accumulation", C.c_uint32),
+        ("keep_dimensions", C.c_uint32), ("epsilon", C.c_float), ("scale", C.c_float),
+        ("count", C.c_uint64), ("largest", C.c_uint32), ("input_count", C.c_uint32),
+        ("inputs", TensorDescC * MAX_INPUTS),
+    ]
+
+
+EXPORTS = {
+    # name: (restype, argtypes)
+    "hyle_hip_abi_version": (C.c_uint32, []),
+    "hyle_hip_last_error": (C.c_char_p, []),
+    "hyle_hip_status_name": (C.c_char_p, [C.c_int]),
+    "hyle_hip_context_create": (C.c_int, [C.c_int, C.POINTER(C.c_void_p)]),
+    "hyle_hip_context_destroy": (None, [C.c_void_p]),
+    "hyle_hip_context_compute_units": (C.c_int, [C.c_void_p]),
+    "hyle_hip_infer_outputs": (C.c_int, [C.POINTER(OpDescC), C.POINTER(TensorDescC), C.POINTER(C.c_uint32)]),
+    "hyle_hip_plan_create": (C.c_int, [C.c_void_p, C.POINTER(OpDescC), C.POINTER(TensorDescC), C.c_uint32,
+                                       C.POINTER(C.c_void_p)]),
+    "hyle_hip_plan_destroy": (None, [C.c_void_p]),
+    "hyle_hip_plan_workspace": (C.c_int, [C.c_void_p, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "hyle_hip_plan_outputs": (C.c_int, [C.c_void_p, C.POINTER(TensorDescC), C.POINTER(C.c_uint32)]),
+    "hyle_hip_plan_alias_support": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32]),
+    "hyle_hip_plan_dispatch_count": (C.c_uint32, [C.c_void_p]),
+    "hyle_hip_plan_route_name": (C.c_char_p, [C.c_void_p]),
+    "hyle_hip_plan_launch": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_uint32, C.POINTER(C.c_void_p),
+                                       C.c_uint32, C.c_void_p, C.c_size_t, C.c_void_p]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load libhyle_hip.so and bind every symbol include/hyle_hip.h declares."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: the gfx950 library has not been built "
+            "(run `python -m hyle_amd.build`); there is no CPU fallback")
+    lib = C.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in EXPORTS.items():
+        fn = getattr(lib, name)  # AttributeError here means the ABI and the header disagree
+        fn.restype, fn.argtypes = restype, argtypes
+    if lib.hyle_hip_abi_version() != ABI_VERSION:
+        raise RuntimeError("libhyle_hip.so ABI version differs from hyle_amd/capi.py")
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().hyle_hip_last_error().decode()
+
+
+def status_name(code: int) -> str:
+    return load().hyle_hip_status_name(code).decode()

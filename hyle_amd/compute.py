@@ -1,0 +1,460 @@
+"""Host-side mirror of the slice of `hyle::compute` that the tensor hot path uses, over the
+C ABI of libhyle_hip.so.
+
+Names, argument meaning and error behaviour follow the reference so that tests read like the
+reference's own provider tests:
+
+    context  = Context.create(device=0)                         # include/hyle/compute/device.h:124-140
+    prepared = prepare(context, Binary(BinaryKind.kAdd), a, b)  # include/hyle/compute/prepared_operation.h:313-317
+    run      = prepared.create_invocation(workspace)            # ...prepared_operation.h:144-291
+    run.submit(stream, inputs, outputs)                         # enqueue only; never blocks
+
+Errors surface as StatusError carrying the reference's StatusCode; `is_unimplemented()` is the
+clean decline a route table moves past (src/compute/operation.cc:1259-1266).  There is no CPU
+fallback anywhere in this module: without the built library it cannot be imported.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import enum
+from dataclasses import dataclass, field
+from typing import Optional, Sequence
+
+from . import capi
+
+
+# ---- status ---------------------------------------------------------------------------
+class StatusCode(enum.IntEnum):  # include/hyle/error/status.h:18-38
+    kOk = 0
+    kInvalidArgument = 3
+    kResourceExhausted = 8
+    kFailedPrecondition = 9
+    kOutOfRange = 11
+    kUnimplemented = 12
+    kInternal = 13
+    kUnavailable = 14
+
+
+class StatusError(RuntimeError):
+    def __init__(self, code: int, message: str):
+        super().__init__(f"{capi.status_name(code)}: {message}")
+        self.code = StatusCode(code)
+        self.message = message
+
+    def is_unimplemented(self) -> bool:
+        return self.code == StatusCode.kUnimplemented
+
+    def is_invalid_argument(self) -> bool:
+        return self.code == StatusCode.kInvalidArgument
+
+    def is_out_of_range(self) -> bool:
+        return self.code == StatusCode.kOutOfRange
+
+    def is_failed_precondition(self) -> bool:
+        return self.code == StatusCode.kFailedPrecondition
+
+
+def _check(code: int) -> None:
+    if code != capi.OK:
+        raise StatusError(code, capi.last_error())
+
+
+# ---- descriptors ------------------------------------------------------------------------
+class DataType(enum.IntEnum):  # include/hyle/compute/tensor_desc.h:17-34
+    kUnknown = 0
+    kBool = 1
+    kFloat16 = 4
+    kBFloat16 = 5
+    kFloat32 = 6
+    kInt8 = 8
+    kUInt8 = 9
+    kInt32 = 12
+
+
+_SIZES = {DataType.kBool: 1, DataType.kInt8: 1, DataType.kUInt8: 1, DataType.kFloat16: 2,
+          DataType.kBFloat16: 2, DataType.kFloat32: 4, DataType.kInt32: 4}
+
+
+def data_type_size(dtype: DataType) -> int:
+    return _SIZES.get(DataType(dtype), 0)
+
+
+@dataclass(frozen=True)
+class TensorDesc:
+    """Logical dims + byte strides (include/hyle/compute/tensor_desc.h:141-225)."""
+    data_type: DataType
+    dimensions: tuple
+    byte_strides: tuple
+    blocked: bool = False
+    block_axis: int = 0
+    elements_per_block: int = 1
+    bytes_per_block: int = 0
+
+    @staticmethod
+    def dense(data_type: DataType, dimensions: Sequence[int]) -> "TensorDesc":
+        dims = tuple(int(d) for d in dimensions)
+        if len(dims) > capi.MAX_RANK:
+            raise StatusError(capi.INVALID_ARGUMENT, "tensor shape rank exceeds kMaxTensorRank")
+        if any(d < 0 for d in dims):
+            raise StatusError(capi.INVALID_ARGUMENT, "tensor shape dimension is negative")
+        if 0 in dims:  # src/compute_ops/tensor_desc.cc:219-222
+            return TensorDesc(DataType(data_type), dims, tuple(0 for _ in dims))
+        strides, step = [], data_type_size(data_type)
+        for d in reversed(dims):
+            strides.append(step)
+            step *= d
+        return TensorDesc(DataType(data_type), dims, tuple(reversed(strides)))
+
+    @staticmethod
+    def strided_bytes(data_type: DataType, dimensions: Sequence[int], byte_strides: Sequence[int]) -> "TensorDesc":
+        if len(dimensions) != len(byte_strides):
+            raise StatusError(capi.INVALID_ARGUMENT, "stride count differs from rank")
+        return TensorDesc(DataType(data_type), tuple(int(d) for d in dimensions),
+                          tuple(int(s) for s in byte_strides))
+
+    @staticmethod
+    def gguf_q8_0_weight(logical_type: DataType, k: int, n: int, row_stride: Optional[int] = None) -> "TensorDesc":
+        """gguf_weight_description(kQ8_0, type, k, n): logical [K, N], physical rows of K/32
+        34-byte blocks (src/compute_ops/low_precision.cc:269-297)."""
+        if k <= 0 or n <= 0 or k % 32 != 0:
+            raise StatusError(capi.INVALID_ARGUMENT, "GGUF weight dimensions do not contain complete K blocks")
+        stride = (k // 32) * 34 if row_stride is None else int(row_stride)
+        return TensorDesc(DataType(logical_type), (k, n), (34, stride), blocked=True, block_axis=0,
+                          elements_per_block=32, bytes_per_block=34)
+
+    @property
+    def rank(self) -> int:
+        return len(self.dimensions)
+
+    def element_count(self) -> int:
+        n = 1
+        for d in self.dimensions:
+            n *= d
+        return n
+
+    def is_plain(self) -> bool:
+        return not self.blocked
+
+    def is_dense(self) -> bool:
+        return (not self.blocked) and self == TensorDesc.dense(self.data_type, self.dimensions)
+
+    def required_bytes(self) -> int:  # src/compute_ops/tensor_desc.cc:494-540
+        if 0 in self.dimensions:
+            return 0
+        last = 0
+        for axis, (d, s) in enumerate(zip(self.dimensions, self.byte_strides)):
+            units = d // self.elements_per_block if (self.blocked and axis == self.block_axis) else d
+            last += (units - 1) * s
+        return last + (self.bytes_per_block if self.blocked else data_type_size(self.data_type))
+
+    def to_c(self) -> capi.TensorDescC:
+        c = capi.TensorDescC()
+        c.dtype, c.rank = int(self.data_type), len(self.dimensions)
+        c.storage = 1 if self.blocked else 0
+        c.block_axis = self.block_axis
+        c.elements_per_block, c.bytes_per_block = self.elements_per_block, self.bytes_per_block
+        for i, (d, s) in enumerate(zip(self.dimensions, self.byte_strides)):
+            c.dims[i], c.byte_strides[i] = d, s
+        return c
+
+    @staticmethod
+    def from_c(c: capi.TensorDescC) -> "TensorDesc":
+        dims = tuple(int(c.dims[i]) for i in range(c.rank))
+        strides = tuple(int(c.byte_strides[i]) for i in range(c.rank))
+        if c.storage == 1:
+            return TensorDesc(DataType(c.dtype), dims, strides, True, c.block_axis,
+                              c.elements_per_block, c.bytes_per_block)
+        return TensorDesc(DataType(c.dtype), dims, strides)
+
+
+# ---- operations (include/hyle/compute/operation.h) -----------------------------------------
+class OperationKind(enum.IntEnum):
+    kUnary = 5
+    kBinary = 6
+    kReduce = 8
+    kRmsNorm = 9
+    kGatedActivation = 12
+    kSoftmax = 18
+    kTopK = 19
+    kBinaryChain = 0x100
+    kQ8_0DequantSumSquares = 0x101
+
+
+class UnaryKind(enum.IntEnum):
+    kAbs = 0
+    kNeg = 1
+    kExp = 2
+    kLog = 3
+    kSqrt = 4
+    kRsqrt = 5
+    kTanh = 6
+    kSigmoid = 7
+    kRelu = 8
+    kGelu = 9
+    kGeluTanh = 10
+    kSilu = 11
+    kSoftplus = 12
+
+
+class BinaryKind(enum.IntEnum):
+    kAdd = 0
+    kSubtract = 1
+    kMultiply = 2
+    kDivide = 3
+    kMinimum = 4
+    kMaximum = 5
+
+
+class ReductionKind(enum.IntEnum):
+    kSum = 0
+    kMean = 1
+    kMinimum = 2
+    kMaximum = 3
+
+
+class GatedActivationKind(enum.IntEnum):
+    kSilu = 0
+    kGelu = 1
+    kGeluTanh = 2
+
+
+class GatedInputKind(enum.IntEnum):
+    kPackedHalves = 0
+    kSeparate = 1
+
+
+class SoftmaxKind(enum.IntEnum):
+    kSoftmax = 0
+    kLogSoftmax = 1
+
+
+class MaskKind(enum.IntEnum):
+    kNone = 0
+    kAdditive = 1
+    kBoolean = 2
+
+
+@dataclass(frozen=True)
+class Unary:
+    kind: UnaryKind = UnaryKind.kAbs
+
+
+@dataclass(frozen=True)
+class Binary:
+    kind: BinaryKind = BinaryKind.kAdd
+
+
+@dataclass(frozen=True)
+class BinaryChain:
+    """out = (in0 first in1) second in2 with the intermediate rounded to storage."""
+    first: BinaryKind = BinaryKind.kAdd
+    second: BinaryKind = BinaryKind.kMultiply
+
+
+@dataclass(frozen=True)
+class Reduce:
+    kind: ReductionKind = ReductionKind.kSum
+    axis: int = -1
+    keep_dimensions: bool = False
+    accumulation_type: DataType = DataType.kUnknown
+
+
+@dataclass(frozen=True)
+class RmsNorm:
+    epsilon: float = 1.0e-5
+    accumulation_type: DataType = DataType.kFloat32
+
+
+@dataclass(frozen=True)
+class GatedActivation:
+    activation: GatedActivationKind = GatedActivationKind.kSilu
+    inputs: GatedInputKind = GatedInputKind.kPackedHalves
+
+
+@dataclass(frozen=True)
+class Softmax:
+    axis: int = -1
+    scale: float = 1.0
+    kind: SoftmaxKind = SoftmaxKind.kSoftmax
+    mask: MaskKind = MaskKind.kNone
+    accumulation_type: DataType = DataType.kFloat32
+
+
+@dataclass(frozen=True)
+class TopK:
+    count: int = 1
+    axis: int = -1
+    largest: bool = True
+    sorted: bool = True
+    stable: bool = True
+
+
+@dataclass(frozen=True)
+class Q8_0DequantSumSquares:
+    pass
+
+
+def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
+    c = capi.OpDescC()
+    c.abi_version = capi.ABI_VERSION
+    c.scale, c.largest = 1.0, 1
+    if isinstance(operation, Unary):
+        c.op, c.kind = OperationKind.kUnary, int(operation.kind)
+    elif isinstance(operation, Binary):
+        c.op, c.kind = OperationKind.kBinary, int(operation.kind)
+    elif isinstance(operation, BinaryChain):
+        c.op, c.kind, c.kind2 = OperationKind.kBinaryChain, int(operation.first), int(operation.second)
+    elif isinstance(operation, Reduce):
+        c.op, c.kind, c.axis = OperationKind.kReduce, int(operation.kind), operation.axis
+        c.keep_dimensions, c.accumulation = int(operation.keep_dimensions), int(operation.accumulation_type)
+    elif isinstance(operation, RmsNorm):
+        c.op, c.epsilon, c.accumulation = OperationKind.kRmsNorm, operation.epsilon, int(operation.accumulation_type)
+    elif isinstance(operation, GatedActivation):
+        c.op, c.kind, c.kind2 = OperationKind.kGatedActivation, int(operation.activation), int(operation.inputs)
+    elif isinstance(operation, Softmax):
+        c.op, c.axis, c.scale = OperationKind.kSoftmax, operation.axis, operation.scale
+        c.kind2, c.mask, c.accumulation = int(operation.kind), int(operation.mask), int(operation.accumulation_type)
+    elif isinstance(operation, TopK):
+        c.op, c.count, c.axis, c.largest = OperationKind.kTopK, operation.count, operation.axis, int(operation.largest)
+    elif isinstance(operation, Q8_0DequantSumSquares):
+        c.op = OperationKind.kQ8_0DequantSumSquares
+    else:
+        raise StatusError(capi.UNIMPLEMENTED, f"operation {type(operation).__name__} is not served by this provider")
+    if len(inputs) > capi.MAX_INPUTS:
+        raise StatusError(capi.INVALID_ARGUMENT, "operation input count does not match its typed contract")
+    c.input_count = len(inputs)
+    for i, desc in enumerate(inputs):
+        c.inputs[i] = desc.to_c()
+    return c
+
+
+def infer_output_descriptions(operation, inputs: Sequence[TensorDesc]) -> list:
+    """src/compute_ops/operation.cc:1214-1704 for the operations of this provider."""
+    req = _op_desc(operation, inputs)
+    outs = (capi.TensorDescC * capi.MAX_OUTPUTS)()
+    count = C.c_uint32(0)
+    _check(capi.load().hyle_hip_infer_outputs(C.byref(req), outs, C.byref(count)))
+    return [TensorDesc.from_c(outs[i]) for i in range(count.value)]
+
+
+# ---- context / prepare / submit ----------------------------------------------------------
+class Context:
+    """One HIP device bound to the provider (ProviderVTable::create_context)."""
+
+    def __init__(self, handle: Optional[int], device: int):
+        self._handle, self.device = handle, device
+
+    @staticmethod
+    def create(device: int = 0) -> "Context":
+        handle = C.c_void_p()
+        _check(capi.load().hyle_hip_context_create(device, C.byref(handle)))
+        return Context(handle.value, device)
+
+    @staticmethod
+    def planning_only() -> "Context":
+        """No device: plans can be built and inspected (cold path), never launched."""
+        capi.load()
+        return Context(None, -1)
+
+    @property
+    def compute_units(self) -> int:
+        return capi.load().hyle_hip_context_compute_units(self._handle)
+
+    def close(self) -> None:
+        if self._handle:
+            capi.load().hyle_hip_context_destroy(self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+@dataclass(frozen=True)
+class WorkspaceRequirement:
+    size: int = 0
+    alignment: int = 1
+
+
+class PreparedOperation:
+    def __init__(self, context: Context, handle: int, inputs: Sequence[TensorDesc]):
+        self._context, self._handle, self._inputs = context, handle, list(inputs)
+        lib = capi.load()
+        outs = (capi.TensorDescC * capi.MAX_OUTPUTS)()
+        count = C.c_uint32(0)
+        _check(lib.hyle_hip_plan_outputs(handle, outs, C.byref(count)))
+        self._outputs = [TensorDesc.from_c(outs[i]) for i in range(count.value)]
+        size, align = C.c_size_t(0), C.c_size_t(1)
+        _check(lib.hyle_hip_plan_workspace(handle, C.byref(size), C.byref(align)))
+        self._workspace = WorkspaceRequirement(size.value, align.value)
+
+    def output_descriptions(self) -> list:
+        return list(self._outputs)
+
+    def output_description(self) -> TensorDesc:
+        return self._outputs[0]
+
+    def workspace_requirement(self) -> WorkspaceRequirement:
+        return self._workspace
+
+    def alias_support(self, output_index: int, input_index: int) -> bool:
+        return bool(capi.load().hyle_hip_plan_alias_support(self._handle, output_index, input_index))
+
+    def dispatch_count(self) -> int:
+        return capi.load().hyle_hip_plan_dispatch_count(self._handle)
+
+    def route_name(self) -> str:
+        return capi.load().hyle_hip_plan_route_name(self._handle).decode()
+
+    def create_invocation(self, workspace: int = 0, workspace_size: int = 0) -> "OperationInvocation":
+        """`workspace` is a device address the caller owns for the invocation's lifetime."""
+        if self._workspace.size and (not workspace or workspace_size < self._workspace.size):
+            raise StatusError(capi.INVALID_ARGUMENT, "workspace is smaller than the plan requires")
+        return OperationInvocation(self, workspace, workspace_size)
+
+    def close(self) -> None:
+        if self._handle:
+            capi.load().hyle_hip_plan_destroy(self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+class OperationInvocation:
+    def __init__(self, prepared: PreparedOperation, workspace: int, workspace_size: int):
+        self._prepared, self._workspace, self._workspace_size = prepared, workspace, workspace_size
+        self._in = (C.c_void_p * capi.MAX_INPUTS)()
+        self._out = (C.c_void_p * capi.MAX_OUTPUTS)()
+
+    def submit(self, stream: int, inputs: Sequence[int], outputs: Sequence[int]) -> None:
+        """Enqueue on HIP stream handle `stream` (0 = default stream) and return at once.
+        `inputs` / `outputs` are device addresses."""
+        for i, p in enumerate(inputs):
+            self._in[i] = p
+        for i, p in enumerate(outputs):
+            self._out[i] = p
+        _check(capi.load().hyle_hip_plan_launch(
+            self._prepared._handle, self._in, len(inputs), self._out, len(outputs),
+            self._workspace, self._workspace_size, stream))
+
+
+def prepare(context: Context, operation, *inputs: TensorDesc,
+            outputs: Optional[Sequence[TensorDesc]] = None) -> PreparedOperation:
+    """hyle::compute::prepare(context, operation, input descriptors...)."""
+    req = _op_desc(operation, inputs)
+    handle = C.c_void_p()
+    if outputs is None:
+        outs, count = None, 0
+    else:
+        outs = (capi.TensorDescC * capi.MAX_OUTPUTS)()
+        for i, d in enumerate(outputs):
+            outs[i] = d.to_c()
+        count = len(outputs)
+    _check(capi.load().hyle_hip_plan_create(context._handle, C.byref(req), outs, count, C.byref(handle)))
+    return PreparedOperation(context, handle.value, inputs)

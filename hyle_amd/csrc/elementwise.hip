@@ -1,0 +1,412 @@
+// elementwise.hip -- Binary (broadcast), BinaryChain, Unary SiLU and SwiGLU for
+// gfx950.  Pure streaming kernels: 128-bit global loads and stores, several
+// independent vectors in flight per lane, f32 arithmetic, one rounding per
+// stored value.
+//
+// Semantics follow the reference's CPU native provider:
+//   Binary        src/compute_provider_native/elementwise.cc:102-169 (decode ->
+//                 f32 op -> one RN-even store), broadcast offsets of
+//                 src/compute_provider_native/native_plan.h:152-174
+//   SiLU / SwiGLU src/simd/math/activations.cc:21-25,44-47,114-122
+#include "device_common.h"
+#include "kernels.h"
+
+namespace hyle_hip {
+namespace {
+
+constexpr int kUnroll = 4;
+
+// ---- scalar semantics --------------------------------------------------------
+enum : int { kAdd = 0, kSub = 1, kMul = 2, kDiv = 3, kMin = 4, kMax = 5 };
+
+template <int kKind> __device__ __forceinline__ float binary_apply(float x, float y) {
+  if constexpr (kKind == kAdd) return x + y;
+  else if constexpr (kKind == kSub) return x - y;
+  else if constexpr (kKind == kMul) return x * y;
+  else if constexpr (kKind == kDiv) return x / y;
+  else if constexpr (kKind == kMin) return fminf(x, y);
+  else return fmaxf(x, y);
+}
+__device__ __forceinline__ float binary_apply_rt(int kind, float x, float y) {
+  switch (kind) {
+    case kAdd: return x + y;
+    case kSub: return x - y;
+    case kMul: return x * y;
+    case kDiv: return x / y;
+    case kMin: return fminf(x, y);
+    default: return fmaxf(x, y);
+  }
+}
+
+// Exact form, operation for operation the reference's scalar floor
+// (src/simd/math/activations.cc:21-25,44-47): used for f32 storage.
+__device__ __forceinline__ float silu_exact(float x) {
+  if (x == -INFINITY) return 0.0f;
+  float s;
+  if (x != x) {
+    s = x;
+  } else {
+    const float e = expf(-fabsf(x));
+    s = (x < 0.0f ? e : 1.0f) / (1.0f + e);
+  }
+  return x * s;
+}
+
+// Narrow storage keeps 8 (bf16) or 11 (f16) significand bits, so the sigmoid is
+// evaluated as 1 / (1 + exp(-x)) with the hardware exp2 and reciprocal (about
+// 1e-6 relative).  exp(-x) is carried scaled by 2^-32 so that it stays finite
+// down to x = -110, where silu(x) itself underflows every storage type:
+//   sigmoid = 2^-32 / (exp(-x) * 2^-32 + 2^-32).
+// The final product uses the "zero wins" multiply so that silu(-inf) is +0 as
+// in the reference rather than -inf * 0.
+__device__ __forceinline__ float silu_fast(float x) {
+  constexpr float kNegLog2e = -1.44269504088896340736f;
+  constexpr float kTwoM32 = 2.3283064365386963e-10f;
+  const float scaled = __builtin_amdgcn_exp2f(__builtin_fmaf(x, kNegLog2e, -32.0f));
+  const float sigmoid = __builtin_amdgcn_rcpf(scaled + kTwoM32) * kTwoM32;
+  return mul_zero_wins(x, sigmoid);
+}
+
+template <class T> __device__ __forceinline__ float silu_for(float x) {
+  if constexpr (Traits<T>::kSize == 4) return silu_exact(x);
+  else return silu_fast(x);
+}
+
+template <int kKind> struct BinaryFn {
+  static constexpr int kInputs = 2;
+  template <class T> __device__ __forceinline__ float operator()(T, float x, float y, float) const {
+    return binary_apply<kKind>(x, y);
+  }
+};
+template <int kKind0, int kKind1> struct ChainFn {
+  static constexpr int kInputs = 3;
+  template <class T> __device__ __forceinline__ float operator()(T, float x, float y, float z) const {
+    return binary_apply<kKind1>(Traits<T>::round(binary_apply<kKind0>(x, y)), z);
+  }
+};
+struct SiluFn {
+  static constexpr int kInputs = 1;
+  template <class T> __device__ __forceinline__ float operator()(T, float x, float, float) const {
+    return silu_for<T>(x);
+  }
+};
+struct SwigluFn {
+  static constexpr int kInputs = 2;
+  template <class T> __device__ __forceinline__ float operator()(T, float g, float u, float) const {
+    return silu_for<T>(g) * u;
+  }
+};
+// One functor for the slow routes: the operation is a launch-uniform value.
+struct RuntimeFn {
+  EwOp op;
+  int kind0, kind1;
+  template <class T> __device__ __forceinline__ float operator()(T, float x, float y, float z) const {
+    switch (op) {
+      case EwOp::kBinary: return binary_apply_rt(kind0, x, y);
+      case EwOp::kChain:
+        return binary_apply_rt(kind1, Traits<T>::round(binary_apply_rt(kind0, x, y)), z);
+      case EwOp::kSilu: return silu_for<T>(x);
+      default: return silu_for<T>(x) * y;
+    }
+  }
+};
+
+// ---- flat vectorised kernel ----------------------------------------------------
+// Operand addressing inside the flat kernels.  `period` is in elements: 0 = the
+// operand is as long as the output, 1 = one value for every element, otherwise
+// the operand repeats every `period` elements (a dense broadcast suffix).  The
+// vectorised kernel needs period % vector width == 0 (`period_vec`).  Element
+// counts are at most INT32_MAX, so 32-bit indices suffice.
+struct Operand {
+  const void *base;
+  uint32_t period;
+  uint32_t period_vec;
+};
+
+template <class T>
+__device__ __forceinline__ void fetch(const Operand &op, uint32_t vec, float (&v)[Traits<T>::kVec]) {
+  constexpr int kVec = Traits<T>::kVec;
+  if (op.period == 0) {
+    Traits<T>::unpack(load16_stream(op.base, vec), v);
+  } else if (op.period == 1) {
+    const float s = Traits<T>::load(op.base, 0);
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) v[j] = s;
+  } else {
+    Traits<T>::unpack(load16(op.base, vec % op.period_vec), v);
+  }
+}
+
+template <class T>
+__device__ __forceinline__ float fetch1(const Operand &op, uint32_t e) {
+  return Traits<T>::load(op.base, op.period ? e % op.period : e);
+}
+
+template <class T, class Fn>
+__global__ __launch_bounds__(kBlockThreads) void ew_flat_vec(Operand a, Operand b, Operand c,
+                                                             void *out, uint32_t vectors,
+                                                             uint32_t elements, Fn fn) {
+  constexpr int kVec = Traits<T>::kVec;
+  const uint32_t first = blockIdx.x * (kUnroll * kBlockThreads) + threadIdx.x;
+  float x[kUnroll][kVec], y[kUnroll][kVec], z[kUnroll][kVec];
+#pragma unroll
+  for (int k = 0; k < kUnroll; ++k) {
+    const uint32_t vec = first + k * kBlockThreads;
+    if (vec < vectors) {
+      fetch<T>(a, vec, x[k]);
+      if constexpr (Fn::kInputs > 1) fetch<T>(b, vec, y[k]);
+      if constexpr (Fn::kInputs > 2) fetch<T>(c, vec, z[k]);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kUnroll; ++k) {
+    const uint32_t vec = first + k * kBlockThreads;
+    if (vec < vectors) {
+      float r[kVec];
+#pragma unroll
+      for (int j = 0; j < kVec; ++j)
+        r[j] = fn(T{}, x[k][j], Fn::kInputs > 1 ? y[k][j] : 0.0f, Fn::kInputs > 2 ? z[k][j] : 0.0f);
+      store16_stream(out, vec, Traits<T>::pack(r));
+    }
+  }
+  // elements past the last whole vector
+  if (blockIdx.x == 0) {
+    const uint32_t e = vectors * kVec + threadIdx.x;
+    if (e < elements) {
+      const float xs = fetch1<T>(a, e);
+      const float ys = Fn::kInputs > 1 ? fetch1<T>(b, e) : 0.0f;
+      const float zs = Fn::kInputs > 2 ? fetch1<T>(c, e) : 0.0f;
+      Traits<T>::store(out, e, fn(T{}, xs, ys, zs));
+    }
+  }
+}
+
+// Same addressing, one element per lane: used when a pointer is not 16-byte
+// aligned or a period is not a whole number of vectors.
+template <class T>
+__global__ __launch_bounds__(kBlockThreads) void ew_flat_scalar(Operand a, Operand b, Operand c,
+                                                                void *out, uint32_t elements,
+                                                                int inputs, RuntimeFn fn) {
+  const uint32_t e = blockIdx.x * kBlockThreads + threadIdx.x;
+  if (e >= elements) return;
+  const float xs = fetch1<T>(a, e);
+  const float ys = inputs > 1 ? fetch1<T>(b, e) : 0.0f;
+  const float zs = inputs > 2 ? fetch1<T>(c, e) : 0.0f;
+  Traits<T>::store(out, e, fn(T{}, xs, ys, zs));
+}
+
+// ---- general strided kernel ------------------------------------------------------
+struct GeneralLayout {
+  int32_t rank;
+  uint32_t dims[kMaxRank];
+  int64_t strides[3][kMaxRank];
+};
+
+template <class T>
+__global__ __launch_bounds__(kBlockThreads) void ew_general(const char *a, const char *b,
+                                                            const char *c, void *out,
+                                                            uint64_t elements, int inputs,
+                                                            GeneralLayout layout, RuntimeFn fn) {
+  const uint64_t e = (uint64_t)blockIdx.x * kBlockThreads + threadIdx.x;
+  if (e >= elements) return;
+  uint64_t rest = e;
+  int64_t off[3] = {0, 0, 0};
+  for (int axis = layout.rank - 1; axis >= 0; --axis) {
+    const uint32_t extent = layout.dims[axis];
+    const uint64_t coordinate = rest % extent;
+    rest /= extent;
+    off[0] += (int64_t)coordinate * layout.strides[0][axis];
+    off[1] += (int64_t)coordinate * layout.strides[1][axis];
+    off[2] += (int64_t)coordinate * layout.strides[2][axis];
+  }
+  const float xs = Traits<T>::load(a + off[0], 0);
+  const float ys = inputs > 1 ? Traits<T>::load(b + off[1], 0) : 0.0f;
+  const float zs = inputs > 2 ? Traits<T>::load(c + off[2], 0) : 0.0f;
+  Traits<T>::store(out, e, fn(T{}, xs, ys, zs));
+}
+
+// ---- packed SwiGLU -----------------------------------------------------------------
+template <class T>
+__global__ __launch_bounds__(kBlockThreads) void swiglu_packed_vec(const void *packed, void *out,
+                                                                   uint32_t row_vectors,
+                                                                   uint64_t vectors) {
+  constexpr int kVec = Traits<T>::kVec;
+  const uint64_t first = (uint64_t)blockIdx.x * (kUnroll * kBlockThreads) + threadIdx.x;
+  float g[kUnroll][kVec], u[kUnroll][kVec];
+#pragma unroll
+  for (int k = 0; k < kUnroll; ++k) {
+    const uint64_t vec = first + (uint64_t)k * kBlockThreads;
+    if (vec < vectors) {
+      const uint64_t row = vec / row_vectors, col = vec % row_vectors;
+      Traits<T>::unpack(load16_stream(packed, row * 2 * row_vectors + col), g[k]);
+      Traits<T>::unpack(load16_stream(packed, row * 2 * row_vectors + row_vectors + col), u[k]);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kUnroll; ++k) {
+    const uint64_t vec = first + (uint64_t)k * kBlockThreads;
+    if (vec < vectors) {
+      float r[kVec];
+#pragma unroll
+      for (int j = 0; j < kVec; ++j) r[j] = silu_for<T>(g[k][j]) * u[k][j];
+      store16_stream(out, vec, Traits<T>::pack(r));
+    }
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(kBlockThreads) void swiglu_packed_scalar(const void *packed, void *out,
+                                                                      uint32_t hidden,
+                                                                      uint64_t elements) {
+  const uint64_t e = (uint64_t)blockIdx.x * kBlockThreads + threadIdx.x;
+  if (e >= elements) return;
+  const uint64_t row = e / hidden, col = e % hidden;
+  const float g = Traits<T>::load(packed, row * 2 * hidden + col);
+  const float u = Traits<T>::load(packed, row * 2 * hidden + hidden + col);
+  Traits<T>::store(out, e, silu_for<T>(g) * u);
+}
+
+// ---- host dispatch -------------------------------------------------------------------
+Operand make_operand(const void *base, uint32_t period, int vec) {
+  Operand op;
+  op.base = base;
+  op.period = period;
+  op.period_vec = (period > 1 && period % vec == 0) ? period / vec : 0;
+  return op;
+}
+
+template <class T, class Fn>
+hipError_t run_vec(const EwFlat &p, Operand a, Operand b, Operand c, void *out, hipStream_t s) {
+  constexpr int kVec = Traits<T>::kVec;
+  const uint64_t vectors = p.elements / kVec;
+  const uint64_t per_block = (uint64_t)kUnroll * kBlockThreads;
+  uint64_t blocks = (vectors + per_block - 1) / per_block;
+  if (blocks == 0) blocks = 1;  // the tail still needs block 0
+  hipLaunchKernelGGL((ew_flat_vec<T, Fn>), dim3((uint32_t)blocks), dim3(kBlockThreads), 0, s, a, b,
+                     c, out, (uint32_t)vectors, (uint32_t)p.elements, Fn{});
+  return hipGetLastError();
+}
+
+template <class T, int kKind0>
+hipError_t run_chain(const EwFlat &p, Operand a, Operand b, Operand c, void *out, hipStream_t s) {
+  switch (p.kind1) {
+    case kAdd: return run_vec<T, ChainFn<kKind0, kAdd>>(p, a, b, c, out, s);
+    case kSub: return run_vec<T, ChainFn<kKind0, kSub>>(p, a, b, c, out, s);
+    case kMul: return run_vec<T, ChainFn<kKind0, kMul>>(p, a, b, c, out, s);
+    default: return hipErrorInvalidValue;
+  }
+}
+
+template <class T>
+hipError_t run_flat(const EwFlat &p, const void *a, const void *b, const void *c, void *out,
+                    bool vectorised, hipStream_t s) {
+  constexpr int kVec = Traits<T>::kVec;
+  const Operand oa = make_operand(a, p.period[0], kVec);
+  const Operand ob = make_operand(b, p.period[1], kVec);
+  const Operand oc = make_operand(c, p.period[2], kVec);
+  const bool chain_fast = p.op != EwOp::kChain || (p.kind0 <= kMul && p.kind1 <= kMul);
+  bool whole_vectors = true;
+  for (int i = 0; i < p.inputs; ++i)
+    whole_vectors = whole_vectors && (p.period[i] <= 1 || p.period[i] % kVec == 0);
+  if (!vectorised || !chain_fast || !whole_vectors) {
+    const uint64_t blocks = (p.elements + kBlockThreads - 1) / kBlockThreads;
+    hipLaunchKernelGGL((ew_flat_scalar<T>), dim3((uint32_t)blocks), dim3(kBlockThreads), 0, s, oa,
+                       ob, oc, out, (uint32_t)p.elements, (int)p.inputs,
+                       RuntimeFn{p.op, (int)p.kind0, (int)p.kind1});
+    return hipGetLastError();
+  }
+  switch (p.op) {
+    case EwOp::kBinary:
+      switch (p.kind0) {
+        case kAdd: return run_vec<T, BinaryFn<kAdd>>(p, oa, ob, oc, out, s);
+        case kSub: return run_vec<T, BinaryFn<kSub>>(p, oa, ob, oc, out, s);
+        case kMul: return run_vec<T, BinaryFn<kMul>>(p, oa, ob, oc, out, s);
+        case kDiv: return run_vec<T, BinaryFn<kDiv>>(p, oa, ob, oc, out, s);
+        case kMin: return run_vec<T, BinaryFn<kMin>>(p, oa, ob, oc, out, s);
+        case kMax: return run_vec<T, BinaryFn<kMax>>(p, oa, ob, oc, out, s);
+        default: return hipErrorInvalidValue;
+      }
+    case EwOp::kChain:
+      switch (p.kind0) {
+        case kAdd: return run_chain<T, kAdd>(p, oa, ob, oc, out, s);
+        case kSub: return run_chain<T, kSub>(p, oa, ob, oc, out, s);
+        case kMul: return run_chain<T, kMul>(p, oa, ob, oc, out, s);
+        default: return hipErrorInvalidValue;
+      }
+    case EwOp::kSilu: return run_vec<T, SiluFn>(p, oa, ob, oc, out, s);
+    case EwOp::kSwiglu: return run_vec<T, SwigluFn>(p, oa, ob, oc, out, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+template <class T>
+hipError_t run_general(const EwGeneral &p, const void *a, const void *b, const void *c, void *out,
+                       hipStream_t s) {
+  GeneralLayout layout;
+  layout.rank = p.rank;
+  for (int i = 0; i < kMaxRank; ++i) {
+    layout.dims[i] = p.dims[i];
+    for (int k = 0; k < 3; ++k) layout.strides[k][i] = p.strides[k][i];
+  }
+  const uint64_t blocks = (p.elements + kBlockThreads - 1) / kBlockThreads;
+  hipLaunchKernelGGL((ew_general<T>), dim3((uint32_t)blocks), dim3(kBlockThreads), 0, s,
+                     static_cast<const char *>(a), static_cast<const char *>(b),
+                     static_cast<const char *>(c), out, p.elements, (int)p.inputs, layout,
+                     RuntimeFn{p.op, (int)p.kind0, (int)p.kind1});
+  return hipGetLastError();
+}
+
+template <class T>
+hipError_t run_packed(const EwPacked &p, const void *packed, void *out, bool vectorised,
+                      hipStream_t s) {
+  constexpr int kVec = Traits<T>::kVec;
+  const uint64_t elements = p.rows * p.hidden;
+  if (vectorised && p.hidden % kVec == 0) {
+    const uint64_t vectors = elements / kVec;
+    const uint64_t per_block = (uint64_t)kUnroll * kBlockThreads;
+    hipLaunchKernelGGL((swiglu_packed_vec<T>), dim3((uint32_t)((vectors + per_block - 1) / per_block)),
+                       dim3(kBlockThreads), 0, s, packed, out, p.hidden / kVec, vectors);
+  } else {
+    hipLaunchKernelGGL((swiglu_packed_scalar<T>),
+                       dim3((uint32_t)((elements + kBlockThreads - 1) / kBlockThreads)),
+                       dim3(kBlockThreads), 0, s, packed, out, p.hidden, elements);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_ew_flat(Elem type, const EwFlat &p, const void *a, const void *b, const void *c,
+                          void *out, bool vectorised, hipStream_t stream) {
+  if (p.elements == 0) return hipSuccess;
+  switch (type) {
+    case Elem::kF32: return run_flat<F32>(p, a, b, c, out, vectorised, stream);
+    case Elem::kF16: return run_flat<F16>(p, a, b, c, out, vectorised, stream);
+    case Elem::kBF16: return run_flat<BF16>(p, a, b, c, out, vectorised, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_ew_general(Elem type, const EwGeneral &p, const void *a, const void *b,
+                             const void *c, void *out, hipStream_t stream) {
+  if (p.elements == 0) return hipSuccess;
+  switch (type) {
+    case Elem::kF32: return run_general<F32>(p, a, b, c, out, stream);
+    case Elem::kF16: return run_general<F16>(p, a, b, c, out, stream);
+    case Elem::kBF16: return run_general<BF16>(p, a, b, c, out, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_swiglu_packed(Elem type, const EwPacked &p, const void *packed, void *out,
+                                bool vectorised, hipStream_t stream) {
+  if (p.rows == 0 || p.hidden == 0) return hipSuccess;
+  switch (type) {
+    case Elem::kF32: return run_packed<F32>(p, packed, out, vectorised, stream);
+    case Elem::kF16: return run_packed<F16>(p, packed, out, vectorised, stream);
+    case Elem::kBF16: return run_packed<BF16>(p, packed, out, vectorised, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace hyle_hip

@@ -1,0 +1,135 @@
+// kernels.h -- host-callable launchers of the gfx950 kernels.  Each launcher
+// only enqueues on the given stream; shapes were validated when the plan was
+// built, pointer alignment is checked by the caller at launch time.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace hyle_hip {
+
+enum class Elem : uint8_t { kF32 = 0, kF16 = 1, kBF16 = 2 };
+
+inline int elem_size(Elem e) { return e == Elem::kF32 ? 4 : 2; }
+inline int elem_vec(Elem e) { return e == Elem::kF32 ? 4 : 8; }
+
+constexpr int kMaxRank = 8;
+
+// ---- elementwise ------------------------------------------------------------
+enum class EwOp : uint8_t { kBinary = 0, kChain, kSilu, kSwiglu };
+
+// How one input is addressed by the flat (vectorised) kernel: every `period`
+// elements the operand repeats (0 = never, the operand is as large as the
+// output); period 1 is a scalar splat.
+struct EwFlat {
+  uint64_t elements = 0;      // output elements
+  uint32_t period[3] = {0, 0, 0};
+  EwOp op = EwOp::kBinary;
+  uint8_t kind0 = 0, kind1 = 0;
+  uint8_t inputs = 2;
+};
+
+// Fully general addressing: dense output of `rank` dims, per-input byte strides
+// (0 on broadcast axes).
+struct EwGeneral {
+  uint64_t elements = 0;
+  int32_t rank = 0;
+  uint32_t dims[kMaxRank] = {};
+  int64_t strides[3][kMaxRank] = {};
+  EwOp op = EwOp::kBinary;
+  uint8_t kind0 = 0, kind1 = 0;
+  uint8_t inputs = 2;
+};
+
+// Packed SwiGLU: rows of [gate | value], each `hidden` wide.
+struct EwPacked {
+  uint64_t rows = 0;
+  uint32_t hidden = 0;
+};
+
+hipError_t launch_ew_flat(Elem type, const EwFlat &p, const void *a, const void *b, const void *c,
+                          void *out, bool vectorised, hipStream_t stream);
+hipError_t launch_ew_general(Elem type, const EwGeneral &p, const void *a, const void *b,
+                             const void *c, void *out, hipStream_t stream);
+hipError_t launch_swiglu_packed(Elem type, const EwPacked &p, const void *packed, void *out,
+                                bool vectorised, hipStream_t stream);
+
+// ---- row kernels ------------------------------------------------------------
+struct RowShape {
+  uint64_t rows = 0;
+  uint32_t width = 0;
+};
+
+struct NormParams {
+  RowShape shape;
+  float epsilon = 0;
+  bool has_weight = false;
+  bool weight_f32 = false;  // f32 weight with a narrow input
+};
+hipError_t launch_rms_norm(Elem type, const NormParams &p, const void *x, const void *w, void *y,
+                           bool vectorised, hipStream_t stream);
+
+// Softmax over the last axis of a dense [rows, width] tensor.  The mask row of
+// logical row r starts at mask + sum_k coord_k(r) * outer_stride[k]; inside the
+// row the mask advances by `mask_inner_stride` bytes per column (0 = one value
+// for the whole row).
+struct SoftmaxParams {
+  RowShape shape;
+  float scale = 1.0f;
+  uint8_t mask_kind = 0;  // HYLE_HIP_MASK_*
+  bool log = false;
+  int32_t outer_rank = 0;
+  uint32_t outer_dims[kMaxRank] = {};
+  int64_t mask_outer_strides[kMaxRank] = {};
+  int64_t mask_inner_stride = 0;
+  // rows r and r + mask_period share one mask row (0 = no such structure)
+  uint64_t mask_period = 0;
+};
+hipError_t launch_softmax(Elem type, const SoftmaxParams &p, const void *x, const void *mask,
+                          void *y, bool vectorised, int compute_units, hipStream_t stream);
+
+// Softmax along any axis of a strided tensor: rows = outer * inner.
+struct SoftmaxGeneralParams {
+  uint64_t outer = 0, inner = 0;
+  uint32_t width = 0;
+  float scale = 1.0f;
+  uint8_t mask_kind = 0;
+  bool log = false;
+  int32_t rank = 0;
+  int32_t axis = 0;
+  uint32_t dims[kMaxRank] = {};
+  int64_t in_strides[kMaxRank] = {};
+  int64_t mask_strides[kMaxRank] = {};
+};
+hipError_t launch_softmax_general(Elem type, const SoftmaxGeneralParams &p, const void *x,
+                                  const void *mask, void *y, hipStream_t stream);
+
+struct ReduceParams {
+  RowShape shape;
+  uint8_t kind = 0;  // HYLE_HIP_REDUCE_*
+};
+hipError_t launch_reduce_rows(Elem type, const ReduceParams &p, const void *x, void *y,
+                              bool vectorised, hipStream_t stream);
+
+// TopK(count = 1): two dispatches, per-tile candidates in the workspace.
+struct ArgmaxParams {
+  RowShape shape;
+  uint32_t tiles = 0;        // tiles per row
+  uint32_t tile_elems = 0;   // elements per tile (multiple of 1024)
+};
+void argmax_plan(uint64_t rows, uint32_t width, int compute_units, ArgmaxParams *p);
+size_t argmax_workspace_bytes(const ArgmaxParams &p);
+hipError_t launch_argmax(Elem type, const ArgmaxParams &p, const void *x, void *values,
+                         int32_t *indices, void *workspace, bool vectorised, hipStream_t stream);
+
+// Q8_0 rows of k/32 blocks {f16 d; int8 qs[32]} -> bf16 [rows, k] + f32 sumsq[rows].
+struct Q8Params {
+  uint64_t rows = 0;
+  uint32_t k = 0;
+  uint64_t row_stride = 0;  // bytes between physical rows
+};
+hipError_t launch_q8_0_dequant(const Q8Params &p, const void *blocks, void *out, float *sumsq,
+                               bool vectorised, hipStream_t stream);
+
+}  // namespace hyle_hip

@@ -1,0 +1,984 @@
+// plan.hip -- the C ABI of include/hyle_hip.h: operator schema (output inference),
+// admission of a request into a kernel route (the reference's propose + prepare),
+// and the allocation-free launch (shared_submit).  Host code only; the kernels
+// live in the sibling .hip files behind kernels.h.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <limits>
+#include <new>
+
+#include "../../include/hyle_hip.h"
+#include "kernels.h"
+
+using namespace hyle_hip;
+
+// ---------------------------------------------------------------------------------
+// errors
+// ---------------------------------------------------------------------------------
+namespace {
+
+thread_local char g_error[320] = "";
+
+hyle_hip_status fail(hyle_hip_status status, const char *format, ...) {
+  va_list args;
+  va_start(args, format);
+  vsnprintf(g_error, sizeof g_error, format, args);
+  va_end(args);
+  return status;
+}
+
+hyle_hip_status hip_fail(hipError_t error, const char *what) {
+  return fail(HYLE_HIP_INTERNAL, "%s: %s", what, hipGetErrorString(error));
+}
+
+// ---------------------------------------------------------------------------------
+// descriptors
+// ---------------------------------------------------------------------------------
+typedef hyle_hip_tensor_desc Desc;
+
+size_t dtype_size(uint8_t dtype) {
+  switch (dtype) {
+    case HYLE_HIP_DTYPE_BOOL:
+    case HYLE_HIP_DTYPE_I8:
+    case HYLE_HIP_DTYPE_U8: return 1;
+    case HYLE_HIP_DTYPE_F16:
+    case HYLE_HIP_DTYPE_BF16: return 2;
+    case HYLE_HIP_DTYPE_F32:
+    case HYLE_HIP_DTYPE_I32: return 4;
+    default: return 0;
+  }
+}
+bool is_floating(uint8_t dtype) {
+  return dtype == HYLE_HIP_DTYPE_F16 || dtype == HYLE_HIP_DTYPE_BF16 || dtype == HYLE_HIP_DTYPE_F32;
+}
+bool is_numeric(uint8_t dtype) {
+  return is_floating(dtype) || dtype == HYLE_HIP_DTYPE_I8 || dtype == HYLE_HIP_DTYPE_U8 ||
+         dtype == HYLE_HIP_DTYPE_I32;
+}
+bool to_elem(uint8_t dtype, Elem *out) {
+  switch (dtype) {
+    case HYLE_HIP_DTYPE_F32: *out = Elem::kF32; return true;
+    case HYLE_HIP_DTYPE_F16: *out = Elem::kF16; return true;
+    case HYLE_HIP_DTYPE_BF16: *out = Elem::kBF16; return true;
+    default: return false;
+  }
+}
+
+bool has_zero_extent(const Desc &d) {
+  for (int i = 0; i < d.rank; ++i)
+    if (d.dims[i] == 0) return true;
+  return false;
+}
+
+// element count with overflow check; false on overflow
+bool element_count(const Desc &d, uint64_t *count) {
+  if (has_zero_extent(d)) {
+    *count = 0;
+    return true;
+  }
+  uint64_t n = 1;
+  for (int i = 0; i < d.rank; ++i) {
+    const uint64_t e = (uint64_t)d.dims[i];
+    if (e != 0 && n > std::numeric_limits<uint64_t>::max() / e) return false;
+    n *= e;
+  }
+  *count = n;
+  return true;
+}
+
+// TensorDesc::dense of the reference (src/compute_ops/tensor_desc.cc:211-243): canonical
+// row-major byte strides; a shape with a zero extent gets all-zero strides.
+hyle_hip_status make_dense(uint8_t dtype, const int64_t *dims, int rank, Desc *out) {
+  if (rank < 0 || rank > HYLE_HIP_MAX_RANK)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "tensor shape rank exceeds kMaxTensorRank");
+  if (dtype_size(dtype) == 0) return fail(HYLE_HIP_INVALID_ARGUMENT, "tensor data type is invalid");
+  std::memset(out, 0, sizeof *out);
+  out->dtype = dtype;
+  out->rank = (uint8_t)rank;
+  out->storage = HYLE_HIP_STORAGE_PLAIN;
+  out->elements_per_block = 1;
+  bool zero = false;
+  for (int i = 0; i < rank; ++i) {
+    if (dims[i] < 0) return fail(HYLE_HIP_INVALID_ARGUMENT, "tensor shape dimension is negative");
+    out->dims[i] = dims[i];
+    zero = zero || dims[i] == 0;
+  }
+  if (zero) return HYLE_HIP_OK;
+  uint64_t stride = dtype_size(dtype);
+  for (int i = rank - 1; i >= 0; --i) {
+    if (stride > (uint64_t)std::numeric_limits<int64_t>::max())
+      return fail(HYLE_HIP_OUT_OF_RANGE, "dense tensor byte stride overflows");
+    out->byte_strides[i] = (int64_t)stride;
+    const uint64_t e = (uint64_t)dims[i];
+    if (e != 0 && stride > std::numeric_limits<uint64_t>::max() / e)
+      return fail(HYLE_HIP_OUT_OF_RANGE, "dense tensor byte stride overflows size_t");
+    stride *= e;
+  }
+  return HYLE_HIP_OK;
+}
+
+bool same_desc(const Desc &a, const Desc &b) {
+  if (a.dtype != b.dtype || a.rank != b.rank || a.storage != b.storage) return false;
+  if (a.storage == HYLE_HIP_STORAGE_BLOCKED &&
+      (a.block_axis != b.block_axis || a.elements_per_block != b.elements_per_block ||
+       a.bytes_per_block != b.bytes_per_block))
+    return false;
+  for (int i = 0; i < a.rank; ++i)
+    if (a.dims[i] != b.dims[i] || a.byte_strides[i] != b.byte_strides[i]) return false;
+  return true;
+}
+
+bool is_plain(const Desc &d) { return d.storage == HYLE_HIP_STORAGE_PLAIN; }
+
+// TensorDesc::is_dense (src/compute_ops/tensor_desc.cc:542-552): exactly the canonical strides.
+bool is_dense(const Desc &d) {
+  if (!is_plain(d)) return false;
+  Desc canonical;
+  if (make_dense(d.dtype, d.dims, d.rank, &canonical) != HYLE_HIP_OK) return false;
+  return same_desc(canonical, d);
+}
+
+// validate_description of the reference: known type, bounded rank, non-negative extents and
+// strides (negative strides are outside the public contract, tensor_desc.h:136-139).
+hyle_hip_status validate_desc(const Desc &d, const char *what) {
+  if (d.rank > HYLE_HIP_MAX_RANK)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "%s: rank exceeds kMaxTensorRank", what);
+  if (dtype_size(d.dtype) == 0)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "%s: data type is invalid", what);
+  if (d.storage != HYLE_HIP_STORAGE_PLAIN && d.storage != HYLE_HIP_STORAGE_BLOCKED)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "%s: storage format kind is invalid", what);
+  for (int i = 0; i < d.rank; ++i) {
+    if (d.dims[i] < 0) return fail(HYLE_HIP_INVALID_ARGUMENT, "%s: dimension is negative", what);
+    if (d.byte_strides[i] < 0)
+      return fail(HYLE_HIP_INVALID_ARGUMENT, "%s: negative byte stride", what);
+  }
+  if (d.storage == HYLE_HIP_STORAGE_BLOCKED) {
+    if (d.elements_per_block == 0 || d.bytes_per_block == 0)
+      return fail(HYLE_HIP_INVALID_ARGUMENT, "%s: blocked storage needs non-zero block geometry",
+                  what);
+    if (d.block_axis >= d.rank)
+      return fail(HYLE_HIP_INVALID_ARGUMENT, "%s: block axis is outside the tensor rank", what);
+    if (d.dims[d.block_axis] % d.elements_per_block != 0)
+      return fail(HYLE_HIP_INVALID_ARGUMENT, "%s: block axis does not hold whole blocks", what);
+  }
+  uint64_t count;
+  if (!element_count(d, &count))
+    return fail(HYLE_HIP_OUT_OF_RANGE, "%s: element count overflows size_t", what);
+  return HYLE_HIP_OK;
+}
+
+// broadcast_shape (src/compute_ops/operation.cc:249-278)
+hyle_hip_status broadcast_shape(const int64_t *l, int lr, const int64_t *r, int rr, int64_t *out,
+                                int *out_rank) {
+  const int rank = lr > rr ? lr : rr;
+  if (rank > HYLE_HIP_MAX_RANK)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "broadcast result rank exceeds limit");
+  for (int rev = 0; rev < rank; ++rev) {
+    const int64_t a = rev < lr ? l[lr - 1 - rev] : 1;
+    const int64_t b = rev < rr ? r[rr - 1 - rev] : 1;
+    int64_t e;
+    if (a == b) e = a;
+    else if (a == 1) e = b;
+    else if (b == 1) e = a;
+    else return fail(HYLE_HIP_INVALID_ARGUMENT, "tensor dimensions cannot be broadcast");
+    out[rank - 1 - rev] = e;
+  }
+  *out_rank = rank;
+  return HYLE_HIP_OK;
+}
+
+// normalize_axis (src/compute_ops/operation.cc:228-243)
+hyle_hip_status normalize_axis(int32_t axis, int rank, int *out) {
+  if (rank == 0) return fail(HYLE_HIP_OUT_OF_RANGE, "operation axis requires rank >= 1");
+  const int64_t n = axis < 0 ? (int64_t)rank + axis : (int64_t)axis;
+  if (n < 0 || n >= rank) return fail(HYLE_HIP_OUT_OF_RANGE, "operation axis is outside tensor rank");
+  *out = (int)n;
+  return HYLE_HIP_OK;
+}
+
+hyle_hip_status validate_accumulation(uint32_t type) {
+  if (type == HYLE_HIP_DTYPE_UNKNOWN) return HYLE_HIP_OK;
+  if (type > 255 || !is_numeric((uint8_t)type))
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "operation accumulation type must be numeric");
+  return HYLE_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------------
+// schema: output inference (src/compute_ops/operation.cc:1214-1704)
+// ---------------------------------------------------------------------------------
+hyle_hip_status expect_inputs(const hyle_hip_op_desc &r, uint32_t low, uint32_t high) {
+  if (r.input_count < low || r.input_count > high || r.input_count > HYLE_HIP_MAX_INPUTS)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "operation input count does not match its typed contract");
+  return HYLE_HIP_OK;
+}
+
+hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count) {
+  if (r.abi_version != HYLE_HIP_ABI_VERSION)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "hyle_hip_op_desc ABI version %u is not %u", r.abi_version,
+                HYLE_HIP_ABI_VERSION);
+  if (r.input_count > HYLE_HIP_MAX_INPUTS)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "operation input count does not match its typed contract");
+  for (uint32_t i = 0; i < r.input_count; ++i) {
+    hyle_hip_status s = validate_desc(r.inputs[i], "input");
+    if (s != HYLE_HIP_OK) return s;
+  }
+  const Desc *in = r.inputs;
+  hyle_hip_status s;
+  *out_count = 1;
+  switch (r.op) {
+    case HYLE_HIP_OP_UNARY: {
+      if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
+      if (r.kind > 12) return fail(HYLE_HIP_INVALID_ARGUMENT, "Unary kind is invalid");
+      const bool broad = r.kind == 0 /*abs*/ || r.kind == 1 /*neg*/ || r.kind == 8 /*relu*/;
+      if ((!broad && !is_floating(in[0].dtype)) || (broad && !is_numeric(in[0].dtype)))
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Unary mode does not support the input data type");
+      return make_dense(in[0].dtype, in[0].dims, in[0].rank, &outs[0]);
+    }
+    case HYLE_HIP_OP_BINARY: {
+      if ((s = expect_inputs(r, 2, 2)) != HYLE_HIP_OK) return s;
+      if (r.kind > HYLE_HIP_BINARY_MAXIMUM)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Binary kind is invalid");
+      if (in[0].dtype != in[1].dtype)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "binary input data types differ");
+      int64_t dims[HYLE_HIP_MAX_RANK];
+      int rank;
+      if ((s = broadcast_shape(in[0].dims, in[0].rank, in[1].dims, in[1].rank, dims, &rank)) != HYLE_HIP_OK)
+        return s;
+      return make_dense(in[0].dtype, dims, rank, &outs[0]);
+    }
+    case HYLE_HIP_OP_BINARY_CHAIN: {
+      if ((s = expect_inputs(r, 3, 3)) != HYLE_HIP_OK) return s;
+      if (r.kind > HYLE_HIP_BINARY_MAXIMUM || r.kind2 > HYLE_HIP_BINARY_MAXIMUM)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Binary kind is invalid");
+      if (in[0].dtype != in[1].dtype || in[0].dtype != in[2].dtype)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "binary input data types differ");
+      int64_t first[HYLE_HIP_MAX_RANK], dims[HYLE_HIP_MAX_RANK];
+      int first_rank, rank;
+      if ((s = broadcast_shape(in[0].dims, in[0].rank, in[1].dims, in[1].rank, first, &first_rank)) != HYLE_HIP_OK)
+        return s;
+      if ((s = broadcast_shape(first, first_rank, in[2].dims, in[2].rank, dims, &rank)) != HYLE_HIP_OK)
+        return s;
+      return make_dense(in[0].dtype, dims, rank, &outs[0]);
+    }
+    case HYLE_HIP_OP_REDUCE: {
+      if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
+      if (r.kind > HYLE_HIP_REDUCE_MAXIMUM)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Reduce kind is invalid");
+      if (!is_numeric(in[0].dtype))
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Reduce requires a numeric input");
+      if ((s = validate_accumulation(r.accumulation)) != HYLE_HIP_OK) return s;
+      int axis;
+      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
+      int64_t dims[HYLE_HIP_MAX_RANK];
+      int rank = 0;
+      for (int a = 0; a < in[0].rank; ++a) {
+        if (a == axis) {
+          if (r.keep_dimensions) dims[rank++] = 1;
+        } else {
+          dims[rank++] = in[0].dims[a];
+        }
+      }
+      return make_dense(in[0].dtype, dims, rank, &outs[0]);
+    }
+    case HYLE_HIP_OP_RMS_NORM: {
+      if ((s = expect_inputs(r, 1, 2)) != HYLE_HIP_OK) return s;
+      if (!std::isfinite(r.epsilon) || r.epsilon < 0.0f)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "RMSNorm epsilon must be finite and non-negative");
+      if ((s = validate_accumulation(r.accumulation)) != HYLE_HIP_OK) return s;
+      if (!is_floating(in[0].dtype) || in[0].rank == 0)
+        return fail(HYLE_HIP_INVALID_ARGUMENT,
+                    "normalization requires a floating tensor with rank >= 1");
+      if (r.input_count == 2) {
+        const bool promoted = in[0].dtype != HYLE_HIP_DTYPE_F32 && in[1].dtype == HYLE_HIP_DTYPE_F32;
+        if ((!promoted && in[1].dtype != in[0].dtype) || in[1].rank != 1 ||
+            in[1].dims[0] != in[0].dims[in[0].rank - 1])
+          return fail(HYLE_HIP_INVALID_ARGUMENT,
+                      "normalization scale must match the last input dimension");
+      }
+      return make_dense(in[0].dtype, in[0].dims, in[0].rank, &outs[0]);
+    }
+    case HYLE_HIP_OP_GATED_ACTIVATION: {
+      if (r.kind > 2 || r.kind2 > HYLE_HIP_GATED_SEPARATE)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "GatedActivation mode is invalid");
+      const bool separate = r.kind2 == HYLE_HIP_GATED_SEPARATE;
+      if ((s = expect_inputs(r, separate ? 2 : 1, separate ? 2 : 1)) != HYLE_HIP_OK) return s;
+      if (!is_floating(in[0].dtype) || in[0].rank == 0)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "GatedActivation requires floating rank >= 1 inputs");
+      if (separate) {
+        bool same = in[0].dtype == in[1].dtype && in[0].rank == in[1].rank;
+        for (int a = 0; same && a < in[0].rank; ++a) same = in[0].dims[a] == in[1].dims[a];
+        if (!same)
+          return fail(HYLE_HIP_INVALID_ARGUMENT,
+                      "separate gate/value tensors must have equal type and shape");
+        return make_dense(in[0].dtype, in[0].dims, in[0].rank, &outs[0]);
+      }
+      if ((in[0].dims[in[0].rank - 1] & 1) != 0)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "packed gate/value last dimension must be even");
+      int64_t dims[HYLE_HIP_MAX_RANK];
+      for (int a = 0; a < in[0].rank; ++a) dims[a] = in[0].dims[a];
+      dims[in[0].rank - 1] /= 2;
+      return make_dense(in[0].dtype, dims, in[0].rank, &outs[0]);
+    }
+    case HYLE_HIP_OP_SOFTMAX: {
+      if (r.kind2 > HYLE_HIP_LOG_SOFTMAX || r.mask > HYLE_HIP_MASK_BOOLEAN)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Softmax mode is invalid");
+      const uint32_t want = r.mask == HYLE_HIP_MASK_NONE ? 1 : 2;
+      if ((s = expect_inputs(r, want, want)) != HYLE_HIP_OK) return s;
+      if (!is_floating(in[0].dtype) || in[0].rank == 0 || !std::isfinite(r.scale))
+        return fail(HYLE_HIP_INVALID_ARGUMENT,
+                    "Softmax requires floating rank >= 1 input and finite scale");
+      int axis;
+      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
+      if ((s = validate_accumulation(r.accumulation)) != HYLE_HIP_OK) return s;
+      if (r.mask != HYLE_HIP_MASK_NONE) {
+        if (r.mask == HYLE_HIP_MASK_BOOLEAN && in[1].dtype != HYLE_HIP_DTYPE_BOOL)
+          return fail(HYLE_HIP_INVALID_ARGUMENT, "boolean mask requires Bool data type");
+        if (r.mask == HYLE_HIP_MASK_ADDITIVE && !is_floating(in[1].dtype))
+          return fail(HYLE_HIP_INVALID_ARGUMENT, "additive mask requires a floating data type");
+        int64_t dims[HYLE_HIP_MAX_RANK];
+        int rank;
+        if ((s = broadcast_shape(in[1].dims, in[1].rank, in[0].dims, in[0].rank, dims, &rank)) != HYLE_HIP_OK)
+          return s;
+        bool same = rank == in[0].rank;
+        for (int a = 0; same && a < rank; ++a) same = dims[a] == in[0].dims[a];
+        if (!same)
+          return fail(HYLE_HIP_INVALID_ARGUMENT,
+                      "tensor is not broadcast-compatible with target shape");
+      }
+      return make_dense(in[0].dtype, in[0].dims, in[0].rank, &outs[0]);
+    }
+    case HYLE_HIP_OP_TOP_K: {
+      if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
+      if (!is_numeric(in[0].dtype) || in[0].rank == 0)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "TopK requires numeric rank >= 1 input");
+      int axis;
+      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
+      if (in[0].dims[axis] > (int64_t)std::numeric_limits<int32_t>::max())
+        return fail(HYLE_HIP_OUT_OF_RANGE,
+                    "TopK selected dimension cannot be represented by i32 indices");
+      if (r.count > (uint64_t)in[0].dims[axis])
+        return fail(HYLE_HIP_OUT_OF_RANGE, "TopK count exceeds selected dimension");
+      int64_t dims[HYLE_HIP_MAX_RANK];
+      for (int a = 0; a < in[0].rank; ++a) dims[a] = in[0].dims[a];
+      dims[axis] = (int64_t)r.count;
+      if ((s = make_dense(in[0].dtype, dims, in[0].rank, &outs[0])) != HYLE_HIP_OK) return s;
+      *out_count = 2;
+      return make_dense(HYLE_HIP_DTYPE_I32, dims, in[0].rank, &outs[1]);
+    }
+    case HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ: {
+      if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
+      // gguf_weight_description(kQ8_0, ..., k, n): logical [K, N], blocks along axis 0
+      // (src/compute_ops/low_precision.cc:269-297)
+      if (in[0].storage != HYLE_HIP_STORAGE_BLOCKED || in[0].elements_per_block != 32 ||
+          in[0].bytes_per_block != 34 || in[0].rank != 2 || in[0].block_axis != 0)
+        return fail(HYLE_HIP_INVALID_ARGUMENT,
+                    "Q8_0 weight must be blocked [K, N] storage with 32-element 34-byte blocks on axis 0");
+      if (!is_floating(in[0].dtype))
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "GGUF weight requires a floating logical type");
+      const int64_t dims0[2] = {in[0].dims[1], in[0].dims[0]};
+      if ((s = make_dense(HYLE_HIP_DTYPE_BF16, dims0, 2, &outs[0])) != HYLE_HIP_OK) return s;
+      *out_count = 2;
+      return make_dense(HYLE_HIP_DTYPE_F32, &in[0].dims[1], 1, &outs[1]);
+    }
+    default:
+      return fail(HYLE_HIP_UNIMPLEMENTED, "operation kind %u is not served by this provider", r.op);
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// plans
+// ---------------------------------------------------------------------------------
+enum class Route : uint8_t {
+  kNoOp = 0,
+  kEwFlat,
+  kEwGeneral,
+  kSwigluPacked,
+  kRmsNorm,
+  kSoftmax,
+  kReduceRows,
+  kArgmax,
+  kQ8Dequant,
+};
+
+const char *route_name(Route r) {
+  switch (r) {
+    case Route::kNoOp: return "no-op";
+    case Route::kEwFlat: return "elementwise-flat";
+    case Route::kEwGeneral: return "elementwise-strided";
+    case Route::kSwigluPacked: return "swiglu-packed";
+    case Route::kRmsNorm: return "rms-norm-rows";
+    case Route::kSoftmax: return "softmax-rows";
+    case Route::kReduceRows: return "reduce-rows";
+    case Route::kArgmax: return "argmax-tiles";
+    case Route::kQ8Dequant: return "q8_0-dequant-rows";
+  }
+  return "?";
+}
+
+constexpr uint64_t kMaxElements = (uint64_t)std::numeric_limits<int32_t>::max();
+
+}  // namespace
+
+struct hyle_hip_context {
+  int device = 0;
+  int compute_units = 0;
+};
+
+struct hyle_hip_plan {
+  const hyle_hip_context *context = nullptr;
+  hyle_hip_op_desc request{};
+  Desc outputs[HYLE_HIP_MAX_OUTPUTS]{};
+  uint32_t output_count = 0;
+  Route route = Route::kNoOp;
+  Elem elem = Elem::kF32;
+  uint8_t alias_inputs[HYLE_HIP_MAX_OUTPUTS] = {0, 0};  // bit i: output may alias input i
+  uint32_t dispatches = 0;
+  size_t workspace_size = 0, workspace_alignment = 1;
+  size_t input_alignment[HYLE_HIP_MAX_INPUTS] = {1, 1, 1, 1};   // element alignment (required)
+  size_t output_alignment[HYLE_HIP_MAX_OUTPUTS] = {1, 1};
+  uint64_t input_elements[HYLE_HIP_MAX_INPUTS] = {0, 0, 0, 0};
+  uint64_t output_elements[HYLE_HIP_MAX_OUTPUTS] = {0, 0};
+  // route parameters
+  EwFlat flat;
+  EwGeneral general;
+  EwPacked packed;
+  NormParams norm;
+  SoftmaxParams softmax;
+  SoftmaxGeneralParams softmax_general;
+  bool softmax_rows_ok = false;     // the row kernel applies (dense last-axis layout)
+  bool softmax_mask_vector_ok = false;
+  ReduceParams reduce;
+  ArgmaxParams argmax;
+  Q8Params q8;
+};
+
+namespace {
+
+bool dims_equal(const Desc &a, const Desc &b) {
+  if (a.rank != b.rank) return false;
+  for (int i = 0; i < a.rank; ++i)
+    if (a.dims[i] != b.dims[i]) return false;
+  return true;
+}
+
+// A dense input that is a trailing slice of the output shape (leading axes absent or 1):
+// it repeats every `period` elements of the flat output
+// (dense_broadcast_suffix, src/compute_provider_native/elementwise.cc:540-571).
+bool suffix_period(const Desc &in, const Desc &out, uint64_t out_elements, uint32_t *period) {
+  if (!is_dense(in)) return false;
+  uint64_t count = 1;
+  bool leading = false;  // once an axis is broadcast, every axis left of it must be too
+  for (int rev = 0; rev < out.rank; ++rev) {
+    const int64_t oe = out.dims[out.rank - 1 - rev];
+    const int64_t ie = rev < in.rank ? in.dims[in.rank - 1 - rev] : 1;
+    if (!leading && ie == oe) {
+      count *= (uint64_t)ie;
+      continue;
+    }
+    if (ie != 1) return false;
+    leading = true;
+  }
+  if (count == out_elements) *period = 0;
+  else *period = (uint32_t)count;
+  return true;
+}
+
+hyle_hip_status admit_elementwise(hyle_hip_plan *p, EwOp op, int inputs) {
+  const hyle_hip_op_desc &r = p->request;
+  const Desc &out = p->outputs[0];
+  if (!to_elem(out.dtype, &p->elem))
+    return fail(HYLE_HIP_UNIMPLEMENTED, "elementwise arithmetic requires plain float32/float16/bfloat16");
+  for (int i = 0; i < inputs; ++i)
+    if (!is_plain(r.inputs[i]) || r.inputs[i].dtype != out.dtype)
+      return fail(HYLE_HIP_UNIMPLEMENTED, "elementwise arithmetic requires plain float32/float16/bfloat16");
+  const uint64_t n = p->output_elements[0];
+  if (n > kMaxElements)
+    return fail(HYLE_HIP_UNIMPLEMENTED, "elementwise output exceeds INT32_MAX elements");
+  if (n == 0) {
+    p->route = Route::kNoOp;
+    return HYLE_HIP_OK;
+  }
+  // alias only when an input descriptor equals the output descriptor
+  // (src/compute_provider_native/elementwise.cc:645-655; gated routes take no alias)
+  if (op != EwOp::kSwiglu)
+    for (int i = 0; i < inputs; ++i)
+      if (same_desc(r.inputs[i], out)) p->alias_inputs[0] |= (uint8_t)(1u << i);
+
+  uint32_t period[3] = {0, 0, 0};
+  bool flat = true;
+  for (int i = 0; i < inputs && flat; ++i) flat = suffix_period(r.inputs[i], out, n, &period[i]);
+  p->dispatches = 1;
+  if (flat) {
+    p->route = Route::kEwFlat;
+    p->flat.elements = n;
+    p->flat.op = op;
+    p->flat.kind0 = (uint8_t)r.kind;
+    p->flat.kind1 = (uint8_t)r.kind2;
+    p->flat.inputs = (uint8_t)inputs;
+    for (int i = 0; i < 3; ++i) p->flat.period[i] = period[i];
+    return HYLE_HIP_OK;
+  }
+  p->route = Route::kEwGeneral;
+  EwGeneral &g = p->general;
+  g.elements = n;
+  g.rank = out.rank;
+  g.op = op;
+  g.kind0 = (uint8_t)r.kind;
+  g.kind1 = (uint8_t)r.kind2;
+  g.inputs = (uint8_t)inputs;
+  for (int a = 0; a < out.rank; ++a) g.dims[a] = (uint32_t)out.dims[a];
+  for (int i = 0; i < inputs; ++i) {
+    const Desc &in = r.inputs[i];
+    for (int rev = 0; rev < out.rank; ++rev) {
+      const int oa = out.rank - 1 - rev;
+      int64_t stride = 0;
+      if (rev < in.rank) {
+        const int ia = in.rank - 1 - rev;
+        // logical_broadcast_byte_offset: an input axis of extent 1 contributes nothing
+        if (in.dims[ia] != 1) stride = in.byte_strides[ia];
+      }
+      g.strides[i][oa] = stride;
+    }
+  }
+  return HYLE_HIP_OK;
+}
+
+hyle_hip_status require_f32_accumulation(const hyle_hip_plan *p, uint8_t input_dtype, const char *op) {
+  const uint32_t acc = p->request.accumulation;
+  if (acc == HYLE_HIP_DTYPE_F32) return HYLE_HIP_OK;
+  if (acc == HYLE_HIP_DTYPE_UNKNOWN && input_dtype == HYLE_HIP_DTYPE_F32) return HYLE_HIP_OK;
+  return fail(HYLE_HIP_UNIMPLEMENTED, "%s supports float32 accumulation (explicit for half inputs)", op);
+}
+
+hyle_hip_status admit(hyle_hip_plan *p) {
+  const hyle_hip_op_desc &r = p->request;
+  const Desc *in = r.inputs;
+  const Desc &out = p->outputs[0];
+  hyle_hip_status s;
+  switch (r.op) {
+    case HYLE_HIP_OP_UNARY:
+      if (r.kind != HYLE_HIP_UNARY_SILU)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "only Unary SiLU is served by this provider");
+      return admit_elementwise(p, EwOp::kSilu, 1);
+    case HYLE_HIP_OP_BINARY:
+      return admit_elementwise(p, EwOp::kBinary, 2);
+    case HYLE_HIP_OP_BINARY_CHAIN:
+      return admit_elementwise(p, EwOp::kChain, 3);
+    case HYLE_HIP_OP_GATED_ACTIVATION: {
+      if (r.kind != HYLE_HIP_GATED_SILU)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "gated activation serves SiLU only");
+      // dense inputs and output (src/compute_provider_cuda/cuda_provider.cc:86-139)
+      for (uint32_t i = 0; i < r.input_count; ++i)
+        if (!is_dense(in[i]))
+          return fail(HYLE_HIP_UNIMPLEMENTED, "gated activation requires dense plain input");
+      if (r.kind2 == HYLE_HIP_GATED_SEPARATE) return admit_elementwise(p, EwOp::kSwiglu, 2);
+      if (!to_elem(out.dtype, &p->elem))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "gated activation requires dense FP16/BF16/FP32");
+      if (p->output_elements[0] > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "gated activation requires at most INT32_MAX elements");
+      if (p->output_elements[0] == 0) return HYLE_HIP_OK;
+      p->route = Route::kSwigluPacked;
+      p->packed.hidden = (uint32_t)out.dims[out.rank - 1];
+      p->packed.rows = p->output_elements[0] / p->packed.hidden;
+      p->dispatches = 1;
+      return HYLE_HIP_OK;
+    }
+    case HYLE_HIP_OP_RMS_NORM: {
+      if (r.accumulation != HYLE_HIP_DTYPE_F32)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "normalization supports float32 accumulation");
+      if (!to_elem(in[0].dtype, &p->elem) || !is_dense(in[0]))
+        return fail(HYLE_HIP_UNIMPLEMENTED,
+                    "normalization requires dense plain float32/float16/bfloat16");
+      if (r.input_count == 2 && !is_dense(in[1]))
+        return fail(HYLE_HIP_UNIMPLEMENTED,
+                    "normalization requires dense plain float32/float16/bfloat16");
+      if (p->output_elements[0] > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "normalization requires at most INT32_MAX elements");
+      p->alias_inputs[0] = 1;  // reductions finish before the first write
+      if (p->output_elements[0] == 0) return HYLE_HIP_OK;
+      p->route = Route::kRmsNorm;
+      p->norm.shape.width = (uint32_t)in[0].dims[in[0].rank - 1];
+      p->norm.shape.rows = p->output_elements[0] / p->norm.shape.width;
+      p->norm.epsilon = r.epsilon;
+      p->norm.has_weight = r.input_count == 2;
+      p->norm.weight_f32 = r.input_count == 2 && in[1].dtype == HYLE_HIP_DTYPE_F32 &&
+                           in[0].dtype != HYLE_HIP_DTYPE_F32;
+      p->dispatches = 1;
+      return HYLE_HIP_OK;
+    }
+    case HYLE_HIP_OP_SOFTMAX: {
+      if (!to_elem(in[0].dtype, &p->elem) || !is_plain(in[0]))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Softmax requires plain float32/float16/bfloat16");
+      if ((s = require_f32_accumulation(p, in[0].dtype, "Softmax")) != HYLE_HIP_OK) return s;
+      if (r.mask != HYLE_HIP_MASK_NONE) {
+        if (!is_plain(in[1]) || (r.mask == HYLE_HIP_MASK_ADDITIVE && in[1].dtype != in[0].dtype))
+          return fail(HYLE_HIP_UNIMPLEMENTED,
+                      "Softmax requires plain Bool or matching floating masks");
+      }
+      if (p->output_elements[0] > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Softmax requires at most INT32_MAX elements");
+      if (same_desc(in[0], out)) p->alias_inputs[0] = 1;
+      if (p->output_elements[0] == 0) return HYLE_HIP_OK;
+      int axis;
+      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
+      p->route = Route::kSoftmax;
+      p->dispatches = 1;
+      const int rank = in[0].rank;
+      const uint32_t width = (uint32_t)in[0].dims[axis];
+      // general description (any axis, any strides)
+      SoftmaxGeneralParams &g = p->softmax_general;
+      g.width = width;
+      g.scale = r.scale;
+      g.mask_kind = (uint8_t)r.mask;
+      g.log = r.kind2 == HYLE_HIP_LOG_SOFTMAX;
+      g.rank = rank;
+      g.axis = axis;
+      g.outer = g.inner = 1;
+      for (int a = 0; a < rank; ++a) {
+        g.dims[a] = (uint32_t)in[0].dims[a];
+        g.in_strides[a] = in[0].byte_strides[a];
+        if (a < axis) g.outer *= (uint64_t)in[0].dims[a];
+        if (a > axis) g.inner *= (uint64_t)in[0].dims[a];
+      }
+      if (r.mask != HYLE_HIP_MASK_NONE) {
+        for (int rev = 0; rev < rank; ++rev) {
+          const int a = rank - 1 - rev;
+          int64_t stride = 0;
+          if (rev < in[1].rank) {
+            const int ma = in[1].rank - 1 - rev;
+            if (in[1].dims[ma] != 1) stride = in[1].byte_strides[ma];
+          }
+          g.mask_strides[a] = stride;
+        }
+      }
+      // row kernel: dense input, last axis
+      p->softmax_rows_ok = axis == rank - 1 && is_dense(in[0]);
+      if (p->softmax_rows_ok) {
+        SoftmaxParams &sp = p->softmax;
+        sp.shape.width = width;
+        sp.shape.rows = p->output_elements[0] / width;
+        sp.scale = r.scale;
+        sp.mask_kind = (uint8_t)r.mask;
+        sp.log = g.log;
+        sp.outer_rank = rank - 1;
+        for (int a = 0; a < rank - 1; ++a) {
+          sp.outer_dims[a] = g.dims[a];
+          sp.mask_outer_strides[a] = g.mask_strides[a];
+        }
+        sp.mask_inner_stride = g.mask_strides[rank - 1];
+        p->softmax_mask_vector_ok = true;
+        if (r.mask != HYLE_HIP_MASK_NONE) {
+          const int64_t unit = (int64_t)dtype_size(in[1].dtype);
+          if (sp.mask_inner_stride != 0 && sp.mask_inner_stride != unit)
+            p->softmax_mask_vector_ok = false;
+          // a mask row is read as whole vectors: one byte per column for Bool, one
+          // element per column for an additive mask
+          const int64_t row_alignment = r.mask == HYLE_HIP_MASK_BOOLEAN ? elem_vec(p->elem) : 16;
+          for (int a = 0; a < rank - 1; ++a)
+            if (sp.mask_outer_strides[a] % row_alignment != 0) p->softmax_mask_vector_ok = false;
+          // rows r and r + period share a mask row when the mask is a dense trailing
+          // slice of the input shape (e.g. [q, k] under [heads, q, k])
+          uint32_t period_elements = 0;
+          if (suffix_period(in[1], in[0], p->output_elements[0], &period_elements) &&
+              period_elements != 0 && period_elements % width == 0)
+            sp.mask_period = period_elements / width;
+        }
+      }
+      return HYLE_HIP_OK;
+    }
+    case HYLE_HIP_OP_REDUCE: {
+      if (!to_elem(in[0].dtype, &p->elem) || !is_dense(in[0]))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Reduce requires dense plain float32/float16/bfloat16");
+      if ((s = require_f32_accumulation(p, in[0].dtype, "Reduce")) != HYLE_HIP_OK) return s;
+      int axis;
+      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
+      if (axis != in[0].rank - 1)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Reduce serves the last axis only");
+      if (p->input_elements[0] > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Reduce requires at most INT32_MAX elements");
+      if (p->output_elements[0] == 0) return HYLE_HIP_OK;
+      p->route = Route::kReduceRows;
+      p->reduce.shape.width = (uint32_t)in[0].dims[axis];
+      p->reduce.shape.rows = p->output_elements[0];
+      p->reduce.kind = (uint8_t)r.kind;
+      p->dispatches = 1;
+      return HYLE_HIP_OK;
+    }
+    case HYLE_HIP_OP_TOP_K: {
+      if (r.count != 1 || !r.largest)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK serves count = 1, largest only");
+      if (!to_elem(in[0].dtype, &p->elem) || !is_dense(in[0]))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK requires dense plain float32/float16/bfloat16");
+      int axis;
+      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
+      if (axis != in[0].rank - 1)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK serves the last axis only");
+      if (p->input_elements[0] > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK requires at most INT32_MAX elements");
+      if (p->output_elements[0] == 0) return HYLE_HIP_OK;
+      p->route = Route::kArgmax;
+      argmax_plan(p->output_elements[0], (uint32_t)in[0].dims[axis],
+                  p->context ? p->context->compute_units : 256, &p->argmax);
+      p->workspace_size = argmax_workspace_bytes(p->argmax);
+      p->workspace_alignment = 16;
+      p->dispatches = 2;
+      return HYLE_HIP_OK;
+    }
+    case HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ: {
+      const int64_t k = in[0].dims[0], n = in[0].dims[1];
+      if (in[0].byte_strides[0] != 34)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Q8_0 blocks of a row must be contiguous (34-byte block stride)");
+      if (k > 0 && n > 1 && in[0].byte_strides[1] < (k / 32) * 34)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Q8_0 row stride is shorter than a row of blocks");
+      if ((uint64_t)k * (uint64_t)n > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Q8_0 dequant requires at most INT32_MAX elements");
+      p->elem = Elem::kBF16;
+      if (n == 0) return HYLE_HIP_OK;
+      // with K == 0 the bf16 output is empty but every row still gets sumsq = 0
+      p->route = Route::kQ8Dequant;
+      p->q8.rows = (uint64_t)n;
+      p->q8.k = (uint32_t)k;
+      p->q8.row_stride = (uint64_t)in[0].byte_strides[1];
+      p->dispatches = 1;
+      return HYLE_HIP_OK;
+    }
+    default:
+      return fail(HYLE_HIP_UNIMPLEMENTED, "operation kind %u is not served by this provider", r.op);
+  }
+}
+
+bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------
+// C ABI
+// ---------------------------------------------------------------------------------
+extern "C" {
+
+uint32_t hyle_hip_abi_version(void) { return HYLE_HIP_ABI_VERSION; }
+
+const char *hyle_hip_last_error(void) { return g_error; }
+
+const char *hyle_hip_status_name(hyle_hip_status status) {
+  switch (status) {
+    case HYLE_HIP_OK: return "OK";
+    case HYLE_HIP_INVALID_ARGUMENT: return "INVALID_ARGUMENT";
+    case HYLE_HIP_RESOURCE_EXHAUSTED: return "RESOURCE_EXHAUSTED";
+    case HYLE_HIP_FAILED_PRECONDITION: return "FAILED_PRECONDITION";
+    case HYLE_HIP_OUT_OF_RANGE: return "OUT_OF_RANGE";
+    case HYLE_HIP_UNIMPLEMENTED: return "UNIMPLEMENTED";
+    case HYLE_HIP_INTERNAL: return "INTERNAL";
+    case HYLE_HIP_UNAVAILABLE: return "UNAVAILABLE";
+  }
+  return "UNKNOWN";
+}
+
+hyle_hip_status hyle_hip_context_create(int device, hyle_hip_context **context) {
+  if (context == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "context output is null");
+  *context = nullptr;
+  int count = 0;
+  hipError_t err = hipGetDeviceCount(&count);
+  if (err != hipSuccess || count <= 0) {
+    (void)hipGetLastError();
+    return fail(HYLE_HIP_UNAVAILABLE, "no HIP device is visible");
+  }
+  if (device < 0 || device >= count)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "device %d is outside [0, %d)", device, count);
+  hipDeviceProp_t props;
+  err = hipGetDeviceProperties(&props, device);
+  if (err != hipSuccess) return hip_fail(err, "hipGetDeviceProperties");
+  if (std::strncmp(props.gcnArchName, "gfx950", 6) != 0)
+    return fail(HYLE_HIP_UNAVAILABLE, "device %d is %s; this provider carries gfx950 code only", device,
+                props.gcnArchName);
+  auto *ctx = new (std::nothrow) hyle_hip_context;
+  if (ctx == nullptr) return fail(HYLE_HIP_RESOURCE_EXHAUSTED, "out of host memory");
+  ctx->device = device;
+  ctx->compute_units = props.multiProcessorCount;
+  *context = ctx;
+  return HYLE_HIP_OK;
+}
+
+void hyle_hip_context_destroy(hyle_hip_context *context) { delete context; }
+
+int hyle_hip_context_compute_units(const hyle_hip_context *context) {
+  return context ? context->compute_units : 0;
+}
+
+hyle_hip_status hyle_hip_infer_outputs(const hyle_hip_op_desc *request, hyle_hip_tensor_desc *outputs,
+                                       uint32_t *output_count) {
+  if (request == nullptr || outputs == nullptr || output_count == nullptr)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "null argument");
+  Desc local[HYLE_HIP_MAX_OUTPUTS];
+  uint32_t count = 0;
+  hyle_hip_status s = infer(*request, local, &count);
+  if (s != HYLE_HIP_OK) return s;
+  for (uint32_t i = 0; i < count; ++i) outputs[i] = local[i];
+  *output_count = count;
+  return HYLE_HIP_OK;
+}
+
+hyle_hip_status hyle_hip_plan_create(hyle_hip_context *context, const hyle_hip_op_desc *request,
+                                     const hyle_hip_tensor_desc *outputs, uint32_t output_count,
+                                     hyle_hip_plan **plan) {
+  if (plan == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "plan output is null");
+  *plan = nullptr;
+  if (request == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "request is null");
+  auto *p = new (std::nothrow) hyle_hip_plan;
+  if (p == nullptr) return fail(HYLE_HIP_RESOURCE_EXHAUSTED, "out of host memory");
+  p->context = context;
+  p->request = *request;
+  hyle_hip_status s = infer(p->request, p->outputs, &p->output_count);
+  if (s == HYLE_HIP_OK && outputs != nullptr) {
+    if (output_count != p->output_count)
+      s = fail(HYLE_HIP_INVALID_ARGUMENT, "operation output span must have the exact output count");
+    for (uint32_t i = 0; s == HYLE_HIP_OK && i < output_count; ++i)
+      if (!same_desc(outputs[i], p->outputs[i]))
+        s = fail(HYLE_HIP_INVALID_ARGUMENT,
+                 "output %u descriptor differs from the inferred dense description", i);
+  }
+  if (s == HYLE_HIP_OK) {
+    for (uint32_t i = 0; i < p->request.input_count; ++i) {
+      element_count(p->request.inputs[i], &p->input_elements[i]);
+      p->input_alignment[i] =
+          is_plain(p->request.inputs[i]) ? dtype_size(p->request.inputs[i].dtype) : 1;
+    }
+    for (uint32_t i = 0; i < p->output_count; ++i) {
+      element_count(p->outputs[i], &p->output_elements[i]);
+      p->output_alignment[i] = dtype_size(p->outputs[i].dtype);
+    }
+    s = admit(p);
+  }
+  if (s != HYLE_HIP_OK) {
+    delete p;
+    return s;
+  }
+  *plan = p;
+  return HYLE_HIP_OK;
+}
+
+void hyle_hip_plan_destroy(hyle_hip_plan *plan) { delete plan; }
+
+hyle_hip_status hyle_hip_plan_workspace(const hyle_hip_plan *plan, size_t *size, size_t *alignment) {
+  if (plan == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "plan is null");
+  if (size) *size = plan->workspace_size;
+  if (alignment) *alignment = plan->workspace_alignment;
+  return HYLE_HIP_OK;
+}
+
+hyle_hip_status hyle_hip_plan_outputs(const hyle_hip_plan *plan, hyle_hip_tensor_desc *outputs,
+                                      uint32_t *output_count) {
+  if (plan == nullptr || outputs == nullptr || output_count == nullptr)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "null argument");
+  for (uint32_t i = 0; i < plan->output_count; ++i) outputs[i] = plan->outputs[i];
+  *output_count = plan->output_count;
+  return HYLE_HIP_OK;
+}
+
+int hyle_hip_plan_alias_support(const hyle_hip_plan *plan, uint32_t output_index, uint32_t input_index) {
+  if (plan == nullptr || output_index >= plan->output_count ||
+      input_index >= plan->request.input_count)
+    return 0;
+  return (plan->alias_inputs[output_index] >> input_index) & 1u;
+}
+
+uint32_t hyle_hip_plan_dispatch_count(const hyle_hip_plan *plan) { return plan ? plan->dispatches : 0; }
+
+const char *hyle_hip_plan_route_name(const hyle_hip_plan *plan) {
+  return plan ? route_name(plan->route) : "";
+}
+
+hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *const *inputs,
+                                     uint32_t input_count, void *const *outputs, uint32_t output_count,
+                                     void *workspace, size_t workspace_size, void *stream_handle) {
+  if (plan == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "plan is null");
+  if (input_count != plan->request.input_count || output_count != plan->output_count)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "launch binding counts differ from the plan");
+  if (plan->route == Route::kNoOp) return HYLE_HIP_OK;  // zero elements: storage is never touched
+  if (plan->context == nullptr)
+    return fail(HYLE_HIP_FAILED_PRECONDITION, "plan was built without a device context");
+  if (inputs == nullptr || outputs == nullptr)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "binding arrays are null");
+  bool vector = true;
+  for (uint32_t i = 0; i < input_count; ++i) {
+    if (plan->input_elements[i] == 0) continue;
+    if (inputs[i] == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "input %u is null", i);
+    if (!aligned(inputs[i], plan->input_alignment[i]))
+      return fail(HYLE_HIP_FAILED_PRECONDITION, "input %u does not satisfy tensor alignment", i);
+    // a one-element operand is read with a scalar load and never limits vector access
+    if (plan->input_elements[i] > 1) vector = vector && aligned(inputs[i], 16);
+  }
+  for (uint32_t o = 0; o < output_count; ++o) {
+    if (plan->output_elements[o] == 0) continue;
+    if (outputs[o] == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "output %u is null", o);
+    if (!aligned(outputs[o], plan->output_alignment[o]))
+      return fail(HYLE_HIP_FAILED_PRECONDITION, "output %u does not satisfy tensor alignment", o);
+    if (o == 0) vector = vector && aligned(outputs[o], 16);
+    for (uint32_t i = 0; i < input_count; ++i)
+      if (outputs[o] == inputs[i] && plan->input_elements[i] != 0 &&
+          ((plan->alias_inputs[o] >> i) & 1u) == 0)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "input %u cannot alias output %u on this route", i, o);
+  }
+  if (plan->workspace_size != 0) {
+    if (workspace == nullptr || workspace_size < plan->workspace_size)
+      return fail(HYLE_HIP_INVALID_ARGUMENT, "workspace is smaller than the plan requires");
+    if (!aligned(workspace, plan->workspace_alignment))
+      return fail(HYLE_HIP_FAILED_PRECONDITION, "workspace does not satisfy its alignment");
+  }
+  hipStream_t stream = static_cast<hipStream_t>(stream_handle);
+  hipError_t err = hipSuccess;
+  switch (plan->route) {
+    case Route::kNoOp: break;
+    case Route::kEwFlat:
+      err = launch_ew_flat(plan->elem, plan->flat, inputs[0], input_count > 1 ? inputs[1] : nullptr,
+                           input_count > 2 ? inputs[2] : nullptr, outputs[0], vector, stream);
+      break;
+    case Route::kEwGeneral:
+      err = launch_ew_general(plan->elem, plan->general, inputs[0],
+                              input_count > 1 ? inputs[1] : nullptr,
+                              input_count > 2 ? inputs[2] : nullptr, outputs[0], stream);
+      break;
+    case Route::kSwigluPacked:
+      err = launch_swiglu_packed(plan->elem, plan->packed, inputs[0], outputs[0], vector, stream);
+      break;
+    case Route::kRmsNorm:
+      err = launch_rms_norm(plan->elem, plan->norm, inputs[0], input_count > 1 ? inputs[1] : nullptr,
+                            outputs[0], vector, stream);
+      break;
+    case Route::kSoftmax: {
+      const void *mask = input_count > 1 ? inputs[1] : nullptr;
+      const int kvec = elem_vec(plan->elem);
+      const bool rows = plan->softmax_rows_ok && plan->softmax_mask_vector_ok &&
+                        aligned(inputs[0], 16) && aligned(outputs[0], 16) &&
+                        (mask == nullptr || aligned(mask, 16)) &&
+                        plan->softmax.shape.width % kvec == 0 &&
+                        plan->softmax.shape.width / kvec <= 16u * 256u;
+      if (rows)
+        err = launch_softmax(plan->elem, plan->softmax, inputs[0], mask, outputs[0], true,
+                             plan->context->compute_units, stream);
+      else
+        err = launch_softmax_general(plan->elem, plan->softmax_general, inputs[0], mask, outputs[0],
+                                     stream);
+      break;
+    }
+    case Route::kReduceRows:
+      err = launch_reduce_rows(plan->elem, plan->reduce, inputs[0], outputs[0], vector, stream);
+      break;
+    case Route::kArgmax:
+      err = launch_argmax(plan->elem, plan->argmax, inputs[0], outputs[0],
+                          static_cast<int32_t *>(outputs[1]), workspace, aligned(inputs[0], 16), stream);
+      break;
+    case Route::kQ8Dequant:
+      err = launch_q8_0_dequant(plan->q8, inputs[0], outputs[0], static_cast<float *>(outputs[1]),
+                                aligned(inputs[0], 16) && aligned(outputs[0], 16), stream);
+      break;
+  }
+  if (err != hipSuccess) return hip_fail(err, "kernel launch");
+  return HYLE_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,477 @@
+// softmax.hip -- row Softmax / LogSoftmax with scale and broadcast mask, and
+// last-axis Reduce (sum, mean, min, max) for gfx950.
+//
+// Softmax reads every row from HBM once: the row lives in registers across the
+// max reduction, the exponential pass and the normalised store.  Semantics are
+// those of the reference's CPU path
+// (src/compute_provider_native/transformer.cc:44-57,165-191 and
+//  src/simd/math/activations.cc:177-192,301-340):
+//   v = x * scale; Boolean mask 0 -> -inf; additive mask -> v + mask;
+//   a row holding a NaN or +inf, or no finite value at all, becomes all NaN;
+//   otherwise out = exp(v - max) / sum, with masked lanes exactly 0.
+// The exponential sum is accumulated in f32 (the reference's scalar floor uses
+// double); the exponentials are carried scaled by 2^32 and the scale is folded
+// into the normaliser, so results down to the smallest subnormal are produced by
+// an ordinary multiply instead of being flushed by the hardware exp2.
+#include "device_common.h"
+#include "kernels.h"
+
+namespace hyle_hip {
+namespace {
+
+enum : int { kMaskNone = 0, kMaskAdditive = 1, kMaskBoolean = 2 };
+
+template <int kLanes> __device__ __forceinline__ float row_sum(float v, float *joint) {
+  if constexpr (kLanes <= kWaveLanes) {
+    return group_sum<kLanes>(v);
+  } else {
+    v = group_sum<kWaveLanes>(v);
+    if ((threadIdx.x & (kWaveLanes - 1)) == 0) joint[threadIdx.x / kWaveLanes] = v;
+    __syncthreads();
+    return (joint[0] + joint[1]) + (joint[2] + joint[3]);
+  }
+}
+template <int kLanes> __device__ __forceinline__ float row_max(float v, float *joint) {
+  if constexpr (kLanes <= kWaveLanes) {
+    return group_max<kLanes>(v);
+  } else {
+    v = group_max<kWaveLanes>(v);
+    if ((threadIdx.x & (kWaveLanes - 1)) == 0) joint[threadIdx.x / kWaveLanes] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(joint[0], joint[1]), fmaxf(joint[2], joint[3]));
+  }
+}
+
+// exp(t) * 2^32 for t <= 0, about 2 ulp.  t * log2(e) is split into a rounded
+// product and its exact residual so the hardware exp2 sees an accurate argument.
+__device__ __forceinline__ float exp_scaled(float t) {
+  constexpr float kLog2eHi = 1.44269502162933349609f;   // f32(log2 e)
+  constexpr float kLog2eLo = 1.92596299112661746e-08f;  // log2 e - f32(log2 e)
+  constexpr float kLn2 = 0.69314718055994530942f;
+  t = fmaxf(t, -200.0f);  // exp(-200) * 2^32 is below every subnormal; also tames -inf
+  const float hi = t * kLog2eHi;
+  float lo = __builtin_fmaf(t, kLog2eHi, -hi);
+  lo = __builtin_fmaf(t, kLog2eLo, lo);
+  const float p = __builtin_amdgcn_exp2f(hi + 32.0f);
+  return __builtin_fmaf(p, lo * kLn2, p);
+}
+
+struct MaskRows {
+  int32_t outer_rank;
+  uint32_t outer_dims[kMaxRank];
+  int64_t outer_strides[kMaxRank];
+  int64_t inner_stride;
+};
+
+__device__ __forceinline__ int64_t mask_row_offset(const MaskRows &m, uint32_t row) {
+  int64_t offset = 0;
+  uint32_t rest = row;
+  for (int axis = m.outer_rank - 1; axis >= 0; --axis) {
+    const uint32_t extent = m.outer_dims[axis];
+    offset += (int64_t)(rest % extent) * m.outer_strides[axis];
+    rest /= extent;
+  }
+  return offset;
+}
+
+// Rows that share a mask row are steered onto one XCD, close in time, so the mask
+// row is fetched from memory once per XCD and then served by that XCD's L2.
+// Workgroups are dealt to the 8 XCDs round-robin by index.
+struct RowOrder {
+  uint32_t period;  // rows r and r + period share a mask row; 0 = plain order
+  uint32_t groups;  // blocks per mask row = (rows / period) / rows-per-block
+};
+template <int kRowsPerBlock>
+__device__ __forceinline__ uint32_t assigned_row(const RowOrder &o, uint32_t block, uint32_t slot) {
+  if (o.period == 0) return block * kRowsPerBlock + slot;
+  const uint32_t xcd = block & 7u, j = block >> 3;
+  const uint32_t mask_row = (j / o.groups) * 8u + xcd;
+  const uint32_t repeat = (j % o.groups) * kRowsPerBlock + slot;
+  return repeat * o.period + mask_row;
+}
+
+template <class T, int kLanes, int kVpl>
+__global__ __launch_bounds__(kBlockThreads) void softmax_rows(const void *x, const void *mask,
+                                                              void *y, uint32_t rows,
+                                                              uint32_t row_vectors, float scale,
+                                                              int mask_kind, int log_form,
+                                                              MaskRows mrows, RowOrder order) {
+  constexpr int kVec = Traits<T>::kVec;
+  constexpr int kRowsPerBlock = kBlockThreads / kLanes;
+  __shared__ float joint_max[4], joint_bad[4], joint_sum[4];
+  const uint32_t lane = threadIdx.x % kLanes;
+  const uint32_t row = assigned_row<kRowsPerBlock>(order, blockIdx.x, threadIdx.x / kLanes);
+  const bool row_ok = row < rows;
+  const size_t row_base = (size_t)row * row_vectors;
+  const char *mask_row = nullptr;
+  if (mask_kind != kMaskNone && row_ok)
+    mask_row = static_cast<const char *>(mask) + mask_row_offset(mrows, row);
+
+  float v[kVpl][kVec];
+  // ---- load, scale, mask ------------------------------------------------------
+#pragma unroll
+  for (int k = 0; k < kVpl; ++k) {
+    const uint32_t vec = lane + k * kLanes;
+    const bool ok = row_ok && vec < row_vectors;
+    if (ok) {
+      Traits<T>::unpack(load16_stream(x, row_base + vec), v[k]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < kVec; ++j) v[k][j] = -INFINITY;
+    }
+  }
+  if (mask_kind == kMaskBoolean) {
+#pragma unroll
+    for (int k = 0; k < kVpl; ++k) {
+      const uint32_t vec = lane + k * kLanes;
+      if (row_ok && vec < row_vectors) {
+        uint32_t bits[kVec / 4];
+        if (mrows.inner_stride == 0) {
+          const uint32_t one = *reinterpret_cast<const uint8_t *>(mask_row) ? 0x01010101u : 0u;
+#pragma unroll
+          for (int q = 0; q < kVec / 4; ++q) bits[q] = one;
+        } else {
+          const uint32_t *words = reinterpret_cast<const uint32_t *>(mask_row) + (size_t)vec * (kVec / 4);
+#pragma unroll
+          for (int q = 0; q < kVec / 4; ++q) bits[q] = words[q];
+        }
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) {
+          const bool keep = ((bits[j / 4] >> (8 * (j % 4))) & 0xFFu) != 0;
+          v[k][j] = keep ? v[k][j] * scale : -INFINITY;
+        }
+      }
+    }
+  } else if (mask_kind == kMaskAdditive) {
+#pragma unroll
+    for (int k = 0; k < kVpl; ++k) {
+      const uint32_t vec = lane + k * kLanes;
+      if (row_ok && vec < row_vectors) {
+        float m[kVec];
+        if (mrows.inner_stride == 0) {
+          const float one = Traits<T>::load(mask_row, 0);
+#pragma unroll
+          for (int j = 0; j < kVec; ++j) m[j] = one;
+        } else {
+          Traits<T>::unpack(load16(mask_row, vec), m);
+        }
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) v[k][j] = v[k][j] * scale + m[j];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < kVpl; ++k)
+#pragma unroll
+      for (int j = 0; j < kVec; ++j) v[k][j] = v[k][j] * scale;
+  }
+
+  // ---- row maximum and validity -------------------------------------------------
+  float peak = -INFINITY, bad = 0.0f;
+#pragma unroll
+  for (int k = 0; k < kVpl; ++k)
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) {
+      const float e = v[k][j];
+      bad = (e != e || e == INFINITY) ? 1.0f : bad;
+      peak = e > peak ? e : peak;  // a NaN never replaces the running value
+    }
+  peak = row_max<kLanes>(peak, joint_max);
+  bad = row_max<kLanes>(bad, joint_bad);
+  const bool invalid = bad != 0.0f || peak == -INFINITY;
+
+  // ---- exponentials and their sum -------------------------------------------------
+  float total = 0.0f;
+#pragma unroll
+  for (int k = 0; k < kVpl; ++k)
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) {
+      const float shifted = v[k][j] - peak;
+      if (log_form) {
+        total += exp_scaled(shifted);
+        v[k][j] = shifted;
+      } else {
+        v[k][j] = exp_scaled(shifted);
+        total += v[k][j];
+      }
+    }
+  total = row_sum<kLanes>(total, joint_sum);  // = 2^32 * sum(exp)
+
+  // ---- normalise and store ------------------------------------------------------------
+  // softmax: e * 2^32 * (1 / (sum * 2^32)).  log-softmax: (v - max) - log(sum).
+  const float normaliser = log_form ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
+  const float nan = __builtin_nanf("");
+#pragma unroll
+  for (int k = 0; k < kVpl; ++k) {
+    const uint32_t vec = lane + k * kLanes;
+    if (row_ok && vec < row_vectors) {
+      float r[kVec];
+#pragma unroll
+      for (int j = 0; j < kVec; ++j) {
+        const float value = log_form ? v[k][j] - normaliser : v[k][j] * normaliser;
+        r[j] = invalid ? nan : value;
+      }
+      store16_stream(y, row_base + vec, Traits<T>::pack(r));
+    }
+  }
+}
+
+// ---- any axis, any strides: one block per (outer, inner) row, three passes ----------
+struct GeneralLayout {
+  int32_t rank, axis;
+  uint32_t dims[kMaxRank];
+  int64_t in_strides[kMaxRank];
+  int64_t mask_strides[kMaxRank];
+  uint32_t inner;
+};
+
+template <class T>
+__device__ __forceinline__ float general_value(const char *x, const char *mask,
+                                               const GeneralLayout &g, uint32_t outer,
+                                               uint32_t inner, uint32_t column, float scale,
+                                               int mask_kind) {
+  // logical index = (outer * width + column) * inner_count + inner, decoded axis by axis
+  int64_t in_off = 0, mask_off = 0;
+  uint32_t rest_inner = inner, rest_outer = outer;
+  for (int axis = g.rank - 1; axis >= 0; --axis) {
+    uint32_t coordinate;
+    if (axis > g.axis) {
+      coordinate = rest_inner % g.dims[axis];
+      rest_inner /= g.dims[axis];
+    } else if (axis == g.axis) {
+      coordinate = column;
+    } else {
+      coordinate = rest_outer % g.dims[axis];
+      rest_outer /= g.dims[axis];
+    }
+    in_off += (int64_t)coordinate * g.in_strides[axis];
+    mask_off += (int64_t)coordinate * g.mask_strides[axis];
+  }
+  float v = Traits<T>::load(x + in_off, 0) * scale;
+  if (mask_kind == kMaskBoolean)
+    v = *reinterpret_cast<const uint8_t *>(mask + mask_off) ? v : -INFINITY;
+  else if (mask_kind == kMaskAdditive)
+    v = v + Traits<T>::load(mask + mask_off, 0);
+  return v;
+}
+
+template <class T>
+__global__ __launch_bounds__(kBlockThreads) void softmax_general(const char *x, const char *mask,
+                                                                 void *y, uint32_t width,
+                                                                 float scale, int mask_kind,
+                                                                 int log_form, GeneralLayout g) {
+  __shared__ float joint_max[4], joint_bad[4], joint_sum[4];
+  const uint32_t outer = blockIdx.x / g.inner, inner = blockIdx.x % g.inner;
+  float peak = -INFINITY, bad = 0.0f;
+  for (uint32_t c = threadIdx.x; c < width; c += kBlockThreads) {
+    const float e = general_value<T>(x, mask, g, outer, inner, c, scale, mask_kind);
+    bad = (e != e || e == INFINITY) ? 1.0f : bad;
+    peak = e > peak ? e : peak;
+  }
+  peak = row_max<kBlockThreads>(peak, joint_max);
+  bad = row_max<kBlockThreads>(bad, joint_bad);
+  const bool invalid = bad != 0.0f || peak == -INFINITY;
+  float total = 0.0f;
+  for (uint32_t c = threadIdx.x; c < width; c += kBlockThreads)
+    total += exp_scaled(general_value<T>(x, mask, g, outer, inner, c, scale, mask_kind) - peak);
+  total = row_sum<kBlockThreads>(total, joint_sum);
+  const float normaliser = log_form ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
+  // every read of this row is complete: an exact input alias may now be overwritten
+  __syncthreads();
+  for (uint32_t c = threadIdx.x; c < width; c += kBlockThreads) {
+    const float shifted = general_value<T>(x, mask, g, outer, inner, c, scale, mask_kind) - peak;
+    const float value = log_form ? shifted - normaliser : exp_scaled(shifted) * normaliser;
+    const size_t logical = ((size_t)outer * width + c) * g.inner + inner;
+    Traits<T>::store(y, logical, invalid ? __builtin_nanf("") : value);
+  }
+}
+
+// ---- last-axis Reduce -------------------------------------------------------------------
+enum : int { kSum = 0, kMean = 1, kMinimum = 2, kMaximum = 3 };
+
+template <int kKind> __device__ __forceinline__ float reduce_identity() {
+  return kKind == kMinimum ? INFINITY : kKind == kMaximum ? -INFINITY : 0.0f;
+}
+template <int kKind> __device__ __forceinline__ float reduce_step(float acc, float v) {
+  if constexpr (kKind == kMinimum) return min_propagate(acc, v);
+  else if constexpr (kKind == kMaximum) return max_propagate(acc, v);
+  else return acc + v;
+}
+
+template <class T, int kKind, int kLanes, bool kVector>
+__global__ __launch_bounds__(kBlockThreads) void reduce_rows(const void *x, void *y, uint32_t rows,
+                                                             uint32_t width) {
+  constexpr int kVec = Traits<T>::kVec;
+  constexpr int kRowsPerBlock = kBlockThreads / kLanes;
+  __shared__ float joint[4];
+  const uint32_t lane = threadIdx.x % kLanes;
+  const uint32_t row = blockIdx.x * kRowsPerBlock + threadIdx.x / kLanes;
+  const bool row_ok = row < rows;
+  float acc = reduce_identity<kKind>();
+  if (row_ok) {
+    if constexpr (kVector) {
+      const uint32_t vectors = width / kVec;
+      const size_t base = (size_t)row * vectors;
+      for (uint32_t vec = lane; vec < vectors; vec += kLanes) {
+        float v[kVec];
+        Traits<T>::unpack(load16_stream(x, base + vec), v);
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) acc = reduce_step<kKind>(acc, v[j]);
+      }
+    } else {
+      const size_t base = (size_t)row * width;
+      for (uint32_t i = lane; i < width; i += kLanes)
+        acc = reduce_step<kKind>(acc, Traits<T>::load(x, base + i));
+    }
+  }
+  auto combine = [](LaneF32 a, LaneF32 b) { return LaneF32{reduce_step<kKind>(a.x, b.x)}; };
+  acc = group_reduce<(kLanes < kWaveLanes ? kLanes : kWaveLanes)>(LaneF32{acc}, combine).x;
+  if constexpr (kLanes > kWaveLanes) {
+    if ((threadIdx.x & (kWaveLanes - 1)) == 0) joint[threadIdx.x / kWaveLanes] = acc;
+    __syncthreads();
+    acc = reduce_step<kKind>(reduce_step<kKind>(joint[0], joint[1]),
+                             reduce_step<kKind>(joint[2], joint[3]));
+  }
+  if (row_ok && lane == 0) {
+    if constexpr (kKind == kMean) acc = width == 0 ? __builtin_nanf("") : acc / (float)width;
+    Traits<T>::store(y, row, acc);
+  }
+}
+
+// ---- host dispatch ----------------------------------------------------------------------------
+template <class T, int kLanes, int kVpl>
+hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, void *y,
+                    hipStream_t s) {
+  constexpr int kRowsPerBlock = kBlockThreads / kLanes;
+  const uint32_t rows = (uint32_t)p.shape.rows;
+  const uint32_t blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+  MaskRows m{};
+  m.outer_rank = p.outer_rank;
+  for (int i = 0; i < kMaxRank; ++i) {
+    m.outer_dims[i] = p.outer_dims[i];
+    m.outer_strides[i] = p.mask_outer_strides[i];
+  }
+  m.inner_stride = p.mask_inner_stride;
+  RowOrder order{0, 0};
+  if (p.mask_kind != kMaskNone && p.mask_period != 0 && p.mask_period % 8 == 0 &&
+      p.shape.rows % p.mask_period == 0) {
+    const uint64_t repeats = p.shape.rows / p.mask_period;
+    if (repeats > 1 && repeats % kRowsPerBlock == 0) {
+      order.period = (uint32_t)p.mask_period;
+      order.groups = (uint32_t)(repeats / kRowsPerBlock);
+    }
+  }
+  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl>), dim3(blocks), dim3(kBlockThreads), 0, s, x,
+                     mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, (int)p.mask_kind,
+                     p.log ? 1 : 0, m, order);
+  return hipGetLastError();
+}
+
+template <class T>
+hipError_t run_softmax(const SoftmaxParams &p, const void *x, const void *mask, void *y,
+                       hipStream_t s) {
+  const uint32_t vectors = p.shape.width / Traits<T>::kVec;
+  if (vectors <= 8) return run_rows<T, 8, 1>(p, x, mask, y, s);
+  if (vectors <= 16) return run_rows<T, 16, 1>(p, x, mask, y, s);
+  if (vectors <= 32) return run_rows<T, 32, 1>(p, x, mask, y, s);
+  if (vectors <= 64) return run_rows<T, 64, 1>(p, x, mask, y, s);
+  if (vectors <= 128) return run_rows<T, 64, 2>(p, x, mask, y, s);
+  if (vectors <= 256) return run_rows<T, 64, 4>(p, x, mask, y, s);
+  if (vectors <= 512) return run_rows<T, 64, 8>(p, x, mask, y, s);
+  if (vectors <= 1024) return run_rows<T, 256, 4>(p, x, mask, y, s);
+  if (vectors <= 2048) return run_rows<T, 256, 8>(p, x, mask, y, s);
+  return run_rows<T, 256, 16>(p, x, mask, y, s);
+}
+
+template <class T>
+hipError_t run_general(const SoftmaxGeneralParams &p, const void *x, const void *mask, void *y,
+                       hipStream_t s) {
+  GeneralLayout g{};
+  g.rank = p.rank;
+  g.axis = p.axis;
+  g.inner = (uint32_t)p.inner;
+  for (int i = 0; i < kMaxRank; ++i) {
+    g.dims[i] = p.dims[i];
+    g.in_strides[i] = p.in_strides[i];
+    g.mask_strides[i] = p.mask_strides[i];
+  }
+  hipLaunchKernelGGL((softmax_general<T>), dim3((uint32_t)(p.outer * p.inner)), dim3(kBlockThreads),
+                     0, s, static_cast<const char *>(x), static_cast<const char *>(mask), y, p.width,
+                     p.scale, (int)p.mask_kind, p.log ? 1 : 0, g);
+  return hipGetLastError();
+}
+
+template <class T, int kKind>
+hipError_t run_reduce_kind(const ReduceParams &p, const void *x, void *y, bool vectorised,
+                           hipStream_t s) {
+  const uint32_t rows = (uint32_t)p.shape.rows, width = p.shape.width;
+  const bool vec = vectorised && width % Traits<T>::kVec == 0;
+  const bool wide = (size_t)width * Traits<T>::kSize >= 8192;
+  if (wide) {
+    if (vec)
+      hipLaunchKernelGGL((reduce_rows<T, kKind, kBlockThreads, true>), dim3(rows),
+                         dim3(kBlockThreads), 0, s, x, y, rows, width);
+    else
+      hipLaunchKernelGGL((reduce_rows<T, kKind, kBlockThreads, false>), dim3(rows),
+                         dim3(kBlockThreads), 0, s, x, y, rows, width);
+  } else {
+    const uint32_t blocks = (rows + 3) / 4;
+    if (vec)
+      hipLaunchKernelGGL((reduce_rows<T, kKind, kWaveLanes, true>), dim3(blocks),
+                         dim3(kBlockThreads), 0, s, x, y, rows, width);
+    else
+      hipLaunchKernelGGL((reduce_rows<T, kKind, kWaveLanes, false>), dim3(blocks),
+                         dim3(kBlockThreads), 0, s, x, y, rows, width);
+  }
+  return hipGetLastError();
+}
+
+template <class T>
+hipError_t run_reduce(const ReduceParams &p, const void *x, void *y, bool vectorised,
+                      hipStream_t s) {
+  switch (p.kind) {
+    case kSum: return run_reduce_kind<T, kSum>(p, x, y, vectorised, s);
+    case kMean: return run_reduce_kind<T, kMean>(p, x, y, vectorised, s);
+    case kMinimum: return run_reduce_kind<T, kMinimum>(p, x, y, vectorised, s);
+    case kMaximum: return run_reduce_kind<T, kMaximum>(p, x, y, vectorised, s);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace
+
+hipError_t launch_softmax(Elem type, const SoftmaxParams &p, const void *x, const void *mask,
+                          void *y, bool vectorised, int /*compute_units*/, hipStream_t stream) {
+  if (p.shape.rows == 0 || p.shape.width == 0) return hipSuccess;
+  if (!vectorised) return hipErrorInvalidValue;  // the caller routes those to the general kernel
+  switch (type) {
+    case Elem::kF32: return run_softmax<F32>(p, x, mask, y, stream);
+    case Elem::kF16: return run_softmax<F16>(p, x, mask, y, stream);
+    case Elem::kBF16: return run_softmax<BF16>(p, x, mask, y, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_softmax_general(Elem type, const SoftmaxGeneralParams &p, const void *x,
+                                  const void *mask, void *y, hipStream_t stream) {
+  if (p.outer == 0 || p.inner == 0 || p.width == 0) return hipSuccess;
+  switch (type) {
+    case Elem::kF32: return run_general<F32>(p, x, mask, y, stream);
+    case Elem::kF16: return run_general<F16>(p, x, mask, y, stream);
+    case Elem::kBF16: return run_general<BF16>(p, x, mask, y, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+hipError_t launch_reduce_rows(Elem type, const ReduceParams &p, const void *x, void *y,
+                              bool vectorised, hipStream_t stream) {
+  if (p.shape.rows == 0) return hipSuccess;
+  switch (type) {
+    case Elem::kF32: return run_reduce<F32>(p, x, y, vectorised, stream);
+    case Elem::kF16: return run_reduce<F16>(p, x, y, vectorised, stream);
+    case Elem::kBF16: return run_reduce<BF16>(p, x, y, vectorised, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace hyle_hip

@@ -1,0 +1,218 @@
+/*
+ * hyle_hip.h -- C ABI of the MI355X (gfx950) compute provider for HYLE's tensor
+ * hot path: broadcast Binary, Unary SiLU, GatedActivation (SwiGLU), RMSNorm,
+ * row Softmax, last-axis Reduce, TopK(count = 1) and Q8_0 block dequant.
+ *
+ * The surface is what a `hyle::compute` provider for this path binds: one cold
+ * "plan" per (Operation, input descriptors) pair -- the reference's
+ * propose + prepare -- and one allocation-free, non-blocking launch per
+ * submit on a caller-owned HIP stream.  Plain pointers and sizes only.
+ *
+ * Enumerator values are the reference's own so that an adapter can cast:
+ *   hyle_hip_status     <- hyle::StatusCode          (include/hyle/error/status.h:18-38)
+ *   hyle_hip_dtype      <- hyle::compute::DataType   (include/hyle/compute/tensor_desc.h:17-34)
+ *   hyle_hip_op_kind    <- hyle::compute::OperationKind (include/hyle/compute/operation.h:22-48)
+ *   sub-kinds           <- UnaryKind / BinaryKind / ReductionKind /
+ *                          GatedActivationKind / GatedInputKind / SoftmaxKind /
+ *                          MaskKind (include/hyle/compute/operation.h:57-126)
+ */
+#ifndef HYLE_HIP_H_
+#define HYLE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define HYLE_HIP_API __attribute__((visibility("default")))
+#else
+#define HYLE_HIP_API
+#endif
+
+#define HYLE_HIP_MAX_RANK 8      /* hyle::compute::kMaxTensorRank */
+#define HYLE_HIP_MAX_INPUTS 4
+#define HYLE_HIP_MAX_OUTPUTS 2
+#define HYLE_HIP_ABI_VERSION 1u
+
+/* hyle::StatusCode.  UNIMPLEMENTED from plan_create is a clean decline (the
+ * caller tries its next provider, src/compute/operation.cc:1259-1266); every
+ * other non-OK code is an error. */
+typedef enum hyle_hip_status {
+  HYLE_HIP_OK = 0,
+  HYLE_HIP_INVALID_ARGUMENT = 3,
+  HYLE_HIP_RESOURCE_EXHAUSTED = 8,
+  HYLE_HIP_FAILED_PRECONDITION = 9,
+  HYLE_HIP_OUT_OF_RANGE = 11,
+  HYLE_HIP_UNIMPLEMENTED = 12,
+  HYLE_HIP_INTERNAL = 13,
+  HYLE_HIP_UNAVAILABLE = 14
+} hyle_hip_status;
+
+typedef enum hyle_hip_dtype {
+  HYLE_HIP_DTYPE_UNKNOWN = 0,
+  HYLE_HIP_DTYPE_BOOL = 1,
+  HYLE_HIP_DTYPE_F16 = 4,
+  HYLE_HIP_DTYPE_BF16 = 5,
+  HYLE_HIP_DTYPE_F32 = 6,
+  HYLE_HIP_DTYPE_I8 = 8,
+  HYLE_HIP_DTYPE_U8 = 9,
+  HYLE_HIP_DTYPE_I32 = 12
+} hyle_hip_dtype;
+
+typedef enum hyle_hip_op_kind {
+  HYLE_HIP_OP_UNARY = 5,
+  HYLE_HIP_OP_BINARY = 6,
+  HYLE_HIP_OP_REDUCE = 8,
+  HYLE_HIP_OP_RMS_NORM = 9,
+  HYLE_HIP_OP_GATED_ACTIVATION = 12,
+  HYLE_HIP_OP_SOFTMAX = 18,
+  HYLE_HIP_OP_TOP_K = 19,
+  /* Fused forms with no single counterpart in the reference schema; a HYLE
+   * adapter reaches them through OperationKind::kCustom (24). */
+  /* out = (in0 kind in1) kind2 in2, the intermediate rounded to the storage
+   * type: bit-identical to two chained Binary operations. */
+  HYLE_HIP_OP_BINARY_CHAIN = 0x100,
+  /* in0: Q8_0 blocked weight, logical [K, N], physical rows of K/32 blocks;
+   * out0: bf16 [N, K] dense; out1: f32 [N] row sum of squares of the exact
+   * f32 products. */
+  HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ = 0x101
+} hyle_hip_op_kind;
+
+/* UnaryKind (include/hyle/compute/operation.h:57-73); only SiLU is on the path. */
+enum { HYLE_HIP_UNARY_SILU = 11 };
+/* BinaryKind (include/hyle/compute/operation.h:75-82) */
+enum {
+  HYLE_HIP_BINARY_ADD = 0,
+  HYLE_HIP_BINARY_SUBTRACT = 1,
+  HYLE_HIP_BINARY_MULTIPLY = 2,
+  HYLE_HIP_BINARY_DIVIDE = 3,
+  HYLE_HIP_BINARY_MINIMUM = 4,
+  HYLE_HIP_BINARY_MAXIMUM = 5
+};
+/* ReductionKind (include/hyle/compute/operation.h:84-89) */
+enum {
+  HYLE_HIP_REDUCE_SUM = 0,
+  HYLE_HIP_REDUCE_MEAN = 1,
+  HYLE_HIP_REDUCE_MINIMUM = 2,
+  HYLE_HIP_REDUCE_MAXIMUM = 3
+};
+/* GatedActivationKind / GatedInputKind (include/hyle/compute/operation.h:91-100) */
+enum { HYLE_HIP_GATED_SILU = 0 };
+enum { HYLE_HIP_GATED_PACKED_HALVES = 0, HYLE_HIP_GATED_SEPARATE = 1 };
+/* SoftmaxKind / MaskKind (include/hyle/compute/operation.h:117-126) */
+enum { HYLE_HIP_SOFTMAX = 0, HYLE_HIP_LOG_SOFTMAX = 1 };
+enum { HYLE_HIP_MASK_NONE = 0, HYLE_HIP_MASK_ADDITIVE = 1, HYLE_HIP_MASK_BOOLEAN = 2 };
+
+/* StorageFormatKind (include/hyle/compute/tensor_desc.h:77-81) */
+enum { HYLE_HIP_STORAGE_PLAIN = 0, HYLE_HIP_STORAGE_BLOCKED = 1 };
+
+/* hyle::compute::TensorDesc as plain data
+ * (include/hyle/compute/tensor_desc.h:141-225): logical dims, BYTE strides, a
+ * zero stride on an axis of extent > 1 is a broadcast; blocked storage names
+ * its block axis and block geometry. */
+typedef struct hyle_hip_tensor_desc {
+  uint8_t dtype;        /* hyle_hip_dtype */
+  uint8_t rank;         /* 0..8 */
+  uint8_t storage;      /* HYLE_HIP_STORAGE_* */
+  uint8_t block_axis;   /* valid when storage == BLOCKED */
+  uint32_t elements_per_block;
+  uint32_t bytes_per_block;
+  uint32_t reserved;
+  int64_t dims[HYLE_HIP_MAX_RANK];
+  int64_t byte_strides[HYLE_HIP_MAX_RANK];
+} hyle_hip_tensor_desc;
+
+/* One hyle::compute::Operation plus its exact input descriptors
+ * (ProviderOperationRequest, src/compute/provider_internal.h:45-53). */
+typedef struct hyle_hip_op_desc {
+  uint32_t abi_version;      /* HYLE_HIP_ABI_VERSION */
+  uint32_t op;               /* hyle_hip_op_kind */
+  uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind */
+  uint32_t kind2;            /* BINARY_CHAIN: second BinaryKind; GATED: GatedInputKind;
+                                SOFTMAX: SoftmaxKind */
+  int32_t axis;              /* Softmax / TopK / Reduce axis (negative counts from the end) */
+  uint32_t mask;             /* Softmax MaskKind */
+  uint32_t accumulation;     /* hyle_hip_dtype; UNKNOWN or F32 */
+  uint32_t keep_dimensions;  /* Reduce */
+  float epsilon;             /* RmsNorm */
+  float scale;               /* Softmax */
+  uint64_t count;            /* TopK count (only 1 is implemented) */
+  uint32_t largest;          /* TopK */
+  uint32_t input_count;
+  hyle_hip_tensor_desc inputs[HYLE_HIP_MAX_INPUTS];
+} hyle_hip_op_desc;
+
+typedef struct hyle_hip_context hyle_hip_context;
+typedef struct hyle_hip_plan hyle_hip_plan;
+
+/* ProviderVTable::create_context / destroy_context
+ * (src/compute/provider_internal.h:124-129).  Binds one HIP device; fails with
+ * UNAVAILABLE when no gfx950 device is present. */
+HYLE_HIP_API hyle_hip_status hyle_hip_context_create(int device, hyle_hip_context **context);
+HYLE_HIP_API void hyle_hip_context_destroy(hyle_hip_context *context);
+/* Compute units of the bound device. */
+HYLE_HIP_API int hyle_hip_context_compute_units(const hyle_hip_context *context);
+
+/* Provider-neutral output inference, hyle::compute::infer_output_descriptions
+ * (src/compute_ops/operation.cc:1214-1704) for the operations above.  Needs no
+ * device.  Writes up to HYLE_HIP_MAX_OUTPUTS descriptors. */
+HYLE_HIP_API hyle_hip_status hyle_hip_infer_outputs(const hyle_hip_op_desc *request,
+                                                    hyle_hip_tensor_desc *outputs,
+                                                    uint32_t *output_count);
+
+/* ProviderVTable::propose + prepare (src/compute/provider_internal.h:130-142):
+ * validates the request against the schema, then admits it into a kernel route.
+ * `outputs` may be NULL (inferred dense outputs) or the caller's exact output
+ * descriptors, which must equal the inferred ones. */
+HYLE_HIP_API hyle_hip_status hyle_hip_plan_create(hyle_hip_context *context,
+                                                  const hyle_hip_op_desc *request,
+                                                  const hyle_hip_tensor_desc *outputs,
+                                                  uint32_t output_count, hyle_hip_plan **plan);
+/* ProviderPreparedVTable::destroy_prepared
+ * (include/hyle/compute/detail/prepared_callbacks.h:15-16). */
+HYLE_HIP_API void hyle_hip_plan_destroy(hyle_hip_plan *plan);
+
+/* ProviderPrepared::workspace (src/compute/provider_internal.h:85-88):
+ * caller-owned device scratch the launch needs; size 0 for most routes. */
+HYLE_HIP_API hyle_hip_status hyle_hip_plan_workspace(const hyle_hip_plan *plan, size_t *size,
+                                                     size_t *alignment);
+/* The inferred output descriptors of a plan. */
+HYLE_HIP_API hyle_hip_status hyle_hip_plan_outputs(const hyle_hip_plan *plan,
+                                                   hyle_hip_tensor_desc *outputs,
+                                                   uint32_t *output_count);
+/* ProviderPreparedVTable::alias_support
+ * (include/hyle/compute/detail/prepared_callbacks.h:17-18): 1 when output
+ * `output_index` may share exact storage with input `input_index`. */
+HYLE_HIP_API int hyle_hip_plan_alias_support(const hyle_hip_plan *plan, uint32_t output_index,
+                                             uint32_t input_index);
+/* ProviderRouteCostFacts::dispatch_count
+ * (include/hyle/compute/prepared_operation.h:51-67): kernels one launch enqueues. */
+HYLE_HIP_API uint32_t hyle_hip_plan_dispatch_count(const hyle_hip_plan *plan);
+/* Name of the kernel route the plan selected (diagnostics, profiling). */
+HYLE_HIP_API const char *hyle_hip_plan_route_name(const hyle_hip_plan *plan);
+
+/* ProviderPreparedVTable::shared_submit
+ * (include/hyle/compute/detail/prepared_callbacks.h:26-30): enqueue on `stream`
+ * (a hipStream_t; NULL is the default stream) and return without waiting.
+ * Pointers are device addresses of the tensors' first logical element.  No
+ * allocation, no synchronisation.  A non-OK return means nothing was enqueued
+ * (EnqueueResult::rejected).  Zero-element tensors succeed without touching
+ * storage. */
+HYLE_HIP_API hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan,
+                                                  const void *const *inputs, uint32_t input_count,
+                                                  void *const *outputs, uint32_t output_count,
+                                                  void *workspace, size_t workspace_size,
+                                                  void *stream);
+
+/* Text of the last non-OK status returned on the calling thread. */
+HYLE_HIP_API const char *hyle_hip_last_error(void);
+HYLE_HIP_API const char *hyle_hip_status_name(hyle_hip_status status);
+HYLE_HIP_API uint32_t hyle_hip_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HYLE_HIP_H_ */
