@@ -1,0 +1,394 @@
+#!/usr/bin/env python3
+"""Measures the tensor hot path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input: the largest shape of
+each of the five benchmark configurations, seven kernels launched back to back through the
+C ABI of libhyle_hip.so on one HIP stream:
+
+    cfg1  f32  (A[4096,2048] + b[2048]) * 0.5          BinaryChain (add, multiply)
+    cfg2  bf16 RMSNorm X[8192,2048], w[2048], eps 1e-6
+    cfg3  bf16 SwiGLU gate/up[8192,6144]                GatedActivation (SiLU, separate)
+    cfg3' bf16 R[8192,2048] += Y                        Binary add, output aliases input 0
+    cfg4  f32  softmax S[32,4096,4096] + causal Bool mask [4096,4096]
+    cfg4' f32  argmax logits[64,151936]                 TopK(count = 1)
+    cfg5  Q8_0 W[6144 rows x 2048] -> bf16 + f32 row sum of squares
+
+Inputs are resident in HBM before the timed region.  Shapes whose traffic fits the 256 MB
+memory-side cache rotate over several buffer sets (> 512 MB in total) so that HBM, not the
+cache, is measured.  `value` is algorithmic bytes per step / step time; `roofline` describes
+the dominant kernel (softmax) timed with HIP events inside the timed region; `per_op` holds
+each kernel's own figure from an event-timed loop of back-to-back launches; `cpu_baseline`
+times the CPU oracle ("port" of the reference's CPU path) on a bounded sample of the same
+workload on the host cores.
+
+Prints one JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=5)
+    p.add_argument("--op-reps", type=int, default=200, help="launches per kernel in the per-op timing loops")
+    p.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    p.add_argument("--cpu-seconds", type=float, default=2.0, help="target CPU seconds per kernel sample")
+    p.add_argument("--only", default="", help="comma-separated op names: run and time just these kernels")
+    return p.parse_args()
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from hyle_amd import compute as hc
+    from hyle_amd import torch_io as tio
+    from hyle_amd import workloads as wl
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        return 2
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    ctx = hc.Context.create(0)
+    stream = torch.cuda.current_stream().cuda_stream
+    BK = hc.BinaryKind
+
+    def bf16(bits):
+        return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).to(dev).view(torch.bfloat16)
+
+    class Op:
+        """One kernel of the step: a prepared operation plus `sets` rotating buffer sets."""
+
+        def __init__(self, name, operation, descs, make_set, sets, algorithmic_bytes, elements, dtype):
+            self.name, self.bytes, self.elements, self.dtype = name, algorithmic_bytes, elements, dtype
+            self.bound = tio.Bound(ctx, operation, descs, device=dev)
+            self.route = self.bound.prepared.route_name()
+            self.sets = [make_set(i) for i in range(sets)]  # each: (inputs, outputs)
+            self.addresses = [([t.data_ptr() for t in i], [t.data_ptr() for t in o]) for i, o in self.sets]
+            self.turn = 0
+
+        def launch(self, on_stream):
+            """Enqueue on the HIP stream `on_stream`, rotating to the next buffer set."""
+            inputs, outputs = self.addresses[self.turn]
+            self.turn = (self.turn + 1) % len(self.sets)
+            self.bound.invocation.submit(on_stream, inputs, outputs)
+
+    D = hc.TensorDesc.dense
+    F32, BF = hc.DataType.kFloat32, hc.DataType.kBFloat16
+    ops = []
+    wanted = {n for n in args.only.split(",") if n}
+
+    def want(name):
+        return not wanted or name in wanted
+
+    # ---- cfg1 ---------------------------------------------------------------------------
+    if want("cfg1_broadcast_add_mul_f32"):
+        a, b, s = wl.config1()
+        db, ds = torch.from_numpy(b).to(dev), torch.from_numpy(s).to(dev)
+
+        def set1(i):
+            da = torch.from_numpy(np.roll(a, i, axis=0)).to(dev)
+            return [da, db, ds], [torch.empty_like(da)]
+        ops.append(Op("cfg1_broadcast_add_mul_f32", hc.BinaryChain(BK.kAdd, BK.kMultiply),
+                      [D(F32, [4096, 2048]), D(F32, [2048]), D(F32, [1])], set1, 10,
+                      wl.ALGORITHMIC_BYTES["cfg1_broadcast_add_mul_f32"], 4096 * 2048, "f32"))
+    # ---- cfg2 ---------------------------------------------------------------------------
+    if want("cfg2_rmsnorm_bf16"):
+        x, w = wl.config2()
+        dw = bf16(w)
+
+        def set2(i):
+            dx = bf16(np.roll(x, i, axis=0))
+            return [dx, dw], [torch.empty_like(dx)]
+        ops.append(Op("cfg2_rmsnorm_bf16", hc.RmsNorm(epsilon=1e-6), [D(BF, [8192, 2048]), D(BF, [2048])], set2, 10,
+                      wl.ALGORITHMIC_BYTES["cfg2_rmsnorm_bf16"], 8192 * 2048, "bf16"))
+    # ---- cfg3 ---------------------------------------------------------------------------
+    if want("cfg3_swiglu_bf16"):
+        gate, up = wl.config3_swiglu()
+
+        def set3(i):
+            dg, du = bf16(np.roll(gate, i, axis=0)), bf16(np.roll(up, i, axis=0))
+            return [dg, du], [torch.empty_like(dg)]
+        ops.append(Op("cfg3_swiglu_bf16", hc.GatedActivation(hc.GatedActivationKind.kSilu, hc.GatedInputKind.kSeparate),
+                      [D(BF, [8192, 6144]), D(BF, [8192, 6144])], set3, 3,
+                      wl.ALGORITHMIC_BYTES["cfg3_swiglu_bf16"], 8192 * 6144, "bf16"))
+    if want("cfg3_residual_add_bf16"):
+        r, y = wl.config3_residual()
+
+        def set3r(i):
+            dr, dy = bf16(np.roll(r, i, axis=0)), bf16(np.roll(y, i, axis=0))
+            return [dr, dy], [dr]  # R += Y
+        ops.append(Op("cfg3_residual_add_bf16", hc.Binary(BK.kAdd), [D(BF, [8192, 2048]), D(BF, [8192, 2048])],
+                      set3r, 10, wl.ALGORITHMIC_BYTES["cfg3_residual_add_bf16"], 8192 * 2048, "bf16"))
+    # ---- cfg4 ---------------------------------------------------------------------------
+    if want("cfg4_softmax_f32_causal"):
+        gen = torch.Generator(device=dev).manual_seed(3)
+        big = torch.randn((32, 4096, 4096), generator=gen, device=dev, dtype=torch.float32).mul_(3.0)
+        causal = torch.ones((4096, 4096), dtype=torch.bool, device=dev).tril_()
+        big_out = torch.empty_like(big)
+        ops.append(Op("cfg4_softmax_f32_causal", hc.Softmax(mask=hc.MaskKind.kBoolean),
+                      [D(F32, [32, 4096, 4096]), D(hc.DataType.kBool, [4096, 4096])],
+                      lambda i: ([big, causal], [big_out]), 1,
+                      wl.ALGORITHMIC_BYTES["cfg4_softmax_f32_causal"], 32 * 4096 * 4096, "f32"))
+    if want("cfg4_argmax_f32"):
+        logits = wl.config4_argmax()
+
+        def set4a(i):
+            dl = torch.from_numpy(np.roll(logits, i, axis=0)).to(dev)
+            return [dl], [torch.empty((64, 1), dtype=torch.float32, device=dev),
+                          torch.empty((64, 1), dtype=torch.int32, device=dev)]
+        ops.append(Op("cfg4_argmax_f32", hc.TopK(), [D(F32, [64, 151936])], set4a, 16,
+                      wl.ALGORITHMIC_BYTES["cfg4_argmax_f32"], 64 * 151936, "f32"))
+    # ---- cfg5 ---------------------------------------------------------------------------
+    if want("cfg5_q8_0_dequant_sumsq"):
+        blocks = wl.config5()
+
+        def set5(i):
+            dbk = torch.from_numpy(np.roll(blocks, i, axis=0)).to(dev)
+            return [dbk], [torch.empty((6144, 2048), dtype=torch.bfloat16, device=dev),
+                           torch.empty(6144, dtype=torch.float32, device=dev)]
+        ops.append(Op("cfg5_q8_0_dequant_sumsq", hc.Q8_0DequantSumSquares(),
+                      [hc.TensorDesc.gguf_q8_0_weight(BF, 2048, 6144)], set5, 16,
+                      wl.ALGORITHMIC_BYTES["cfg5_q8_0_dequant_sumsq"], 6144 * 2048, "u8/bf16"))
+    if not ops:
+        print("no kernel selected", file=sys.stderr)
+        return 2
+
+    dominant = max(ops, key=lambda o: o.bytes)
+    step_bytes = sum(o.bytes for o in ops)
+    step_elements = sum(o.elements for o in ops)
+    before = ops[:ops.index(dominant)]
+    after = ops[ops.index(dominant) + 1:]
+
+    # Every kernel runs once eagerly (code objects load on first use), then the short
+    # kernels are captured into HIP graphs: their 5-50 us run times are of the order of
+    # one launch call, so eager submission would measure the host, not the GPU.  The
+    # reference replays captured graphs the same way (capture_compatible,
+    # include/hyle/compute/provider.h:136-139).  One graph per rotation phase.
+    for op in ops:
+        op.launch(stream)
+    torch.cuda.synchronize()
+    PHASES = 16
+
+    def capture(members, launches_each=1):
+        graphs = []
+        if not members:
+            return graphs
+        for _ in range(PHASES if launches_each == 1 else 1):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                s = torch.cuda.current_stream().cuda_stream
+                for _ in range(launches_each):
+                    for op in members:
+                        op.launch(s)
+            graphs.append(g)
+        return graphs
+
+    graphs_before, graphs_after = capture(before), capture(after)
+
+    def step(i, events=None):
+        if graphs_before:
+            graphs_before[i % PHASES].replay()
+        if events is not None:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            dominant.launch(stream)
+            e1.record()
+            events.append((e0, e1))
+        else:
+            dominant.launch(stream)
+        if graphs_after:
+            graphs_after[i % PHASES].replay()
+
+    # ---- whole-step timing ----------------------------------------------------------------
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    events = []
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i, events)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    dominant_us = sum(a.elapsed_time(b) for a, b in events) * 1e3 / len(events)
+
+    # ---- per-kernel timing: a graph of back-to-back launches between two HIP events ---------
+    per_op = []
+    for op in ops:
+        reps = args.op_reps if op.bytes < (1 << 30) else max(10, args.op_reps // 10)
+        (graph,) = capture([op], launches_each=reps)
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / reps
+        gbps = op.bytes / us / 1e3
+        per_op.append({"op": op.name, "route": op.route, "dtype": op.dtype, "bytes": op.bytes,
+                       "buffer_sets": len(op.sets), "launches": reps, "us": round(us, 3),
+                       "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                       "gelem_per_s": round(op.elements / us / 1e3, 2)})
+        del graph
+
+    achieved = dominant.bytes / dominant_us / 1e3
+    result = {
+        "metric": "achieved HBM GB/s and % of 8 TB/s peak per op (RMSNorm, SwiGLU, softmax)",
+        "value": round(step_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32+bf16+u8", "data": "synthetic",
+        "config": {"workload": "one pass over the largest shape of configs 1-5: " + ", ".join(o.name for o in ops),
+                   "algorithmic_bytes_per_step": step_bytes, "elements_per_step": step_elements,
+                   "gelem_per_s": round(step_elements / (ms_per_step * 1e-3) / 1e9, 2),
+                   "buffer_rotation": "shapes under 256 MB rotate over buffer sets totalling > 512 MB"},
+        "roofline": {"bound": "hbm", "kernel": dominant.name, "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "us_per_launch": round(dominant_us, 2), "traffic": TRAFFIC.get(dominant.name)},
+        "per_op": per_op,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(args, ops, np, torch, wl)
+    print(json.dumps(result))
+    return 0
+
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# (summaries under profiles/); None until measured.
+TRAFFIC = {}
+
+
+def cpu_baseline(args, ops, np, torch, wl):
+    """Times the CPU oracle's dense row loops (the "port" of the reference's CPU provider path)
+    on a bounded sample of each kernel's workload, rows fanned out over threads with the
+    reference's rule: tasks = min(cores, rows, ceil(rows * width / 16384)), contiguous ranges,
+    remainder over the first tasks (src/compute_provider_native/native_provider.cc:47-69,
+    native_plan.h:74-111)."""
+    import ctypes as C
+
+    from oracle import lib as orc
+
+    lib = C.CDLL(os.path.join(ROOT, "oracle", "libhyle_oracle.so"))
+    vp, sz = C.c_void_p, C.c_size_t
+    cores = min(len(os.sched_getaffinity(0)), 16)
+    pool = ThreadPoolExecutor(max_workers=cores)
+
+    def ptr(a):
+        return a.ctypes.data_as(vp)
+
+    def fan_out(rows, width, call):
+        tasks = max(1, min(cores, rows, -(-rows * width // 16384)))
+        base, rem = divmod(rows, tasks)
+        ranges, begin = [], 0
+        for i in range(tasks):
+            end = begin + base + (1 if i < rem else 0)
+            ranges.append((begin, end))
+            begin = end
+        list(pool.map(lambda be: call(*be), ranges))
+
+    def timed(rows_full, width, bytes_full, make_call):
+        """Grow the sample until it costs about --cpu-seconds; return (rows, seconds)."""
+        rows = max(cores, min(rows_full, 64))
+        while True:
+            call = make_call(rows)
+            t0 = time.perf_counter()
+            fan_out(rows, width, call)
+            dt = time.perf_counter() - t0
+            if dt >= args.cpu_seconds * 0.5 or rows == rows_full:
+                return rows, dt
+            grow = max(2.0, min(16.0, args.cpu_seconds / max(dt, 1e-4)))
+            rows = int(min(rows_full, rows * grow))
+
+    names = {o.name for o in ops}
+    samples, total_seconds_full = [], 0.0
+
+    def record(name, rows_full, rows, dt, bytes_full):
+        nonlocal total_seconds_full
+        full = dt * rows_full / rows
+        total_seconds_full += full
+        samples.append(f"{name}: {rows}/{rows_full} rows in {dt:.2f}s = {bytes_full * rows / rows_full / dt / 1e9:.2f} GB/s")
+
+    if "cfg1_broadcast_add_mul_f32" in names:
+        a, b, s = wl.config1()
+        out = np.empty_like(a)
+        fn = lib.hyle_oracle_rows_add_row_scale_f32
+        fn.argtypes = [vp, vp, C.c_float, vp, sz, sz, sz]
+        rows, dt = timed(4096, 2048, 0, lambda n: (lambda b0, e0: fn(ptr(a), ptr(b), 0.5, ptr(out), 2048, b0, e0)))
+        record("cfg1", 4096, rows, dt, wl.ALGORITHMIC_BYTES["cfg1_broadcast_add_mul_f32"])
+    if "cfg2_rmsnorm_bf16" in names:
+        x, w = wl.config2()
+        out = np.empty_like(x)
+        fn = lib.hyle_oracle_rows_rms_norm_bf16
+        fn.argtypes = [vp, vp, vp, sz, C.c_float, sz, sz]
+        rows, dt = timed(8192, 2048, 0, lambda n: (lambda b0, e0: fn(ptr(x), ptr(w), ptr(out), 2048, 1e-6, b0, e0)))
+        record("cfg2", 8192, rows, dt, wl.ALGORITHMIC_BYTES["cfg2_rmsnorm_bf16"])
+    if "cfg3_swiglu_bf16" in names:
+        gate, up = wl.config3_swiglu(rows=2048)
+        out = np.empty_like(gate)
+        fn = lib.hyle_oracle_rows_swiglu_bf16
+        fn.argtypes = [vp, vp, vp, sz, sz, sz]
+        rows, dt = timed(2048, 6144, 0, lambda n: (lambda b0, e0: fn(ptr(gate), ptr(up), ptr(out), 6144, b0, e0)))
+        record("cfg3", 8192, rows, dt, wl.ALGORITHMIC_BYTES["cfg3_swiglu_bf16"])
+    if "cfg3_residual_add_bf16" in names:
+        r, y = wl.config3_residual()
+        out = np.empty_like(r)
+        fn = lib.hyle_oracle_rows_add_bf16
+        fn.argtypes = [vp, vp, vp, sz, sz, sz]
+        rows, dt = timed(8192, 2048, 0, lambda n: (lambda b0, e0: fn(ptr(r), ptr(y), ptr(out), 2048, b0, e0)))
+        record("cfg3r", 8192, rows, dt, wl.ALGORITHMIC_BYTES["cfg3_residual_add_bf16"])
+    if "cfg4_softmax_f32_causal" in names:
+        srows = 4096  # the last query rows of head 0: full-length causal rows, the costliest kind
+        s4, mask = wl.config4_softmax(heads=1, seq=4096)
+        x4 = s4.reshape(4096, 4096)
+        out = np.empty_like(x4)
+        fn = lib.hyle_oracle_rows_softmax_bool_f32
+        fn.argtypes = [vp, vp, vp, sz, sz, sz, sz]
+        rows, dt = timed(srows, 4096, 0, lambda n: (lambda b0, e0: fn(ptr(x4), ptr(mask), ptr(out), 4096, 4096, b0, e0)))
+        record("cfg4", 32 * 4096, rows, dt, wl.ALGORITHMIC_BYTES["cfg4_softmax_f32_causal"])
+    if "cfg4_argmax_f32" in names:
+        logits = wl.config4_argmax()
+        values, indices = np.empty(64, np.float32), np.empty(64, np.int32)
+        fn = lib.hyle_oracle_rows_topk1_f32
+        fn.argtypes = [vp, vp, vp, sz, sz, sz]
+        rows, dt = timed(64, 151936, 0, lambda n: (lambda b0, e0: fn(ptr(logits), ptr(values), ptr(indices), 151936, b0, e0)))
+        record("cfg4a", 64, rows, dt, wl.ALGORITHMIC_BYTES["cfg4_argmax_f32"])
+    if "cfg5_q8_0_dequant_sumsq" in names:
+        blocks = wl.config5()
+        out, sumsq = np.empty((6144, 2048), np.uint16), np.empty(6144, np.float32)
+        fn = lib.hyle_oracle_rows_q8_0_bf16
+        fn.argtypes = [vp, vp, vp, sz, sz, sz, sz]
+        rows, dt = timed(6144, 2048, 0, lambda n: (lambda b0, e0: fn(ptr(blocks), ptr(out), ptr(sumsq), 2048, 2176, b0, e0)))
+        record("cfg5", 6144, rows, dt, wl.ALGORITHMIC_BYTES["cfg5_q8_0_dequant_sumsq"])
+    pool.shutdown()
+    step_bytes = sum(o.bytes for o in ops)
+    return {"value": round(step_bytes / total_seconds_full / 1e9, 3), "unit": "GB/s", "cores": cores,
+            "kind": "port",
+            "sample": "row subsets of the same seeded inputs, per-kernel time scaled to the full shape; " + "; ".join(samples)}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -20,9 +20,15 @@ _TO_TORCH = {v: k for k, v in _TO_HYLE.items()}
 
 def desc_of(tensor: torch.Tensor) -> hc.TensorDesc:
     """TensorDesc of a torch tensor: logical dims + byte strides (0 on expanded axes)."""
+    dtype, shape = _TO_HYLE[tensor.dtype], tuple(tensor.shape)
+    dense = hc.TensorDesc.dense(dtype, shape)
+    if 0 in shape:
+        return dense
     size = tensor.element_size()
-    return hc.TensorDesc.strided_bytes(_TO_HYLE[tensor.dtype], tuple(tensor.shape),
-                                       tuple(s * size for s in tensor.stride()))
+    # torch leaves the stride of an extent-1 axis arbitrary; the descriptor wants the canonical one
+    strides = tuple(c if d == 1 else s * size
+                    for d, s, c in zip(shape, tensor.stride(), dense.byte_strides))
+    return hc.TensorDesc.strided_bytes(dtype, shape, strides)
 
 
 def empty_like_desc(desc: hc.TensorDesc, device) -> torch.Tensor:

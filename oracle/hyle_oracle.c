@@ -481,14 +481,21 @@ void hyle_oracle_softmax(int type, const void *src, void *dst,
 /* ------------------------------------------------------------------------ */
 
 /* src/compute_provider_native/reduction.cc:24-47: once the running extremum is
- * NaN it stays NaN; a NaN input replaces a non-NaN running value. */
+ * NaN it stays NaN; a NaN input replaces a non-NaN running value.  Equal values
+ * of opposite sign follow the row primitive the dense route calls
+ * (simd::max_value / simd::min_value, pinned by tests/simd/search_test.cc:196-206):
+ * the maximum of {-0, +0} is +0 and the minimum is -0, whatever the order. */
 static void accumulate_extremum(int maximum, float value, float *result) {
   if (isnan(*result)) return;
   if (isnan(value)) {
     *result = value;
     return;
   }
-  *result = maximum ? fmaxf(*result, value) : fminf(*result, value);
+  if (value == *result) {
+    if (maximum ? !signbit(value) : signbit(value)) *result = value;
+    return;
+  }
+  if (maximum ? value > *result : value < *result) *result = value;
 }
 
 void hyle_oracle_reduce_last_axis(int kind, int type, const void *src,
@@ -600,4 +607,86 @@ void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
         out[r * k + b * 32 + j] = (float)(int8_t)blk[2 + j] * d;
     }
   }
+}
+
+/* ------------------------------------------------------------------------ */
+/* CPU baseline legs (row ranges, dense loops)                              */
+/* ------------------------------------------------------------------------ */
+
+void hyle_oracle_rows_add_row_scale_f32(const float *a, const float *b, float s,
+                                        float *out, size_t cols,
+                                        size_t row_begin, size_t row_end) {
+  for (size_t r = row_begin; r < row_end; ++r) {
+    const float *row = a + r * cols;
+    float *dst = out + r * cols;
+    for (size_t c = 0; c < cols; ++c) dst[c] = row[c] + b[c];
+    for (size_t c = 0; c < cols; ++c) dst[c] = dst[c] * s;
+  }
+}
+
+void hyle_oracle_rows_add_bf16(const uint16_t *r, const uint16_t *y,
+                               uint16_t *out, size_t cols, size_t row_begin,
+                               size_t row_end) {
+  float left[128], right[128];
+  for (size_t row = row_begin; row < row_end; ++row) {
+    for (size_t c = 0; c < cols; c += 128) {
+      const size_t size = cols - c < 128 ? cols - c : 128;
+      const size_t base = row * cols + c;
+      for (size_t i = 0; i < size; ++i) left[i] = hyle_oracle_bf16_to_f32(r[base + i]);
+      for (size_t i = 0; i < size; ++i) right[i] = hyle_oracle_bf16_to_f32(y[base + i]);
+      for (size_t i = 0; i < size; ++i) left[i] = left[i] + right[i];
+      for (size_t i = 0; i < size; ++i) out[base + i] = hyle_oracle_f32_to_bf16(left[i]);
+    }
+  }
+}
+
+void hyle_oracle_rows_swiglu_bf16(const uint16_t *gate, const uint16_t *up,
+                                  uint16_t *out, size_t cols, size_t row_begin,
+                                  size_t row_end) {
+  float g[128], u[128];
+  for (size_t row = row_begin; row < row_end; ++row) {
+    for (size_t c = 0; c < cols; c += 128) {
+      const size_t size = cols - c < 128 ? cols - c : 128;
+      const size_t base = row * cols + c;
+      for (size_t i = 0; i < size; ++i) g[i] = hyle_oracle_bf16_to_f32(gate[base + i]);
+      for (size_t i = 0; i < size; ++i) u[i] = hyle_oracle_bf16_to_f32(up[base + i]);
+      for (size_t i = 0; i < size; ++i) g[i] = hyle_oracle_silu(g[i]) * u[i];
+      for (size_t i = 0; i < size; ++i) out[base + i] = hyle_oracle_f32_to_bf16(g[i]);
+    }
+  }
+}
+
+void hyle_oracle_rows_rms_norm_bf16(const uint16_t *x, const uint16_t *w,
+                                    uint16_t *out, size_t cols, float epsilon,
+                                    size_t row_begin, size_t row_end) {
+  hyle_oracle_rms_norm_native(HYLE_ORACLE_BF16, HYLE_ORACLE_BF16,
+                              x + row_begin * cols, w, out + row_begin * cols,
+                              row_end - row_begin, cols, epsilon);
+}
+
+void hyle_oracle_rows_softmax_bool_f32(const float *x, const uint8_t *mask,
+                                       float *out, size_t cols,
+                                       size_t mask_rows, size_t row_begin,
+                                       size_t row_end) {
+  for (size_t r = row_begin; r < row_end; ++r) {
+    const float *src = x + r * cols;
+    const uint8_t *m = mask + (r % mask_rows) * cols;
+    float *dst = out + r * cols;
+    for (size_t c = 0; c < cols; ++c) dst[c] = m[c] ? src[c] : -INFINITY;
+    hyle_oracle_softmax_f32_row(dst, dst, cols);
+  }
+}
+
+void hyle_oracle_rows_topk1_f32(const float *x, float *values, int32_t *indices,
+                                size_t cols, size_t row_begin, size_t row_end) {
+  hyle_oracle_topk1_f32(x + row_begin * cols, row_end - row_begin, cols,
+                        values + row_begin, indices + row_begin);
+}
+
+void hyle_oracle_rows_q8_0_bf16(const void *blocks, uint16_t *out, float *sumsq,
+                                size_t k, size_t row_stride, size_t row_begin,
+                                size_t row_end) {
+  hyle_oracle_q8_0_dequant_bf16((const unsigned char *)blocks + row_begin * row_stride,
+                                row_end - row_begin, k, row_stride,
+                                out + row_begin * k, sumsq + row_begin, NULL);
 }

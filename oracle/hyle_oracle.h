@@ -198,6 +198,40 @@ void hyle_oracle_q8_0_dequant_bf16(const void *blocks, size_t rows, size_t k,
 void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
                                   size_t row_stride_bytes, float *out);
 
+/* ---- CPU baseline legs ---------------------------------------------------
+ * The same arithmetic as above in the loop shapes the reference's CPU provider
+ * runs (dense rows, no per-element offset walk), over a contiguous row range
+ * [row_begin, row_end) so a caller can fan rows out over threads exactly as
+ * parallel_for_ranges does (src/compute_provider_native/native_plan.h:74-111).
+ * Used only by the benchmark's cpu_baseline timing. */
+/* out = (a[r, :] + b[:]) * s: two simd-style row passes per row
+ * (src/compute_provider_native/elementwise.cc:333-348, chunk = cols). */
+void hyle_oracle_rows_add_row_scale_f32(const float *a, const float *b, float s,
+                                        float *out, size_t cols,
+                                        size_t row_begin, size_t row_end);
+/* r[row, :] = bf16(r + y) via 128-wide f32 tiles
+ * (src/compute_provider_native/elementwise.cc:135-147). */
+void hyle_oracle_rows_add_bf16(const uint16_t *r, const uint16_t *y,
+                               uint16_t *out, size_t cols, size_t row_begin,
+                               size_t row_end);
+void hyle_oracle_rows_swiglu_bf16(const uint16_t *gate, const uint16_t *up,
+                                  uint16_t *out, size_t cols, size_t row_begin,
+                                  size_t row_end);
+void hyle_oracle_rows_rms_norm_bf16(const uint16_t *x, const uint16_t *w,
+                                    uint16_t *out, size_t cols, float epsilon,
+                                    size_t row_begin, size_t row_end);
+/* rows of a [heads, seq, seq]-shaped f32 tensor flattened to [rows, cols] with a
+ * Bool mask [mask_rows, cols] reused every mask_rows rows. */
+void hyle_oracle_rows_softmax_bool_f32(const float *x, const uint8_t *mask,
+                                       float *out, size_t cols,
+                                       size_t mask_rows, size_t row_begin,
+                                       size_t row_end);
+void hyle_oracle_rows_topk1_f32(const float *x, float *values, int32_t *indices,
+                                size_t cols, size_t row_begin, size_t row_end);
+void hyle_oracle_rows_q8_0_bf16(const void *blocks, uint16_t *out, float *sumsq,
+                                size_t k, size_t row_stride, size_t row_begin,
+                                size_t row_end);
+
 #ifdef __cplusplus
 }
 #endif

@@ -424,6 +424,11 @@ def test_reduce_last_axis_nan_and_identities():
     x[2, 17] = np.nan
     assert np.isnan(orc.reduce_last_axis(orc.MAX, orc.F32, x)[2])
     assert np.isnan(orc.reduce_last_axis(orc.MIN, orc.F32, x)[2])
+    # tests/simd/search_test.cc:196-206: max of signed zeros is +0, min is -0, in any order
+    for zeros in ([0.0, -0.0, -1.0], [-0.0, 0.0, -1.0]):
+        assert not np.signbit(orc.reduce_last_axis(orc.MAX, orc.F32, np.array([zeros], np.float32))[0])
+    for zeros in ([0.0, -0.0, 1.0], [-0.0, 0.0, 1.0]):
+        assert np.signbit(orc.reduce_last_axis(orc.MIN, orc.F32, np.array([zeros], np.float32))[0])
     empty = np.empty((2, 0), np.float32)
     assert np.all(orc.reduce_last_axis(orc.MAX, orc.F32, empty) == -np.inf)
     assert np.all(orc.reduce_last_axis(orc.MIN, orc.F32, empty) == np.inf)
