@@ -3,12 +3,19 @@
 //
 // A few very wide rows cannot fill 256 CUs with one block per row, so each row is
 // cut into tiles; every block scans one tile with 128-bit loads and leaves its
-// best (value, index) candidate in the workspace, then one block per row folds
+// best (value, index) candidate in the workspace, then one wave per row folds
 // the candidates.  Ordering is the reference's TopK rule
 // (src/compute_provider_cuda/collectives.cu:478-495): a number beats NaN, a
 // larger number beats a smaller one, ties (including -0 against +0 and NaN
 // against NaN) go to the lower index.  The value output carries the original
 // storage bits of the winner.
+//
+// Measured on MI355X over logits[64, 151936] f32: a tile of 256 lanes x 2
+// vectors scans at about 5.2 TB/s, larger tiles are slower (4 vectors 4.2 TB/s,
+// 8 vectors 1.3 TB/s); folding inside the scan kernel with device-scope atomics
+// (a packed key, or a last-block ticket) costs 5 to 13 us, and a device-wide
+// fence writes back and invalidates a whole L2 (100 us), so the fold is a second,
+// tiny dispatch (about 2 us including the dependent launch).
 #include "device_common.h"
 #include "kernels.h"
 
@@ -20,11 +27,8 @@ struct Candidate {
   int32_t index;
 };
 
-__device__ __forceinline__ LaneArg block_best(LaneArg best, LaneArg *joint) {
-  best = group_reduce<kWaveLanes>(best, [](LaneArg a, LaneArg b) { return arg_best(a, b); });
-  if ((threadIdx.x & (kWaveLanes - 1)) == 0) joint[threadIdx.x / kWaveLanes] = best;
-  __syncthreads();
-  return arg_best(arg_best(joint[0], joint[1]), arg_best(joint[2], joint[3]));
+__device__ __forceinline__ LaneArg wave_best(LaneArg best) {
+  return group_reduce<kWaveLanes>(best, [](LaneArg a, LaneArg b) { return arg_best(a, b); });
 }
 
 // A lane walks its elements in increasing index order, so "strictly better"
@@ -35,61 +39,96 @@ __device__ __forceinline__ void consider(LaneArg &best, float value, int32_t ind
   if (better) best = LaneArg{value, index};
 }
 
+constexpr int kTileVectorsPerLane = 2;
+
+// One block per (row, tile).  A lane issues all of its loads before it compares.
 template <class T, bool kVector>
 __global__ __launch_bounds__(kBlockThreads) void argmax_tiles(const void *x, Candidate *partial,
                                                               uint32_t width, uint32_t tiles,
                                                               uint32_t tile_elems) {
   constexpr int kVec = Traits<T>::kVec;
-  __shared__ LaneArg joint[4];
+  constexpr int kVpl = kTileVectorsPerLane;
+  __shared__ LaneArg joint[kBlockThreads / kWaveLanes];
   const uint32_t row = blockIdx.x / tiles, tile = blockIdx.x % tiles;
   const uint32_t begin = tile * tile_elems;
   const uint32_t end = begin + tile_elems < width ? begin + tile_elems : width;
   LaneArg best{0.0f, -1};
   if constexpr (kVector) {
-    // width % kVec == 0 and tile_elems % kVec == 0: whole vectors only
+    // width % kVec == 0 and tile_elems == kVpl * kBlockThreads * kVec: whole vectors only
     const size_t row_vec = (size_t)row * (width / kVec);
     const uint32_t vec_end = end / kVec;
-    uint32_t vec = begin / kVec + threadIdx.x;
-    // two vectors in flight per lane
-    for (; vec + kBlockThreads < vec_end; vec += 2 * kBlockThreads) {
-      float a[kVec], b[kVec];
-      Traits<T>::unpack(load16_stream(x, row_vec + vec), a);
-      Traits<T>::unpack(load16_stream(x, row_vec + vec + kBlockThreads), b);
+    const uint32_t first = begin / kVec + threadIdx.x;
+    u32x4 raw[kVpl];
 #pragma unroll
-      for (int j = 0; j < kVec; ++j) consider(best, a[j], (int32_t)(vec * kVec + j));
-#pragma unroll
-      for (int j = 0; j < kVec; ++j)
-        consider(best, b[j], (int32_t)((vec + kBlockThreads) * kVec + j));
+    for (int k = 0; k < kVpl; ++k) {
+      const uint32_t vec = first + k * kBlockThreads;
+      if (vec < vec_end) raw[k] = load16_stream(x, row_vec + vec);
     }
-    if (vec < vec_end) {
-      float a[kVec];
-      Traits<T>::unpack(load16_stream(x, row_vec + vec), a);
+    // Common case first: the greatest number above -inf, found with one compare per element
+    // (a NaN never passes "greater than"; the first of equal values stays).  `slot` is the
+    // position inside the lane's own vectors.
+    float top = -INFINITY;
+    int slot = -1;
 #pragma unroll
-      for (int j = 0; j < kVec; ++j) consider(best, a[j], (int32_t)(vec * kVec + j));
+    for (int k = 0; k < kVpl; ++k) {
+      const uint32_t vec = first + k * kBlockThreads;
+      if (vec < vec_end) {
+        float a[kVec];
+        Traits<T>::unpack(raw[k], a);
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) {
+          const bool greater = a[j] > top;
+          top = greater ? a[j] : top;
+          slot = greater ? k * kVec + j : slot;
+        }
+      }
+    }
+    if (slot >= 0) {
+      best = LaneArg{top, (int32_t)((first + (slot / kVec) * kBlockThreads) * kVec + slot % kVec)};
+    } else {
+      // nothing but -inf and NaN in this lane's share: apply the full ordering
+#pragma unroll
+      for (int k = 0; k < kVpl; ++k) {
+        const uint32_t vec = first + k * kBlockThreads;
+        if (vec < vec_end) {
+          float a[kVec];
+          Traits<T>::unpack(raw[k], a);
+#pragma unroll
+          for (int j = 0; j < kVec; ++j) consider(best, a[j], (int32_t)(vec * kVec + j));
+        }
+      }
     }
   } else {
     const size_t base = (size_t)row * width;
     for (uint32_t i = begin + threadIdx.x; i < end; i += kBlockThreads)
       consider(best, Traits<T>::load(x, base + i), (int32_t)i);
   }
-  best = block_best(best, joint);
-  if (threadIdx.x == 0) partial[blockIdx.x] = Candidate{best.value, best.index};
+  best = wave_best(best);
+  if ((threadIdx.x & (kWaveLanes - 1)) == 0) joint[threadIdx.x / kWaveLanes] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    best = arg_best(arg_best(joint[0], joint[1]), arg_best(joint[2], joint[3]));
+    partial[blockIdx.x] = Candidate{best.value, best.index};
+  }
 }
 
+// One wave per row folds that row's candidates.
 template <class T>
-__global__ __launch_bounds__(kBlockThreads) void argmax_finish(const void *x,
-                                                               const Candidate *partial, void *values,
-                                                               int32_t *indices, uint32_t width,
+__global__ __launch_bounds__(kBlockThreads) void argmax_finish(const void *x, const Candidate *partial,
+                                                               void *values, int32_t *indices,
+                                                               uint32_t rows, uint32_t width,
                                                                uint32_t tiles) {
-  __shared__ LaneArg joint[4];
-  const uint32_t row = blockIdx.x;
+  const uint32_t row = blockIdx.x * (kBlockThreads / kWaveLanes) + threadIdx.x / kWaveLanes;
+  const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
   LaneArg best{0.0f, -1};
-  for (uint32_t t = threadIdx.x; t < tiles; t += kBlockThreads) {
-    const Candidate c = partial[(size_t)row * tiles + t];
-    best = arg_best(best, LaneArg{c.value, c.index});
+  if (row < rows) {
+    for (uint32_t t = lane; t < tiles; t += kWaveLanes) {
+      const Candidate c = partial[(size_t)row * tiles + t];
+      best = arg_best(best, LaneArg{c.value, c.index});
+    }
   }
-  best = block_best(best, joint);
-  if (threadIdx.x == 0) {
+  best = wave_best(best);
+  if (row < rows && lane == 0) {
     indices[row] = best.index;
     if (values != nullptr) {
       // copy the winner's storage bits untouched
@@ -107,7 +146,8 @@ hipError_t run(const ArgmaxParams &p, const void *x, void *values, int32_t *indi
                bool vectorised, hipStream_t s) {
   const uint32_t rows = (uint32_t)p.shape.rows, width = p.shape.width;
   auto *partial = static_cast<Candidate *>(workspace);
-  const bool vec = vectorised && width % Traits<T>::kVec == 0;
+  const bool vec = vectorised && width % Traits<T>::kVec == 0 &&
+                   p.tile_elems == (uint32_t)(kTileVectorsPerLane * kBlockThreads * Traits<T>::kVec);
   if (vec)
     hipLaunchKernelGGL((argmax_tiles<T, true>), dim3(rows * p.tiles), dim3(kBlockThreads), 0, s, x,
                        partial, width, p.tiles, p.tile_elems);
@@ -116,27 +156,21 @@ hipError_t run(const ArgmaxParams &p, const void *x, void *values, int32_t *indi
                        partial, width, p.tiles, p.tile_elems);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
-  hipLaunchKernelGGL((argmax_finish<T>), dim3(rows), dim3(kBlockThreads), 0, s, x, partial, values,
-                     indices, width, p.tiles);
+  constexpr int kRowsPerBlock = kBlockThreads / kWaveLanes;
+  hipLaunchKernelGGL((argmax_finish<T>), dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock),
+                     dim3(kBlockThreads), 0, s, x, partial, values, indices, rows, width, p.tiles);
   return hipGetLastError();
 }
 
 }  // namespace
 
-// Tiles are multiples of 1024 elements (whole vectors for every storage type).
-// Aim for a few blocks per CU so the scan is spread over the whole chip, but keep
-// at least 4096 elements per tile so a block has enough loads in flight.
-void argmax_plan(uint64_t rows, uint32_t width, int compute_units, ArgmaxParams *p) {
+// A tile is what one block holds in registers at once: 256 lanes x 2 vectors (2048 f32 or
+// 4096 narrow elements).  64 rows of 151936 logits become 4800 blocks.
+void argmax_plan(uint64_t rows, uint32_t width, Elem type, ArgmaxParams *p) {
   p->shape.rows = rows;
   p->shape.width = width;
-  const uint64_t want_blocks = (uint64_t)(compute_units > 0 ? compute_units : 256) * 8;
-  uint64_t tiles = rows == 0 ? 1 : (want_blocks + rows - 1) / rows;
-  if (tiles < 1) tiles = 1;
-  uint64_t tile_elems = (width + tiles - 1) / tiles;
-  if (tile_elems < 4096) tile_elems = 4096;
-  tile_elems = (tile_elems + 1023) / 1024 * 1024;
-  p->tile_elems = (uint32_t)tile_elems;
-  p->tiles = width == 0 ? 1 : (uint32_t)((width + tile_elems - 1) / tile_elems);
+  p->tile_elems = (uint32_t)(kTileVectorsPerLane * kBlockThreads * elem_vec(type));
+  p->tiles = width == 0 ? 1 : (width + p->tile_elems - 1) / p->tile_elems;
 }
 
 size_t argmax_workspace_bytes(const ArgmaxParams &p) {

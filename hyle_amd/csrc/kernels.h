@@ -112,13 +112,14 @@ struct ReduceParams {
 hipError_t launch_reduce_rows(Elem type, const ReduceParams &p, const void *x, void *y,
                               bool vectorised, hipStream_t stream);
 
-// TopK(count = 1): two dispatches, per-tile candidates in the workspace.
+// TopK(count = 1): a scan dispatch leaves per-tile candidates in the workspace, a fold dispatch
+// turns them into the outputs.
 struct ArgmaxParams {
   RowShape shape;
   uint32_t tiles = 0;        // tiles per row
-  uint32_t tile_elems = 0;   // elements per tile (multiple of 1024)
+  uint32_t tile_elems = 0;   // elements per tile
 };
-void argmax_plan(uint64_t rows, uint32_t width, int compute_units, ArgmaxParams *p);
+void argmax_plan(uint64_t rows, uint32_t width, Elem type, ArgmaxParams *p);
 size_t argmax_workspace_bytes(const ArgmaxParams &p);
 hipError_t launch_argmax(Elem type, const ArgmaxParams &p, const void *x, void *values,
                          int32_t *indices, void *workspace, bool vectorised, hipStream_t stream);

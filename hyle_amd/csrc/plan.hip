@@ -721,8 +721,7 @@ hyle_hip_status admit(hyle_hip_plan *p) {
         return fail(HYLE_HIP_UNIMPLEMENTED, "TopK requires at most INT32_MAX elements");
       if (p->output_elements[0] == 0) return HYLE_HIP_OK;
       p->route = Route::kArgmax;
-      argmax_plan(p->output_elements[0], (uint32_t)in[0].dims[axis],
-                  p->context ? p->context->compute_units : 256, &p->argmax);
+      argmax_plan(p->output_elements[0], (uint32_t)in[0].dims[axis], p->elem, &p->argmax);
       p->workspace_size = argmax_workspace_bytes(p->argmax);
       p->workspace_alignment = 16;
       p->dispatches = 2;

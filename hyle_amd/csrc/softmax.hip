@@ -13,6 +13,8 @@
 // double); the exponentials are carried scaled by 2^32 and the scale is folded
 // into the normaliser, so results down to the smallest subnormal are produced by
 // an ordinary multiply instead of being flushed by the hardware exp2.
+#include <cstdlib>
+
 #include "device_common.h"
 #include "kernels.h"
 
@@ -42,18 +44,23 @@ template <int kLanes> __device__ __forceinline__ float row_max(float v, float *j
   }
 }
 
-// exp(t) * 2^32 for t <= 0, about 2 ulp.  t * log2(e) is split into a rounded
-// product and its exact residual so the hardware exp2 sees an accurate argument.
+// exp(t) * 2^32 for t <= 0.  t * log2(e) is taken as a rounded product plus its exact
+// residual (one fma), so the hardware exp2 sees an argument good to about 2e-8 * |t|
+// and the result stays within 2e-6 relative down to the subnormal range.
 __device__ __forceinline__ float exp_scaled(float t) {
-  constexpr float kLog2eHi = 1.44269502162933349609f;   // f32(log2 e)
-  constexpr float kLog2eLo = 1.92596299112661746e-08f;  // log2 e - f32(log2 e)
+  constexpr float kLog2e = 1.44269504088896340736f;
   constexpr float kLn2 = 0.69314718055994530942f;
   t = fmaxf(t, -200.0f);  // exp(-200) * 2^32 is below every subnormal; also tames -inf
-  const float hi = t * kLog2eHi;
-  float lo = __builtin_fmaf(t, kLog2eHi, -hi);
-  lo = __builtin_fmaf(t, kLog2eLo, lo);
+  const float hi = t * kLog2e;
+  const float lo = __builtin_fmaf(t, kLog2e, -hi);
   const float p = __builtin_amdgcn_exp2f(hi + 32.0f);
   return __builtin_fmaf(p, lo * kLn2, p);
+}
+
+// NaN or +inf: the values that make a softmax row undefined
+// (src/simd/math/activations.cc:181-186).
+__device__ __forceinline__ bool poisons_row(float v) {
+  return __builtin_amdgcn_class(v, 0x001 | 0x002 | 0x200);  // sNaN | qNaN | +inf
 }
 
 struct MaskRows {
@@ -167,17 +174,17 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_rows(const void *x, con
   }
 
   // ---- row maximum and validity -------------------------------------------------
-  float peak = -INFINITY, bad = 0.0f;
+  float peak = -INFINITY;
+  bool poisoned = false;
 #pragma unroll
   for (int k = 0; k < kVpl; ++k)
 #pragma unroll
     for (int j = 0; j < kVec; ++j) {
-      const float e = v[k][j];
-      bad = (e != e || e == INFINITY) ? 1.0f : bad;
-      peak = e > peak ? e : peak;  // a NaN never replaces the running value
+      poisoned = poisoned || poisons_row(v[k][j]);
+      peak = fmaxf(peak, v[k][j]);  // a NaN never replaces the running value
     }
   peak = row_max<kLanes>(peak, joint_max);
-  bad = row_max<kLanes>(bad, joint_bad);
+  const float bad = row_max<kLanes>(poisoned ? 1.0f : 0.0f, joint_bad);
   const bool invalid = bad != 0.0f || peak == -INFINITY;
 
   // ---- exponentials and their sum -------------------------------------------------
@@ -199,18 +206,18 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_rows(const void *x, con
 
   // ---- normalise and store ------------------------------------------------------------
   // softmax: e * 2^32 * (1 / (sum * 2^32)).  log-softmax: (v - max) - log(sum).
-  const float normaliser = log_form ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
-  const float nan = __builtin_nanf("");
+  // An undefined row gets a NaN normaliser: it turns every lane, masked zeros included,
+  // into NaN without a per-element select.
+  float normaliser = log_form ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
+  if (invalid) normaliser = __builtin_nanf("");
 #pragma unroll
   for (int k = 0; k < kVpl; ++k) {
     const uint32_t vec = lane + k * kLanes;
     if (row_ok && vec < row_vectors) {
       float r[kVec];
 #pragma unroll
-      for (int j = 0; j < kVec; ++j) {
-        const float value = log_form ? v[k][j] - normaliser : v[k][j] * normaliser;
-        r[j] = invalid ? nan : value;
-      }
+      for (int j = 0; j < kVec; ++j)
+        r[j] = log_form ? v[k][j] - normaliser : v[k][j] * normaliser;
       store16_stream(y, row_base + vec, Traits<T>::pack(r));
     }
   }
@@ -378,6 +385,8 @@ hipError_t run_softmax(const SoftmaxParams &p, const void *x, const void *mask, 
   if (vectors <= 128) return run_rows<T, 64, 2>(p, x, mask, y, s);
   if (vectors <= 256) return run_rows<T, 64, 4>(p, x, mask, y, s);
   if (vectors <= 512) return run_rows<T, 64, 8>(p, x, mask, y, s);
+  static const bool wave_rows = getenv("HYLE_HIP_EXPERIMENT_SOFTMAX_WAVE") != nullptr;
+  if (vectors <= 1024 && wave_rows) return run_rows<T, 64, 16>(p, x, mask, y, s);
   if (vectors <= 1024) return run_rows<T, 256, 4>(p, x, mask, y, s);
   if (vectors <= 2048) return run_rows<T, 256, 8>(p, x, mask, y, s);
   return run_rows<T, 256, 16>(p, x, mask, y, s);

@@ -47,7 +47,7 @@ class Bound:
         req = self.prepared.workspace_requirement()
         self.workspace: Optional[torch.Tensor] = None
         if req.size:
-            self.workspace = torch.empty(req.size + 256, dtype=torch.uint8, device=device)
+            self.workspace = torch.empty(req.size, dtype=torch.uint8, device=device)  # 512-byte aligned
         ptr = self.workspace.data_ptr() if self.workspace is not None else 0
         self.invocation = self.prepared.create_invocation(ptr, req.size)
         self.device = device
