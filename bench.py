@@ -48,6 +48,9 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     p.add_argument("--cpu-seconds", type=float, default=2.0, help="target CPU seconds per kernel sample")
     p.add_argument("--only", default="", help="comma-separated op names: run and time just these kernels")
+    p.add_argument("--copy-probe", action="store_true",
+                   help="also run three plain device copies of 1 GiB (a kernel of known traffic that "
+                        "calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     return p.parse_args()
 
 
@@ -252,6 +255,14 @@ def main() -> int:
                        "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
                        "gelem_per_s": round(op.elements / us / 1e3, 2)})
         del graph
+
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)  # one elementwise kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     achieved = dominant.bytes / dominant_us / 1e3
     result = {

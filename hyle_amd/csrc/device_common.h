@@ -208,6 +208,31 @@ template <int kLanes> __device__ __forceinline__ float group_max(float v) {
   }).x;
 }
 
+// A row handled by `kLanes` adjacent lanes of a block: a slice of a wave, one wave, or
+// several whole waves.  Waves of one row meet through `joint` (one float per wave of the
+// block) and one block barrier; each call needs its own `joint` array.
+template <int kLanes, class Op>
+__device__ __forceinline__ float row_reduce(float v, float *joint, Op op) {
+  constexpr int kGroup = kLanes < kWaveLanes ? kLanes : kWaveLanes;
+  v = group_reduce<kGroup>(LaneF32{v}, [op](LaneF32 a, LaneF32 b) { return LaneF32{op(a.x, b.x)}; }).x;
+  if constexpr (kLanes > kWaveLanes) {
+    constexpr int kWavesPerRow = kLanes / kWaveLanes;
+    if ((threadIdx.x & (kWaveLanes - 1)) == 0) joint[threadIdx.x / kWaveLanes] = v;
+    __syncthreads();
+    const int first = (threadIdx.x / kLanes) * kWavesPerRow;
+    v = joint[first];
+#pragma unroll
+    for (int w = 1; w < kWavesPerRow; ++w) v = op(v, joint[first + w]);
+  }
+  return v;
+}
+template <int kLanes> __device__ __forceinline__ float row_sum(float v, float *joint) {
+  return row_reduce<kLanes>(v, joint, [](float a, float b) { return a + b; });
+}
+template <int kLanes> __device__ __forceinline__ float row_max(float v, float *joint) {
+  return row_reduce<kLanes>(v, joint, [](float a, float b) { return a > b ? a : b; });
+}
+
 // NaN-propagating extrema of the reference's Reduce
 // (src/compute_provider_native/reduction.cc:34-47): the first NaN met sticks;
 // +0 ranks above -0 (tests/simd/search_test.cc:203-206).

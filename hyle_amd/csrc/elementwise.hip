@@ -142,7 +142,7 @@ __device__ __forceinline__ float fetch1(const Operand &op, uint32_t e) {
   return Traits<T>::load(op.base, op.period ? e % op.period : e);
 }
 
-template <class T, class Fn>
+template <class T, class Fn, int kUnroll>
 __global__ __launch_bounds__(kBlockThreads) void ew_flat_vec(Operand a, Operand b, Operand c,
                                                              void *out, uint32_t vectors,
                                                              uint32_t elements, Fn fn) {
@@ -275,16 +275,30 @@ Operand make_operand(const void *base, uint32_t period, int vec) {
   return op;
 }
 
-template <class T, class Fn>
-hipError_t run_vec(const EwFlat &p, Operand a, Operand b, Operand c, void *out, hipStream_t s) {
+template <class T, class Fn, int kUnroll>
+hipError_t run_vec_unrolled(const EwFlat &p, Operand a, Operand b, Operand c, void *out,
+                            hipStream_t s) {
   constexpr int kVec = Traits<T>::kVec;
   const uint64_t vectors = p.elements / kVec;
   const uint64_t per_block = (uint64_t)kUnroll * kBlockThreads;
   uint64_t blocks = (vectors + per_block - 1) / per_block;
   if (blocks == 0) blocks = 1;  // the tail still needs block 0
-  hipLaunchKernelGGL((ew_flat_vec<T, Fn>), dim3((uint32_t)blocks), dim3(kBlockThreads), 0, s, a, b,
-                     c, out, (uint32_t)vectors, (uint32_t)p.elements, Fn{});
+  hipLaunchKernelGGL((ew_flat_vec<T, Fn, kUnroll>), dim3((uint32_t)blocks), dim3(kBlockThreads), 0, s,
+                     a, b, c, out, (uint32_t)vectors, (uint32_t)p.elements, Fn{});
   return hipGetLastError();
+}
+
+// Vectors per lane, chosen from what was measured on MI355X: launches that move less than
+// about 80 MB finish in a few microseconds and do best with four vectors in flight per lane
+// (fewer, fatter blocks: (A[4096,2048] + b) * s takes 11.8 us against 12.7 us); larger ones
+// do best with one vector per lane (SwiGLU over [8192,6144] bf16: 47.8 us against 50.3 us).
+template <class T, class Fn>
+hipError_t run_vec(const EwFlat &p, Operand a, Operand b, Operand c, void *out, hipStream_t s) {
+  uint64_t streams = 1;  // the output
+  for (int i = 0; i < p.inputs; ++i) streams += p.period[i] == 0 ? 1 : 0;
+  const uint64_t traffic = streams * p.elements * Traits<T>::kSize;
+  if (traffic > (80ull << 20)) return run_vec_unrolled<T, Fn, 1>(p, a, b, c, out, s);
+  return run_vec_unrolled<T, Fn, 4>(p, a, b, c, out, s);
 }
 
 template <class T, int kKind0>

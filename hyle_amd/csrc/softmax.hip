@@ -23,27 +23,6 @@ namespace {
 
 enum : int { kMaskNone = 0, kMaskAdditive = 1, kMaskBoolean = 2 };
 
-template <int kLanes> __device__ __forceinline__ float row_sum(float v, float *joint) {
-  if constexpr (kLanes <= kWaveLanes) {
-    return group_sum<kLanes>(v);
-  } else {
-    v = group_sum<kWaveLanes>(v);
-    if ((threadIdx.x & (kWaveLanes - 1)) == 0) joint[threadIdx.x / kWaveLanes] = v;
-    __syncthreads();
-    return (joint[0] + joint[1]) + (joint[2] + joint[3]);
-  }
-}
-template <int kLanes> __device__ __forceinline__ float row_max(float v, float *joint) {
-  if constexpr (kLanes <= kWaveLanes) {
-    return group_max<kLanes>(v);
-  } else {
-    v = group_max<kWaveLanes>(v);
-    if ((threadIdx.x & (kWaveLanes - 1)) == 0) joint[threadIdx.x / kWaveLanes] = v;
-    __syncthreads();
-    return fmaxf(fmaxf(joint[0], joint[1]), fmaxf(joint[2], joint[3]));
-  }
-}
-
 // exp(t) * 2^32 for t <= 0.  t * log2(e) is taken as a rounded product plus its exact
 // residual (one fma), so the hardware exp2 sees an argument good to about 2e-8 * |t|
 // and the result stays within 2e-6 relative down to the subnormal range.
@@ -97,15 +76,15 @@ __device__ __forceinline__ uint32_t assigned_row(const RowOrder &o, uint32_t blo
   return repeat * o.period + mask_row;
 }
 
-template <class T, int kLanes, int kVpl>
-__global__ __launch_bounds__(kBlockThreads) void softmax_rows(const void *x, const void *mask,
-                                                              void *y, uint32_t rows,
-                                                              uint32_t row_vectors, float scale,
-                                                              int mask_kind, int log_form,
-                                                              MaskRows mrows, RowOrder order) {
+template <class T, int kLanes, int kVpl, int kThreads>
+__global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const void *mask, void *y,
+                                                         uint32_t rows, uint32_t row_vectors,
+                                                         float scale, int mask_kind, int log_form,
+                                                         MaskRows mrows, RowOrder order) {
   constexpr int kVec = Traits<T>::kVec;
-  constexpr int kRowsPerBlock = kBlockThreads / kLanes;
-  __shared__ float joint_max[4], joint_bad[4], joint_sum[4];
+  constexpr int kRowsPerBlock = kThreads / kLanes;
+  constexpr int kWaves = kThreads / kWaveLanes;
+  __shared__ float joint_max[kWaves], joint_bad[kWaves], joint_sum[kWaves];
   const uint32_t lane = threadIdx.x % kLanes;
   const uint32_t row = assigned_row<kRowsPerBlock>(order, blockIdx.x, threadIdx.x / kLanes);
   const bool row_ok = row < rows;
@@ -267,7 +246,8 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_general(const char *x, 
                                                                  void *y, uint32_t width,
                                                                  float scale, int mask_kind,
                                                                  int log_form, GeneralLayout g) {
-  __shared__ float joint_max[4], joint_bad[4], joint_sum[4];
+  constexpr int kWaves = kBlockThreads / kWaveLanes;
+  __shared__ float joint_max[kWaves], joint_bad[kWaves], joint_sum[kWaves];
   const uint32_t outer = blockIdx.x / g.inner, inner = blockIdx.x % g.inner;
   float peak = -INFINITY, bad = 0.0f;
   for (uint32_t c = threadIdx.x; c < width; c += kBlockThreads) {
@@ -346,10 +326,10 @@ __global__ __launch_bounds__(kBlockThreads) void reduce_rows(const void *x, void
 }
 
 // ---- host dispatch ----------------------------------------------------------------------------
-template <class T, int kLanes, int kVpl>
+template <class T, int kLanes, int kVpl, int kThreads = kBlockThreads>
 hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, void *y,
                     hipStream_t s) {
-  constexpr int kRowsPerBlock = kBlockThreads / kLanes;
+  constexpr int kRowsPerBlock = kThreads / kLanes;
   const uint32_t rows = (uint32_t)p.shape.rows;
   const uint32_t blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
   MaskRows m{};
@@ -360,7 +340,8 @@ hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, voi
   }
   m.inner_stride = p.mask_inner_stride;
   RowOrder order{0, 0};
-  if (p.mask_kind != kMaskNone && p.mask_period != 0 && p.mask_period % 8 == 0 &&
+  if (getenv("HYLE_HIP_EXPERIMENT_PLAIN_ORDER") == nullptr &&
+      p.mask_kind != kMaskNone && p.mask_period != 0 && p.mask_period % 8 == 0 &&
       p.shape.rows % p.mask_period == 0) {
     const uint64_t repeats = p.shape.rows / p.mask_period;
     if (repeats > 1 && repeats % kRowsPerBlock == 0) {
@@ -368,7 +349,7 @@ hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, voi
       order.groups = (uint32_t)(repeats / kRowsPerBlock);
     }
   }
-  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl>), dim3(blocks), dim3(kBlockThreads), 0, s, x,
+  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads>), dim3(blocks), dim3(kThreads), 0, s, x,
                      mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, (int)p.mask_kind,
                      p.log ? 1 : 0, m, order);
   return hipGetLastError();
@@ -385,9 +366,10 @@ hipError_t run_softmax(const SoftmaxParams &p, const void *x, const void *mask, 
   if (vectors <= 128) return run_rows<T, 64, 2>(p, x, mask, y, s);
   if (vectors <= 256) return run_rows<T, 64, 4>(p, x, mask, y, s);
   if (vectors <= 512) return run_rows<T, 64, 8>(p, x, mask, y, s);
-  static const bool wave_rows = getenv("HYLE_HIP_EXPERIMENT_SOFTMAX_WAVE") != nullptr;
-  if (vectors <= 1024 && wave_rows) return run_rows<T, 64, 16>(p, x, mask, y, s);
-  if (vectors <= 1024) return run_rows<T, 256, 4>(p, x, mask, y, s);
+  // Measured on MI355X for S[32,4096,4096] f32 with a causal mask (us per launch): two waves
+  // per row with 8 vectors per lane 785; four waves x 4 vectors 813; eight waves x 2 vectors
+  // 827; sixteen waves x 1 vector 1224; one wave x 16 vectors 834.
+  if (vectors <= 1024) return run_rows<T, 128, 8>(p, x, mask, y, s);
   if (vectors <= 2048) return run_rows<T, 256, 8>(p, x, mask, y, s);
   return run_rows<T, 256, 16>(p, x, mask, y, s);
 }
