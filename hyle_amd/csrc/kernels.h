@@ -83,8 +83,6 @@ struct SoftmaxParams {
   uint32_t outer_dims[kMaxRank] = {};
   int64_t mask_outer_strides[kMaxRank] = {};
   int64_t mask_inner_stride = 0;
-  // rows r and r + mask_period share one mask row (0 = no such structure)
-  uint64_t mask_period = 0;
 };
 hipError_t launch_softmax(Elem type, const SoftmaxParams &p, const void *x, const void *mask,
                           void *y, bool vectorised, int compute_units, hipStream_t stream);

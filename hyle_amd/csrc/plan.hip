@@ -680,12 +680,6 @@ hyle_hip_status admit(hyle_hip_plan *p) {
           const int64_t row_alignment = r.mask == HYLE_HIP_MASK_BOOLEAN ? elem_vec(p->elem) : 16;
           for (int a = 0; a < rank - 1; ++a)
             if (sp.mask_outer_strides[a] % row_alignment != 0) p->softmax_mask_vector_ok = false;
-          // rows r and r + period share a mask row when the mask is a dense trailing
-          // slice of the input shape (e.g. [q, k] under [heads, q, k])
-          uint32_t period_elements = 0;
-          if (suffix_period(in[1], in[0], p->output_elements[0], &period_elements) &&
-              period_elements != 0 && period_elements % width == 0)
-            sp.mask_period = period_elements / width;
         }
       }
       return HYLE_HIP_OK;

@@ -13,8 +13,6 @@
 // double); the exponentials are carried scaled by 2^32 and the scale is folded
 // into the normaliser, so results down to the smallest subnormal are produced by
 // an ordinary multiply instead of being flushed by the hardware exp2.
-#include <cstdlib>
-
 #include "device_common.h"
 #include "kernels.h"
 
@@ -60,33 +58,22 @@ __device__ __forceinline__ int64_t mask_row_offset(const MaskRows &m, uint32_t r
   return offset;
 }
 
-// Rows that share a mask row are steered onto one XCD, close in time, so the mask
-// row is fetched from memory once per XCD and then served by that XCD's L2.
-// Workgroups are dealt to the 8 XCDs round-robin by index.
-struct RowOrder {
-  uint32_t period;  // rows r and r + period share a mask row; 0 = plain order
-  uint32_t groups;  // blocks per mask row = (rows / period) / rows-per-block
-};
-template <int kRowsPerBlock>
-__device__ __forceinline__ uint32_t assigned_row(const RowOrder &o, uint32_t block, uint32_t slot) {
-  if (o.period == 0) return block * kRowsPerBlock + slot;
-  const uint32_t xcd = block & 7u, j = block >> 3;
-  const uint32_t mask_row = (j / o.groups) * 8u + xcd;
-  const uint32_t repeat = (j % o.groups) * kRowsPerBlock + slot;
-  return repeat * o.period + mask_row;
-}
-
+// Rows are taken in storage order.  A mask broadcast over leading axes (a [q, k] mask under
+// [heads, q, k]) is re-read by every head; the FETCH_SIZE counter shows those re-reads never
+// reach HBM (the mask's 16 MiB are fetched once per launch), and steering the heads of one
+// mask row onto one XCD changed neither the counter nor the run time, so there is no such
+// remapping here.
 template <class T, int kLanes, int kVpl, int kThreads>
 __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const void *mask, void *y,
                                                          uint32_t rows, uint32_t row_vectors,
                                                          float scale, int mask_kind, int log_form,
-                                                         MaskRows mrows, RowOrder order) {
+                                                         MaskRows mrows) {
   constexpr int kVec = Traits<T>::kVec;
   constexpr int kRowsPerBlock = kThreads / kLanes;
   constexpr int kWaves = kThreads / kWaveLanes;
   __shared__ float joint_max[kWaves], joint_bad[kWaves], joint_sum[kWaves];
   const uint32_t lane = threadIdx.x % kLanes;
-  const uint32_t row = assigned_row<kRowsPerBlock>(order, blockIdx.x, threadIdx.x / kLanes);
+  const uint32_t row = blockIdx.x * kRowsPerBlock + threadIdx.x / kLanes;
   const bool row_ok = row < rows;
   const size_t row_base = (size_t)row * row_vectors;
   const char *mask_row = nullptr;
@@ -339,19 +326,9 @@ hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, voi
     m.outer_strides[i] = p.mask_outer_strides[i];
   }
   m.inner_stride = p.mask_inner_stride;
-  RowOrder order{0, 0};
-  if (getenv("HYLE_HIP_EXPERIMENT_PLAIN_ORDER") == nullptr &&
-      p.mask_kind != kMaskNone && p.mask_period != 0 && p.mask_period % 8 == 0 &&
-      p.shape.rows % p.mask_period == 0) {
-    const uint64_t repeats = p.shape.rows / p.mask_period;
-    if (repeats > 1 && repeats % kRowsPerBlock == 0) {
-      order.period = (uint32_t)p.mask_period;
-      order.groups = (uint32_t)(repeats / kRowsPerBlock);
-    }
-  }
   hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads>), dim3(blocks), dim3(kThreads), 0, s, x,
                      mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, (int)p.mask_kind,
-                     p.log ? 1 : 0, m, order);
+                     p.log ? 1 : 0, m);
   return hipGetLastError();
 }
 

@@ -1,0 +1,71 @@
+"""The launches are capture-compatible (ProviderRuntimeProperties::capture_compatible,
+include/hyle/compute/provider.h:136-139): a captured HIP graph of the hot-path kernels replays
+to the same bits as eager submission, replay after replay, with eager work in between."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from hyle_amd import compute as hc
+from hyle_amd import torch_io as tio
+from hyle_amd import workloads as wl
+
+from gpu_support import DEVICE, context, note, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def test_captured_step_replays_bit_identically():
+    ctx = context()
+    x, w = wl.config2(rows=512)
+    gate, up = wl.config3_swiglu(rows=64)
+    logits = wl.config4_argmax(rows=8)
+    s, mask = wl.config4_softmax(heads=2, seq=256)
+    blocks = wl.config5(rows=128)
+    dx, dw = to_device(x, "bf16"), to_device(w, "bf16")
+    dg, du = to_device(gate, "bf16"), to_device(up, "bf16")
+    dl = to_device(logits, "f32")
+    ds = to_device(s, "f32")
+    dm = torch.from_numpy(mask).to(DEVICE).view(torch.bool)
+    db = torch.from_numpy(blocks).to(DEVICE)
+
+    ops = [
+        (tio.Bound(ctx, hc.RmsNorm(1e-6), [tio.desc_of(dx), tio.desc_of(dw)]), [dx, dw]),
+        (tio.Bound(ctx, hc.GatedActivation(hc.GatedActivationKind.kSilu, hc.GatedInputKind.kSeparate),
+                   [tio.desc_of(dg), tio.desc_of(du)]), [dg, du]),
+        (tio.Bound(ctx, hc.TopK(), [tio.desc_of(dl)]), [dl]),
+        (tio.Bound(ctx, hc.Softmax(mask=hc.MaskKind.kBoolean), [tio.desc_of(ds), tio.desc_of(dm)]), [ds, dm]),
+        (tio.Bound(ctx, hc.Q8_0DequantSumSquares(), [hc.TensorDesc.gguf_q8_0_weight(hc.DataType.kBFloat16, 2048, 128)]),
+         [db]),
+    ]
+    note("eager pass of rmsnorm, swiglu, argmax, softmax, q8_0")
+    eager_outs = []
+    for bound, inputs in ops:
+        outs = bound.outputs()
+        bound.submit(inputs, outs)
+        eager_outs.append(outs)
+    torch.cuda.synchronize()
+    want = [[to_host(t).copy() for t in outs] for outs in eager_outs]
+
+    note("capture the same five launches into one HIP graph")
+    graph_outs = [bound.outputs() for bound, _ in ops]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        stream = torch.cuda.current_stream().cuda_stream
+        for (bound, inputs), outs in zip(ops, graph_outs):
+            bound.submit(inputs, outs, stream=stream)
+    for replay in range(3):
+        note(f"graph replay {replay}")
+        for outs in graph_outs:
+            for t in outs:
+                t.zero_()
+        # unrelated eager work and a synchronisation between replays
+        scratch = torch.randn(1 << 20, device=DEVICE).sum().item()
+        assert np.isfinite(scratch)
+        graph.replay()
+        torch.cuda.synchronize()
+        for outs, expected in zip(graph_outs, want):
+            for t, e in zip(outs, expected):
+                got = to_host(t)
+                assert np.array_equal(got.view(np.uint8), e.view(np.uint8))

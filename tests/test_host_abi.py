@@ -1,0 +1,247 @@
+"""CPU-side checks of the drop-in boundary: the C ABI loads and exports what include/hyle_hip.h
+declares, the schema (output inference) and the admission logic behave like the reference's,
+and nothing here needs or touches a GPU.
+
+Reference behaviour cited per case: src/compute_ops/operation.cc (inference),
+src/compute_provider_native/*.cc and src/compute_provider_cuda/*_provider.cc (admission),
+tests/compute/custom_kernel_test.cc (decline vs error at the provider boundary).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import re
+import subprocess
+import tempfile
+
+import pytest
+
+from hyle_amd import capi
+from hyle_amd import compute as hc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hyle_hip.h")
+DT = hc.DataType
+D = hc.TensorDesc.dense
+CTX = hc.Context.planning_only()
+
+
+def test_library_exports_every_declared_symbol():
+    text = open(HEADER).read()
+    declared = set(re.findall(r"HYLE_HIP_API\s+[\w\s\*]+?\b(hyle_hip_\w+)\s*\(", text))
+    assert declared, "no declarations parsed"
+    lib = capi.load()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared but not exported"
+    assert declared == set(capi.EXPORTS), (declared ^ set(capi.EXPORTS))
+    assert lib.hyle_hip_abi_version() == capi.ABI_VERSION
+
+
+def test_header_is_plain_c_and_struct_layout_matches_ctypes():
+    probe = r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "hyle_hip.h"
+int main(void) {
+  printf("%zu %zu %zu %zu %zu %zu %zu\n", sizeof(hyle_hip_tensor_desc), offsetof(hyle_hip_tensor_desc, dims),
+         offsetof(hyle_hip_tensor_desc, byte_strides), sizeof(hyle_hip_op_desc),
+         offsetof(hyle_hip_op_desc, count), offsetof(hyle_hip_op_desc, input_count),
+         offsetof(hyle_hip_op_desc, inputs));
+  return 0;
+}
+'''
+    with tempfile.TemporaryDirectory() as tmp:
+        src = os.path.join(tmp, "probe.c")
+        open(src, "w").write(probe)
+        exe = os.path.join(tmp, "probe")
+        subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.dirname(HEADER), src, "-o", exe],
+                       check=True)
+        got = [int(v) for v in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()]
+    want = [C.sizeof(capi.TensorDescC), capi.TensorDescC.dims.offset, capi.TensorDescC.byte_strides.offset,
+            C.sizeof(capi.OpDescC), capi.OpDescC.count.offset, capi.OpDescC.input_count.offset,
+            capi.OpDescC.inputs.offset]
+    assert got == want
+
+
+def test_no_device_here_is_reported_as_unavailable_not_hidden():
+    try:
+        import torch
+        if torch.cuda.is_available():
+            pytest.skip("a HIP device is present")
+    except ImportError:
+        pass
+    with pytest.raises(hc.StatusError) as err:
+        hc.Context.create(0)
+    assert err.value.code == hc.StatusCode.kUnavailable
+
+
+# ---------------------------------------------------------------- inference ----
+def test_infer_binary_broadcast_and_type_rules():
+    # src/compute_ops/operation.cc:249-278,480-490
+    out = hc.infer_output_descriptions(hc.Binary(), [D(DT.kFloat32, [4096, 2048]), D(DT.kFloat32, [2048])])
+    assert out == [D(DT.kFloat32, [4096, 2048])]
+    out = hc.infer_output_descriptions(hc.Binary(), [D(DT.kBFloat16, [2, 1, 5]), D(DT.kBFloat16, [7, 1])])
+    assert out == [D(DT.kBFloat16, [2, 7, 5])]
+    assert hc.infer_output_descriptions(hc.Binary(), [D(DT.kFloat32, []), D(DT.kFloat32, [])]) == [D(DT.kFloat32, [])]
+    assert hc.infer_output_descriptions(hc.Binary(), [D(DT.kFloat32, [0, 3]), D(DT.kFloat32, [1])])[0].byte_strides == (0, 0)
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Binary(), [D(DT.kFloat32, [2, 3]), D(DT.kFloat32, [4])])
+    assert err.value.is_invalid_argument() and "cannot be broadcast" in err.value.message
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Binary(), [D(DT.kFloat32, [3]), D(DT.kBFloat16, [3])])
+    assert err.value.is_invalid_argument() and "data types differ" in err.value.message
+    with pytest.raises(hc.StatusError) as err:  # arity (operation.cc:1222-1225)
+        hc.infer_output_descriptions(hc.Binary(), [D(DT.kFloat32, [3])])
+    assert err.value.is_invalid_argument()
+    chain = hc.infer_output_descriptions(hc.BinaryChain(), [D(DT.kFloat32, [8, 4]), D(DT.kFloat32, [4]), D(DT.kFloat32, [1])])
+    assert chain == [D(DT.kFloat32, [8, 4])]
+
+
+def test_infer_unary_gated_norm_rules():
+    # src/compute_ops/operation.cc:1291-1305 (Unary), 1439-1469 (gated), 492-536 + 1395-1409 (norm)
+    assert hc.infer_output_descriptions(hc.Unary(hc.UnaryKind.kSilu), [D(DT.kBFloat16, [3, 5])]) == [D(DT.kBFloat16, [3, 5])]
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Unary(hc.UnaryKind.kSilu), [D(DT.kInt32, [3])])
+    assert err.value.is_invalid_argument()
+    sep = hc.GatedActivation(hc.GatedActivationKind.kSilu, hc.GatedInputKind.kSeparate)
+    assert hc.infer_output_descriptions(sep, [D(DT.kBFloat16, [8, 64]), D(DT.kBFloat16, [8, 64])]) == [D(DT.kBFloat16, [8, 64])]
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(sep, [D(DT.kBFloat16, [8, 64]), D(DT.kBFloat16, [8, 32])])
+    assert "equal type and shape" in err.value.message
+    packed = hc.GatedActivation(hc.GatedActivationKind.kSilu, hc.GatedInputKind.kPackedHalves)
+    assert hc.infer_output_descriptions(packed, [D(DT.kFloat16, [4, 10])]) == [D(DT.kFloat16, [4, 5])]
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(packed, [D(DT.kFloat16, [4, 9])])
+    assert "must be even" in err.value.message
+    x = D(DT.kBFloat16, [8192, 2048])
+    assert hc.infer_output_descriptions(hc.RmsNorm(1e-6), [x, D(DT.kBFloat16, [2048])]) == [x]
+    assert hc.infer_output_descriptions(hc.RmsNorm(1e-6), [x, D(DT.kFloat32, [2048])]) == [x]  # promoted scale
+    assert hc.infer_output_descriptions(hc.RmsNorm(1e-6), [x]) == [x]
+    for bad_scale in (D(DT.kBFloat16, [2047]), D(DT.kBFloat16, [1, 2048]), D(DT.kFloat16, [2048])):
+        with pytest.raises(hc.StatusError) as err:
+            hc.infer_output_descriptions(hc.RmsNorm(), [x, bad_scale])
+        assert "scale must match" in err.value.message
+    with pytest.raises(hc.StatusError):  # f32 input does not take a narrow scale
+        hc.infer_output_descriptions(hc.RmsNorm(), [D(DT.kFloat32, [4, 8]), D(DT.kBFloat16, [8])])
+    for eps in (-1.0, float("inf"), float("nan")):
+        with pytest.raises(hc.StatusError) as err:
+            hc.infer_output_descriptions(hc.RmsNorm(epsilon=eps), [x])
+        assert "epsilon" in err.value.message
+
+
+def test_infer_softmax_reduce_topk_rules():
+    # src/compute_ops/operation.cc:696-711,1593-1621 (softmax), 1345-1394 (reduce), 1622-1660 (TopK)
+    s = D(DT.kFloat32, [32, 64, 64])
+    boolean = hc.Softmax(mask=hc.MaskKind.kBoolean)
+    assert hc.infer_output_descriptions(boolean, [s, D(DT.kBool, [64, 64])]) == [s]
+    assert hc.infer_output_descriptions(boolean, [s, D(DT.kBool, [1, 64, 64])]) == [s]
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(boolean, [s, D(DT.kFloat32, [64, 64])])
+    assert "Bool data type" in err.value.message
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(boolean, [s, D(DT.kBool, [63, 64])])
+    assert err.value.is_invalid_argument()
+    with pytest.raises(hc.StatusError) as err:  # a mask larger than the input is not a broadcast onto it
+        hc.infer_output_descriptions(boolean, [D(DT.kFloat32, [1, 64]), D(DT.kBool, [5, 64])])
+    assert "broadcast-compatible" in err.value.message
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Softmax(mask=hc.MaskKind.kAdditive), [s, D(DT.kBool, [64, 64])])
+    assert "floating" in err.value.message
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Softmax(axis=3), [s])
+    assert err.value.is_out_of_range()
+    with pytest.raises(hc.StatusError):
+        hc.infer_output_descriptions(hc.Softmax(scale=float("inf")), [s])
+    with pytest.raises(hc.StatusError):  # mask supplied for a no-mask operation is an arity error
+        hc.infer_output_descriptions(hc.Softmax(), [s, D(DT.kBool, [64, 64])])
+    r = hc.Reduce(hc.ReductionKind.kMaximum, axis=-1)
+    assert hc.infer_output_descriptions(r, [s]) == [D(DT.kFloat32, [32, 64])]
+    keep = hc.Reduce(hc.ReductionKind.kSum, axis=-1, keep_dimensions=True)
+    assert hc.infer_output_descriptions(keep, [s]) == [D(DT.kFloat32, [32, 64, 1])]
+    logits = D(DT.kFloat32, [64, 151936])
+    values, indices = hc.infer_output_descriptions(hc.TopK(), [logits])
+    assert values == D(DT.kFloat32, [64, 1]) and indices == D(DT.kInt32, [64, 1])
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.TopK(count=151937), [logits])
+    assert err.value.is_out_of_range()
+
+
+def test_infer_q8_0_descriptor():
+    # src/compute_ops/low_precision.cc:28-29,269-297: logical [K, N], 34-byte blocks on axis 0
+    w = hc.TensorDesc.gguf_q8_0_weight(DT.kBFloat16, 2048, 6144)
+    assert w.byte_strides == (34, 2176) and w.required_bytes() == 13369344
+    out, sumsq = hc.infer_output_descriptions(hc.Q8_0DequantSumSquares(), [w])
+    assert out == D(DT.kBFloat16, [6144, 2048]) and sumsq == D(DT.kFloat32, [6144])
+    with pytest.raises(hc.StatusError):
+        hc.infer_output_descriptions(hc.Q8_0DequantSumSquares(), [D(DT.kBFloat16, [2048, 6144])])
+    with pytest.raises(hc.StatusError):
+        hc.TensorDesc.gguf_q8_0_weight(DT.kBFloat16, 2047, 8)
+
+
+# ---------------------------------------------------------------- admission ----
+def test_routes_alias_support_and_cost_facts():
+    a, b, s = D(DT.kFloat32, [4096, 2048]), D(DT.kFloat32, [2048]), D(DT.kFloat32, [1])
+    fused = hc.prepare(CTX, hc.BinaryChain(), a, b, s)
+    assert fused.route_name() == "elementwise-flat" and fused.dispatch_count() == 1
+    assert fused.workspace_requirement().size == 0
+    # only an input whose descriptor equals the output may alias it
+    # (src/compute_provider_native/elementwise.cc:645-655)
+    assert fused.alias_support(0, 0) and not fused.alias_support(0, 1) and not fused.alias_support(0, 2)
+    same = hc.prepare(CTX, hc.Binary(), a, a)
+    assert same.alias_support(0, 0) and same.alias_support(0, 1)
+    column = hc.prepare(CTX, hc.Binary(), D(DT.kFloat32, [3, 1]), D(DT.kFloat32, [1, 5]))
+    assert column.route_name() == "elementwise-strided"
+    strided = hc.prepare(CTX, hc.Binary(), hc.TensorDesc.strided_bytes(DT.kFloat32, [6, 16], [160, 8]),
+                         hc.TensorDesc.strided_bytes(DT.kFloat32, [6, 16], [0, 4]))
+    assert strided.route_name() == "elementwise-strided" and not strided.alias_support(0, 0)
+    norm = hc.prepare(CTX, hc.RmsNorm(1e-6), D(DT.kBFloat16, [8192, 2048]), D(DT.kBFloat16, [2048]))
+    assert norm.route_name() == "rms-norm-rows" and norm.alias_support(0, 0) and not norm.alias_support(0, 1)
+    gated = hc.prepare(CTX, hc.GatedActivation(hc.GatedActivationKind.kSilu, hc.GatedInputKind.kSeparate),
+                       D(DT.kBFloat16, [8, 64]), D(DT.kBFloat16, [8, 64]))
+    assert not gated.alias_support(0, 0)  # src/compute_provider_cuda/cuda_provider.cc:219-221
+    soft = hc.prepare(CTX, hc.Softmax(mask=hc.MaskKind.kBoolean), D(DT.kFloat32, [32, 64, 64]), D(DT.kBool, [64, 64]))
+    assert soft.route_name() == "softmax-rows" and soft.alias_support(0, 0)
+    topk = hc.prepare(CTX, hc.TopK(), D(DT.kFloat32, [64, 151936]))
+    assert topk.route_name() == "argmax-tiles" and topk.dispatch_count() == 2
+    need = topk.workspace_requirement()
+    assert need.size == 64 * 75 * 8 and need.alignment == 16
+    with pytest.raises(hc.StatusError) as err:  # workspace is the caller's to supply
+        topk.create_invocation()
+    assert err.value.is_invalid_argument()
+
+
+def test_declines_are_unimplemented_and_errors_are_not():
+    x = D(DT.kBFloat16, [4, 64])
+    declines = [
+        lambda: hc.prepare(CTX, hc.Unary(hc.UnaryKind.kTanh), x),
+        lambda: hc.prepare(CTX, hc.RmsNorm(accumulation_type=DT.kBFloat16), x),
+        lambda: hc.prepare(CTX, hc.Softmax(accumulation_type=DT.kUnknown), x),   # half needs explicit f32
+        lambda: hc.prepare(CTX, hc.Reduce(hc.ReductionKind.kSum, axis=0, accumulation_type=DT.kFloat32), x),
+        lambda: hc.prepare(CTX, hc.TopK(count=2), x),
+        lambda: hc.prepare(CTX, hc.TopK(largest=False), x),
+        lambda: hc.prepare(CTX, hc.Binary(), D(DT.kInt32, [4]), D(DT.kInt32, [4])),
+        lambda: hc.prepare(CTX, hc.GatedActivation(hc.GatedActivationKind.kGelu, hc.GatedInputKind.kSeparate), x, x),
+        lambda: hc.prepare(CTX, hc.RmsNorm(), hc.TensorDesc.strided_bytes(DT.kBFloat16, [4, 64], [256, 2])),
+    ]
+    for attempt in declines:
+        with pytest.raises(hc.StatusError) as err:
+            attempt()
+        assert err.value.is_unimplemented(), err.value
+    with pytest.raises(hc.StatusError) as err:  # a wrong output descriptor is the caller's error
+        hc.prepare(CTX, hc.Binary(), x, x, outputs=[D(DT.kBFloat16, [64, 4])])
+    assert err.value.is_invalid_argument()
+    assert hc.prepare(CTX, hc.Binary(), x, x, outputs=[x]).output_description() == x
+
+
+def test_zero_elements_are_a_no_op_and_launch_needs_a_device():
+    # src/compute_provider_native/elementwise.cc:222-223: success without touching storage
+    empty = hc.prepare(CTX, hc.Binary(), D(DT.kFloat32, [0, 16]), D(DT.kFloat32, [16]))
+    assert empty.route_name() == "no-op" and empty.dispatch_count() == 0
+    empty.create_invocation().submit(0, [0, 0], [0])
+    real = hc.prepare(CTX, hc.Binary(), D(DT.kFloat32, [4, 16]), D(DT.kFloat32, [16]))
+    with pytest.raises(hc.StatusError) as err:
+        real.create_invocation().submit(0, [16, 16], [32])
+    assert err.value.is_failed_precondition()
+    with pytest.raises(hc.StatusError) as err:  # binding count is checked first
+        real.create_invocation().submit(0, [16], [32])
+    assert err.value.is_invalid_argument()
