@@ -60,5 +60,30 @@ def build(verbose: bool = True) -> str:
     return LIB
 
 
+HOST_TEST_SOURCE = os.path.join(os.path.dirname(HERE), "tests", "cpp", "hip_provider_test.cc")
+HOST_TEST_BINARY = os.path.join(os.path.dirname(HERE), "tests", "cpp", "hip_provider_test")
+
+
+def build_host_tests(verbose: bool = True) -> str:
+    """Compiles the C++ tests of the host mirror (include/hyle_hip_compute.hpp) with g++ against
+    the built library, the HIP runtime and the C oracle (the checker)."""
+    root = os.path.dirname(HERE)
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [
+        "g++", "-std=c++20", "-O1", "-Wall", "-D__HIP_PLATFORM_AMD__",
+        "-I" + os.path.join(root, "include"), "-I" + os.path.join(root, "oracle"), "-I" + os.path.join(rocm, "include"),
+        HOST_TEST_SOURCE, "-o", HOST_TEST_BINARY,
+        "-L" + HERE, "-lhyle_hip", "-L" + os.path.join(root, "oracle"), "-lhyle_oracle",
+        "-L" + os.path.join(rocm, "lib"), "-lamdhip64",
+        "-Wl,-rpath,$ORIGIN/../../hyle_amd:$ORIGIN/../../oracle:" + os.path.join(rocm, "lib"),
+    ]
+    done = subprocess.run(cmd, capture_output=True, text=True)
+    if done.returncode != 0:
+        raise RuntimeError(f"g++ failed on the host tests:\n{done.stderr}")
+    if verbose:
+        print(f"built {HOST_TEST_BINARY}")
+    return HOST_TEST_BINARY
+
+
 if __name__ == "__main__":
     build()

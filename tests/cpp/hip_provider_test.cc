@@ -1,0 +1,382 @@
+// Tests of the C++ host mirror (include/hyle_hip_compute.hpp) in the shape of the reference's
+// provider tests (tests/compute_provider_native/elementwise_test.cc, normalization_test.cc,
+// transformer_test.cc, reduction_test.cc; tests/compute_provider_cuda/native_reduction_test.cc):
+// describe -> prepare -> create_invocation -> submit -> wait -> compare.
+//
+//   hip_provider_test --host     schema, inference, admission and error behaviour; no device used
+//   hip_provider_test --device   the same calls executed on device 0, compared with the CPU oracle
+//
+// The oracle (oracle/hyle_oracle.h) is linked here as the checker only.
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <limits>
+#include <random>
+#include <string>
+#include <vector>
+
+#include "hyle_hip_compute.hpp"
+#include "hyle_oracle.h"
+
+namespace {
+
+using namespace hyle::compute;
+using hyle::Status;
+
+struct Case { const char *name; bool device; std::function<void()> body; };
+std::vector<Case> &cases() { static std::vector<Case> all; return all; }
+int failures = 0;
+
+struct Registrar {
+  Registrar(const char *name, bool device, std::function<void()> body) { cases().push_back({name, device, std::move(body)}); }
+};
+#define HOST_TEST(name) void name(); Registrar reg_##name(#name, false, name); void name()
+#define DEVICE_TEST(name) void name(); Registrar reg_##name(#name, true, name); void name()
+#define EXPECT(cond) do { if (!(cond)) { ++failures; std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); } } while (0)
+#define REQUIRE(cond) do { if (!(cond)) { ++failures; std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond); return; } } while (0)
+
+constexpr float kInf = std::numeric_limits<float>::infinity();
+constexpr float kNaN = std::numeric_limits<float>::quiet_NaN();
+
+TensorDesc dense(DataType type, std::initializer_list<std::int64_t> dims) { return TensorDesc::dense(type, dims).value(); }
+
+// ---------------------------------------------------------------- host ----------------------------
+HOST_TEST(TensorDescDenseStridesAndZeroExtents) {
+  const TensorDesc d = dense(DataType::kBFloat16, {4, 3, 8});
+  EXPECT(d.rank() == 3 && d.is_dense());
+  EXPECT(d.byte_strides()[0] == 48 && d.byte_strides()[1] == 16 && d.byte_strides()[2] == 2);
+  EXPECT(d.element_count() == 96 && d.required_bytes() == 192);
+  const TensorDesc empty = dense(DataType::kFloat32, {4, 0, 8});
+  EXPECT(empty.is_dense() && empty.required_bytes() == 0);
+  EXPECT(empty.byte_strides()[0] == 0 && empty.byte_strides()[2] == 0);
+  EXPECT(TensorDesc::dense(DataType::kFloat32, {2, -1}).error().IsInvalidArgument());
+  const auto broadcast = TensorDesc::strided_bytes(DataType::kFloat32, {4, 8}, {0, 4});
+  REQUIRE(broadcast.has_value());
+  EXPECT(!broadcast->is_dense() && broadcast->required_bytes() == 32);
+  const auto q8 = TensorDesc::gguf_q8_0_weight(DataType::kBFloat16, 2048, 16);
+  REQUIRE(q8.has_value());
+  EXPECT(!q8->is_plain() && q8->required_bytes() == 16 * 64 * 34);
+  EXPECT(TensorDesc::gguf_q8_0_weight(DataType::kBFloat16, 2040, 16).error().IsInvalidArgument());
+}
+
+HOST_TEST(InfersOutputsLikeTheSchema) {
+  auto out = infer_output_descriptions(Binary{BinaryKind::kAdd},
+                                       {dense(DataType::kFloat32, {6, 1, 5}), dense(DataType::kFloat32, {4, 5})});
+  REQUIRE(out.has_value() && out->size() == 1);
+  EXPECT((*out)[0] == dense(DataType::kFloat32, {6, 4, 5}));
+  EXPECT(infer_output_descriptions(Binary{}, {dense(DataType::kFloat32, {3}), dense(DataType::kFloat32, {4})})
+             .error().IsInvalidArgument());
+  EXPECT(infer_output_descriptions(Binary{}, {dense(DataType::kFloat32, {3}), dense(DataType::kBFloat16, {3})})
+             .error().IsInvalidArgument());
+  out = infer_output_descriptions(TopK{}, {dense(DataType::kFloat32, {7, 100})});
+  REQUIRE(out.has_value() && out->size() == 2);
+  EXPECT((*out)[0] == dense(DataType::kFloat32, {7, 1}) && (*out)[1] == dense(DataType::kInt32, {7, 1}));
+  out = infer_output_descriptions(GatedActivation{}, {dense(DataType::kBFloat16, {9, 64})});
+  REQUIRE(out.has_value());
+  EXPECT((*out)[0] == dense(DataType::kBFloat16, {9, 32}));
+  EXPECT(infer_output_descriptions(GatedActivation{}, {dense(DataType::kBFloat16, {9, 63})}).error().IsInvalidArgument());
+  out = infer_output_descriptions(Reduce{ReductionKind::kMaximum, -1, true}, {dense(DataType::kFloat32, {3, 9})});
+  REQUIRE(out.has_value());
+  EXPECT((*out)[0] == dense(DataType::kFloat32, {3, 1}));
+  out = infer_output_descriptions(Q8_0DequantSumSquares{}, {*TensorDesc::gguf_q8_0_weight(DataType::kBFloat16, 64, 5)});
+  REQUIRE(out.has_value() && out->size() == 2);
+  EXPECT((*out)[0] == dense(DataType::kBFloat16, {5, 64}) && (*out)[1] == dense(DataType::kFloat32, {5}));
+  EXPECT(infer_output_descriptions(RmsNorm{}, {dense(DataType::kBFloat16, {4, 64}), dense(DataType::kBFloat16, {32})})
+             .error().IsInvalidArgument());
+  EXPECT(infer_output_descriptions(Softmax{.axis = 2}, {dense(DataType::kFloat32, {4, 64})}).error().IsOutOfRange() ||
+         infer_output_descriptions(Softmax{.axis = 2}, {dense(DataType::kFloat32, {4, 64})}).error().IsInvalidArgument());
+}
+
+HOST_TEST(PreparesRoutesAndDeclinesCleanly) {
+  const Context context = Context::planning_only();
+  auto add = prepare(context, Binary{BinaryKind::kAdd}, dense(DataType::kFloat32, {32, 256}), dense(DataType::kFloat32, {256}));
+  REQUIRE(add.has_value());
+  EXPECT(add->dispatch_count() == 1 && add->workspace_requirement().size == 0);
+  EXPECT(add->alias_support(0, 0)->supported && !add->alias_support(0, 1)->supported);
+  EXPECT(*add->output_description() == dense(DataType::kFloat32, {32, 256}));
+  auto top = prepare(context, TopK{}, dense(DataType::kFloat32, {8, 151936}));
+  REQUIRE(top.has_value());
+  EXPECT(top->dispatch_count() == 2 && top->workspace_requirement().size > 0);
+  EXPECT(top->create_invocation().error().IsInvalidArgument());  // needs its workspace
+  // Declines are Unimplemented, never an error a router would have to surface.
+  EXPECT(prepare(context, TopK{.count = 4}, dense(DataType::kFloat32, {8, 128})).error().IsUnimplemented());
+  EXPECT(prepare(context, Unary{UnaryKind::kTanh}, dense(DataType::kFloat32, {8})).error().IsUnimplemented());
+  EXPECT(prepare(context, GatedActivation{GatedActivationKind::kGelu}, dense(DataType::kBFloat16, {8, 64})).error().IsUnimplemented());
+  EXPECT(prepare(context, Binary{}, dense(DataType::kInt32, {8}), dense(DataType::kInt32, {8})).error().IsUnimplemented());
+  // Schema violations stay InvalidArgument.
+  EXPECT(prepare(context, Binary{}, dense(DataType::kFloat32, {3}), dense(DataType::kFloat32, {4})).error().IsInvalidArgument());
+  // Zero elements: prepared, nothing to dispatch.
+  auto none = prepare(context, Binary{}, dense(DataType::kFloat32, {0, 8}), dense(DataType::kFloat32, {8}));
+  REQUIRE(none.has_value());
+  EXPECT(none->dispatch_count() == 0);
+}
+
+HOST_TEST(SubmitWithoutDeviceIsFailedPrecondition) {
+  Context context = Context::planning_only();
+  EXPECT(context.create_queue().error().IsFailedPrecondition());
+}
+
+// -------------------------------------------------------------- device ----------------------------
+struct Fixture {
+  Context context = Context::create(hip::device(0)).value();
+  Queue queue = context.create_queue().value();
+};
+Fixture &fixture() { static Fixture f; return f; }
+
+template <class T> DeviceBuffer upload(const std::vector<T> &host) {
+  DeviceBuffer b = DeviceBuffer::create(host.size() * sizeof(T)).value();
+  EXPECT(b.write(host.data(), host.size() * sizeof(T)).ok());
+  return b;
+}
+template <class T> std::vector<T> download(const DeviceBuffer &b, std::size_t count) {
+  std::vector<T> host(count);
+  EXPECT(b.read(host.data(), count * sizeof(T)).ok());
+  return host;
+}
+std::vector<float> normal(std::size_t n, unsigned seed, float sigma = 1.0F) {
+  std::mt19937 rng(seed);
+  std::normal_distribution<float> dist(0.0F, sigma);
+  std::vector<float> v(n);
+  for (float &x : v) x = dist(rng);
+  return v;
+}
+std::vector<std::uint16_t> to_bf16(const std::vector<float> &v) {
+  std::vector<std::uint16_t> r(v.size());
+  hyle_oracle_convert_from_f32(HYLE_ORACLE_BF16, v.data(), r.data(), v.size());
+  return r;
+}
+bool same_bits(const void *a, const void *b, std::size_t bytes) { return std::memcmp(a, b, bytes) == 0; }
+// bf16 results may differ from the oracle by one unit in the last place (fused vs. scalar order).
+bool within_one_ulp_bf16(const std::vector<std::uint16_t> &got, const std::vector<std::uint16_t> &want) {
+  for (std::size_t i = 0; i < got.size(); ++i) {
+    const auto key = [](std::uint16_t b) { return (b & 0x8000U) ? -static_cast<int>(b & 0x7FFFU) : static_cast<int>(b & 0x7FFFU); };
+    const bool nan_g = (got[i] & 0x7FFFU) > 0x7F80U, nan_w = (want[i] & 0x7FFFU) > 0x7F80U;
+    if (nan_g != nan_w) return false;
+    if (!nan_g && std::abs(key(got[i]) - key(want[i])) > 1) return false;
+  }
+  return true;
+}
+
+DEVICE_TEST(BinaryAddBroadcastsRowVectorBitExactly) {
+  constexpr std::int64_t rows = 37, cols = 1000;  // not a multiple of the vector width
+  const auto a = normal(rows * cols, 1), b = normal(cols, 2);
+  const TensorDesc da = dense(DataType::kFloat32, {rows, cols}), db = dense(DataType::kFloat32, {cols});
+  auto prepared = prepare(fixture().context, Binary{BinaryKind::kAdd}, da, db);
+  REQUIRE(prepared.has_value());
+  DeviceBuffer left = upload(a), right = upload(b), out = DeviceBuffer::create(a.size() * 4).value();
+  auto invocation = prepared->create_invocation();
+  REQUIRE(invocation.has_value());
+  auto completion = invocation->submit(fixture().queue, *ConstTensorView::create(da, left), *ConstTensorView::create(db, right),
+                                       *TensorView::create(da, out));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<float> want(a.size());
+  const std::int64_t ad[2] = {rows, cols}, as[2] = {cols * 4, 4}, bd[1] = {cols}, bs[1] = {4};
+  hyle_oracle_binary(HYLE_ORACLE_ADD, HYLE_ORACLE_F32, a.data(), ad, as, 2, b.data(), bd, bs, 1, want.data(), ad, 2);
+  EXPECT(same_bits(download<float>(out, a.size()).data(), want.data(), a.size() * 4));
+  // In place over the left operand, which the plan reports as supported.
+  EXPECT(prepared->alias_support(0, 0)->supported);
+  completion = invocation->submit(fixture().queue, *ConstTensorView::create(da, left), *ConstTensorView::create(db, right),
+                                  *TensorView::create(da, left));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  EXPECT(same_bits(download<float>(left, a.size()).data(), want.data(), a.size() * 4));
+}
+
+DEVICE_TEST(BinaryChainEqualsTwoBinaries) {
+  constexpr std::int64_t rows = 64, cols = 512;
+  const auto a = normal(rows * cols, 3), b = normal(cols, 4);
+  const std::vector<float> s{0.125F};
+  const TensorDesc da = dense(DataType::kFloat32, {rows, cols}), db = dense(DataType::kFloat32, {cols}),
+                   ds = dense(DataType::kFloat32, {});
+  auto prepared = prepare(fixture().context, BinaryChain{BinaryKind::kAdd, BinaryKind::kMultiply}, da, db, ds);
+  REQUIRE(prepared.has_value());
+  DeviceBuffer ba = upload(a), bb = upload(b), bs = upload(s), out = DeviceBuffer::create(a.size() * 4).value();
+  auto invocation = prepared->create_invocation().value();
+  auto completion = invocation.submit(fixture().queue,
+                                      {*ConstTensorView::create(da, ba), *ConstTensorView::create(db, bb), *ConstTensorView::create(ds, bs)},
+                                      {*TensorView::create(da, out)});
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  const auto got = download<float>(out, a.size());
+  bool same = true;
+  for (std::int64_t r = 0; r < rows && same; ++r)
+    for (std::int64_t c = 0; c < cols; ++c) {
+      const float want = (a[r * cols + c] + b[c]) * s[0];
+      same = same && same_bits(&want, &got[r * cols + c], 4);
+    }
+  EXPECT(same);
+}
+
+DEVICE_TEST(RmsNormBf16WithinOneUlpOfScalarFloor) {
+  constexpr std::int64_t rows = 33, hidden = 2048;
+  const auto x = to_bf16(normal(rows * hidden, 5, 2.0F)), w = to_bf16(normal(hidden, 6));
+  const TensorDesc dx = dense(DataType::kBFloat16, {rows, hidden}), dw = dense(DataType::kBFloat16, {hidden});
+  auto prepared = prepare(fixture().context, RmsNorm{1.0e-6F}, dx, dw);
+  REQUIRE(prepared.has_value());
+  DeviceBuffer bx = upload(x), bw = upload(w), out = DeviceBuffer::create(x.size() * 2).value();
+  auto completion = prepared->create_invocation()->submit(fixture().queue, *ConstTensorView::create(dx, bx),
+                                                          *ConstTensorView::create(dw, bw), *TensorView::create(dx, out));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<std::uint16_t> want(x.size());
+  hyle_oracle_rms_norm(HYLE_ORACLE_BF16, HYLE_ORACLE_BF16, x.data(), w.data(), want.data(), rows, hidden, 1.0e-6F);
+  EXPECT(within_one_ulp_bf16(download<std::uint16_t>(out, x.size()), want));
+}
+
+DEVICE_TEST(SwigluSeparateBf16WithinOneUlp) {
+  constexpr std::int64_t rows = 17, width = 6144;
+  auto g = normal(rows * width, 7, 3.0F);
+  g[0] = -kInf; g[1] = kInf; g[2] = kNaN; g[3] = -0.0F; g[4] = -100.0F;
+  const auto gate = to_bf16(g), up = to_bf16(normal(rows * width, 8));
+  const TensorDesc d = dense(DataType::kBFloat16, {rows, width});
+  auto prepared = prepare(fixture().context, GatedActivation{GatedActivationKind::kSilu, GatedInputKind::kSeparate}, d, d);
+  REQUIRE(prepared.has_value());
+  DeviceBuffer bg = upload(gate), bu = upload(up), out = DeviceBuffer::create(gate.size() * 2).value();
+  auto completion = prepared->create_invocation()->submit(fixture().queue, *ConstTensorView::create(d, bg),
+                                                          *ConstTensorView::create(d, bu), *TensorView::create(d, out));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<std::uint16_t> want(gate.size());
+  hyle_oracle_swiglu(HYLE_ORACLE_BF16, gate.data(), up.data(), want.data(), gate.size());
+  EXPECT(within_one_ulp_bf16(download<std::uint16_t>(out, gate.size()), want));
+}
+
+DEVICE_TEST(SoftmaxBooleanMaskAndInvalidRows) {
+  constexpr std::int64_t heads = 3, seq = 192;
+  auto x = normal(heads * seq * seq, 9, 4.0F);
+  std::vector<std::uint8_t> mask(seq * seq);
+  for (std::int64_t q = 0; q < seq; ++q)
+    for (std::int64_t k = 0; k < seq; ++k) mask[q * seq + k] = k <= q;
+  for (std::int64_t k = 0; k < seq; ++k) mask[5 * seq + k] = 0;  // a fully masked row -> NaN row
+  x[(seq + 7) * seq + 3] = kNaN;                                   // head 1, row 7 holds a NaN -> NaN row
+  const TensorDesc dx = dense(DataType::kFloat32, {heads, seq, seq}), dm = dense(DataType::kBool, {seq, seq});
+  auto prepared = prepare(fixture().context, Softmax{.mask = MaskKind::kBoolean}, dx, dm);
+  REQUIRE(prepared.has_value());
+  DeviceBuffer bx = upload(x), bm = upload(mask), out = DeviceBuffer::create(x.size() * 4).value();
+  auto completion = prepared->create_invocation()->submit(fixture().queue, *ConstTensorView::create(dx, bx),
+                                                          *ConstTensorView::create(dm, bm), *TensorView::create(dx, out));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<float> want(x.size());
+  const std::int64_t xd[3] = {heads, seq, seq}, md[2] = {seq, seq}, ms[2] = {seq, 1};
+  hyle_oracle_softmax(HYLE_ORACLE_F32, x.data(), want.data(), xd, 3, 1.0F, HYLE_ORACLE_MASK_BOOLEAN, mask.data(), md, ms, 2);
+  const auto got = download<float>(out, x.size());
+  bool close = true;
+  for (std::size_t i = 0; i < got.size() && close; ++i) {
+    if (std::isnan(want[i])) close = std::isnan(got[i]);
+    else close = std::fabs(got[i] - want[i]) <= 1.0e-5F * std::fabs(want[i]) + 1.0e-9F;  // 1e-5 relative
+  }
+  EXPECT(close);
+  EXPECT(std::isnan(got[5 * seq]) && std::isnan(got[(seq + 7) * seq]) && got[0] == 1.0F);
+}
+
+DEVICE_TEST(TopKArgmaxOrdersNaNLastAndTiesLow) {
+  constexpr std::int64_t rows = 6, width = 151936;
+  auto x = normal(rows * width, 10);
+  x[0 * width + 777] = 9.0F; x[0 * width + 140000] = 9.0F;      // tie -> lower index
+  x[1 * width + 5] = kNaN; x[1 * width + 90000] = 8.0F;          // NaN never wins over a number
+  for (std::int64_t i = 0; i < width; ++i) x[2 * width + i] = kNaN;  // all NaN -> index 0
+  for (std::int64_t i = 0; i < width; ++i) x[3 * width + i] = -kInf;
+  x[3 * width + width - 1] = -1.0e30F;
+  x[4 * width + 100] = kInf;
+  const TensorDesc dx = dense(DataType::kFloat32, {rows, width});
+  auto prepared = prepare(fixture().context, TopK{}, dx);
+  REQUIRE(prepared.has_value());
+  const WorkspaceRequirement need = prepared->workspace_requirement();
+  DeviceBuffer bx = upload(x), values = DeviceBuffer::create(rows * 4).value(), indices = DeviceBuffer::create(rows * 4).value(),
+               workspace = DeviceBuffer::create(need.size).value();
+  auto invocation = prepared->create_invocation(workspace.data(), workspace.size());
+  REQUIRE(invocation.has_value());
+  auto completion = invocation->submit(fixture().queue, {*ConstTensorView::create(dx, bx)},
+                                       {*TensorView::create(*prepared->output_description(0), values),
+                                        *TensorView::create(*prepared->output_description(1), indices)});
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<float> want_values(rows);
+  std::vector<std::int32_t> want_indices(rows);
+  hyle_oracle_topk1_f32(x.data(), rows, width, want_values.data(), want_indices.data());
+  const auto got_indices = download<std::int32_t>(indices, rows);
+  EXPECT(got_indices == want_indices);
+  EXPECT(same_bits(download<float>(values, rows).data(), want_values.data(), rows * 4));
+  EXPECT(got_indices[0] == 777 && got_indices[1] == 90000 && got_indices[2] == 0 && got_indices[3] == width - 1 && got_indices[4] == 100);
+}
+
+DEVICE_TEST(Q8_0DequantBitExactWithRowSumSquares) {
+  constexpr std::int64_t n = 96, k = 2048, blocks = k / 32;
+  std::mt19937 rng(11);
+  std::vector<std::uint8_t> weight(n * blocks * 34);
+  for (std::int64_t b = 0; b < n * blocks; ++b) {
+    const std::uint16_t d = hyle_oracle_f32_to_f16(std::ldexp(static_cast<float>(rng() % 2048) / 2048.0F + 0.5F, -static_cast<int>(rng() % 12)));
+    std::memcpy(&weight[b * 34], &d, 2);
+    for (int j = 0; j < 32; ++j) weight[b * 34 + 2 + j] = static_cast<std::uint8_t>(rng());
+  }
+  const TensorDesc dw = *TensorDesc::gguf_q8_0_weight(DataType::kBFloat16, k, n);
+  auto prepared = prepare(fixture().context, Q8_0DequantSumSquares{}, dw);
+  REQUIRE(prepared.has_value());
+  DeviceBuffer bw = upload(weight), out = DeviceBuffer::create(n * k * 2).value(), sumsq = DeviceBuffer::create(n * 4).value();
+  auto completion = prepared->create_invocation()->submit(fixture().queue, {*ConstTensorView::create(dw, bw)},
+                                                          {*TensorView::create(*prepared->output_description(0), out),
+                                                           *TensorView::create(*prepared->output_description(1), sumsq)});
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<std::uint16_t> want(n * k);
+  std::vector<float> want_sumsq(n);
+  hyle_oracle_q8_0_dequant_bf16(weight.data(), n, k, blocks * 34, want.data(), want_sumsq.data(), nullptr);
+  EXPECT(same_bits(download<std::uint16_t>(out, n * k).data(), want.data(), n * k * 2));
+  const auto got_sumsq = download<float>(sumsq, n);
+  bool close = true;
+  for (std::int64_t r = 0; r < n; ++r) close = close && std::fabs(got_sumsq[r] - want_sumsq[r]) <= 1.0e-5F * want_sumsq[r];
+  EXPECT(close);  // summation order differs from the index-order oracle: 1e-5 relative
+}
+
+DEVICE_TEST(RejectedSubmissionsEnqueueNothing) {
+  const TensorDesc d = dense(DataType::kFloat32, {8, 64}), row = dense(DataType::kFloat32, {64});
+  auto prepared = prepare(fixture().context, Binary{BinaryKind::kMultiply}, d, row);
+  REQUIRE(prepared.has_value());
+  std::vector<float> ones(512, 1.0F);
+  DeviceBuffer a = upload(ones), b = upload(ones), out = DeviceBuffer::create(512 * 4).value();
+  auto invocation = prepared->create_invocation().value();
+  // One binding short.
+  auto short_bound = invocation.submit(fixture().queue, {*ConstTensorView::create(d, a)}, {*TensorView::create(d, out)});
+  EXPECT(!short_bound.has_value() && short_bound.error().IsInvalidArgument());
+  // The output may share storage with the left input only (its descriptor equals the output's);
+  // writing over the broadcast right operand is refused.
+  EXPECT(prepared->alias_support(0, 0)->supported && !prepared->alias_support(0, 1)->supported);
+  auto aliased = invocation.submit(fixture().queue, *ConstTensorView::create(d, a), *ConstTensorView::create(row, b),
+                                   *TensorView::create(d, b));
+  EXPECT(!aliased.has_value() && aliased.error().IsInvalidArgument());
+  // Storage too small for the description never reaches the provider.
+  EXPECT(TensorView::create(d, out.data(), 100).error().IsInvalidArgument());
+  // The invocation stays usable after rejections.
+  auto completion = invocation.submit(fixture().queue, *ConstTensorView::create(d, a), *ConstTensorView::create(row, b),
+                                      *TensorView::create(d, out));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  EXPECT(download<float>(out, 512) == ones);
+}
+
+}  // namespace
+
+int main(int argc, char **argv) {
+  const bool device = argc > 1 && std::string(argv[1]) == "--device";
+  if (argc != 2 || (!device && std::string(argv[1]) != "--host")) {
+    std::printf("usage: %s --host | --device\n", argv[0]);
+    return 2;
+  }
+  int ran = 0;
+  for (const Case &c : cases()) {
+    if (c.device != device) continue;
+    std::printf("[ RUN ] %s\n", c.name);
+    std::fflush(stdout);
+    const int before = failures;
+    c.body();
+    std::printf("[ %s ] %s\n", failures == before ? " OK " : "FAIL", c.name);
+    std::fflush(stdout);
+    ++ran;
+  }
+  std::printf("%d tests, %d failed expectations\n", ran, failures);
+  return failures == 0 ? 0 : 1;
+}
