@@ -63,83 +63,108 @@ __device__ __forceinline__ int64_t mask_row_offset(const MaskRows &m, uint32_t r
 // reach HBM (the mask's 16 MiB are fetched once per launch), and steering the heads of one
 // mask row onto one XCD changed neither the counter nor the run time, so there is no such
 // remapping here.
-template <class T, int kLanes, int kVpl, int kThreads>
+//
+// Loads carry no branches: a lane outside the row (or a row outside the tensor) reads a clamped,
+// valid address and discards the value, so all kVpl loads of a lane are in flight together.
+// Under a Boolean mask the mask words are read first and a vector whose elements are all masked
+// is not loaded at all: its values cannot reach the result (masked -> -inf before anything looks
+// at x, src/compute_provider_native/transformer.cc:44-57), so a causal mask saves half the reads.
+template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog>
 __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const void *mask, void *y,
                                                          uint32_t rows, uint32_t row_vectors,
-                                                         float scale, int mask_kind, int log_form,
-                                                         MaskRows mrows) {
+                                                         float scale, MaskRows mrows) {
   constexpr int kVec = Traits<T>::kVec;
+  constexpr int kWords = kVec / 4;  // mask bytes of one vector, as 32-bit words
   constexpr int kRowsPerBlock = kThreads / kLanes;
   constexpr int kWaves = kThreads / kWaveLanes;
-  __shared__ float joint_max[kWaves], joint_bad[kWaves], joint_sum[kWaves];
+  __shared__ float joint_max[kWaves], joint_sum[kWaves];
   const uint32_t lane = threadIdx.x % kLanes;
   const uint32_t row = blockIdx.x * kRowsPerBlock + threadIdx.x / kLanes;
   const bool row_ok = row < rows;
-  const size_t row_base = (size_t)row * row_vectors;
+  const uint32_t row_clamped = row_ok ? row : rows - 1;
+  const size_t row_base = (size_t)row_clamped * row_vectors;
   const char *mask_row = nullptr;
-  if (mask_kind != kMaskNone && row_ok)
-    mask_row = static_cast<const char *>(mask) + mask_row_offset(mrows, row);
+  if (kMask != kMaskNone) mask_row = static_cast<const char *>(mask) + mask_row_offset(mrows, row_clamped);
 
   float v[kVpl][kVec];
-  // ---- load, scale, mask ------------------------------------------------------
+  bool ok[kVpl];
+  uint32_t vec[kVpl];
 #pragma unroll
   for (int k = 0; k < kVpl; ++k) {
-    const uint32_t vec = lane + k * kLanes;
-    const bool ok = row_ok && vec < row_vectors;
-    if (ok) {
-      Traits<T>::unpack(load16_stream(x, row_base + vec), v[k]);
-    } else {
-#pragma unroll
-      for (int j = 0; j < kVec; ++j) v[k][j] = -INFINITY;
-    }
+    const uint32_t wanted = lane + k * kLanes;
+    ok[k] = row_ok && wanted < row_vectors;
+    vec[k] = wanted < row_vectors ? wanted : row_vectors - 1;
   }
-  if (mask_kind == kMaskBoolean) {
+
+  // ---- load, scale, mask ------------------------------------------------------
+  if constexpr (kMask == kMaskBoolean) {
+    uint32_t bits[kVpl][kWords];
+    if (mrows.inner_stride == 0) {
+      const uint32_t one = *reinterpret_cast<const uint8_t *>(mask_row) ? 0x01010101u : 0u;
+#pragma unroll
+      for (int k = 0; k < kVpl; ++k)
+#pragma unroll
+        for (int q = 0; q < kWords; ++q) bits[k][q] = one;
+    } else {
+      const uint32_t *words = reinterpret_cast<const uint32_t *>(mask_row);
+#pragma unroll
+      for (int k = 0; k < kVpl; ++k)
+#pragma unroll
+        for (int q = 0; q < kWords; ++q) bits[k][q] = words[(size_t)vec[k] * kWords + q];
+    }
 #pragma unroll
     for (int k = 0; k < kVpl; ++k) {
-      const uint32_t vec = lane + k * kLanes;
-      if (row_ok && vec < row_vectors) {
-        uint32_t bits[kVec / 4];
-        if (mrows.inner_stride == 0) {
-          const uint32_t one = *reinterpret_cast<const uint8_t *>(mask_row) ? 0x01010101u : 0u;
+      uint32_t any = 0;
 #pragma unroll
-          for (int q = 0; q < kVec / 4; ++q) bits[q] = one;
-        } else {
-          const uint32_t *words = reinterpret_cast<const uint32_t *>(mask_row) + (size_t)vec * (kVec / 4);
+      for (int q = 0; q < kWords; ++q) {
+        bits[k][q] = ok[k] ? bits[k][q] : 0u;
+        any |= bits[k][q];
+      }
+      if (any != 0) {
+        Traits<T>::unpack(load16_stream(x, row_base + vec[k]), v[k]);
+      } else {
 #pragma unroll
-          for (int q = 0; q < kVec / 4; ++q) bits[q] = words[q];
-        }
-#pragma unroll
-        for (int j = 0; j < kVec; ++j) {
-          const bool keep = ((bits[j / 4] >> (8 * (j % 4))) & 0xFFu) != 0;
-          v[k][j] = keep ? v[k][j] * scale : -INFINITY;
-        }
+        for (int j = 0; j < kVec; ++j) v[k][j] = 0.0f;
       }
     }
-  } else if (mask_kind == kMaskAdditive) {
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) {
-      const uint32_t vec = lane + k * kLanes;
-      if (row_ok && vec < row_vectors) {
-        float m[kVec];
-        if (mrows.inner_stride == 0) {
-          const float one = Traits<T>::load(mask_row, 0);
-#pragma unroll
-          for (int j = 0; j < kVec; ++j) m[j] = one;
-        } else {
-          Traits<T>::unpack(load16(mask_row, vec), m);
-        }
-#pragma unroll
-        for (int j = 0; j < kVec; ++j) v[k][j] = v[k][j] * scale + m[j];
-      }
-    }
-  } else {
 #pragma unroll
     for (int k = 0; k < kVpl; ++k)
 #pragma unroll
-      for (int j = 0; j < kVec; ++j) v[k][j] = v[k][j] * scale;
+      for (int j = 0; j < kVec; ++j) {
+        const bool keep = ((bits[k][j / 4] >> (8 * (j % 4))) & 0xFFu) != 0;
+        v[k][j] = keep ? v[k][j] * scale : -INFINITY;
+      }
+  } else {
+#pragma unroll
+    for (int k = 0; k < kVpl; ++k) Traits<T>::unpack(load16_stream(x, row_base + vec[k]), v[k]);
+    if constexpr (kMask == kMaskAdditive) {
+      float m[kVpl][kVec];
+      if (mrows.inner_stride == 0) {
+        const float one = Traits<T>::load(mask_row, 0);
+#pragma unroll
+        for (int k = 0; k < kVpl; ++k)
+#pragma unroll
+          for (int j = 0; j < kVec; ++j) m[k][j] = one;
+      } else {
+#pragma unroll
+        for (int k = 0; k < kVpl; ++k) Traits<T>::unpack(load16(mask_row, vec[k]), m[k]);
+      }
+#pragma unroll
+      for (int k = 0; k < kVpl; ++k)
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) v[k][j] = ok[k] ? v[k][j] * scale + m[k][j] : -INFINITY;
+    } else {
+#pragma unroll
+      for (int k = 0; k < kVpl; ++k)
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) v[k][j] = ok[k] ? v[k][j] * scale : -INFINITY;
+    }
   }
 
   // ---- row maximum and validity -------------------------------------------------
+  // A NaN or +inf anywhere makes the row undefined.  fmaxf never lets a NaN through, so a lane
+  // that met one reports +inf instead: after the reduction an infinite maximum of either sign
+  // (+inf: poisoned, -inf: nothing finite and unmasked) marks the row.
   float peak = -INFINITY;
   bool poisoned = false;
 #pragma unroll
@@ -147,11 +172,10 @@ __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const vo
 #pragma unroll
     for (int j = 0; j < kVec; ++j) {
       poisoned = poisoned || poisons_row(v[k][j]);
-      peak = fmaxf(peak, v[k][j]);  // a NaN never replaces the running value
+      peak = fmaxf(peak, v[k][j]);
     }
-  peak = row_max<kLanes>(peak, joint_max);
-  const float bad = row_max<kLanes>(poisoned ? 1.0f : 0.0f, joint_bad);
-  const bool invalid = bad != 0.0f || peak == -INFINITY;
+  peak = row_max<kLanes>(poisoned ? INFINITY : peak, joint_max);
+  const bool invalid = __builtin_fabsf(peak) == INFINITY;
 
   // ---- exponentials and their sum -------------------------------------------------
   float total = 0.0f;
@@ -160,7 +184,7 @@ __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const vo
 #pragma unroll
     for (int j = 0; j < kVec; ++j) {
       const float shifted = v[k][j] - peak;
-      if (log_form) {
+      if constexpr (kLog) {
         total += exp_scaled(shifted);
         v[k][j] = shifted;
       } else {
@@ -174,17 +198,15 @@ __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const vo
   // softmax: e * 2^32 * (1 / (sum * 2^32)).  log-softmax: (v - max) - log(sum).
   // An undefined row gets a NaN normaliser: it turns every lane, masked zeros included,
   // into NaN without a per-element select.
-  float normaliser = log_form ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
+  float normaliser = kLog ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
   if (invalid) normaliser = __builtin_nanf("");
 #pragma unroll
   for (int k = 0; k < kVpl; ++k) {
-    const uint32_t vec = lane + k * kLanes;
-    if (row_ok && vec < row_vectors) {
+    if (ok[k]) {
       float r[kVec];
 #pragma unroll
-      for (int j = 0; j < kVec; ++j)
-        r[j] = log_form ? v[k][j] - normaliser : v[k][j] * normaliser;
-      store16_stream(y, row_base + vec, Traits<T>::pack(r));
+      for (int j = 0; j < kVec; ++j) r[j] = kLog ? v[k][j] - normaliser : v[k][j] * normaliser;
+      store16_stream(y, (size_t)row * row_vectors + vec[k], Traits<T>::pack(r));
     }
   }
 }
@@ -313,9 +335,9 @@ __global__ __launch_bounds__(kBlockThreads) void reduce_rows(const void *x, void
 }
 
 // ---- host dispatch ----------------------------------------------------------------------------
-template <class T, int kLanes, int kVpl, int kThreads = kBlockThreads>
-hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, void *y,
-                    hipStream_t s) {
+template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog>
+hipError_t run_rows_as(const SoftmaxParams &p, const void *x, const void *mask, void *y,
+                       hipStream_t s) {
   constexpr int kRowsPerBlock = kThreads / kLanes;
   const uint32_t rows = (uint32_t)p.shape.rows;
   const uint32_t blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
@@ -326,10 +348,26 @@ hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, voi
     m.outer_strides[i] = p.mask_outer_strides[i];
   }
   m.inner_stride = p.mask_inner_stride;
-  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads>), dim3(blocks), dim3(kThreads), 0, s, x,
-                     mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, (int)p.mask_kind,
-                     p.log ? 1 : 0, m);
+  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads, kMask, kLog>), dim3(blocks),
+                     dim3(kThreads), 0, s, x, mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, m);
   return hipGetLastError();
+}
+
+template <class T, int kLanes, int kVpl, int kThreads = kBlockThreads>
+hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, void *y,
+                    hipStream_t s) {
+  const bool log_form = p.log;
+  switch ((int)p.mask_kind) {
+    case kMaskBoolean:
+      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, true>(p, x, mask, y, s)
+                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, false>(p, x, mask, y, s);
+    case kMaskAdditive:
+      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, true>(p, x, mask, y, s)
+                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, false>(p, x, mask, y, s);
+    default:
+      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, true>(p, x, mask, y, s)
+                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, false>(p, x, mask, y, s);
+  }
 }
 
 template <class T>
@@ -341,14 +379,20 @@ hipError_t run_softmax(const SoftmaxParams &p, const void *x, const void *mask, 
   if (vectors <= 32) return run_rows<T, 32, 1>(p, x, mask, y, s);
   if (vectors <= 64) return run_rows<T, 64, 1>(p, x, mask, y, s);
   if (vectors <= 128) return run_rows<T, 64, 2>(p, x, mask, y, s);
-  if (vectors <= 256) return run_rows<T, 64, 4>(p, x, mask, y, s);
-  if (vectors <= 512) return run_rows<T, 64, 8>(p, x, mask, y, s);
-  // Measured on MI355X for S[32,4096,4096] f32 with a causal mask (us per launch): two waves
-  // per row with 8 vectors per lane 785; four waves x 4 vectors 813; eight waves x 2 vectors
-  // 827; sixteen waves x 1 vector 1224; one wave x 16 vectors 834.
-  if (vectors <= 1024) return run_rows<T, 128, 8>(p, x, mask, y, s);
-  if (vectors <= 2048) return run_rows<T, 256, 8>(p, x, mask, y, s);
-  return run_rows<T, 256, 16>(p, x, mask, y, s);
+  if (vectors <= 256) return run_rows<T, 128, 2>(p, x, mask, y, s);
+  if (vectors <= 512) return run_rows<T, 256, 2>(p, x, mask, y, s);
+  // Measured on MI355X for S[32,4096,4096] f32 (1024 vectors per row), us per launch.  Every
+  // vector loaded (no mask, additive mask): eight waves x 2 vectors per lane, one row per block
+  // 685; two waves x 8 vectors 706-737; four waves x 4 vectors 731; a plain copy in the same
+  // shapes 688-737.  Boolean causal mask, masked vectors not loaded: four waves x 4 vectors,
+  // two rows per block 523; eight waves x 2 vectors 581; two waves x 8 vectors 569-591.
+  if (vectors <= 1024) {
+    if ((int)p.mask_kind == kMaskBoolean) return run_rows<T, 256, 4, 512>(p, x, mask, y, s);
+    return run_rows<T, 512, 2, 512>(p, x, mask, y, s);
+  }
+  if (vectors <= 2048) return run_rows<T, 512, 4, 512>(p, x, mask, y, s);
+  if (vectors <= 4096) return run_rows<T, 1024, 4, 1024>(p, x, mask, y, s);
+  return run_rows<T, 1024, 8, 1024>(p, x, mask, y, s);
 }
 
 template <class T>

@@ -364,6 +364,44 @@ def test_softmax_widths_masks_every_route(tag):
         softmax_bar(to_host(out), want) if tag == "f32" else assert_narrow_ulp(to_host(out), want, tag)
 
 
+@pytest.mark.parametrize("tag", ["f32", "bf16"])
+def test_softmax_boolean_mask_hides_specials_additive_mask_does_not(tag):
+    # A masked element is replaced by -inf before anything looks at it
+    # (src/compute_provider_native/transformer.cc:44-57): NaN and +inf under a false mask byte
+    # leave the row defined.  Under an additive -inf they still poison it (NaN + -inf, inf - inf).
+    oid = TYPES[tag][1]
+    rng = np.random.default_rng(110)
+    for width in (24, 512, 4096, 9000):
+        x = rng.normal(0, 3, (2, 6, width)).astype(np.float32)
+        keep = np.ones((6, width), np.uint8)
+        keep[:, width // 2:] = 0          # whole vectors masked: never loaded
+        keep[:, 3] = 0                    # a masked element inside a loaded vector
+        x[0, 0, width - 1] = np.nan
+        x[0, 1, width // 2] = np.inf
+        x[1, 2, 3] = np.nan
+        x[1, 3, 3] = np.inf
+        x[1, 4, 1] = np.nan               # unmasked: this row is undefined
+        x = host_values(x, tag)
+        note(f"softmax {tag} width {width}: specials under a Boolean mask")
+        dmask = torch.from_numpy(keep).to(DEVICE).view(torch.bool)
+        (out,) = run(hc.Softmax(mask=hc.MaskKind.kBoolean), to_device(x, tag), dmask)
+        got = to_host(out)
+        want = orc.softmax(oid, x, mask_kind=orc.MASK_BOOLEAN, mask=keep)
+        softmax_bar(got, want) if tag == "f32" else assert_narrow_ulp(got, want, tag)
+        as_f32 = got if tag == "f32" else orc.to_f32(oid, got)
+        assert np.isnan(as_f32[1, 4]).all()
+        assert not np.isnan(np.delete(as_f32.reshape(12, width), 10, axis=0)).any()
+        note(f"softmax {tag} width {width}: the same specials under an additive mask")
+        add = host_values(np.where(keep == 0, -np.inf, 0.0).astype(np.float32), tag)
+        (out,) = run(hc.Softmax(mask=hc.MaskKind.kAdditive), to_device(x, tag), to_device(add, tag))
+        got = to_host(out)
+        want = orc.softmax(oid, x, mask_kind=orc.MASK_ADDITIVE, mask=add)
+        softmax_bar(got, want) if tag == "f32" else assert_narrow_ulp(got, want, tag)
+        as_f32 = got if tag == "f32" else orc.to_f32(oid, got)
+        for h, q in ((0, 0), (0, 1), (1, 2), (1, 3), (1, 4)):
+            assert np.isnan(as_f32[h, q]).all()
+
+
 def test_softmax_subnormal_tail_and_wide_range():
     note("softmax f32 row spanning 160 units of range")
     rng = np.random.default_rng(107)
