@@ -134,6 +134,13 @@ template <> struct Traits<F16> {
   }
 };
 
+// A fence for the compiler only: the loads written before it are issued before it and no
+// later load is hoisted above it, and the named registers must hold their loaded values here.
+// Used after a group of independent loads so that they are all in flight together instead of
+// being sunk next to their first use, one memory latency after another.
+__device__ __forceinline__ void loads_issued(u32x4 &a) { asm volatile("" : "+v"(a) : : "memory"); }
+__device__ __forceinline__ void loads_issued(uint32_t &a) { asm volatile("" : "+v"(a) : : "memory"); }
+
 // 16-byte global access.  Streaming data is touched once, so loads and stores
 // carry the non-temporal hint; small reused operands use the plain forms.
 __device__ __forceinline__ u32x4 load16_stream(const void *base, size_t vec) {

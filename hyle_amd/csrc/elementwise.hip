@@ -124,6 +124,83 @@ struct Operand {
 };
 
 template <class T>
+__device__ __forceinline__ float fetch1(const Operand &op, uint32_t e) {
+  return Traits<T>::load(op.base, op.period ? e % op.period : e);
+}
+
+// ---- every input as long as the output -------------------------------------------------
+// Each lane handles kUnroll vectors, kThreads apart.  Loads carry no branches (a lane past the
+// end reads the last vector and drops it) and no load sits next to its first use:
+// kSerial = false issues every load of the lane before the first value is consumed;
+// kSerial = true takes the vectors one after another (the loads of vector k + 1 are issued
+// while vector k is computed).  Either way the results stay in registers and all stores follow
+// the last load, so a block reads in one phase and writes in another.
+template <class T, class Fn, int kUnroll, int kThreads, bool kSerial>
+__global__ __launch_bounds__(kThreads) void ew_full_vec(const void *a, const void *b, const void *c,
+                                                        void *out, uint32_t vectors,
+                                                        uint32_t elements, Fn fn) {
+  constexpr int kVec = Traits<T>::kVec;
+  const uint32_t first = blockIdx.x * (kUnroll * kThreads) + threadIdx.x;
+  if (vectors != 0) {
+    u32x4 rx[kUnroll], ry[kUnroll], rz[kUnroll], result[kUnroll];
+    auto load = [&](int k) {
+      const uint32_t vec = first + k * kThreads;
+      const uint32_t at = vec < vectors ? vec : vectors - 1;
+      rx[k] = load16_stream(a, at);
+      if constexpr (Fn::kInputs > 1) ry[k] = load16_stream(b, at);
+      if constexpr (Fn::kInputs > 2) rz[k] = load16_stream(c, at);
+    };
+    auto arrived = [&](int k) {
+      loads_issued(rx[k]);
+      if constexpr (Fn::kInputs > 1) loads_issued(ry[k]);
+      if constexpr (Fn::kInputs > 2) loads_issued(rz[k]);
+    };
+    auto compute = [&](int k) {
+      float x[kVec], y[kVec], z[kVec], r[kVec];
+      Traits<T>::unpack(rx[k], x);
+      if constexpr (Fn::kInputs > 1) Traits<T>::unpack(ry[k], y);
+      if constexpr (Fn::kInputs > 2) Traits<T>::unpack(rz[k], z);
+#pragma unroll
+      for (int j = 0; j < kVec; ++j)
+        r[j] = fn(T{}, x[j], Fn::kInputs > 1 ? y[j] : 0.0f, Fn::kInputs > 2 ? z[j] : 0.0f);
+      result[k] = Traits<T>::pack(r);
+    };
+    if constexpr (kSerial) {
+      load(0);
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) {
+        arrived(k);
+        if (k + 1 < kUnroll) load(k + 1);
+        compute(k);
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) load(k);
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) arrived(k);
+#pragma unroll
+      for (int k = 0; k < kUnroll; ++k) compute(k);
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const uint32_t vec = first + k * kThreads;
+      if (vec < vectors) store16_stream(out, vec, result[k]);
+    }
+  }
+  // elements past the last whole vector
+  if (blockIdx.x == 0) {
+    const uint32_t e = vectors * kVec + threadIdx.x;
+    if (e < elements) {
+      const float xs = Traits<T>::load(a, e);
+      const float ys = Fn::kInputs > 1 ? Traits<T>::load(b, e) : 0.0f;
+      const float zs = Fn::kInputs > 2 ? Traits<T>::load(c, e) : 0.0f;
+      Traits<T>::store(out, e, fn(T{}, xs, ys, zs));
+    }
+  }
+}
+
+// ---- broadcast operands (a repeating suffix, a single value) -------------------------------
+template <class T>
 __device__ __forceinline__ void fetch(const Operand &op, uint32_t vec, float (&v)[Traits<T>::kVec]) {
   constexpr int kVec = Traits<T>::kVec;
   if (op.period == 0) {
@@ -137,21 +214,18 @@ __device__ __forceinline__ void fetch(const Operand &op, uint32_t vec, float (&v
   }
 }
 
-template <class T>
-__device__ __forceinline__ float fetch1(const Operand &op, uint32_t e) {
-  return Traits<T>::load(op.base, op.period ? e % op.period : e);
-}
-
-template <class T, class Fn, int kUnroll>
-__global__ __launch_bounds__(kBlockThreads) void ew_flat_vec(Operand a, Operand b, Operand c,
-                                                             void *out, uint32_t vectors,
-                                                             uint32_t elements, Fn fn) {
+// The addressing mode of each operand is a launch-uniform branch around its load and decode,
+// so a lane takes its operands one after another; all stores follow the last load.
+template <class T, class Fn, int kUnroll, int kThreads>
+__global__ __launch_bounds__(kThreads) void ew_flat_vec(Operand a, Operand b, Operand c,
+                                                        void *out, uint32_t vectors,
+                                                        uint32_t elements, Fn fn) {
   constexpr int kVec = Traits<T>::kVec;
-  const uint32_t first = blockIdx.x * (kUnroll * kBlockThreads) + threadIdx.x;
+  const uint32_t first = blockIdx.x * (kUnroll * kThreads) + threadIdx.x;
   float x[kUnroll][kVec], y[kUnroll][kVec], z[kUnroll][kVec];
 #pragma unroll
   for (int k = 0; k < kUnroll; ++k) {
-    const uint32_t vec = first + k * kBlockThreads;
+    const uint32_t vec = first + k * kThreads;
     if (vec < vectors) {
       fetch<T>(a, vec, x[k]);
       if constexpr (Fn::kInputs > 1) fetch<T>(b, vec, y[k]);
@@ -160,7 +234,7 @@ __global__ __launch_bounds__(kBlockThreads) void ew_flat_vec(Operand a, Operand 
   }
 #pragma unroll
   for (int k = 0; k < kUnroll; ++k) {
-    const uint32_t vec = first + k * kBlockThreads;
+    const uint32_t vec = first + k * kThreads;
     if (vec < vectors) {
       float r[kVec];
 #pragma unroll
@@ -275,30 +349,55 @@ Operand make_operand(const void *base, uint32_t period, int vec) {
   return op;
 }
 
-template <class T, class Fn, int kUnroll>
-hipError_t run_vec_unrolled(const EwFlat &p, Operand a, Operand b, Operand c, void *out,
-                            hipStream_t s) {
+template <class T, class Fn, int kUnroll, int kThreads, bool kSerial>
+hipError_t run_full_as(const EwFlat &p, Operand a, Operand b, Operand c, void *out, hipStream_t s) {
   constexpr int kVec = Traits<T>::kVec;
   const uint64_t vectors = p.elements / kVec;
-  const uint64_t per_block = (uint64_t)kUnroll * kBlockThreads;
+  const uint64_t per_block = (uint64_t)kUnroll * kThreads;
   uint64_t blocks = (vectors + per_block - 1) / per_block;
   if (blocks == 0) blocks = 1;  // the tail still needs block 0
-  hipLaunchKernelGGL((ew_flat_vec<T, Fn, kUnroll>), dim3((uint32_t)blocks), dim3(kBlockThreads), 0, s,
+  hipLaunchKernelGGL((ew_full_vec<T, Fn, kUnroll, kThreads, kSerial>), dim3((uint32_t)blocks),
+                     dim3(kThreads), 0, s, a.base, b.base, c.base, out, (uint32_t)vectors,
+                     (uint32_t)p.elements, Fn{});
+  return hipGetLastError();
+}
+
+template <class T, class Fn, int kUnroll, int kThreads = kBlockThreads>
+hipError_t run_flat_as(const EwFlat &p, Operand a, Operand b, Operand c, void *out, hipStream_t s) {
+  constexpr int kVec = Traits<T>::kVec;
+  const uint64_t vectors = p.elements / kVec;
+  const uint64_t per_block = (uint64_t)kUnroll * kThreads;
+  uint64_t blocks = (vectors + per_block - 1) / per_block;
+  if (blocks == 0) blocks = 1;  // the tail still needs block 0
+  hipLaunchKernelGGL((ew_flat_vec<T, Fn, kUnroll, kThreads>), dim3((uint32_t)blocks), dim3(kThreads), 0, s,
                      a, b, c, out, (uint32_t)vectors, (uint32_t)p.elements, Fn{});
   return hipGetLastError();
 }
 
-// Vectors per lane, chosen from what was measured on MI355X: launches that move less than
-// about 80 MB finish in a few microseconds and do best with four vectors in flight per lane
-// (fewer, fatter blocks: (A[4096,2048] + b) * s takes 11.8 us against 12.7 us); larger ones
-// do best with one vector per lane (SwiGLU over [8192,6144] bf16: 47.8 us against 50.3 us).
+// Launch shape from the HBM traffic of the launch (streams as long as the output, the output
+// included), as measured on MI355X.  Inputs all as long as the output: R[8192,2048] += Y bf16
+// (101 MB) takes 16.5 us with 8 vectors per lane taken serially in blocks of 512 threads,
+// against 17.1 (4 at once, 256 threads) and 17.8 (1 vector per lane); SwiGLU over [8192,6144]
+// bf16 (302 MB) takes 46.9 us with 4 vectors at once against 47.5 (1 vector) and 49-53 for the
+// serial forms.  With broadcast operands: (A[4096,2048] + b) * s f32 (67 MB) takes 11.3 us
+// with 4 vectors per lane in blocks of 1024 threads against 11.8 (256 threads) and 12.9
+// (8 vectors).
 template <class T, class Fn>
 hipError_t run_vec(const EwFlat &p, Operand a, Operand b, Operand c, void *out, hipStream_t s) {
   uint64_t streams = 1;  // the output
-  for (int i = 0; i < p.inputs; ++i) streams += p.period[i] == 0 ? 1 : 0;
+  bool all_full = true;
+  for (int i = 0; i < p.inputs; ++i) {
+    streams += p.period[i] == 0 ? 1 : 0;
+    all_full = all_full && p.period[i] == 0;
+  }
   const uint64_t traffic = streams * p.elements * Traits<T>::kSize;
-  if (traffic > (80ull << 20)) return run_vec_unrolled<T, Fn, 1>(p, a, b, c, out, s);
-  return run_vec_unrolled<T, Fn, 4>(p, a, b, c, out, s);
+  if (!all_full) {
+    if (traffic > (80ull << 20)) return run_flat_as<T, Fn, 1, 256>(p, a, b, c, out, s);
+    return run_flat_as<T, Fn, 4, 1024>(p, a, b, c, out, s);
+  }
+  if (traffic > (110ull << 20)) return run_full_as<T, Fn, 4, 256, false>(p, a, b, c, out, s);
+  if (traffic > (48ull << 20)) return run_full_as<T, Fn, 8, 512, true>(p, a, b, c, out, s);
+  return run_full_as<T, Fn, 4, 512, true>(p, a, b, c, out, s);
 }
 
 template <class T, int kKind0>
