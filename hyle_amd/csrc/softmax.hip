@@ -58,47 +58,66 @@ __device__ __forceinline__ int64_t mask_row_offset(const MaskRows &m, uint32_t r
   return offset;
 }
 
-// Rows are taken in storage order.  A mask broadcast over leading axes (a [q, k] mask under
-// [heads, q, k]) is re-read by every head; the FETCH_SIZE counter shows those re-reads never
-// reach HBM (the mask's 16 MiB are fetched once per launch), and steering the heads of one
-// mask row onto one XCD changed neither the counter nor the run time, so there is no such
-// remapping here.
+// A lane group (kLanes lanes, each with kVpl 16-byte vectors) owns one row at a time.
 //
 // Loads carry no branches: a lane outside the row (or a row outside the tensor) reads a clamped,
 // valid address and discards the value, so all kVpl loads of a lane are in flight together.
 // Under a Boolean mask the mask words are read first and a vector whose elements are all masked
 // is not loaded at all: its values cannot reach the result (masked -> -inf before anything looks
 // at x, src/compute_provider_native/transformer.cc:44-57), so a causal mask saves half the reads.
-template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog>
+//
+// A mask broadcast over the leading axes (a [q, k] mask under [heads, q, k]) repeats every
+// `period` rows, `repeats` times.  With kRepeat > 1 a lane group takes row q of kRepeat
+// consecutive repeats: the mask row is read once and kept in registers, and the next row's loads
+// are issued before the current row is reduced.  The re-reads this saves never reached HBM (the
+// FETCH_SIZE counter shows the mask fetched once per launch either way) but they did cross the
+// cache fabric: measured on MI355X for S[32,4096,4096] f32 with an additive f32 mask, 804 us
+// with one head per lane group and 709 us with two.  A Boolean mask (a quarter of the bytes, and
+// half the rows' vectors never loaded) gains nothing from it.
+template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog, int kRepeat>
 __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const void *mask, void *y,
                                                          uint32_t rows, uint32_t row_vectors,
-                                                         float scale, MaskRows mrows) {
+                                                         float scale, MaskRows mrows, uint32_t period,
+                                                         uint32_t repeats) {
   constexpr int kVec = Traits<T>::kVec;
   constexpr int kWords = kVec / 4;  // mask bytes of one vector, as 32-bit words
-  constexpr int kRowsPerBlock = kThreads / kLanes;
+  constexpr int kGroupsPerBlock = kThreads / kLanes;
   constexpr int kWaves = kThreads / kWaveLanes;
-  __shared__ float joint_max[kWaves], joint_sum[kWaves];
+  __shared__ float joint_max[2][kWaves], joint_sum[2][kWaves];
   const uint32_t lane = threadIdx.x % kLanes;
-  const uint32_t row = blockIdx.x * kRowsPerBlock + threadIdx.x / kLanes;
-  const bool row_ok = row < rows;
-  const uint32_t row_clamped = row_ok ? row : rows - 1;
-  const size_t row_base = (size_t)row_clamped * row_vectors;
+  const uint32_t group = blockIdx.x * kGroupsPerBlock + threadIdx.x / kLanes;
+  // row of repeat i: first_row + i * row_step, valid while i < valid_repeats
+  uint32_t first_row, row_step, valid_repeats;
+  if constexpr (kRepeat == 1) {
+    first_row = group;
+    row_step = 0;
+    valid_repeats = group < rows ? 1u : 0u;
+  } else {
+    const uint32_t chunk = group / period, first_repeat = chunk * kRepeat;
+    first_row = first_repeat * period + group % period;
+    row_step = period;
+    valid_repeats = first_repeat < repeats ? repeats - first_repeat : 0u;
+  }
+  const uint32_t mask_row_index = first_row < rows ? first_row : rows - 1;
   const char *mask_row = nullptr;
-  if (kMask != kMaskNone) mask_row = static_cast<const char *>(mask) + mask_row_offset(mrows, row_clamped);
+  if (kMask != kMaskNone) mask_row = static_cast<const char *>(mask) + mask_row_offset(mrows, mask_row_index);
 
-  float v[kVpl][kVec];
   bool ok[kVpl];
   uint32_t vec[kVpl];
 #pragma unroll
   for (int k = 0; k < kVpl; ++k) {
     const uint32_t wanted = lane + k * kLanes;
-    ok[k] = row_ok && wanted < row_vectors;
-    vec[k] = wanted < row_vectors ? wanted : row_vectors - 1;
+    ok[k] = wanted < row_vectors;
+    vec[k] = ok[k] ? wanted : row_vectors - 1;
   }
 
-  // ---- load, scale, mask ------------------------------------------------------
+  // ---- the mask row, once ---------------------------------------------------------------
+  uint32_t bits[kVpl][kWords];
+  float addend[kVpl][kVec];
+  bool wanted_vector[kVpl];
+#pragma unroll
+  for (int k = 0; k < kVpl; ++k) wanted_vector[k] = true;
   if constexpr (kMask == kMaskBoolean) {
-    uint32_t bits[kVpl][kWords];
     if (mrows.inner_stride == 0) {
       const uint32_t one = *reinterpret_cast<const uint8_t *>(mask_row) ? 0x01010101u : 0u;
 #pragma unroll
@@ -120,93 +139,113 @@ __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const vo
         bits[k][q] = ok[k] ? bits[k][q] : 0u;
         any |= bits[k][q];
       }
-      if (any != 0) {
-        Traits<T>::unpack(load16_stream(x, row_base + vec[k]), v[k]);
-      } else {
+      wanted_vector[k] = any != 0;
+    }
+  } else if constexpr (kMask == kMaskAdditive) {
+    if (mrows.inner_stride == 0) {
+      const float one = Traits<T>::load(mask_row, 0);
 #pragma unroll
-        for (int j = 0; j < kVec; ++j) v[k][j] = 0.0f;
+      for (int k = 0; k < kVpl; ++k)
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) addend[k][j] = one;
+    } else {
+#pragma unroll
+      for (int k = 0; k < kVpl; ++k) Traits<T>::unpack(load16(mask_row, vec[k]), addend[k]);
+    }
+  }
+
+  u32x4 current[kVpl], next[kVpl];
+  auto issue = [&](int i, u32x4(&into)[kVpl]) {
+    const uint32_t row = first_row + (uint32_t)i * row_step;
+    const size_t row_base = (size_t)((uint32_t)i < valid_repeats ? row : mask_row_index) * row_vectors;
+#pragma unroll
+    for (int k = 0; k < kVpl; ++k) {
+      into[k] = u32x4{0u, 0u, 0u, 0u};
+      if constexpr (kMask == kMaskBoolean) {
+        if (wanted_vector[k]) into[k] = load16_stream(x, row_base + vec[k]);
+      } else {
+        into[k] = load16_stream(x, row_base + vec[k]);
       }
     }
+  };
+  issue(0, current);
+#pragma unroll
+  for (int i = 0; i < kRepeat; ++i) {
+    if (i + 1 < kRepeat) issue(i + 1, next);
+#pragma unroll
+    for (int k = 0; k < kVpl; ++k) loads_issued(current[k]);
+    const bool row_ok = (uint32_t)i < valid_repeats;
+    const uint32_t row = first_row + (uint32_t)i * row_step;
+
+    // ---- scale, mask --------------------------------------------------------------------
+    float v[kVpl][kVec];
+#pragma unroll
+    for (int k = 0; k < kVpl; ++k) {
+      Traits<T>::unpack(current[k], v[k]);
+#pragma unroll
+      for (int j = 0; j < kVec; ++j) {
+        if constexpr (kMask == kMaskBoolean) {
+          const bool keep = ((bits[k][j / 4] >> (8 * (j % 4))) & 0xFFu) != 0;
+          v[k][j] = keep ? v[k][j] * scale : -INFINITY;
+        } else if constexpr (kMask == kMaskAdditive) {
+          v[k][j] = ok[k] ? v[k][j] * scale + addend[k][j] : -INFINITY;
+        } else {
+          v[k][j] = ok[k] ? v[k][j] * scale : -INFINITY;
+        }
+      }
+    }
+
+    // ---- row maximum and validity -------------------------------------------------------
+    // A NaN or +inf anywhere makes the row undefined.  fmaxf never lets a NaN through, so a
+    // lane that met one reports +inf instead: after the reduction an infinite maximum of either
+    // sign (+inf: poisoned, -inf: nothing finite and unmasked) marks the row.
+    float peak = -INFINITY;
+    bool poisoned = false;
 #pragma unroll
     for (int k = 0; k < kVpl; ++k)
 #pragma unroll
       for (int j = 0; j < kVec; ++j) {
-        const bool keep = ((bits[k][j / 4] >> (8 * (j % 4))) & 0xFFu) != 0;
-        v[k][j] = keep ? v[k][j] * scale : -INFINITY;
+        poisoned = poisoned || poisons_row(v[k][j]);
+        peak = fmaxf(peak, v[k][j]);
       }
-  } else {
+    peak = row_max<kLanes>(poisoned ? INFINITY : peak, joint_max[i & 1]);
+    const bool invalid = __builtin_fabsf(peak) == INFINITY;
+
+    // ---- exponentials and their sum -----------------------------------------------------
+    float total = 0.0f;
 #pragma unroll
-    for (int k = 0; k < kVpl; ++k) Traits<T>::unpack(load16_stream(x, row_base + vec[k]), v[k]);
-    if constexpr (kMask == kMaskAdditive) {
-      float m[kVpl][kVec];
-      if (mrows.inner_stride == 0) {
-        const float one = Traits<T>::load(mask_row, 0);
+    for (int k = 0; k < kVpl; ++k)
 #pragma unroll
-        for (int k = 0; k < kVpl; ++k)
-#pragma unroll
-          for (int j = 0; j < kVec; ++j) m[k][j] = one;
-      } else {
-#pragma unroll
-        for (int k = 0; k < kVpl; ++k) Traits<T>::unpack(load16(mask_row, vec[k]), m[k]);
+      for (int j = 0; j < kVec; ++j) {
+        const float shifted = v[k][j] - peak;
+        if constexpr (kLog) {
+          total += exp_scaled(shifted);
+          v[k][j] = shifted;
+        } else {
+          v[k][j] = exp_scaled(shifted);
+          total += v[k][j];
+        }
       }
-#pragma unroll
-      for (int k = 0; k < kVpl; ++k)
-#pragma unroll
-        for (int j = 0; j < kVec; ++j) v[k][j] = ok[k] ? v[k][j] * scale + m[k][j] : -INFINITY;
-    } else {
-#pragma unroll
-      for (int k = 0; k < kVpl; ++k)
-#pragma unroll
-        for (int j = 0; j < kVec; ++j) v[k][j] = ok[k] ? v[k][j] * scale : -INFINITY;
-    }
-  }
+    total = row_sum<kLanes>(total, joint_sum[i & 1]);  // = 2^32 * sum(exp)
 
-  // ---- row maximum and validity -------------------------------------------------
-  // A NaN or +inf anywhere makes the row undefined.  fmaxf never lets a NaN through, so a lane
-  // that met one reports +inf instead: after the reduction an infinite maximum of either sign
-  // (+inf: poisoned, -inf: nothing finite and unmasked) marks the row.
-  float peak = -INFINITY;
-  bool poisoned = false;
+    // ---- normalise and store ------------------------------------------------------------
+    // softmax: e * 2^32 * (1 / (sum * 2^32)).  log-softmax: (v - max) - log(sum).
+    // An undefined row gets a NaN normaliser: it turns every lane, masked zeros included,
+    // into NaN without a per-element select.
+    float normaliser = kLog ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
+    if (invalid) normaliser = __builtin_nanf("");
 #pragma unroll
-  for (int k = 0; k < kVpl; ++k)
+    for (int k = 0; k < kVpl; ++k) {
+      if (row_ok && ok[k]) {
+        float r[kVec];
 #pragma unroll
-    for (int j = 0; j < kVec; ++j) {
-      poisoned = poisoned || poisons_row(v[k][j]);
-      peak = fmaxf(peak, v[k][j]);
-    }
-  peak = row_max<kLanes>(poisoned ? INFINITY : peak, joint_max);
-  const bool invalid = __builtin_fabsf(peak) == INFINITY;
-
-  // ---- exponentials and their sum -------------------------------------------------
-  float total = 0.0f;
-#pragma unroll
-  for (int k = 0; k < kVpl; ++k)
-#pragma unroll
-    for (int j = 0; j < kVec; ++j) {
-      const float shifted = v[k][j] - peak;
-      if constexpr (kLog) {
-        total += exp_scaled(shifted);
-        v[k][j] = shifted;
-      } else {
-        v[k][j] = exp_scaled(shifted);
-        total += v[k][j];
+        for (int j = 0; j < kVec; ++j) r[j] = kLog ? v[k][j] - normaliser : v[k][j] * normaliser;
+        store16_stream(y, (size_t)row * row_vectors + vec[k], Traits<T>::pack(r));
       }
     }
-  total = row_sum<kLanes>(total, joint_sum);  // = 2^32 * sum(exp)
-
-  // ---- normalise and store ------------------------------------------------------------
-  // softmax: e * 2^32 * (1 / (sum * 2^32)).  log-softmax: (v - max) - log(sum).
-  // An undefined row gets a NaN normaliser: it turns every lane, masked zeros included,
-  // into NaN without a per-element select.
-  float normaliser = kLog ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
-  if (invalid) normaliser = __builtin_nanf("");
+    if (i + 1 < kRepeat) {
 #pragma unroll
-  for (int k = 0; k < kVpl; ++k) {
-    if (ok[k]) {
-      float r[kVec];
-#pragma unroll
-      for (int j = 0; j < kVec; ++j) r[j] = kLog ? v[k][j] - normaliser : v[k][j] * normaliser;
-      store16_stream(y, (size_t)row * row_vectors + vec[k], Traits<T>::pack(r));
+      for (int k = 0; k < kVpl; ++k) current[k] = next[k];
     }
   }
 }
@@ -335,12 +374,35 @@ __global__ __launch_bounds__(kBlockThreads) void reduce_rows(const void *x, void
 }
 
 // ---- host dispatch ----------------------------------------------------------------------------
-template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog>
+// The leading axes a mask is broadcast over: x rows r and r + period share a mask row,
+// `repeats` times.  repeats = 1 when the mask has no such axes (or there is no mask).
+struct MaskRepeat {
+  uint32_t period, repeats;
+};
+MaskRepeat mask_repeat(const SoftmaxParams &p) {
+  MaskRepeat r{(uint32_t)p.shape.rows, 1};
+  if (p.mask_kind == 0) return r;
+  uint64_t repeats = 1;
+  for (int i = 0; i < p.outer_rank; ++i) {
+    if (p.mask_outer_strides[i] != 0 && p.outer_dims[i] != 1) break;
+    repeats *= p.outer_dims[i];
+  }
+  if (repeats > 1 && p.shape.rows % repeats == 0) {
+    r.repeats = (uint32_t)repeats;
+    r.period = (uint32_t)(p.shape.rows / repeats);
+  }
+  return r;
+}
+
+template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog, int kRepeat>
 hipError_t run_rows_as(const SoftmaxParams &p, const void *x, const void *mask, void *y,
                        hipStream_t s) {
-  constexpr int kRowsPerBlock = kThreads / kLanes;
+  constexpr int kGroupsPerBlock = kThreads / kLanes;
   const uint32_t rows = (uint32_t)p.shape.rows;
-  const uint32_t blocks = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+  const MaskRepeat repeat = mask_repeat(p);
+  const uint64_t groups =
+      kRepeat == 1 ? rows : (uint64_t)repeat.period * ((repeat.repeats + kRepeat - 1) / kRepeat);
+  const uint32_t blocks = (uint32_t)((groups + kGroupsPerBlock - 1) / kGroupsPerBlock);
   MaskRows m{};
   m.outer_rank = p.outer_rank;
   for (int i = 0; i < kMaxRank; ++i) {
@@ -348,25 +410,26 @@ hipError_t run_rows_as(const SoftmaxParams &p, const void *x, const void *mask, 
     m.outer_strides[i] = p.mask_outer_strides[i];
   }
   m.inner_stride = p.mask_inner_stride;
-  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads, kMask, kLog>), dim3(blocks),
-                     dim3(kThreads), 0, s, x, mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, m);
+  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads, kMask, kLog, kRepeat>), dim3(blocks),
+                     dim3(kThreads), 0, s, x, mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, m,
+                     repeat.period, repeat.repeats);
   return hipGetLastError();
 }
 
-template <class T, int kLanes, int kVpl, int kThreads = kBlockThreads>
+template <class T, int kLanes, int kVpl, int kThreads = kBlockThreads, int kRepeat = 1>
 hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, void *y,
                     hipStream_t s) {
   const bool log_form = p.log;
   switch ((int)p.mask_kind) {
     case kMaskBoolean:
-      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, true>(p, x, mask, y, s)
-                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, false>(p, x, mask, y, s);
+      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, true, kRepeat>(p, x, mask, y, s)
+                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, false, kRepeat>(p, x, mask, y, s);
     case kMaskAdditive:
-      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, true>(p, x, mask, y, s)
-                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, false>(p, x, mask, y, s);
+      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, true, kRepeat>(p, x, mask, y, s)
+                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, false, kRepeat>(p, x, mask, y, s);
     default:
-      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, true>(p, x, mask, y, s)
-                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, false>(p, x, mask, y, s);
+      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, true, 1>(p, x, mask, y, s)
+                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, false, 1>(p, x, mask, y, s);
   }
 }
 
@@ -381,13 +444,17 @@ hipError_t run_softmax(const SoftmaxParams &p, const void *x, const void *mask, 
   if (vectors <= 128) return run_rows<T, 64, 2>(p, x, mask, y, s);
   if (vectors <= 256) return run_rows<T, 128, 2>(p, x, mask, y, s);
   if (vectors <= 512) return run_rows<T, 256, 2>(p, x, mask, y, s);
-  // Measured on MI355X for S[32,4096,4096] f32 (1024 vectors per row), us per launch.  Every
-  // vector loaded (no mask, additive mask): eight waves x 2 vectors per lane, one row per block
-  // 685; two waves x 8 vectors 706-737; four waves x 4 vectors 731; a plain copy in the same
-  // shapes 688-737.  Boolean causal mask, masked vectors not loaded: four waves x 4 vectors,
-  // two rows per block 523; eight waves x 2 vectors 581; two waves x 8 vectors 569-591.
+  // Measured on MI355X for S[32,4096,4096] f32 (1024 vectors per row), us per launch, variants
+  // compared within one run.  Every vector loaded (no mask): eight waves x 2 vectors per lane,
+  // one row per block 685; two waves x 8 vectors 706-737; four waves x 4 vectors 731; a plain
+  // copy in the same shapes 688-737.  Boolean causal mask, masked vectors not loaded: four waves
+  // x 4 vectors, one row per block 531; two rows per block 557; two or four heads per lane
+  // group 551-716.  Additive causal mask: eight waves x 2 vectors, one head per lane group 804,
+  // two heads 709, four heads 732; four waves x 4 vectors with two or four heads 730-815.
   if (vectors <= 1024) {
-    if ((int)p.mask_kind == kMaskBoolean) return run_rows<T, 256, 4, 512>(p, x, mask, y, s);
+    if ((int)p.mask_kind == kMaskBoolean) return run_rows<T, 256, 4, 256>(p, x, mask, y, s);
+    if ((int)p.mask_kind == kMaskAdditive && mask_repeat(p).repeats >= 2)
+      return run_rows<T, 512, 2, 512, 2>(p, x, mask, y, s);
     return run_rows<T, 512, 2, 512>(p, x, mask, y, s);
   }
   if (vectors <= 2048) return run_rows<T, 512, 4, 512>(p, x, mask, y, s);
