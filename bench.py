@@ -191,8 +191,31 @@ def main() -> int:
         ops.append(Op("cfg5_q8_0_dequant_sumsq", hc.Q8_0DequantSumSquares(),
                       [hc.TensorDesc.gguf_q8_0_weight(BF, 2048, 6144)], set5, 16,
                       wl.ALGORITHMIC_BYTES["cfg5_q8_0_dequant_sumsq"], 6144 * 2048, "u8/bf16"))
-    if not ops:
-        print("no kernel selected", file=sys.stderr)
+    # ---- the next row of the path: Cast and Copy, timed beside the step -------------------------
+    if want("next_cast_f32_to_bf16") or want("next_cast_bf16_to_f32"):
+        x32 = np.random.default_rng(5).normal(0, 2, (8192, 2048)).astype(np.float32)
+
+        def set_narrow(i):
+            dx = torch.from_numpy(np.roll(x32, i, axis=0)).to(dev)
+            return [dx], [torch.empty((8192, 2048), dtype=torch.bfloat16, device=dev)]
+
+        def set_widen(i):
+            dx = torch.from_numpy(np.roll(x32, i, axis=0)).to(dev).to(torch.bfloat16)
+            return [dx], [torch.empty((8192, 2048), dtype=torch.float32, device=dev)]
+        if want("next_cast_f32_to_bf16"):
+            ops.append(Op("next_cast_f32_to_bf16", hc.Cast(BF), [D(F32, [8192, 2048])], set_narrow, 6,
+                          8192 * 2048 * 6, 8192 * 2048, "f32->bf16", in_step=False))
+        if want("next_cast_bf16_to_f32"):
+            ops.append(Op("next_cast_bf16_to_f32", hc.Cast(F32), [D(BF, [8192, 2048])], set_widen, 6,
+                          8192 * 2048 * 6, 8192 * 2048, "bf16->f32", in_step=False))
+    if want("next_copy_bf16"):
+        def set_copy(i):
+            src = torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev).normal_()
+            return [src], [torch.empty_like(src)]
+        ops.append(Op("next_copy_bf16", hc.Copy(), [D(BF, [8192, 6144])], set_copy, 3,
+                      8192 * 6144 * 4, 8192 * 6144, "bf16", in_step=False))
+    if not any(o.in_step for o in ops):
+        print("no kernel of the step selected", file=sys.stderr)
         return 2
 
     step_ops = [o for o in ops if o.in_step]

@@ -169,6 +169,8 @@ class TensorDesc:
 
 # ---- operations (include/hyle/compute/operation.h) -----------------------------------------
 class OperationKind(enum.IntEnum):
+    kCopy = 2
+    kCast = 4
     kUnary = 5
     kBinary = 6
     kReduce = 8
@@ -235,6 +237,16 @@ class MaskKind(enum.IntEnum):
 
 
 @dataclass(frozen=True)
+class Copy:
+    """Materialise any plain tensor (dense or strided) as a dense tensor of the same type."""
+
+
+@dataclass(frozen=True)
+class Cast:
+    output_type: DataType = DataType.kUnknown
+
+
+@dataclass(frozen=True)
 class Unary:
     kind: UnaryKind = UnaryKind.kAbs
 
@@ -298,7 +310,11 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
     c = capi.OpDescC()
     c.abi_version = capi.ABI_VERSION
     c.scale, c.largest = 1.0, 1
-    if isinstance(operation, Unary):
+    if isinstance(operation, Copy):
+        c.op = OperationKind.kCopy
+    elif isinstance(operation, Cast):
+        c.op, c.kind = OperationKind.kCast, int(operation.output_type)
+    elif isinstance(operation, Unary):
         c.op, c.kind = OperationKind.kUnary, int(operation.kind)
     elif isinstance(operation, Binary):
         c.op, c.kind = OperationKind.kBinary, int(operation.kind)

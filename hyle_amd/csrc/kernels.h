@@ -131,4 +131,19 @@ struct Q8Params {
 hipError_t launch_q8_0_dequant(const Q8Params &p, const void *blocks, void *out, float *sumsq,
                                bool vectorised, hipStream_t stream);
 
+// Cast between storage types, or Copy (copy_size = element bytes, types ignored): any plain
+// input (dims + byte strides, elements need not be aligned) to a dense output.
+enum class CastType : uint8_t { kF32 = 0, kF16, kBF16, kBool, kI32 };
+struct CastParams {
+  uint64_t elements = 0;
+  CastType src = CastType::kF32, dst = CastType::kF32;
+  uint8_t copy_size = 0;     // 0: convert; 1, 2, 4: move elements of that size unchanged
+  bool dense_input = false;  // the input is dense too: the flat kernels apply
+  int32_t rank = 0;
+  uint32_t dims[kMaxRank] = {};
+  int64_t strides[kMaxRank] = {};  // input byte strides
+};
+hipError_t launch_cast(const CastParams &p, const void *in, void *out, bool vectorised,
+                       hipStream_t stream);
+
 }  // namespace hyle_hip

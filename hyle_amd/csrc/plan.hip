@@ -230,6 +230,18 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
   hyle_hip_status s;
   *out_count = 1;
   switch (r.op) {
+    case HYLE_HIP_OP_COPY: {  // src/compute_ops/operation.cc:1254-1262
+      if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
+      if (!is_plain(in[0]))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Copy handles plain dense/strided storage");
+      return make_dense(in[0].dtype, in[0].dims, in[0].rank, &outs[0]);
+    }
+    case HYLE_HIP_OP_CAST: {  // src/compute_ops/operation.cc:1276-1285
+      if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
+      if (r.kind > 255 || dtype_size((uint8_t)r.kind) == 0 || !is_plain(in[0]))
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Cast requires a valid destination type and plain input");
+      return make_dense((uint8_t)r.kind, in[0].dims, in[0].rank, &outs[0]);
+    }
     case HYLE_HIP_OP_UNARY: {
       if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
       if (r.kind > 12) return fail(HYLE_HIP_INVALID_ARGUMENT, "Unary kind is invalid");
@@ -402,6 +414,7 @@ enum class Route : uint8_t {
   kReduceRows,
   kArgmax,
   kQ8Dequant,
+  kCast,
 };
 
 const char *route_name(Route r) {
@@ -415,6 +428,7 @@ const char *route_name(Route r) {
     case Route::kReduceRows: return "reduce-rows";
     case Route::kArgmax: return "argmax-tiles";
     case Route::kQ8Dequant: return "q8_0-dequant-rows";
+    case Route::kCast: return "cast-copy";
   }
   return "?";
 }
@@ -454,6 +468,10 @@ struct hyle_hip_plan {
   ReduceParams reduce;
   ArgmaxParams argmax;
   Q8Params q8;
+  CastParams cast;
+  // Cast and Copy take no alias at all (AliasPolicy::kNone, src/compute_ops/operation.cc:935-957):
+  // the bytes the input and the output occupy must not overlap.
+  uint64_t no_overlap_input_bytes = 0, no_overlap_output_bytes = 0;
 };
 
 namespace {
@@ -739,6 +757,53 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }
+    case HYLE_HIP_OP_COPY:
+    case HYLE_HIP_OP_CAST: {
+      // src/compute_provider_native/cast.cc:127-176,256-279 (admitted pairs, plain input, dense
+      // output) and transform.cc:171-179 (Copy of plain storage).
+      CastParams &c = p->cast;
+      auto cast_type = [](uint8_t dtype, CastType *t) {
+        switch (dtype) {
+          case HYLE_HIP_DTYPE_F32: *t = CastType::kF32; return true;
+          case HYLE_HIP_DTYPE_F16: *t = CastType::kF16; return true;
+          case HYLE_HIP_DTYPE_BF16: *t = CastType::kBF16; return true;
+          case HYLE_HIP_DTYPE_BOOL: *t = CastType::kBool; return true;
+          case HYLE_HIP_DTYPE_I32: *t = CastType::kI32; return true;
+          default: return false;
+        }
+      };
+      if (in[0].dtype == out.dtype) {
+        c.copy_size = (uint8_t)dtype_size(out.dtype);  // equal types keep the bytes
+      } else {
+        const bool pair_ok = cast_type(in[0].dtype, &c.src) && cast_type(out.dtype, &c.dst) &&
+                             ((is_floating(in[0].dtype) && is_floating(out.dtype)) ||
+                              (in[0].dtype == HYLE_HIP_DTYPE_I32 && out.dtype == HYLE_HIP_DTYPE_F32) ||
+                              (in[0].dtype == HYLE_HIP_DTYPE_BOOL && is_floating(out.dtype)) ||
+                              (is_floating(in[0].dtype) && out.dtype == HYLE_HIP_DTYPE_BOOL));
+        if (!pair_ok)
+          return fail(HYLE_HIP_UNIMPLEMENTED, "Cast storage conversion pair is not admitted");
+      }
+      const uint64_t n = p->output_elements[0];
+      if (n > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Cast / Copy output exceeds INT32_MAX elements");
+      if (n == 0) return HYLE_HIP_OK;
+      p->route = Route::kCast;
+      p->dispatches = 1;
+      c.elements = n;
+      c.dense_input = is_dense(in[0]);
+      c.rank = in[0].rank;
+      uint64_t last = 0;  // byte offset of the last element: TensorDesc::required_bytes
+      for (int a = 0; a < in[0].rank; ++a) {
+        c.dims[a] = (uint32_t)in[0].dims[a];
+        c.strides[a] = in[0].byte_strides[a];
+        last += (uint64_t)(in[0].dims[a] - 1) * (uint64_t)in[0].byte_strides[a];
+      }
+      // byte strides need not keep elements aligned (cast.cc:113-116): such inputs are read bytewise
+      if (!c.dense_input) p->input_alignment[0] = 1;
+      p->no_overlap_input_bytes = last + dtype_size(in[0].dtype);
+      p->no_overlap_output_bytes = n * dtype_size(out.dtype);
+      return HYLE_HIP_OK;
+    }
     default:
       return fail(HYLE_HIP_UNIMPLEMENTED, "operation kind %u is not served by this provider", r.op);
   }
@@ -922,6 +987,11 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
     if (!aligned(workspace, plan->workspace_alignment))
       return fail(HYLE_HIP_FAILED_PRECONDITION, "workspace does not satisfy its alignment");
   }
+  if (plan->no_overlap_output_bytes != 0) {
+    const uintptr_t in_first = reinterpret_cast<uintptr_t>(inputs[0]), out_first = reinterpret_cast<uintptr_t>(outputs[0]);
+    if (in_first < out_first + plan->no_overlap_output_bytes && out_first < in_first + plan->no_overlap_input_bytes)
+      return fail(HYLE_HIP_INVALID_ARGUMENT, "input and output storage overlap; Cast and Copy take no alias");
+  }
   hipStream_t stream = static_cast<hipStream_t>(stream_handle);
   hipError_t err = hipSuccess;
   switch (plan->route) {
@@ -968,6 +1038,9 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
     case Route::kQ8Dequant:
       err = launch_q8_0_dequant(plan->q8, inputs[0], outputs[0], static_cast<float *>(outputs[1]),
                                 aligned(inputs[0], 16) && aligned(outputs[0], 16), stream);
+      break;
+    case Route::kCast:
+      err = launch_cast(plan->cast, inputs[0], outputs[0], vector, stream);
       break;
   }
   if (err != hipSuccess) return hip_fail(err, "kernel launch");

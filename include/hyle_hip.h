@@ -63,6 +63,12 @@ typedef enum hyle_hip_dtype {
 } hyle_hip_dtype;
 
 typedef enum hyle_hip_op_kind {
+  /* Copy: any plain input (dense or strided) materialised as a dense tensor of the same type.
+   * Cast: the same with a change of storage type, `kind` = destination hyle_hip_dtype
+   * (f32/f16/bf16 among each other, int32 -> f32, Bool <-> float; equal types copy).
+   * Neither takes an alias: input and output bytes must not overlap. */
+  HYLE_HIP_OP_COPY = 2,
+  HYLE_HIP_OP_CAST = 4,
   HYLE_HIP_OP_UNARY = 5,
   HYLE_HIP_OP_BINARY = 6,
   HYLE_HIP_OP_REDUCE = 8,
@@ -130,7 +136,7 @@ typedef struct hyle_hip_tensor_desc {
 typedef struct hyle_hip_op_desc {
   uint32_t abi_version;      /* HYLE_HIP_ABI_VERSION */
   uint32_t op;               /* hyle_hip_op_kind */
-  uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind */
+  uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind; Cast: output hyle_hip_dtype */
   uint32_t kind2;            /* BINARY_CHAIN: second BinaryKind; GATED: GatedInputKind;
                                 SOFTMAX: SoftmaxKind */
   int32_t axis;              /* Softmax / TopK / Reduce axis (negative counts from the end) */

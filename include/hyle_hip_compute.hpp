@@ -218,6 +218,8 @@ enum class GatedInputKind : std::uint8_t { kPackedHalves = 0, kSeparate };
 enum class SoftmaxKind : std::uint8_t { kSoftmax = 0, kLogSoftmax };
 enum class MaskKind : std::uint8_t { kNone = 0, kAdditive, kBoolean };
 
+struct Copy final {};
+struct Cast final { DataType output_type = DataType::kUnknown; };
 struct Unary final { UnaryKind kind = UnaryKind::kAbs; };
 struct Binary final { BinaryKind kind = BinaryKind::kAdd; };
 struct Reduce final {
@@ -243,7 +245,7 @@ struct TopK final { std::size_t count = 1; std::int32_t axis = -1; bool largest 
 struct BinaryChain final { BinaryKind first = BinaryKind::kAdd; BinaryKind second = BinaryKind::kMultiply; };
 struct Q8_0DequantSumSquares final {};
 
-using Operation = std::variant<Unary, Binary, Reduce, RmsNorm, GatedActivation, Softmax, TopK, BinaryChain,
+using Operation = std::variant<Copy, Cast, Unary, Binary, Reduce, RmsNorm, GatedActivation, Softmax, TopK, BinaryChain,
                                Q8_0DequantSumSquares>;
 
 namespace detail {
@@ -254,6 +256,8 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
   r.largest = 1;
   struct Fill {
     hyle_hip_op_desc &r;
+    void operator()(const Copy &) const { r.op = HYLE_HIP_OP_COPY; }
+    void operator()(const Cast &o) const { r.op = HYLE_HIP_OP_CAST; r.kind = static_cast<std::uint32_t>(o.output_type); }
     void operator()(const Unary &o) const { r.op = HYLE_HIP_OP_UNARY; r.kind = static_cast<std::uint32_t>(o.kind); }
     void operator()(const Binary &o) const { r.op = HYLE_HIP_OP_BINARY; r.kind = static_cast<std::uint32_t>(o.kind); }
     void operator()(const Reduce &o) const {

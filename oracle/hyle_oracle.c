@@ -610,6 +610,101 @@ void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
 }
 
 /* ------------------------------------------------------------------------ */
+/* Cast / Copy                                                              */
+/* ------------------------------------------------------------------------ */
+
+/* src/compute_provider_native/cast.cc:19-41: nearest-even IEEE binary32 of an
+ * int32, formed from the integer so it does not depend on the ambient rounding
+ * mode. */
+static float int32_to_float32(int32_t value) {
+  const uint32_t raw = (uint32_t)value;
+  const uint32_t sign = raw & 0x80000000u;
+  const uint32_t magnitude = value < 0 ? 0u - raw : raw;
+  if (magnitude == 0) return 0.0f;
+  unsigned exponent = 31u - (unsigned)__builtin_clz(magnitude);
+  uint32_t significand;
+  if (exponent <= 23) {
+    significand = magnitude << (23 - exponent);
+  } else {
+    const unsigned shift = exponent - 23;
+    significand = magnitude >> shift;
+    const uint32_t remainder = magnitude & ((1u << shift) - 1);
+    const uint32_t halfway = 1u << (shift - 1);
+    if (remainder > halfway || (remainder == halfway && (significand & 1u)))
+      ++significand;
+    if (significand == (1u << 24)) {
+      significand >>= 1;
+      ++exponent;
+    }
+  }
+  const uint32_t bits = sign | ((exponent + 127) << 23) | (significand & 0x7FFFFFu);
+  float out;
+  memcpy(&out, &bits, 4);
+  return out;
+}
+
+static size_t cast_type_size(int type) {
+  switch (type) {
+    case HYLE_ORACLE_F32:
+    case HYLE_ORACLE_I32: return 4;
+    case HYLE_ORACLE_F16:
+    case HYLE_ORACLE_BF16: return 2;
+    case HYLE_ORACLE_BOOL: return 1;
+    default: return 0;
+  }
+}
+
+static int is_float_type(int type) {
+  return type == HYLE_ORACLE_F32 || type == HYLE_ORACLE_F16 || type == HYLE_ORACLE_BF16;
+}
+
+/* src/compute_provider_native/cast.cc:73-92 (convert_value) and 225-238 (the
+ * strided walk); same type: src/compute_provider_native/transform.cc:85-89
+ * (bytes are kept). */
+int hyle_oracle_cast(int src_type, int dst_type, const void *src,
+                     const int64_t *dims, const int64_t *strides, int rank,
+                     void *dst) {
+  const size_t sw = cast_type_size(src_type), dw = cast_type_size(dst_type);
+  if (sw == 0 || dw == 0) return -1;
+  const int same = src_type == dst_type;
+  if (!same) {
+    const int ok = (is_float_type(src_type) && is_float_type(dst_type)) ||
+                   (src_type == HYLE_ORACLE_I32 && dst_type == HYLE_ORACLE_F32) ||
+                   (src_type == HYLE_ORACLE_BOOL && is_float_type(dst_type)) ||
+                   (is_float_type(src_type) && dst_type == HYLE_ORACLE_BOOL);
+    if (!ok) return -1;
+  }
+  const size_t n = element_count(dims, rank);
+  const unsigned char *s = (const unsigned char *)src;
+  unsigned char *d = (unsigned char *)dst;
+  for (size_t i = 0; i < n; ++i) {
+    const unsigned char *from =
+        s + hyle_oracle_logical_byte_offset(dims, strides, rank, i);
+    unsigned char *to = d + i * dw;
+    if (same) {
+      memcpy(to, from, sw);
+    } else if (src_type == HYLE_ORACLE_I32) {
+      int32_t v;
+      memcpy(&v, from, 4);
+      const float f = int32_to_float32(v);
+      memcpy(to, &f, 4);
+    } else if (dst_type == HYLE_ORACLE_BOOL) {
+      /* truth of the stored bits: any nonzero magnitude, subnormals and NaNs
+       * included; both zeros are false */
+      uint32_t bits = 0;
+      memcpy(&bits, from, sw);
+      const uint32_t magnitude = sw == 4 ? 0x7FFFFFFFu : 0x7FFFu;
+      *to = (unsigned char)((bits & magnitude) != 0);
+    } else if (src_type == HYLE_ORACLE_BOOL) {
+      store_from_f32(dst_type, to, *from != 0 ? 1.0f : 0.0f);
+    } else {
+      store_from_f32(dst_type, to, load_as_f32(src_type, from));
+    }
+  }
+  return 0;
+}
+
+/* ------------------------------------------------------------------------ */
 /* CPU baseline legs (row ranges, dense loops)                              */
 /* ------------------------------------------------------------------------ */
 

@@ -43,6 +43,9 @@ enum {
   HYLE_ORACLE_F32 = 0,
   HYLE_ORACLE_F16 = 1,
   HYLE_ORACLE_BF16 = 2,
+  /* Cast only */
+  HYLE_ORACLE_BOOL = 3,
+  HYLE_ORACLE_I32 = 4,
 };
 
 /* include/hyle/compute/operation.h:75-82 */
@@ -197,6 +200,18 @@ void hyle_oracle_q8_0_dequant_bf16(const void *blocks, size_t rows, size_t k,
 /* ggml dequantize_row_q8_0 to f32 */
 void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
                                   size_t row_stride_bytes, float *out);
+
+/* ---- Cast / Copy ------------------------------------------------------- */
+/* Cast of a plain tensor (dims + byte strides, elements need not be aligned) to
+ * a dense tensor of dst_type (src/compute_provider_native/cast.cc:73-92,225-238):
+ * float <-> float decodes to f32 and encodes once (RN-even codecs above);
+ * int32 -> f32 rounds to nearest even; float -> Bool is the truth of the stored
+ * magnitude bits; Bool -> float is 1 or 0; equal types keep the bytes (Copy,
+ * src/compute_provider_native/transform.cc:85-89).  Returns 0, or -1 for a pair
+ * the reference does not define (f32 -> int32, ...). */
+int hyle_oracle_cast(int src_type, int dst_type, const void *src,
+                     const int64_t *dims, const int64_t *strides, int rank,
+                     void *dst);
 
 /* ---- CPU baseline legs ---------------------------------------------------
  * The same arithmetic as above in the loop shapes the reference's CPU provider

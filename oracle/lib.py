@@ -14,11 +14,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libhyle_oracle.so")
 
 F32, F16, BF16 = 0, 1, 2
+BOOL, I32 = 3, 4  # Cast only
 ADD, SUBTRACT, MULTIPLY, DIVIDE, MINIMUM, MAXIMUM = range(6)
 SUM, MEAN, MIN, MAX = range(4)
 MASK_NONE, MASK_ADDITIVE, MASK_BOOLEAN = range(3)
 
-_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16}
+_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16, BOOL: np.uint8, I32: np.int32}
 
 
 def build() -> None:
@@ -76,6 +77,7 @@ _iom = _sig("hyle_oracle_index_of_max_f32", _sz, _vp, _sz)
 _topk1 = _sig("hyle_oracle_topk1_f32", None, _vp, _sz, _sz, _vp, _vp)
 _q8_bf16 = _sig("hyle_oracle_q8_0_dequant_bf16", None, _vp, _sz, _sz, _sz, _vp, _vp, _vp)
 _q8_f32 = _sig("hyle_oracle_q8_0_dequant_f32", None, _vp, _sz, _sz, _sz, _vp)
+_cast = _sig("hyle_oracle_cast", C.c_int, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int, _vp)
 
 
 def _ptr(a: np.ndarray | None):
@@ -317,4 +319,22 @@ def q8_0_dequant_f32(blocks: np.ndarray, rows: int, k: int, row_stride: int | No
     row_stride = (k // 32) * 34 if row_stride is None else row_stride
     out = np.empty((rows, k), np.float32)
     _q8_f32(_ptr(blocks), rows, k, row_stride, _ptr(out))
+    return out
+
+
+# ---- Cast / Copy ------------------------------------------------------------
+def cast(src_type: int, dst_type: int, storage: np.ndarray, dims, byte_strides=None) -> np.ndarray:
+    """Cast a plain tensor held in `storage` (any dtype, read as bytes) with logical `dims` and
+    `byte_strides` (dense when omitted) to a dense array of dst_type's storage dtype."""
+    dims = [int(d) for d in dims]
+    if byte_strides is None:
+        step, byte_strides = np.dtype(_NP[src_type]).itemsize, []
+        for d in reversed(dims):
+            byte_strides.append(step)
+            step *= d
+        byte_strides = list(reversed(byte_strides))
+    raw = np.ascontiguousarray(storage).view(np.uint8).reshape(-1)
+    out = np.empty(dims, _NP[dst_type])
+    if _cast(src_type, dst_type, _ptr(raw), _i64(dims), _i64(byte_strides), len(dims), _ptr(out)) != 0:
+        raise ValueError("the reference does not define this Cast pair")
     return out

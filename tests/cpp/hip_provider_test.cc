@@ -113,6 +113,24 @@ HOST_TEST(PreparesRoutesAndDeclinesCleanly) {
   EXPECT(none->dispatch_count() == 0);
 }
 
+HOST_TEST(CastAndCopyInferDenseOutputsAndDeclineUndefinedPairs) {
+  const Context context = Context::planning_only();
+  const TensorDesc strided = *TensorDesc::strided_bytes(DataType::kFloat16, {2, 2}, {5, 2});
+  auto out = infer_output_descriptions(Cast{DataType::kFloat32}, {strided});
+  REQUIRE(out.has_value());
+  EXPECT((*out)[0] == dense(DataType::kFloat32, {2, 2}));
+  out = infer_output_descriptions(Copy{}, {strided});
+  REQUIRE(out.has_value());
+  EXPECT((*out)[0] == dense(DataType::kFloat16, {2, 2}));
+  EXPECT(infer_output_descriptions(Cast{}, {dense(DataType::kFloat32, {4})}).error().IsInvalidArgument());
+  auto narrow = prepare(context, Cast{DataType::kBFloat16}, dense(DataType::kFloat32, {8192, 2048}));
+  REQUIRE(narrow.has_value());
+  EXPECT(narrow->dispatch_count() == 1 && !narrow->alias_support(0, 0)->supported);
+  // tests/compute_provider_native/cast_test.cc:296-301: the reverse integer pair is not defined
+  EXPECT(prepare(context, Cast{DataType::kInt32}, dense(DataType::kFloat32, {2, 8})).error().IsUnimplemented());
+  EXPECT(prepare(context, Cast{DataType::kFloat32}, dense(DataType::kInt32, {2, 8})).has_value());
+}
+
 HOST_TEST(SubmitWithoutDeviceIsFailedPrecondition) {
   Context context = Context::planning_only();
   EXPECT(context.create_queue().error().IsFailedPrecondition());
@@ -330,6 +348,53 @@ DEVICE_TEST(Q8_0DequantBitExactWithRowSumSquares) {
   bool close = true;
   for (std::int64_t r = 0; r < n; ++r) close = close && std::fabs(got_sumsq[r] - want_sumsq[r]) <= 1.0e-5F * want_sumsq[r];
   EXPECT(close);  // summation order differs from the index-order oracle: 1e-5 relative
+}
+
+DEVICE_TEST(CastNarrowsWidensAndMaterialisesStridedInputBitExactly) {
+  constexpr std::int64_t rows = 257, cols = 2048;
+  auto values = normal(rows * cols, 12, 2.0F);
+  values[0] = kNaN; values[1] = kInf; values[2] = -0.0F; values[3] = 1.0e-40F; values[4] = 3.4e38F;
+  const TensorDesc wide = dense(DataType::kFloat32, {rows, cols}), narrow = dense(DataType::kBFloat16, {rows, cols});
+  auto prepared = prepare(fixture().context, Cast{DataType::kBFloat16}, wide);
+  REQUIRE(prepared.has_value());
+  DeviceBuffer source = upload(values), target = DeviceBuffer::create(values.size() * 2).value();
+  auto completion = prepared->create_invocation()->submit(fixture().queue, *ConstTensorView::create(wide, source),
+                                                          *TensorView::create(narrow, target));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<std::uint16_t> want(values.size());
+  const std::int64_t dims[2] = {rows, cols}, wide_strides[2] = {cols * 4, 4}, narrow_strides[2] = {cols * 2, 2};
+  EXPECT(hyle_oracle_cast(HYLE_ORACLE_F32, HYLE_ORACLE_BF16, values.data(), dims, wide_strides, 2, want.data()) == 0);
+  const auto got = download<std::uint16_t>(target, values.size());
+  EXPECT(same_bits(got.data(), want.data(), want.size() * 2));
+  // and back: bf16 -> f32 is exact
+  auto widen = prepare(fixture().context, Cast{DataType::kFloat32}, narrow);
+  REQUIRE(widen.has_value());
+  DeviceBuffer back = DeviceBuffer::create(values.size() * 4).value();
+  completion = widen->create_invocation()->submit(fixture().queue, *ConstTensorView::create(narrow, target),
+                                                  *TensorView::create(wide, back));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<float> widened(values.size());
+  EXPECT(hyle_oracle_cast(HYLE_ORACLE_BF16, HYLE_ORACLE_F32, want.data(), dims, narrow_strides, 2, widened.data()) == 0);
+  EXPECT(same_bits(download<float>(back, values.size()).data(), widened.data(), widened.size() * 4));
+  // tests/compute_provider_native/cast_test.cc:177-183: f16 [2,2] with byte strides {5,2}
+  std::vector<std::uint8_t> physical(16, 0);
+  const std::uint16_t halves[4] = {0x3C00, 0x4000, 0x4200, 0x4400};
+  const std::size_t offsets[4] = {0, 2, 5, 7};
+  for (int i = 0; i < 4; ++i) std::memcpy(&physical[offsets[i]], &halves[i], 2);
+  const TensorDesc strided = *TensorDesc::strided_bytes(DataType::kFloat16, {2, 2}, {5, 2});
+  auto gather = prepare(fixture().context, Cast{DataType::kFloat32}, strided);
+  REQUIRE(gather.has_value());
+  DeviceBuffer raw = upload(physical), four = DeviceBuffer::create(16).value();
+  completion = gather->create_invocation()->submit(fixture().queue, *ConstTensorView::create(strided, raw),
+                                                   *TensorView::create(dense(DataType::kFloat32, {2, 2}), four));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  EXPECT((download<float>(four, 4) == std::vector<float>{1.0F, 2.0F, 3.0F, 4.0F}));
+  // Cast takes no alias: output over the input is refused
+  EXPECT(prepared->create_invocation()->submit(fixture().queue, *ConstTensorView::create(wide, source),
+                                               *TensorView::create(narrow, source)).error().IsInvalidArgument());
 }
 
 DEVICE_TEST(RejectedSubmissionsEnqueueNothing) {

@@ -245,3 +245,30 @@ def test_zero_elements_are_a_no_op_and_launch_needs_a_device():
     with pytest.raises(hc.StatusError) as err:  # binding count is checked first
         real.create_invocation().submit(0, [16], [32])
     assert err.value.is_invalid_argument()
+
+
+def test_cast_and_copy_inference_and_admission():
+    # src/compute_ops/operation.cc:1254-1285: dense output of the input's shape, Cast in the new type
+    strided = hc.TensorDesc.strided_bytes(DT.kFloat16, [2, 2], [5, 2])
+    assert hc.infer_output_descriptions(hc.Cast(DT.kFloat32), [strided]) == [D(DT.kFloat32, [2, 2])]
+    assert hc.infer_output_descriptions(hc.Copy(), [strided]) == [D(DT.kFloat16, [2, 2])]
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Cast(DT.kUnknown), [D(DT.kFloat32, [4])])
+    assert err.value.is_invalid_argument()
+    with pytest.raises(hc.StatusError) as err:  # blocked storage is Repack's business
+        hc.infer_output_descriptions(hc.Copy(), [hc.TensorDesc.gguf_q8_0_weight(DT.kBFloat16, 64, 2)])
+    assert err.value.is_unimplemented()
+    # admitted pairs (src/compute_provider_native/cast.cc:127-176 plus the float pairs of the
+    # mature providers); one dispatch, no workspace, no alias
+    for src, dst in ((DT.kFloat32, DT.kBFloat16), (DT.kBFloat16, DT.kFloat32), (DT.kFloat16, DT.kBFloat16),
+                     (DT.kInt32, DT.kFloat32), (DT.kBool, DT.kFloat16), (DT.kFloat32, DT.kBool)):
+        prepared = hc.prepare(CTX, hc.Cast(dst), D(src, [8, 16]))
+        assert prepared.route_name() == "cast-copy" and prepared.dispatch_count() == 1
+        assert prepared.workspace_requirement().size == 0 and not prepared.alias_support(0, 0)
+    assert hc.prepare(CTX, hc.Cast(DT.kFloat32), D(DT.kFloat32, [8])).route_name() == "cast-copy"  # = Copy
+    assert hc.prepare(CTX, hc.Copy(), D(DT.kInt8, [3, 5])).dispatch_count() == 1
+    for src, dst in ((DT.kFloat32, DT.kInt32), (DT.kInt32, DT.kBFloat16), (DT.kInt8, DT.kFloat32), (DT.kBool, DT.kInt32)):
+        with pytest.raises(hc.StatusError) as err:
+            hc.prepare(CTX, hc.Cast(dst), D(src, [8]))
+        assert err.value.is_unimplemented()
+    assert hc.prepare(CTX, hc.Copy(), D(DT.kFloat32, [0, 9])).dispatch_count() == 0

@@ -514,3 +514,69 @@ def test_q8_0_every_scale_times_every_quant():
         assert np.array_equal(out[ok], bf16_rne_independent(y32.view(np.uint32))[ok])
         nan = np.isnan(y32)
         assert np.all((out[nan] & 0x7FFF) > 0x7F80)
+
+
+# ---- Cast / Copy ------------------------------------------------------------------------------
+def test_cast_known_answers_from_reference_tests():
+    # tests/compute_provider_native/cast_test.cc:139-143 (f32 -> f16 bit patterns)
+    got = orc.cast(orc.F32, orc.F16, np.array([0.0, 1.0, -2.0, 0.5, 65504.0], np.float32), [5])
+    assert got.tolist() == [0x0000, 0x3C00, 0xC000, 0x3800, 0x7BFF]
+    # :177-183 (f16 [2,2] with byte strides {5,2} -> f32)
+    physical = np.zeros(9, np.uint8)
+    for bits, offset in zip((0x3C00, 0x4000, 0x4200, 0x4400), (0, 2, 5, 7)):
+        physical[offset:offset + 2] = np.frombuffer(np.uint16(bits).tobytes(), np.uint8)
+    got = orc.cast(orc.F16, orc.F32, physical, [2, 2], [5, 2])
+    assert got.tolist() == [[1.0, 2.0], [3.0, 4.0]]
+    # :232-247 (int32 -> f32 on both sides of the 2^24 ties and the 2^31 carry), dense and with
+    # the odd byte strides {51, 5} of the reference test
+    values = np.array([0, 1, -1, 129279, 16777215, 16777216, 16777217, 16777219, -16777217, -16777219,
+                       2147483520, 2147483583, 2147483584, 2**31 - 1, -2**31, -2**31 + 1], np.int64).astype(np.int32)
+    expected = [0x00000000, 0x3F800000, 0xBF800000, 0x47FC7F80, 0x4B7FFFFF, 0x4B800000, 0x4B800000, 0x4B800002,
+                0xCB800000, 0xCB800002, 0x4EFFFFFF, 0x4EFFFFFF, 0x4F000000, 0x4F000000, 0xCF000000, 0xCF000000]
+    assert orc.cast(orc.I32, orc.F32, values, [2, 8]).view(np.uint32).reshape(-1).tolist() == expected
+    physical = np.full(51 + 7 * 5 + 4, 0x5A, np.uint8)
+    for i, v in enumerate(values):
+        offset = (i // 8) * 51 + (i % 8) * 5
+        physical[offset:offset + 4] = np.frombuffer(np.int32(v).tobytes(), np.uint8)
+    assert orc.cast(orc.I32, orc.F32, physical, [2, 8], [51, 5]).view(np.uint32).reshape(-1).tolist() == expected
+    # :389-396 (truth keeps signed zeros false, subnormals / inf / NaN true; Bool -> float is 1 or 0)
+    for type_id, words, one, dtype in (
+            (orc.F32, [0, 0x80000000, 1, 0x80000001, 0x3F800000, 0xBF800000, 0x7F800000, 0x7FC00001], 0x3F800000, np.uint32),
+            (orc.F16, [0, 0x8000, 1, 0x8001, 0x3C00, 0xBC00, 0x7C00, 0x7E01], 0x3C00, np.uint16),
+            (orc.BF16, [0, 0x8000, 1, 0x8001, 0x3F80, 0xBF80, 0x7F80, 0x7FC1], 0x3F80, np.uint16)):
+        assert orc.cast(type_id, orc.BOOL, np.array(words, dtype), [2, 4]).reshape(-1).tolist() == [0, 0, 1, 1, 1, 1, 1, 1]
+        boolean = np.array([0, 1, 2, 255, 1, 0, 0, 1], np.uint8)
+        got = orc.cast(orc.BOOL, type_id, boolean, [2, 4]).view(dtype).reshape(-1).tolist()
+        assert got == [one if b else 0 for b in boolean]
+    # :296-301: the reverse pair is not defined
+    with pytest.raises(ValueError):
+        orc.cast(orc.F32, orc.I32, np.zeros(4, np.float32), [4])
+
+
+def test_cast_matches_independent_conversions():
+    rng = np.random.default_rng(31)
+    # int32 -> f32: numpy converts with round-to-nearest-even
+    ints = np.concatenate([rng.integers(-2**31, 2**31, 200000, dtype=np.int64),
+                           (1 << np.arange(31, dtype=np.int64)), (1 << np.arange(31, dtype=np.int64)) + 1,
+                           -(1 << np.arange(32, dtype=np.int64)), (1 << np.arange(1, 32, dtype=np.int64)) - 1]).astype(np.int32)
+    assert np.array_equal(orc.cast(orc.I32, orc.F32, ints, [ints.size]).view(np.uint32),
+                          ints.astype(np.float32).view(np.uint32))
+    # float -> float: decode to f32 and encode once, i.e. the pinned codecs; f16 -> f32 -> bf16 etc.
+    words = rng.integers(0, 1 << 32, 300000, dtype=np.uint64).astype(np.uint32)
+    finite = f32(words)
+    via_f16 = orc.cast(orc.F32, orc.F16, finite, [finite.size])
+    assert np.array_equal(via_f16, orc.from_f32(orc.F16, finite))
+    same_bits_or_nan32(orc.cast(orc.F16, orc.F32, via_f16, [via_f16.size]), via_f16.view(np.float16).astype(np.float32))
+    via_bf16 = orc.cast(orc.F32, orc.BF16, finite, [finite.size])
+    numbers = ~np.isnan(finite)
+    assert np.array_equal(via_bf16[numbers], bf16_rne_independent(words[numbers]))
+    assert np.array_equal(orc.cast(orc.BF16, orc.F32, via_bf16, [via_bf16.size]).view(np.uint32), via_bf16.astype(np.uint32) << 16)
+    halves = np.arange(1 << 16, dtype=np.uint32).astype(np.uint16)
+    assert np.array_equal(orc.cast(orc.F16, orc.BF16, halves, [halves.size]),
+                          orc.from_f32(orc.BF16, orc.to_f32(orc.F16, halves)))
+    assert np.array_equal(orc.cast(orc.BF16, orc.F16, halves, [halves.size]),
+                          orc.from_f32(orc.F16, orc.to_f32(orc.BF16, halves)))
+    # equal types keep the bytes (Copy), NaN payloads included, through any strides
+    grid = rng.integers(0, 1 << 16, (6, 10), dtype=np.uint32).astype(np.uint16)
+    assert np.array_equal(orc.cast(orc.BF16, orc.BF16, grid, [6, 5], [20, 4]), grid[:, ::2])
+    assert np.array_equal(orc.cast(orc.F32, orc.F32, words, [1000]).view(np.uint32), words[:1000])
