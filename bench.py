@@ -208,6 +208,16 @@ def main() -> int:
         if want("next_cast_bf16_to_f32"):
             ops.append(Op("next_cast_bf16_to_f32", hc.Cast(F32), [D(BF, [8192, 2048])], set_widen, 6,
                           8192 * 2048 * 6, 8192 * 2048, "bf16->f32", in_step=False))
+    if want("next_layer_norm_bf16"):
+        xl, wl_ = wl.config2()
+        bias_bits = wl.config2(rows=1)[0].reshape(-1)  # any bf16 vector of the right length
+
+        def set_ln(i):
+            dx = bf16(np.roll(xl, i, axis=0))
+            return [dx, bf16(wl_), bf16(bias_bits)], [torch.empty_like(dx)]
+        ops.append(Op("next_layer_norm_bf16", hc.LayerNorm(epsilon=1e-6),
+                      [D(BF, [8192, 2048]), D(BF, [2048]), D(BF, [2048])], set_ln, 10,
+                      2 * 8192 * 2048 * 2 + 2 * 4096, 8192 * 2048, "bf16", in_step=False))
     if want("next_copy_bf16"):
         def set_copy(i):
             src = torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev).normal_()

@@ -175,6 +175,7 @@ class OperationKind(enum.IntEnum):
     kBinary = 6
     kReduce = 8
     kRmsNorm = 9
+    kLayerNorm = 10
     kGatedActivation = 12
     kSoftmax = 18
     kTopK = 19
@@ -278,6 +279,12 @@ class RmsNorm:
 
 
 @dataclass(frozen=True)
+class LayerNorm:
+    epsilon: float = 1.0e-5
+    accumulation_type: DataType = DataType.kFloat32
+
+
+@dataclass(frozen=True)
 class GatedActivation:
     activation: GatedActivationKind = GatedActivationKind.kSilu
     inputs: GatedInputKind = GatedInputKind.kPackedHalves
@@ -325,6 +332,8 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
         c.keep_dimensions, c.accumulation = int(operation.keep_dimensions), int(operation.accumulation_type)
     elif isinstance(operation, RmsNorm):
         c.op, c.epsilon, c.accumulation = OperationKind.kRmsNorm, operation.epsilon, int(operation.accumulation_type)
+    elif isinstance(operation, LayerNorm):
+        c.op, c.epsilon, c.accumulation = OperationKind.kLayerNorm, operation.epsilon, int(operation.accumulation_type)
     elif isinstance(operation, GatedActivation):
         c.op, c.kind, c.kind2 = OperationKind.kGatedActivation, int(operation.activation), int(operation.inputs)
     elif isinstance(operation, Softmax):

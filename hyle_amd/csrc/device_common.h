@@ -239,7 +239,6 @@ template <int kLanes> __device__ __forceinline__ float row_sum(float v, float *j
 template <int kLanes> __device__ __forceinline__ float row_max(float v, float *joint) {
   return row_reduce<kLanes>(v, joint, [](float a, float b) { return a > b ? a : b; });
 }
-
 // NaN-propagating extrema of the reference's Reduce
 // (src/compute_provider_native/reduction.cc:34-47): the first NaN met sticks;
 // +0 ranks above -0 (tests/simd/search_test.cc:203-206).

@@ -65,10 +65,12 @@ struct NormParams {
   RowShape shape;
   float epsilon = 0;
   bool has_weight = false;
-  bool weight_f32 = false;  // f32 weight with a narrow input
+  bool weight_f32 = false;  // f32 parameters with a narrow input
+  bool layer = false;       // LayerNorm: subtract the row mean first
+  bool has_bias = false;    // LayerNorm only, together with a weight
 };
-hipError_t launch_rms_norm(Elem type, const NormParams &p, const void *x, const void *w, void *y,
-                           bool vectorised, hipStream_t stream);
+hipError_t launch_norm(Elem type, const NormParams &p, const void *x, const void *w, const void *b,
+                       void *y, bool vectorised, hipStream_t stream);
 
 // Softmax over the last axis of a dense [rows, width] tensor.  The mask row of
 // logical row r starts at mask + sum_k coord_k(r) * outer_stride[k]; inside the

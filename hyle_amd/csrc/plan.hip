@@ -313,6 +313,24 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
       }
       return make_dense(in[0].dtype, in[0].dims, in[0].rank, &outs[0]);
     }
+    case HYLE_HIP_OP_LAYER_NORM: {  // src/compute_ops/operation.cc:506-536,1410-1424
+      if ((s = expect_inputs(r, 1, 3)) != HYLE_HIP_OK) return s;
+      if (!std::isfinite(r.epsilon) || r.epsilon < 0.0f)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "LayerNorm epsilon must be finite and non-negative");
+      if ((s = validate_accumulation(r.accumulation)) != HYLE_HIP_OK) return s;
+      if (!is_floating(in[0].dtype) || in[0].rank == 0)
+        return fail(HYLE_HIP_INVALID_ARGUMENT,
+                    "normalization requires a floating tensor with rank >= 1");
+      for (uint32_t i = 1; i < r.input_count; ++i) {
+        const bool promoted = in[0].dtype != HYLE_HIP_DTYPE_F32 && in[i].dtype == HYLE_HIP_DTYPE_F32;
+        if ((!promoted && in[i].dtype != in[0].dtype) || in[i].rank != 1 ||
+            in[i].dims[0] != in[0].dims[in[0].rank - 1])
+          return fail(HYLE_HIP_INVALID_ARGUMENT,
+                      i == 1 ? "normalization scale must match the last input dimension"
+                             : "LayerNorm bias must match the last input dimension");
+      }
+      return make_dense(in[0].dtype, in[0].dims, in[0].rank, &outs[0]);
+    }
     case HYLE_HIP_OP_GATED_ACTIVATION: {
       if (r.kind > 2 || r.kind2 > HYLE_HIP_GATED_SEPARATE)
         return fail(HYLE_HIP_INVALID_ARGUMENT, "GatedActivation mode is invalid");
@@ -423,7 +441,7 @@ const char *route_name(Route r) {
     case Route::kEwFlat: return "elementwise-flat";
     case Route::kEwGeneral: return "elementwise-strided";
     case Route::kSwigluPacked: return "swiglu-packed";
-    case Route::kRmsNorm: return "rms-norm-rows";
+    case Route::kRmsNorm: return "norm-rows";
     case Route::kSoftmax: return "softmax-rows";
     case Route::kReduceRows: return "reduce-rows";
     case Route::kArgmax: return "argmax-tiles";
@@ -605,15 +623,17 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }
+    case HYLE_HIP_OP_LAYER_NORM:
     case HYLE_HIP_OP_RMS_NORM: {
       if (r.accumulation != HYLE_HIP_DTYPE_F32)
         return fail(HYLE_HIP_UNIMPLEMENTED, "normalization supports float32 accumulation");
       if (!to_elem(in[0].dtype, &p->elem) || !is_dense(in[0]))
         return fail(HYLE_HIP_UNIMPLEMENTED,
                     "normalization requires dense plain float32/float16/bfloat16");
-      if (r.input_count == 2 && !is_dense(in[1]))
-        return fail(HYLE_HIP_UNIMPLEMENTED,
-                    "normalization requires dense plain float32/float16/bfloat16");
+      for (uint32_t i = 1; i < r.input_count; ++i)
+        if (!is_dense(in[i]) || in[i].dtype != in[1].dtype)
+          return fail(HYLE_HIP_UNIMPLEMENTED,
+                      "normalization requires dense plain parameters of one type");
       if (p->output_elements[0] > kMaxElements)
         return fail(HYLE_HIP_UNIMPLEMENTED, "normalization requires at most INT32_MAX elements");
       p->alias_inputs[0] = 1;  // reductions finish before the first write
@@ -622,8 +642,10 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->norm.shape.width = (uint32_t)in[0].dims[in[0].rank - 1];
       p->norm.shape.rows = p->output_elements[0] / p->norm.shape.width;
       p->norm.epsilon = r.epsilon;
-      p->norm.has_weight = r.input_count == 2;
-      p->norm.weight_f32 = r.input_count == 2 && in[1].dtype == HYLE_HIP_DTYPE_F32 &&
+      p->norm.layer = r.op == HYLE_HIP_OP_LAYER_NORM;
+      p->norm.has_weight = r.input_count >= 2;
+      p->norm.has_bias = r.input_count == 3;
+      p->norm.weight_f32 = r.input_count >= 2 && in[1].dtype == HYLE_HIP_DTYPE_F32 &&
                            in[0].dtype != HYLE_HIP_DTYPE_F32;
       p->dispatches = 1;
       return HYLE_HIP_OK;
@@ -1009,8 +1031,8 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
       err = launch_swiglu_packed(plan->elem, plan->packed, inputs[0], outputs[0], vector, stream);
       break;
     case Route::kRmsNorm:
-      err = launch_rms_norm(plan->elem, plan->norm, inputs[0], input_count > 1 ? inputs[1] : nullptr,
-                            outputs[0], vector, stream);
+      err = launch_norm(plan->elem, plan->norm, inputs[0], input_count > 1 ? inputs[1] : nullptr,
+                        input_count > 2 ? inputs[2] : nullptr, outputs[0], vector, stream);
       break;
     case Route::kSoftmax: {
       const void *mask = input_count > 1 ? inputs[1] : nullptr;

@@ -73,6 +73,8 @@ typedef enum hyle_hip_op_kind {
   HYLE_HIP_OP_BINARY = 6,
   HYLE_HIP_OP_REDUCE = 8,
   HYLE_HIP_OP_RMS_NORM = 9,
+  /* in0 [.., n], optional scale [n], optional bias [n] (bias only with a scale) */
+  HYLE_HIP_OP_LAYER_NORM = 10,
   HYLE_HIP_OP_GATED_ACTIVATION = 12,
   HYLE_HIP_OP_SOFTMAX = 18,
   HYLE_HIP_OP_TOP_K = 19,
@@ -143,7 +145,7 @@ typedef struct hyle_hip_op_desc {
   uint32_t mask;             /* Softmax MaskKind */
   uint32_t accumulation;     /* hyle_hip_dtype; UNKNOWN or F32 */
   uint32_t keep_dimensions;  /* Reduce */
-  float epsilon;             /* RmsNorm */
+  float epsilon;             /* RmsNorm, LayerNorm */
   float scale;               /* Softmax */
   uint64_t count;            /* TopK count (only 1 is implemented) */
   uint32_t largest;          /* TopK */

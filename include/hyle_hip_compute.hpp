@@ -229,6 +229,7 @@ struct Reduce final {
   DataType accumulation_type = DataType::kUnknown;
 };
 struct RmsNorm final { float epsilon = 1.0e-5F; DataType accumulation_type = DataType::kFloat32; };
+struct LayerNorm final { float epsilon = 1.0e-5F; DataType accumulation_type = DataType::kFloat32; };
 struct GatedActivation final {
   GatedActivationKind activation = GatedActivationKind::kSilu;
   GatedInputKind inputs = GatedInputKind::kPackedHalves;
@@ -245,7 +246,7 @@ struct TopK final { std::size_t count = 1; std::int32_t axis = -1; bool largest 
 struct BinaryChain final { BinaryKind first = BinaryKind::kAdd; BinaryKind second = BinaryKind::kMultiply; };
 struct Q8_0DequantSumSquares final {};
 
-using Operation = std::variant<Copy, Cast, Unary, Binary, Reduce, RmsNorm, GatedActivation, Softmax, TopK, BinaryChain,
+using Operation = std::variant<Copy, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
                                Q8_0DequantSumSquares>;
 
 namespace detail {
@@ -266,6 +267,9 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
     }
     void operator()(const RmsNorm &o) const {
       r.op = HYLE_HIP_OP_RMS_NORM; r.epsilon = o.epsilon; r.accumulation = static_cast<std::uint32_t>(o.accumulation_type);
+    }
+    void operator()(const LayerNorm &o) const {
+      r.op = HYLE_HIP_OP_LAYER_NORM; r.epsilon = o.epsilon; r.accumulation = static_cast<std::uint32_t>(o.accumulation_type);
     }
     void operator()(const GatedActivation &o) const {
       r.op = HYLE_HIP_OP_GATED_ACTIVATION; r.kind = static_cast<std::uint32_t>(o.activation);

@@ -352,6 +352,55 @@ void hyle_oracle_rms_norm(int type, int weight_type, const void *src,
                              d + r * hidden * w, hidden, epsilon);
 }
 
+/* src/simd/math/activations.cc:148-175: mean from a plain running sum, centred
+ * squares through an fma chain, inverse = 1 / sqrt(ss / n + eps); without
+ * parameters (x - mean) * inverse, with them fma(normalised, scale, bias).
+ * The scalar floor has no scale-only form; the provider level defines it as
+ * normalised * scale (tests/compute_provider_native/normalization_test.cc:69-127). */
+void hyle_oracle_layer_norm_row(int type, int param_type, const void *src,
+                                const void *scale, const void *bias, void *dst,
+                                size_t n, float epsilon) {
+  if (n == 0) return;
+  const unsigned char *s = (const unsigned char *)src;
+  const unsigned char *sp = (const unsigned char *)scale;
+  const unsigned char *bp = (const unsigned char *)bias;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  const size_t pw = type_size(param_type);
+  float sum = 0.0f;
+  for (size_t i = 0; i < n; ++i) sum += load_as_f32(type, s + i * w);
+  const float mean = sum / (float)n;
+  float sum_squares = 0.0f;
+  for (size_t i = 0; i < n; ++i) {
+    const float centered = load_as_f32(type, s + i * w) - mean;
+    sum_squares = fmaf(centered, centered, sum_squares);
+  }
+  const float inverse = 1.0f / sqrtf(sum_squares / (float)n + epsilon);
+  for (size_t i = 0; i < n; ++i) {
+    const float normalized = (load_as_f32(type, s + i * w) - mean) * inverse;
+    if (scale == NULL)
+      store_from_f32(type, d + i * w, normalized);
+    else if (bias == NULL)
+      store_from_f32(type, d + i * w,
+                     normalized * load_as_f32(param_type, sp + i * pw));
+    else
+      store_from_f32(type, d + i * w,
+                     fmaf(normalized, load_as_f32(param_type, sp + i * pw),
+                          load_as_f32(param_type, bp + i * pw)));
+  }
+}
+
+void hyle_oracle_layer_norm(int type, int param_type, const void *src,
+                            const void *scale, const void *bias, void *dst,
+                            size_t rows, size_t hidden, float epsilon) {
+  const unsigned char *s = (const unsigned char *)src;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  for (size_t r = 0; r < rows; ++r)
+    hyle_oracle_layer_norm_row(type, param_type, s + r * hidden * w, scale, bias,
+                               d + r * hidden * w, hidden, epsilon);
+}
+
 /* src/compute_provider_native/normalization.cc:41-80.  The reference sums each
  * tile with simd::dot (a Highway vector dot: lane order is target-dependent),
  * here each tile is summed in index order without fusing; the row total adds

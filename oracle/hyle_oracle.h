@@ -149,6 +149,17 @@ void hyle_oracle_rms_norm_row(int type, int weight_type, const void *src,
 void hyle_oracle_rms_norm(int type, int weight_type, const void *src,
                           const void *weight, void *dst, size_t rows,
                           size_t hidden, float epsilon);
+/* LayerNorm over the last axis, src/simd/math/activations.cc:148-175.  scale
+ * and bias may both be NULL; with scale alone the result is normalised * scale
+ * (the provider-level form of tests/compute_provider_native/normalization_test.cc:69-127,
+ * which the scalar floor does not have).  param_type may be HYLE_ORACLE_F32 for
+ * a narrow input. */
+void hyle_oracle_layer_norm_row(int type, int param_type, const void *src,
+                                const void *scale, const void *bias, void *dst,
+                                size_t n, float epsilon);
+void hyle_oracle_layer_norm(int type, int param_type, const void *src,
+                            const void *scale, const void *bias, void *dst,
+                            size_t rows, size_t hidden, float epsilon);
 /* src/compute_provider_native/normalization.cc:41-80: 128-wide f32 tiles,
  * squares += dot(tile, tile); (x * inv) then * w; one RN-even store. */
 void hyle_oracle_rms_norm_native(int type, int weight_type, const void *src,

@@ -69,6 +69,7 @@ _swiglu = _sig("hyle_oracle_swiglu", None, C.c_int, _vp, _vp, _vp, _sz)
 _swiglu_packed = _sig("hyle_oracle_swiglu_packed", None, C.c_int, _vp, _vp, _sz, _sz)
 _rms = _sig("hyle_oracle_rms_norm", None, C.c_int, C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_float)
 _rms_native = _sig("hyle_oracle_rms_norm_native", None, C.c_int, C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_float)
+_layer = _sig("hyle_oracle_layer_norm", None, C.c_int, C.c_int, _vp, _vp, _vp, _vp, _sz, _sz, C.c_float)
 _softmax_row = _sig("hyle_oracle_softmax_f32_row", None, _vp, _vp, _sz)
 _softmax = _sig("hyle_oracle_softmax", None, C.c_int, _vp, _vp, _i64p, C.c_int, C.c_float,
                 C.c_int, _vp, _i64p, _i64p, C.c_int)
@@ -247,6 +248,20 @@ def rms_norm(type_id, src, weight, epsilon, weight_type=None, native=False):
     out = np.empty_like(src)
     fn = _rms_native if native else _rms
     fn(type_id, weight_type, _ptr(src), _ptr(weight), _ptr(out), rows, hidden, float(epsilon))
+    return out
+
+
+def layer_norm(type_id, src, scale, bias, epsilon, param_type=None):
+    src = _c(src, _NP[type_id])
+    param_type = type_id if param_type is None else param_type
+    if scale is None and bias is not None:
+        raise ValueError("LayerNorm takes a bias only together with a scale")
+    scale = None if scale is None else _c(scale, _NP[param_type])
+    bias = None if bias is None else _c(bias, _NP[param_type])
+    hidden = src.shape[-1]
+    rows = src.size // hidden if hidden else 0
+    out = np.empty_like(src)
+    _layer(type_id, param_type, _ptr(src), _ptr(scale), _ptr(bias), _ptr(out), rows, hidden, float(epsilon))
     return out
 
 

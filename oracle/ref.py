@@ -79,6 +79,16 @@ def rms_norm_row(type_id: int, src: np.ndarray, weight, epsilon: float) -> np.nd
     return out
 
 
+def layer_norm_row(type_id: int, src: np.ndarray, scale, bias, epsilon: float) -> np.ndarray:
+    src = np.ascontiguousarray(src)
+    scale = None if scale is None else np.ascontiguousarray(scale)
+    bias = None if bias is None else np.ascontiguousarray(bias)
+    out = np.empty_like(src)
+    _fn(f"ref_layer_norm_{_SUFFIX[type_id]}", None, _vp, _vp, _vp, _vp, _sz, C.c_float)(
+        _p(src), _p(scale), _p(bias), _p(out), src.size, float(epsilon))
+    return out
+
+
 def softmax_f32(src: np.ndarray) -> np.ndarray:
     src = np.ascontiguousarray(src, np.float32)
     out = np.empty_like(src)

@@ -4,7 +4,7 @@
 // This file contains no arithmetic.  It includes the reference's headers where
 // they lie (the Makefile passes -I<reference> -I<reference>/include) and
 // forwards to the functions the reference compiles from
-//   src/simd/math/activations.cc      (silu / swiglu / rms_norm / softmax)
+//   src/simd/math/activations.cc      (silu / swiglu / rms_norm / layer_norm / softmax)
 //   include/hyle/simd/dtype.h         (f16 / bf16 codecs, header-only)
 // The resulting library lives in oracle/_ref/ and is never committed.
 #include <cstddef>
@@ -86,6 +86,25 @@ void ref_rms_norm_bf16(const std::uint16_t *src, const std::uint16_t *weight,
   hd::rms_norm_bf16_scalar(reinterpret_cast<const hs::bfloat16_t *>(src),
                            reinterpret_cast<const hs::bfloat16_t *>(weight),
                            reinterpret_cast<hs::bfloat16_t *>(dst), n, epsilon);
+}
+
+void ref_layer_norm_f32(const float *src, const float *scale, const float *bias, float *dst,
+                        std::size_t n, float epsilon) {
+  hd::layer_norm_f32_scalar(src, scale, bias, dst, n, epsilon);
+}
+void ref_layer_norm_f16(const std::uint16_t *src, const std::uint16_t *scale, const std::uint16_t *bias,
+                        std::uint16_t *dst, std::size_t n, float epsilon) {
+  hd::layer_norm_f16_scalar(reinterpret_cast<const hs::float16_t *>(src),
+                            reinterpret_cast<const hs::float16_t *>(scale),
+                            reinterpret_cast<const hs::float16_t *>(bias),
+                            reinterpret_cast<hs::float16_t *>(dst), n, epsilon);
+}
+void ref_layer_norm_bf16(const std::uint16_t *src, const std::uint16_t *scale, const std::uint16_t *bias,
+                         std::uint16_t *dst, std::size_t n, float epsilon) {
+  hd::layer_norm_bf16_scalar(reinterpret_cast<const hs::bfloat16_t *>(src),
+                             reinterpret_cast<const hs::bfloat16_t *>(scale),
+                             reinterpret_cast<const hs::bfloat16_t *>(bias),
+                             reinterpret_cast<hs::bfloat16_t *>(dst), n, epsilon);
 }
 
 void ref_softmax_f32(const float *src, float *dst, std::size_t n) {

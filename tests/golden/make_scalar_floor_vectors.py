@@ -105,6 +105,19 @@ def main() -> None:
     out["softmax_x_wide"] = wide
     out["softmax_y_wide_words"] = ref.softmax_f32(wide).view(np.uint32)
 
+    # layer norm rows (drawn last so that every array above keeps its values)
+    for n in (1, 7, 127, 128, 129, 257, 2048):
+        row = (rng.normal(0.5, 1, n) * rng.uniform(0.1, 10)).astype(np.float32)
+        scale = rng.normal(1, 0.1, n).astype(np.float32)
+        bias = rng.normal(0, 0.5, n).astype(np.float32)
+        out[f"ln_x_f32_{n}"], out[f"ln_s_f32_{n}"], out[f"ln_b_f32_{n}"] = row, scale, bias
+        out[f"ln_y_f32_{n}"] = ref.layer_norm_row(0, row, scale, bias, 1e-5)
+        out[f"ln_y_f32_plain_{n}"] = ref.layer_norm_row(0, row, None, None, 1e-6)
+        for tag, type_id, narrow in (("bf16", 2, ref.f32_to_bf16), ("f16", 1, ref.f32_to_f16)):
+            rn, sn, bn = narrow(row), narrow(scale), narrow(bias)
+            out[f"ln_x_{tag}_{n}"], out[f"ln_s_{tag}_{n}"], out[f"ln_b_{tag}_{n}"] = rn, sn, bn
+            out[f"ln_y_{tag}_{n}"] = ref.layer_norm_row(type_id, rn, sn, bn, 1e-5)
+
     np.savez_compressed(OUT, **out)
     print(f"wrote {OUT}: {os.path.getsize(OUT)} bytes, {len(out)} arrays")
 

@@ -195,7 +195,7 @@ def test_routes_alias_support_and_cost_facts():
                          hc.TensorDesc.strided_bytes(DT.kFloat32, [6, 16], [0, 4]))
     assert strided.route_name() == "elementwise-strided" and not strided.alias_support(0, 0)
     norm = hc.prepare(CTX, hc.RmsNorm(1e-6), D(DT.kBFloat16, [8192, 2048]), D(DT.kBFloat16, [2048]))
-    assert norm.route_name() == "rms-norm-rows" and norm.alias_support(0, 0) and not norm.alias_support(0, 1)
+    assert norm.route_name() == "norm-rows" and norm.alias_support(0, 0) and not norm.alias_support(0, 1)
     gated = hc.prepare(CTX, hc.GatedActivation(hc.GatedActivationKind.kSilu, hc.GatedInputKind.kSeparate),
                        D(DT.kBFloat16, [8, 64]), D(DT.kBFloat16, [8, 64]))
     assert not gated.alias_support(0, 0)  # src/compute_provider_cuda/cuda_provider.cc:219-221

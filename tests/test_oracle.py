@@ -347,6 +347,66 @@ def test_rms_norm_matches_reference_floor_live():
         assert np.array_equal(orc.rms_norm(orc.BF16, xb, wb, 1e-6), ref.rms_norm_row(2, xb, wb, 1e-6))
 
 
+# ------------------------------------------------------------ layer norm ---
+def test_layer_norm_golden_bit_exact():
+    for n in (1, 7, 127, 128, 129, 257, 2048):
+        x, s, b = GOLD[f"ln_x_f32_{n}"], GOLD[f"ln_s_f32_{n}"], GOLD[f"ln_b_f32_{n}"]
+        same_bits_or_nan32(orc.layer_norm(orc.F32, x, s, b, 1e-5), GOLD[f"ln_y_f32_{n}"])
+        same_bits_or_nan32(orc.layer_norm(orc.F32, x, None, None, 1e-6), GOLD[f"ln_y_f32_plain_{n}"])
+        for tag, type_id in (("bf16", orc.BF16), ("f16", orc.F16)):
+            got = orc.layer_norm(type_id, GOLD[f"ln_x_{tag}_{n}"], GOLD[f"ln_s_{tag}_{n}"], GOLD[f"ln_b_{tag}_{n}"], 1e-5)
+            assert np.array_equal(got, GOLD[f"ln_y_{tag}_{n}"])
+
+
+def test_layer_norm_closed_form_and_reference_test_cases():
+    # tests/simd/math_test.cc:1168-1231: generator row, affine and plain, constant row -> zeros
+    n, eps = 257, 1e-5
+    i = np.arange(n, dtype=np.float32)
+    x = (3.0 * np.sin(i * np.float32(0.13)) + 0.25).astype(np.float32)
+    w = (0.75 + 0.5 * i / np.float32(n)).astype(np.float32)
+    b = (0.125 * np.cos(i * np.float32(0.07))).astype(np.float32)
+    x64 = x.astype(np.float64)
+    inv = 1.0 / math.sqrt(float(np.mean((x64 - x64.mean()) ** 2)) + eps)
+    want = (x64 - x64.mean()) * inv * w + b
+    got = orc.layer_norm(orc.F32, x, w, b, eps).astype(np.float64)
+    assert np.all(np.abs(got - want) <= np.abs(want) * 3e-5 + 3e-6)
+    plain = orc.layer_norm(orc.F32, x, None, None, eps).astype(np.float64)
+    assert np.all(np.abs(plain - (x64 - x64.mean()) * inv) <= np.abs((x64 - x64.mean()) * inv) * 3e-5 + 3e-6)
+    assert np.array_equal(orc.layer_norm(orc.F32, np.full(17, 3.0, np.float32), None, None, eps), np.zeros(17, np.float32))
+    # tests/compute_provider_native/normalization_test.cc:69-127: plain, scale only, affine (2e-5 absolute)
+    values = np.array([[1, 2, 3], [2, 4, 6]], np.float32)
+    scale, bias = np.array([2, 3, 4], np.float32), np.array([10, 20, 30], np.float32)
+    first = 1.0 / math.sqrt(2.0 / 3.0 + 1e-5)
+    second = 2.0 / math.sqrt(8.0 / 3.0 + 1e-5)
+    normalized = np.array([[-first, 0, first], [-second, 0, second]])
+    assert np.all(np.abs(orc.layer_norm(orc.F32, values, None, None, 1e-5) - normalized) <= 2e-5)
+    assert np.all(np.abs(orc.layer_norm(orc.F32, values, scale, None, 1e-5) - normalized * scale) <= 2e-5)
+    assert np.all(np.abs(orc.layer_norm(orc.F32, values, scale, bias, 1e-5) - (normalized * scale + bias)) <= 2e-5)
+    # shift invariance up to rounding: adding a constant that is exact in f32 leaves the result
+    shifted = orc.layer_norm(orc.F32, (x + np.float32(64.0)).astype(np.float32), None, None, eps).astype(np.float64)
+    assert np.all(np.abs(shifted - plain) <= 2e-4)
+    # narrow inputs with f32 parameters round once
+    xb = orc.from_f32(orc.BF16, x)
+    mixed = orc.layer_norm(orc.BF16, xb, w, b, eps, param_type=orc.F32)
+    xf = orc.to_f32(orc.BF16, xb).astype(np.float64)
+    inv_b = 1.0 / math.sqrt(float(np.mean((xf - xf.mean()) ** 2)) + eps)
+    want_b = orc.from_f32(orc.BF16, ((xf - xf.mean()) * inv_b * w + b).astype(np.float32))
+    assert np.abs(mixed.astype(np.int32) - want_b.astype(np.int32)).max() <= 1
+
+
+@needs_ref
+def test_layer_norm_matches_reference_floor_live():
+    rng = np.random.default_rng(8)
+    for n in (3, 64, 1000, 2048, 6144):
+        x = (rng.normal(0.3, 1, n) * rng.uniform(0.1, 10)).astype(np.float32)
+        s, b = rng.normal(1, 0.1, n).astype(np.float32), rng.normal(0, 0.5, n).astype(np.float32)
+        same_bits_or_nan32(orc.layer_norm(orc.F32, x, s, b, 1e-5), ref.layer_norm_row(0, x, s, b, 1e-5))
+        same_bits_or_nan32(orc.layer_norm(orc.F32, x, None, None, 1e-5), ref.layer_norm_row(0, x, None, None, 1e-5))
+        for type_id in (orc.BF16, orc.F16):
+            xn, sn, bn = orc.from_f32(type_id, x), orc.from_f32(type_id, s), orc.from_f32(type_id, b)
+            assert np.array_equal(orc.layer_norm(type_id, xn, sn, bn, 1e-5), ref.layer_norm_row(type_id, xn, sn, bn, 1e-5))
+
+
 # -------------------------------------------------------------- softmax ---
 def softmax64(x):
     x = np.asarray(x, np.float64)
