@@ -72,6 +72,69 @@ template <class T> __device__ __forceinline__ float silu_for(float x) {
   else return silu_fast(x);
 }
 
+// Unary kinds (include/hyle/compute/operation.h:57-73) in the scalar forms of the reference:
+// src/compute_provider_native/elementwise.cc:30-55 (neg, exp, log, sqrt, rsqrt, tanh, relu, silu),
+// src/simd/math/activations.cc:21-47 (sigmoid, gelu, gelu_tanh, silu) and
+// tests/compute_provider_native/elementwise_test.cc:43-82 (abs, softplus).
+enum : int {
+  kAbs = 0, kNeg, kExp, kLog, kSqrt, kRsqrt, kTanh, kSigmoid, kRelu, kGelu, kGeluTanh, kSiluKind, kSoftplus
+};
+
+__device__ __forceinline__ float sigmoid_exact(float x) {
+  if (x != x) return x;
+  const float e = expf(-fabsf(x));
+  return x < 0.0f ? e / (1.0f + e) : 1.0f / (1.0f + e);
+}
+__device__ __forceinline__ float gelu_erf(float x) {
+  if (x == -INFINITY) return 0.0f;
+  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+__device__ __forceinline__ float gelu_tanh(float x) {
+  if (x == -INFINITY) return 0.0f;
+  const float inner = 0.79788456080286535588f * x * __builtin_fmaf(0.044715f, x * x, 1.0f);
+  return 0.5f * x * (1.0f + tanhf(inner));
+}
+// log1p(exp(x)); the reference evaluates it in double.  max(x, 0) + log1p(exp(-|x|)) is the
+// same function without the overflow, good to a few units of f32 in the last place.
+__device__ __forceinline__ float softplus(float x) {
+  if (x != x) return x;
+  return fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x)));
+}
+
+template <class T> __device__ __forceinline__ float unary_apply_rt(int kind, float x) {
+  switch (kind) {
+    case kAbs: return fabsf(x);
+    case kNeg: return -x;
+    case kExp: return expf(x);
+    case kLog: return logf(x);
+    case kSqrt: return sqrtf(x);
+    case kRsqrt: return 1.0f / sqrtf(x);
+    case kTanh: return tanhf(x);
+    case kSigmoid: return sigmoid_exact(x);
+    case kRelu: return x != x ? x : (x > 0.0f ? x : 0.0f);
+    case kGelu: return gelu_erf(x);
+    case kGeluTanh: return gelu_tanh(x);
+    case kSiluKind: return silu_for<T>(x);
+    default: return softplus(x);
+  }
+}
+template <int kKind> struct UnaryFn {
+  static constexpr int kInputs = 1;
+  template <class T> __device__ __forceinline__ float operator()(T, float x, float, float) const {
+    return unary_apply_rt<T>(kKind, x);  // kKind is a constant: the switch folds away
+  }
+};
+// GatedActivationKind (include/hyle/compute/operation.h:91-95): activation(gate) * value.
+template <class T> __device__ __forceinline__ float gate_apply_rt(int activation, float g) {
+  return activation == 0 ? silu_for<T>(g) : (activation == 1 ? gelu_erf(g) : gelu_tanh(g));
+}
+template <int kActivation> struct GatedFn {
+  static constexpr int kInputs = 2;
+  template <class T> __device__ __forceinline__ float operator()(T, float g, float u, float) const {
+    return gate_apply_rt<T>(kActivation, g) * u;
+  }
+};
+
 template <int kKind> struct BinaryFn {
   static constexpr int kInputs = 2;
   template <class T> __device__ __forceinline__ float operator()(T, float x, float y, float) const {
@@ -106,6 +169,8 @@ struct RuntimeFn {
       case EwOp::kChain:
         return binary_apply_rt(kind1, Traits<T>::round(binary_apply_rt(kind0, x, y)), z);
       case EwOp::kSilu: return silu_for<T>(x);
+      case EwOp::kUnary: return unary_apply_rt<T>(kind0, x);
+      case EwOp::kGated: return gate_apply_rt<T>(kind0, x) * y;
       default: return silu_for<T>(x) * y;
     }
   }
@@ -299,11 +364,11 @@ __global__ __launch_bounds__(kBlockThreads) void ew_general(const char *a, const
   Traits<T>::store(out, e, fn(T{}, xs, ys, zs));
 }
 
-// ---- packed SwiGLU -----------------------------------------------------------------
+// ---- packed gated activation: rows of [gate | value] -----------------------------------------------------------------
 template <class T>
 __global__ __launch_bounds__(kBlockThreads) void swiglu_packed_vec(const void *packed, void *out,
                                                                    uint32_t row_vectors,
-                                                                   uint64_t vectors) {
+                                                                   uint64_t vectors, int activation) {
   constexpr int kVec = Traits<T>::kVec;
   const uint64_t first = (uint64_t)blockIdx.x * (kUnroll * kBlockThreads) + threadIdx.x;
   float g[kUnroll][kVec], u[kUnroll][kVec];
@@ -322,7 +387,7 @@ __global__ __launch_bounds__(kBlockThreads) void swiglu_packed_vec(const void *p
     if (vec < vectors) {
       float r[kVec];
 #pragma unroll
-      for (int j = 0; j < kVec; ++j) r[j] = silu_for<T>(g[k][j]) * u[k][j];
+      for (int j = 0; j < kVec; ++j) r[j] = gate_apply_rt<T>(activation, g[k][j]) * u[k][j];
       store16_stream(out, vec, Traits<T>::pack(r));
     }
   }
@@ -331,13 +396,13 @@ __global__ __launch_bounds__(kBlockThreads) void swiglu_packed_vec(const void *p
 template <class T>
 __global__ __launch_bounds__(kBlockThreads) void swiglu_packed_scalar(const void *packed, void *out,
                                                                       uint32_t hidden,
-                                                                      uint64_t elements) {
+                                                                      uint64_t elements, int activation) {
   const uint64_t e = (uint64_t)blockIdx.x * kBlockThreads + threadIdx.x;
   if (e >= elements) return;
   const uint64_t row = e / hidden, col = e % hidden;
   const float g = Traits<T>::load(packed, row * 2 * hidden + col);
   const float u = Traits<T>::load(packed, row * 2 * hidden + hidden + col);
-  Traits<T>::store(out, e, silu_for<T>(g) * u);
+  Traits<T>::store(out, e, gate_apply_rt<T>(activation, g) * u);
 }
 
 // ---- host dispatch -------------------------------------------------------------------
@@ -448,6 +513,26 @@ hipError_t run_flat(const EwFlat &p, const void *a, const void *b, const void *c
       }
     case EwOp::kSilu: return run_vec<T, SiluFn>(p, oa, ob, oc, out, s);
     case EwOp::kSwiglu: return run_vec<T, SwigluFn>(p, oa, ob, oc, out, s);
+    case EwOp::kUnary:
+      switch (p.kind0) {
+        case kAbs: return run_vec<T, UnaryFn<kAbs>>(p, oa, ob, oc, out, s);
+        case kNeg: return run_vec<T, UnaryFn<kNeg>>(p, oa, ob, oc, out, s);
+        case kExp: return run_vec<T, UnaryFn<kExp>>(p, oa, ob, oc, out, s);
+        case kLog: return run_vec<T, UnaryFn<kLog>>(p, oa, ob, oc, out, s);
+        case kSqrt: return run_vec<T, UnaryFn<kSqrt>>(p, oa, ob, oc, out, s);
+        case kRsqrt: return run_vec<T, UnaryFn<kRsqrt>>(p, oa, ob, oc, out, s);
+        case kTanh: return run_vec<T, UnaryFn<kTanh>>(p, oa, ob, oc, out, s);
+        case kSigmoid: return run_vec<T, UnaryFn<kSigmoid>>(p, oa, ob, oc, out, s);
+        case kRelu: return run_vec<T, UnaryFn<kRelu>>(p, oa, ob, oc, out, s);
+        case kGelu: return run_vec<T, UnaryFn<kGelu>>(p, oa, ob, oc, out, s);
+        case kGeluTanh: return run_vec<T, UnaryFn<kGeluTanh>>(p, oa, ob, oc, out, s);
+        case kSoftplus: return run_vec<T, UnaryFn<kSoftplus>>(p, oa, ob, oc, out, s);
+        default: return hipErrorInvalidValue;
+      }
+    case EwOp::kGated:
+      if (p.kind0 == 1) return run_vec<T, GatedFn<1>>(p, oa, ob, oc, out, s);
+      if (p.kind0 == 2) return run_vec<T, GatedFn<2>>(p, oa, ob, oc, out, s);
+      return hipErrorInvalidValue;
   }
   return hipErrorInvalidValue;
 }
@@ -478,11 +563,11 @@ hipError_t run_packed(const EwPacked &p, const void *packed, void *out, bool vec
     const uint64_t vectors = elements / kVec;
     const uint64_t per_block = (uint64_t)kUnroll * kBlockThreads;
     hipLaunchKernelGGL((swiglu_packed_vec<T>), dim3((uint32_t)((vectors + per_block - 1) / per_block)),
-                       dim3(kBlockThreads), 0, s, packed, out, p.hidden / kVec, vectors);
+                       dim3(kBlockThreads), 0, s, packed, out, p.hidden / kVec, vectors, (int)p.activation);
   } else {
     hipLaunchKernelGGL((swiglu_packed_scalar<T>),
                        dim3((uint32_t)((elements + kBlockThreads - 1) / kBlockThreads)),
-                       dim3(kBlockThreads), 0, s, packed, out, p.hidden, elements);
+                       dim3(kBlockThreads), 0, s, packed, out, p.hidden, elements, (int)p.activation);
   }
   return hipGetLastError();
 }

@@ -17,7 +17,8 @@ inline int elem_vec(Elem e) { return e == Elem::kF32 ? 4 : 8; }
 constexpr int kMaxRank = 8;
 
 // ---- elementwise ------------------------------------------------------------
-enum class EwOp : uint8_t { kBinary = 0, kChain, kSilu, kSwiglu };
+// kUnary: kind0 = UnaryKind; kGated: kind0 = GatedActivationKind (kSilu / kSwiglu are the SiLU forms)
+enum class EwOp : uint8_t { kBinary = 0, kChain, kSilu, kSwiglu, kUnary, kGated };
 
 // How one input is addressed by the flat (vectorised) kernel: every `period`
 // elements the operand repeats (0 = never, the operand is as large as the
@@ -46,6 +47,7 @@ struct EwGeneral {
 struct EwPacked {
   uint64_t rows = 0;
   uint32_t hidden = 0;
+  uint8_t activation = 0;  // GatedActivationKind
 };
 
 hipError_t launch_ew_flat(Elem type, const EwFlat &p, const void *a, const void *b, const void *c,

@@ -540,7 +540,7 @@ hyle_hip_status admit_elementwise(hyle_hip_plan *p, EwOp op, int inputs) {
   }
   // alias only when an input descriptor equals the output descriptor
   // (src/compute_provider_native/elementwise.cc:645-655; gated routes take no alias)
-  if (op != EwOp::kSwiglu)
+  if (op != EwOp::kSwiglu && op != EwOp::kGated)
     for (int i = 0; i < inputs; ++i)
       if (same_desc(r.inputs[i], out)) p->alias_inputs[0] |= (uint8_t)(1u << i);
 
@@ -597,21 +597,20 @@ hyle_hip_status admit(hyle_hip_plan *p) {
   hyle_hip_status s;
   switch (r.op) {
     case HYLE_HIP_OP_UNARY:
-      if (r.kind != HYLE_HIP_UNARY_SILU)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "only Unary SiLU is served by this provider");
-      return admit_elementwise(p, EwOp::kSilu, 1);
+      // integer abs / neg / relu pass the schema but are not served (FP32/FP16/BF16 only,
+      // include/hyle/compute/providers/cuda.h:20-23)
+      return admit_elementwise(p, r.kind == HYLE_HIP_UNARY_SILU ? EwOp::kSilu : EwOp::kUnary, 1);
     case HYLE_HIP_OP_BINARY:
       return admit_elementwise(p, EwOp::kBinary, 2);
     case HYLE_HIP_OP_BINARY_CHAIN:
       return admit_elementwise(p, EwOp::kChain, 3);
     case HYLE_HIP_OP_GATED_ACTIVATION: {
-      if (r.kind != HYLE_HIP_GATED_SILU)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "gated activation serves SiLU only");
-      // dense inputs and output (src/compute_provider_cuda/cuda_provider.cc:86-139)
+      // SiLU, GELU and GELU-tanh (include/hyle/compute/providers/cuda.h:52-54); dense inputs and output (src/compute_provider_cuda/cuda_provider.cc:86-139)
       for (uint32_t i = 0; i < r.input_count; ++i)
         if (!is_dense(in[i]))
           return fail(HYLE_HIP_UNIMPLEMENTED, "gated activation requires dense plain input");
-      if (r.kind2 == HYLE_HIP_GATED_SEPARATE) return admit_elementwise(p, EwOp::kSwiglu, 2);
+      if (r.kind2 == HYLE_HIP_GATED_SEPARATE)
+        return admit_elementwise(p, r.kind == HYLE_HIP_GATED_SILU ? EwOp::kSwiglu : EwOp::kGated, 2);
       if (!to_elem(out.dtype, &p->elem))
         return fail(HYLE_HIP_UNIMPLEMENTED, "gated activation requires dense FP16/BF16/FP32");
       if (p->output_elements[0] > kMaxElements)
@@ -620,6 +619,7 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->route = Route::kSwigluPacked;
       p->packed.hidden = (uint32_t)out.dims[out.rank - 1];
       p->packed.rows = p->output_elements[0] / p->packed.hidden;
+      p->packed.activation = (uint8_t)r.kind;
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }

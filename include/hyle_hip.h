@@ -89,8 +89,22 @@ typedef enum hyle_hip_op_kind {
   HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ = 0x101
 } hyle_hip_op_kind;
 
-/* UnaryKind (include/hyle/compute/operation.h:57-73); only SiLU is on the path. */
-enum { HYLE_HIP_UNARY_SILU = 11 };
+/* UnaryKind (include/hyle/compute/operation.h:57-73) */
+enum {
+  HYLE_HIP_UNARY_ABS = 0,
+  HYLE_HIP_UNARY_NEG = 1,
+  HYLE_HIP_UNARY_EXP = 2,
+  HYLE_HIP_UNARY_LOG = 3,
+  HYLE_HIP_UNARY_SQRT = 4,
+  HYLE_HIP_UNARY_RSQRT = 5,
+  HYLE_HIP_UNARY_TANH = 6,
+  HYLE_HIP_UNARY_SIGMOID = 7,
+  HYLE_HIP_UNARY_RELU = 8,
+  HYLE_HIP_UNARY_GELU = 9,
+  HYLE_HIP_UNARY_GELU_TANH = 10,
+  HYLE_HIP_UNARY_SILU = 11,
+  HYLE_HIP_UNARY_SOFTPLUS = 12
+};
 /* BinaryKind (include/hyle/compute/operation.h:75-82) */
 enum {
   HYLE_HIP_BINARY_ADD = 0,
@@ -108,7 +122,7 @@ enum {
   HYLE_HIP_REDUCE_MAXIMUM = 3
 };
 /* GatedActivationKind / GatedInputKind (include/hyle/compute/operation.h:91-100) */
-enum { HYLE_HIP_GATED_SILU = 0 };
+enum { HYLE_HIP_GATED_SILU = 0, HYLE_HIP_GATED_GELU = 1, HYLE_HIP_GATED_GELU_TANH = 2 };
 enum { HYLE_HIP_GATED_PACKED_HALVES = 0, HYLE_HIP_GATED_SEPARATE = 1 };
 /* SoftmaxKind / MaskKind (include/hyle/compute/operation.h:117-126) */
 enum { HYLE_HIP_SOFTMAX = 0, HYLE_HIP_LOG_SOFTMAX = 1 };

@@ -297,6 +297,67 @@ void hyle_oracle_swiglu(int type, const void *gate, const void *value,
   }
 }
 
+/* ---- every Unary kind and the three gate activations -------------------- */
+/* src/simd/math/activations.cc:27-41 */
+static float gelu_erf(float x) {
+  if (x == -INFINITY) return 0.0f;
+  return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f));
+}
+static float gelu_tanh(float x) {
+  if (x == -INFINITY) return 0.0f;
+  const float inner = 0.79788456080286535588f * x * fmaf(0.044715f, x * x, 1.0f);
+  return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+/* UnaryKind order of include/hyle/compute/operation.h:57-73.  neg, exp, log,
+ * sqrt, rsqrt, tanh, relu, silu: src/compute_provider_native/elementwise.cc:30-55;
+ * sigmoid, gelu, gelu_tanh: src/simd/math/activations.cc:21-41; abs and
+ * softplus (evaluated in double): tests/compute_provider_native/elementwise_test.cc:43-82.
+ * exp, log, tanh, erf are the host libm's. */
+float hyle_oracle_unary_scalar(int kind, float x) {
+  switch (kind) {
+    case 0: return fabsf(x);
+    case 1: return -x;
+    case 2: return expf(x);
+    case 3: return logf(x);
+    case 4: return sqrtf(x);
+    case 5: return 1.0f / sqrtf(x);
+    case 6: return tanhf(x);
+    case 7: return hyle_oracle_sigmoid(x);
+    case 8: return isnan(x) ? x : (x > 0.0f ? x : 0.0f);
+    case 9: return gelu_erf(x);
+    case 10: return gelu_tanh(x);
+    case 11: return hyle_oracle_silu(x);
+    default: return (float)log1p(exp((double)x));
+  }
+}
+
+/* decode -> f32 function -> one rounding
+ * (src/compute_provider_native/elementwise.cc:83-99, src/simd/math/activations.cc:106-112) */
+void hyle_oracle_unary(int kind, int type, const void *src, void *dst, size_t n) {
+  const unsigned char *s = (const unsigned char *)src;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  for (size_t i = 0; i < n; ++i)
+    store_from_f32(type, d + i * w, hyle_oracle_unary_scalar(kind, load_as_f32(type, s + i * w)));
+}
+
+/* src/simd/math/activations.cc:114-122 with activation = silu (0), gelu (1),
+ * gelu_tanh (2): GatedActivationKind of include/hyle/compute/operation.h:91-95 */
+void hyle_oracle_gated(int activation, int type, const void *gate, const void *value,
+                       void *dst, size_t n) {
+  const unsigned char *g = (const unsigned char *)gate;
+  const unsigned char *v = (const unsigned char *)value;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  for (size_t i = 0; i < n; ++i) {
+    const float gv = load_as_f32(type, g + i * w);
+    const float lv = load_as_f32(type, v + i * w);
+    const float a = activation == 0 ? hyle_oracle_silu(gv) : (activation == 1 ? gelu_erf(gv) : gelu_tanh(gv));
+    store_from_f32(type, d + i * w, a * lv);
+  }
+}
+
 /* src/compute_provider_native/elementwise.cc:192-208: value = gate + hidden */
 void hyle_oracle_swiglu_packed(int type, const void *packed, void *dst,
                                size_t rows, size_t hidden) {

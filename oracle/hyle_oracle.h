@@ -134,6 +134,17 @@ void hyle_oracle_silu_rows(int type, const void *src, void *dst, size_t n);
 /* src/simd/math/activations.cc:114-122 (gated_storage, activation = silu) */
 void hyle_oracle_swiglu(int type, const void *gate, const void *value,
                         void *dst, size_t n);
+/* Every UnaryKind (include/hyle/compute/operation.h:57-73: abs 0, neg 1, exp 2,
+ * log 3, sqrt 4, rsqrt 5, tanh 6, sigmoid 7, relu 8, gelu 9, gelu_tanh 10,
+ * silu 11, softplus 12) in the reference's scalar forms
+ * (src/compute_provider_native/elementwise.cc:30-55, src/simd/math/activations.cc:21-47,
+ * tests/compute_provider_native/elementwise_test.cc:43-82). */
+float hyle_oracle_unary_scalar(int kind, float x);
+void hyle_oracle_unary(int kind, int type, const void *src, void *dst, size_t n);
+/* activation(gate) * value, activation = silu 0, gelu 1, gelu_tanh 2
+ * (src/simd/math/activations.cc:114-122). */
+void hyle_oracle_gated(int activation, int type, const void *gate, const void *value,
+                       void *dst, size_t n);
 /* GatedInputKind::kPackedHalves: row = [gate half | value half]
  * (src/compute_provider_native/elementwise.cc:192-208). */
 void hyle_oracle_swiglu_packed(int type, const void *packed, void *dst,

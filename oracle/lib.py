@@ -66,6 +66,9 @@ _sigmoid = _sig("hyle_oracle_sigmoid", C.c_float, C.c_float)
 _silu1 = _sig("hyle_oracle_silu", C.c_float, C.c_float)
 _silu = _sig("hyle_oracle_silu_rows", None, C.c_int, _vp, _vp, _sz)
 _swiglu = _sig("hyle_oracle_swiglu", None, C.c_int, _vp, _vp, _vp, _sz)
+_unary = _sig("hyle_oracle_unary", None, C.c_int, C.c_int, _vp, _vp, _sz)
+_unary1 = _sig("hyle_oracle_unary_scalar", C.c_float, C.c_int, C.c_float)
+_gated = _sig("hyle_oracle_gated", None, C.c_int, C.c_int, _vp, _vp, _vp, _sz)
 _swiglu_packed = _sig("hyle_oracle_swiglu_packed", None, C.c_int, _vp, _vp, _sz, _sz)
 _rms = _sig("hyle_oracle_rms_norm", None, C.c_int, C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_float)
 _rms_native = _sig("hyle_oracle_rms_norm_native", None, C.c_int, C.c_int, _vp, _vp, _vp, _sz, _sz, C.c_float)
@@ -225,6 +228,20 @@ def swiglu(type_id, gate, value):
     assert gate.shape == value.shape
     out = np.empty_like(gate)
     _swiglu(type_id, _ptr(gate), _ptr(value), _ptr(out), gate.size)
+    return out
+
+
+def unary(kind: int, type_id: int, src):
+    src = _c(src, _NP[type_id])
+    out = np.empty_like(src)
+    _unary(int(kind), type_id, _ptr(src), _ptr(out), src.size)
+    return out
+
+
+def gated(activation: int, type_id: int, gate, value):
+    gate, value = _c(gate, _NP[type_id]), _c(value, _NP[type_id])
+    out = np.empty_like(gate)
+    _gated(int(activation), type_id, _ptr(gate), _ptr(value), _ptr(out), gate.size)
     return out
 
 

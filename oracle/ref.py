@@ -79,6 +79,22 @@ def rms_norm_row(type_id: int, src: np.ndarray, weight, epsilon: float) -> np.nd
     return out
 
 
+def activation(name: str, type_id: int, src: np.ndarray) -> np.ndarray:
+    """name: gelu, gelu_tanh (f32/f16/bf16), sigmoid, relu (f32)."""
+    src = np.ascontiguousarray(src)
+    out = np.empty_like(src)
+    _fn(f"ref_{name}_{_SUFFIX[type_id]}", None, _vp, _vp, _sz)(_p(src), _p(out), src.size)
+    return out
+
+
+def gated(name: str, type_id: int, gate: np.ndarray, value: np.ndarray) -> np.ndarray:
+    """name: geglu, geglu_tanh (f32/bf16)."""
+    gate, value = np.ascontiguousarray(gate), np.ascontiguousarray(value)
+    out = np.empty_like(gate)
+    _fn(f"ref_{name}_{_SUFFIX[type_id]}", None, _vp, _vp, _vp, _sz)(_p(gate), _p(value), _p(out), gate.size)
+    return out
+
+
 def layer_norm_row(type_id: int, src: np.ndarray, scale, bias, epsilon: float) -> np.ndarray:
     src = np.ascontiguousarray(src)
     scale = None if scale is None else np.ascontiguousarray(scale)

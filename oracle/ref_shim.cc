@@ -71,6 +71,38 @@ void ref_swiglu_bf16(const std::uint16_t *gate, const std::uint16_t *value,
                          reinterpret_cast<hs::bfloat16_t *>(dst), n);
 }
 
+// gelu / gelu_tanh / sigmoid / relu and the gated forms built on them
+void ref_gelu_f32(const float *src, float *dst, std::size_t n) { hd::gelu_f32_scalar(src, dst, n); }
+void ref_gelu_tanh_f32(const float *src, float *dst, std::size_t n) { hd::gelu_tanh_f32_scalar(src, dst, n); }
+void ref_sigmoid_f32(const float *src, float *dst, std::size_t n) { hd::sigmoid_f32_scalar(src, dst, n); }
+void ref_relu_f32(const float *src, float *dst, std::size_t n) { hd::relu_f32_scalar(src, dst, n); }
+void ref_gelu_f16(const std::uint16_t *src, std::uint16_t *dst, std::size_t n) {
+  hd::gelu_f16_scalar(reinterpret_cast<const hs::float16_t *>(src), reinterpret_cast<hs::float16_t *>(dst), n);
+}
+void ref_gelu_bf16(const std::uint16_t *src, std::uint16_t *dst, std::size_t n) {
+  hd::gelu_bf16_scalar(reinterpret_cast<const hs::bfloat16_t *>(src), reinterpret_cast<hs::bfloat16_t *>(dst), n);
+}
+void ref_gelu_tanh_f16(const std::uint16_t *src, std::uint16_t *dst, std::size_t n) {
+  hd::gelu_tanh_f16_scalar(reinterpret_cast<const hs::float16_t *>(src), reinterpret_cast<hs::float16_t *>(dst), n);
+}
+void ref_gelu_tanh_bf16(const std::uint16_t *src, std::uint16_t *dst, std::size_t n) {
+  hd::gelu_tanh_bf16_scalar(reinterpret_cast<const hs::bfloat16_t *>(src), reinterpret_cast<hs::bfloat16_t *>(dst), n);
+}
+void ref_geglu_f32(const float *gate, const float *value, float *dst, std::size_t n) {
+  hd::geglu_f32_scalar(gate, value, dst, n);
+}
+void ref_geglu_tanh_f32(const float *gate, const float *value, float *dst, std::size_t n) {
+  hd::geglu_tanh_f32_scalar(gate, value, dst, n);
+}
+void ref_geglu_bf16(const std::uint16_t *gate, const std::uint16_t *value, std::uint16_t *dst, std::size_t n) {
+  hd::geglu_bf16_scalar(reinterpret_cast<const hs::bfloat16_t *>(gate), reinterpret_cast<const hs::bfloat16_t *>(value),
+                        reinterpret_cast<hs::bfloat16_t *>(dst), n);
+}
+void ref_geglu_tanh_bf16(const std::uint16_t *gate, const std::uint16_t *value, std::uint16_t *dst, std::size_t n) {
+  hd::geglu_tanh_bf16_scalar(reinterpret_cast<const hs::bfloat16_t *>(gate), reinterpret_cast<const hs::bfloat16_t *>(value),
+                             reinterpret_cast<hs::bfloat16_t *>(dst), n);
+}
+
 void ref_rms_norm_f32(const float *src, const float *weight, float *dst,
                       std::size_t n, float epsilon) {
   hd::rms_norm_f32_scalar(src, weight, dst, n, epsilon);

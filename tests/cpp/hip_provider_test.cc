@@ -102,8 +102,10 @@ HOST_TEST(PreparesRoutesAndDeclinesCleanly) {
   EXPECT(top->create_invocation().error().IsInvalidArgument());  // needs its workspace
   // Declines are Unimplemented, never an error a router would have to surface.
   EXPECT(prepare(context, TopK{.count = 4}, dense(DataType::kFloat32, {8, 128})).error().IsUnimplemented());
-  EXPECT(prepare(context, Unary{UnaryKind::kTanh}, dense(DataType::kFloat32, {8})).error().IsUnimplemented());
-  EXPECT(prepare(context, GatedActivation{GatedActivationKind::kGelu}, dense(DataType::kBFloat16, {8, 64})).error().IsUnimplemented());
+  EXPECT(prepare(context, Unary{UnaryKind::kAbs}, dense(DataType::kInt32, {8})).error().IsUnimplemented());
+  EXPECT(prepare(context, LayerNorm{1.0e-5F, DataType::kFloat16}, dense(DataType::kFloat16, {8, 64})).error().IsUnimplemented());
+  EXPECT(prepare(context, Unary{UnaryKind::kTanh}, dense(DataType::kFloat32, {8})).has_value());
+  EXPECT(prepare(context, GatedActivation{GatedActivationKind::kGelu}, dense(DataType::kBFloat16, {8, 64})).has_value());
   EXPECT(prepare(context, Binary{}, dense(DataType::kInt32, {8}), dense(DataType::kInt32, {8})).error().IsUnimplemented());
   // Schema violations stay InvalidArgument.
   EXPECT(prepare(context, Binary{}, dense(DataType::kFloat32, {3}), dense(DataType::kFloat32, {4})).error().IsInvalidArgument());

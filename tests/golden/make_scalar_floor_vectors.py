@@ -118,6 +118,23 @@ def main() -> None:
             out[f"ln_x_{tag}_{n}"], out[f"ln_s_{tag}_{n}"], out[f"ln_b_{tag}_{n}"] = rn, sn, bn
             out[f"ln_y_{tag}_{n}"] = ref.layer_norm_row(type_id, rn, sn, bn, 1e-5)
 
+    # the other activations of the floor and the gates built on them (drawn last, see above)
+    xa = np.concatenate([SPECIAL_F32, rng.normal(0, 3, 800).astype(np.float32),
+                         rng.uniform(-12, 12, 400).astype(np.float32)]).astype(np.float32)
+    ua = rng.normal(0, 2, xa.size).astype(np.float32)
+    out["more_x_f32_words"], out["more_u_f32_words"] = xa.view(np.uint32), ua.view(np.uint32)
+    for name in ("gelu", "gelu_tanh", "sigmoid", "relu"):
+        out[f"{name}_f32_words"] = ref.activation(name, 0, xa).view(np.uint32)
+    out["geglu_f32_words"] = ref.gated("geglu", 0, xa, ua).view(np.uint32)
+    out["geglu_tanh_f32_words"] = ref.gated("geglu_tanh", 0, xa, ua).view(np.uint32)
+    for tag, type_id, narrow in (("bf16", 2, ref.f32_to_bf16), ("f16", 1, ref.f32_to_f16)):
+        xn, un = narrow(xa), narrow(ua)
+        out[f"more_x_{tag}"], out[f"more_u_{tag}"] = xn, un
+        out[f"gelu_{tag}"] = ref.activation("gelu", type_id, xn)
+        out[f"gelu_tanh_{tag}"] = ref.activation("gelu_tanh", type_id, xn)
+    out["geglu_bf16"] = ref.gated("geglu", 2, out["more_x_bf16"], out["more_u_bf16"])
+    out["geglu_tanh_bf16"] = ref.gated("geglu_tanh", 2, out["more_x_bf16"], out["more_u_bf16"])
+
     np.savez_compressed(OUT, **out)
     print(f"wrote {OUT}: {os.path.getsize(OUT)} bytes, {len(out)} arrays")
 

@@ -199,6 +199,15 @@ def test_routes_alias_support_and_cost_facts():
     gated = hc.prepare(CTX, hc.GatedActivation(hc.GatedActivationKind.kSilu, hc.GatedInputKind.kSeparate),
                        D(DT.kBFloat16, [8, 64]), D(DT.kBFloat16, [8, 64]))
     assert not gated.alias_support(0, 0)  # src/compute_provider_cuda/cuda_provider.cc:219-221
+    for kind in hc.UnaryKind:  # every Unary kind is served for floating storage, in place allowed
+        unary = hc.prepare(CTX, hc.Unary(kind), D(DT.kFloat16, [8, 64]))
+        assert unary.route_name() == "elementwise-flat" and unary.alias_support(0, 0)
+    for activation in hc.GatedActivationKind:
+        for inputs, descs in ((hc.GatedInputKind.kSeparate, [D(DT.kBFloat16, [8, 64])] * 2),
+                              (hc.GatedInputKind.kPackedHalves, [D(DT.kBFloat16, [8, 128])])):
+            served = hc.prepare(CTX, hc.GatedActivation(activation, inputs), *descs)
+            assert served.dispatch_count() == 1 and not served.alias_support(0, 0)
+            assert served.output_description() == D(DT.kBFloat16, [8, 64])
     soft = hc.prepare(CTX, hc.Softmax(mask=hc.MaskKind.kBoolean), D(DT.kFloat32, [32, 64, 64]), D(DT.kBool, [64, 64]))
     assert soft.route_name() == "softmax-rows" and soft.alias_support(0, 0)
     topk = hc.prepare(CTX, hc.TopK(), D(DT.kFloat32, [64, 151936]))
@@ -213,14 +222,14 @@ def test_routes_alias_support_and_cost_facts():
 def test_declines_are_unimplemented_and_errors_are_not():
     x = D(DT.kBFloat16, [4, 64])
     declines = [
-        lambda: hc.prepare(CTX, hc.Unary(hc.UnaryKind.kTanh), x),
+        lambda: hc.prepare(CTX, hc.Unary(hc.UnaryKind.kAbs), D(DT.kInt32, [4])),   # integer Unary
         lambda: hc.prepare(CTX, hc.RmsNorm(accumulation_type=DT.kBFloat16), x),
         lambda: hc.prepare(CTX, hc.Softmax(accumulation_type=DT.kUnknown), x),   # half needs explicit f32
         lambda: hc.prepare(CTX, hc.Reduce(hc.ReductionKind.kSum, axis=0, accumulation_type=DT.kFloat32), x),
         lambda: hc.prepare(CTX, hc.TopK(count=2), x),
         lambda: hc.prepare(CTX, hc.TopK(largest=False), x),
         lambda: hc.prepare(CTX, hc.Binary(), D(DT.kInt32, [4]), D(DT.kInt32, [4])),
-        lambda: hc.prepare(CTX, hc.GatedActivation(hc.GatedActivationKind.kGelu, hc.GatedInputKind.kSeparate), x, x),
+        lambda: hc.prepare(CTX, hc.LayerNorm(accumulation_type=DT.kFloat16), D(DT.kFloat16, [4, 64])),
         lambda: hc.prepare(CTX, hc.RmsNorm(), hc.TensorDesc.strided_bytes(DT.kBFloat16, [4, 64], [256, 2])),
     ]
     for attempt in declines:

@@ -347,6 +347,103 @@ def test_rms_norm_matches_reference_floor_live():
         assert np.array_equal(orc.rms_norm(orc.BF16, xb, wb, 1e-6), ref.rms_norm_row(2, xb, wb, 1e-6))
 
 
+# ------------------------------------------- every unary kind, gated forms ---
+ABS, NEG, EXP, LOG, SQRT, RSQRT, TANH, SIGMOID, RELU, GELU, GELU_TANH, SILU, SOFTPLUS = range(13)
+
+
+def test_unary_and_gated_golden_bit_exact():
+    x, u = f32(GOLD["more_x_f32_words"]), f32(GOLD["more_u_f32_words"])
+    for name, kind in (("gelu", GELU), ("gelu_tanh", GELU_TANH), ("sigmoid", SIGMOID), ("relu", RELU)):
+        same_bits_or_nan32(orc.unary(kind, orc.F32, x), f32(GOLD[f"{name}_f32_words"]))
+    same_bits_or_nan32(orc.gated(1, orc.F32, x, u), f32(GOLD["geglu_f32_words"]))
+    same_bits_or_nan32(orc.gated(2, orc.F32, x, u), f32(GOLD["geglu_tanh_f32_words"]))
+    for tag, type_id in (("bf16", orc.BF16), ("f16", orc.F16)):
+        assert np.array_equal(orc.unary(GELU, type_id, GOLD[f"more_x_{tag}"]), GOLD[f"gelu_{tag}"])
+        assert np.array_equal(orc.unary(GELU_TANH, type_id, GOLD[f"more_x_{tag}"]), GOLD[f"gelu_tanh_{tag}"])
+    assert np.array_equal(orc.gated(1, orc.BF16, GOLD["more_x_bf16"], GOLD["more_u_bf16"]), GOLD["geglu_bf16"])
+    assert np.array_equal(orc.gated(2, orc.BF16, GOLD["more_x_bf16"], GOLD["more_u_bf16"]), GOLD["geglu_tanh_bf16"])
+    # activation 0 is the SwiGLU already pinned above
+    assert np.array_equal(orc.gated(0, orc.BF16, GOLD["act_x_bf16"], GOLD["act_u_bf16"]), GOLD["swiglu_bf16"])
+    assert np.array_equal(orc.unary(SILU, orc.BF16, GOLD["act_x_bf16"]), GOLD["silu_bf16"])
+
+
+def test_unary_closed_forms_and_reference_test_values():
+    rng = np.random.default_rng(41)
+    x = np.concatenate([rng.normal(0, 3, 4000), rng.uniform(-80, 80, 1000)]).astype(np.float32)
+    pos = np.abs(x) + np.float32(1e-3)
+    x64, pos64 = x.astype(np.float64), pos.astype(np.float64)
+    # exact kinds
+    assert np.array_equal(orc.unary(ABS, orc.F32, x), np.abs(x))
+    assert np.array_equal(orc.unary(NEG, orc.F32, x), -x)
+    assert np.array_equal(orc.unary(SQRT, orc.F32, pos), np.sqrt(pos))          # correctly rounded both sides
+    assert np.array_equal(orc.unary(RELU, orc.F32, x), np.maximum(x, np.float32(0)))
+    # libm kinds against float64, a few units in the last place
+    def close(got, want, rel=4e-7):
+        got = got.astype(np.float64)
+        assert np.all(np.abs(got - want) <= rel * np.abs(want) + 1e-45)
+    with np.errstate(over="ignore"):
+        close(orc.unary(EXP, orc.F32, x), np.exp(x64).astype(np.float32).astype(np.float64))
+        close(orc.unary(LOG, orc.F32, pos), np.log(pos64))
+        close(orc.unary(RSQRT, orc.F32, pos), 1.0 / np.sqrt(pos64))
+        close(orc.unary(TANH, orc.F32, x), np.tanh(x64))
+        close(orc.unary(SIGMOID, orc.F32, x), 1.0 / (1.0 + np.exp(-x64)), rel=1e-6)
+        close(orc.unary(SOFTPLUS, orc.F32, x), np.log1p(np.exp(x64)), rel=2e-7)
+        inner = 0.79788456080286535588 * x64 * (1 + 0.044715 * x64 * x64)
+        # 1 + tanh(.) cancels for negative arguments in f32, as in the reference's own formula
+        got = orc.unary(GELU_TANH, orc.F32, x[:4000]).astype(np.float64)
+        want = (0.5 * x64 * (1 + np.tanh(inner)))[:4000]
+        assert np.all(np.abs(got - want) <= 2e-6 * np.abs(want) + 2e-7 * np.abs(x64[:4000]))
+    # special values of the scalar forms
+    inf, nan = np.float32(np.inf), np.float32(np.nan)
+    for kind in (GELU, GELU_TANH, SILU):
+        got = orc.unary(kind, orc.F32, np.array([-inf, inf, nan, 0.0, -0.0], np.float32))
+        assert got[0] == 0 and not np.signbit(got[0]) and got[1] == inf and np.isnan(got[2]) and got[3] == 0
+    assert np.isnan(orc.unary(RELU, orc.F32, np.array([nan], np.float32))[0])
+    relu_zero = orc.unary(RELU, orc.F32, np.array([-0.0, -1.0], np.float32))
+    assert not np.signbit(relu_zero).any() and (relu_zero == 0).all()
+    assert np.isnan(orc.unary(SIGMOID, orc.F32, np.array([nan], np.float32))[0])
+    assert orc.unary(SIGMOID, orc.F32, np.array([-inf, inf], np.float32)).tolist() == [0.0, 1.0]
+    assert orc.unary(SOFTPLUS, orc.F32, np.array([-inf, 100.0, inf], np.float32)).tolist() == [0.0, 100.0, np.inf]
+    # tests/compute_provider_native/elementwise_test.cc:127-178: seven values, every kind, 3e-4 relative
+    values = np.array([-2.0, -0.0, 0.25, 0.5, 1.0, 2.0, 4.0], np.float32)
+    v64 = values.astype(np.float64)
+    from math import erf
+    with np.errstate(divide="ignore", invalid="ignore"):
+        expected = {ABS: np.abs(v64), NEG: -v64, EXP: np.exp(v64), LOG: np.log(v64), SQRT: np.sqrt(v64),
+                    RSQRT: 1 / np.sqrt(v64), TANH: np.tanh(v64), SIGMOID: 1 / (1 + np.exp(-v64)),
+                    RELU: np.maximum(v64, 0), GELU: np.array([0.5 * v * (1 + erf(v * 0.7071067811865476)) for v in v64]),
+                    SILU: v64 / (1 + np.exp(-v64)), SOFTPLUS: np.log1p(np.exp(v64))}
+    for kind, want in expected.items():
+        got = orc.unary(kind, orc.F32, values).astype(np.float64)
+        for g, w in zip(got, want):
+            if np.isnan(w):
+                assert np.isnan(g)
+            elif np.isinf(w):
+                assert g == w
+            else:
+                assert abs(g - w) <= abs(w) * 3e-4 + 3e-6
+    # narrow storage: decode, apply, round once
+    xb = orc.from_f32(orc.BF16, x[:2000])
+    for kind in (EXP, TANH, SOFTPLUS, NEG, ABS):
+        want = orc.from_f32(orc.BF16, orc.unary(kind, orc.F32, orc.to_f32(orc.BF16, xb)))
+        assert np.array_equal(orc.unary(kind, orc.BF16, xb), want)
+
+
+@needs_ref
+def test_unary_and_gated_match_reference_floor_live():
+    rng = np.random.default_rng(42)
+    x = np.concatenate([rng.normal(0, 3, 20000), rng.uniform(-100, 100, 5000)]).astype(np.float32)
+    u = rng.normal(0, 2, x.size).astype(np.float32)
+    for name, kind in (("gelu", GELU), ("gelu_tanh", GELU_TANH), ("sigmoid", SIGMOID), ("relu", RELU)):
+        same_bits_or_nan32(orc.unary(kind, orc.F32, x), ref.activation(name, 0, x))
+    same_bits_or_nan32(orc.gated(1, orc.F32, x, u), ref.gated("geglu", 0, x, u))
+    same_bits_or_nan32(orc.gated(2, orc.F32, x, u), ref.gated("geglu_tanh", 0, x, u))
+    all16 = np.arange(1 << 16, dtype=np.uint32).astype(np.uint16)
+    for type_id in (orc.BF16, orc.F16):
+        assert np.array_equal(orc.unary(GELU, type_id, all16), ref.activation("gelu", type_id, all16))
+        assert np.array_equal(orc.unary(GELU_TANH, type_id, all16), ref.activation("gelu_tanh", type_id, all16))
+
+
 # ------------------------------------------------------------ layer norm ---
 def test_layer_norm_golden_bit_exact():
     for n in (1, 7, 127, 128, 129, 257, 2048):
