@@ -218,6 +218,24 @@ def main() -> int:
         ops.append(Op("next_layer_norm_bf16", hc.LayerNorm(epsilon=1e-6),
                       [D(BF, [8192, 2048]), D(BF, [2048]), D(BF, [2048])], set_ln, 10,
                       2 * 8192 * 2048 * 2 + 2 * 4096, 8192 * 2048, "bf16", in_step=False))
+    if want("next_geglu_tanh_bf16") or want("next_gelu_bf16"):
+        gate_g, up_g = wl.config3_swiglu()
+
+        def set_geglu(i):
+            dg, du = bf16(np.roll(gate_g, i, axis=0)), bf16(np.roll(up_g, i, axis=0))
+            return [dg, du], [torch.empty_like(dg)]
+
+        def set_gelu(i):
+            dg = bf16(np.roll(gate_g, i, axis=0))
+            return [dg], [torch.empty_like(dg)]
+        if want("next_geglu_tanh_bf16"):
+            ops.append(Op("next_geglu_tanh_bf16",
+                          hc.GatedActivation(hc.GatedActivationKind.kGeluTanh, hc.GatedInputKind.kSeparate),
+                          [D(BF, [8192, 6144]), D(BF, [8192, 6144])], set_geglu, 3,
+                          3 * 8192 * 6144 * 2, 8192 * 6144, "bf16", in_step=False))
+        if want("next_gelu_bf16"):
+            ops.append(Op("next_gelu_bf16", hc.Unary(hc.UnaryKind.kGelu), [D(BF, [8192, 6144])], set_gelu, 3,
+                          2 * 8192 * 6144 * 2, 8192 * 6144, "bf16", in_step=False))
     if want("next_copy_bf16"):
         def set_copy(i):
             src = torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev).normal_()

@@ -101,6 +101,46 @@ __device__ __forceinline__ float softplus(float x) {
   return fmaxf(x, 0.0f) + log1pf(expf(-fabsf(x)));
 }
 
+// Forms for narrow storage (8 or 11 significand bits), built on the hardware exp2 and
+// reciprocal like silu_fast; each is good to about 2e-7 of the result's scale, far inside half
+// a unit of bf16 / f16, and none of them subtracts nearly equal numbers.
+__device__ __forceinline__ float sigmoid_fast(float x) {
+  constexpr float kNegLog2e = -1.44269504088896340736f;
+  constexpr float kTwoM32 = 2.3283064365386963e-10f;
+  const float scaled = __builtin_amdgcn_exp2f(__builtin_fmaf(x, kNegLog2e, -32.0f));
+  return __builtin_amdgcn_rcpf(scaled + kTwoM32) * kTwoM32;
+}
+// 0.5 * (1 + tanh(u)) = sigmoid(2u): the tanh form of GELU without the cancelling 1 + tanh.
+__device__ __forceinline__ float gelu_tanh_fast(float x) {
+  const float inner = 0.79788456080286535588f * x * __builtin_fmaf(0.044715f, x * x, 1.0f);
+  return mul_zero_wins(x, sigmoid_fast(2.0f * inner));
+}
+// 1 - erf(z) for z >= 0 is poly(t) * exp(-z^2), t = 1 / (1 + p z) (Abramowitz and Stegun
+// 7.1.26, absolute error 1.5e-7); the negative side of 1 + erf is that product itself.
+__device__ __forceinline__ float gelu_erf_fast(float x) {
+  const float z = fabsf(x) * 0.70710678118654752440f;
+  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, z, 1.0f));
+  float poly = __builtin_fmaf(t, 1.061405429f, -1.453152027f);
+  poly = __builtin_fmaf(t, poly, 1.421413741f);
+  poly = __builtin_fmaf(t, poly, -0.284496736f);
+  poly = __builtin_fmaf(t, poly, 0.254829592f);
+  const float tail = mul_zero_wins(poly * t, __builtin_amdgcn_exp2f(-1.44269504088896340736f * z * z));
+  const float one_plus_erf = x < 0.0f ? tail : 2.0f - tail;
+  return mul_zero_wins(x, 0.5f * one_plus_erf);
+}
+template <class T> __device__ __forceinline__ float sigmoid_for(float x) {
+  if constexpr (Traits<T>::kSize == 4) return sigmoid_exact(x);
+  else return sigmoid_fast(x);
+}
+template <class T> __device__ __forceinline__ float gelu_for(float x) {
+  if constexpr (Traits<T>::kSize == 4) return gelu_erf(x);
+  else return gelu_erf_fast(x);
+}
+template <class T> __device__ __forceinline__ float gelu_tanh_for(float x) {
+  if constexpr (Traits<T>::kSize == 4) return gelu_tanh(x);
+  else return gelu_tanh_fast(x);
+}
+
 template <class T> __device__ __forceinline__ float unary_apply_rt(int kind, float x) {
   switch (kind) {
     case kAbs: return fabsf(x);
@@ -110,10 +150,10 @@ template <class T> __device__ __forceinline__ float unary_apply_rt(int kind, flo
     case kSqrt: return sqrtf(x);
     case kRsqrt: return 1.0f / sqrtf(x);
     case kTanh: return tanhf(x);
-    case kSigmoid: return sigmoid_exact(x);
+    case kSigmoid: return sigmoid_for<T>(x);
     case kRelu: return x != x ? x : (x > 0.0f ? x : 0.0f);
-    case kGelu: return gelu_erf(x);
-    case kGeluTanh: return gelu_tanh(x);
+    case kGelu: return gelu_for<T>(x);
+    case kGeluTanh: return gelu_tanh_for<T>(x);
     case kSiluKind: return silu_for<T>(x);
     default: return softplus(x);
   }
@@ -126,7 +166,7 @@ template <int kKind> struct UnaryFn {
 };
 // GatedActivationKind (include/hyle/compute/operation.h:91-95): activation(gate) * value.
 template <class T> __device__ __forceinline__ float gate_apply_rt(int activation, float g) {
-  return activation == 0 ? silu_for<T>(g) : (activation == 1 ? gelu_erf(g) : gelu_tanh(g));
+  return activation == 0 ? silu_for<T>(g) : (activation == 1 ? gelu_for<T>(g) : gelu_tanh_for<T>(g));
 }
 template <int kActivation> struct GatedFn {
   static constexpr int kInputs = 2;
