@@ -236,6 +236,26 @@ def main() -> int:
         if want("next_gelu_bf16"):
             ops.append(Op("next_gelu_bf16", hc.Unary(hc.UnaryKind.kGelu), [D(BF, [8192, 6144])], set_gelu, 3,
                           2 * 8192 * 6144 * 2, 8192 * 6144, "bf16", in_step=False))
+    # Reduce over the innermost axis, over the leading axis and over every axis (two dispatches
+    # that meet in the workspace when there are too few results to fill the chip).
+    reduce_lines = (
+        ("next_reduce_sum_rows_bf16", hc.ReductionKind.kSum, [-1], BF, torch.bfloat16, [8192, 2048], 16, 2 * 8192),
+        ("next_reduce_sum_columns_bf16", hc.ReductionKind.kSum, [0], BF, torch.bfloat16, [8192, 2048], 16, 2 * 2048),
+        ("next_reduce_max_all_f32", hc.ReductionKind.kMaximum, None, F32, torch.float32, [4096, 4096], 8, 4),
+    )
+    for name, kind, axes, dtype, torch_dtype, dims, sets, out_bytes in reduce_lines:
+        if not want(name):
+            continue
+
+        def set_reduce(i, dims=dims, torch_dtype=torch_dtype, axes=axes):
+            src = torch.empty(dims, dtype=torch_dtype, device=dev).normal_()
+            shape = [] if axes is None else [d for a, d in enumerate(dims) if a != axes[0] % len(dims)]
+            return [src], [torch.empty(shape, dtype=torch_dtype, device=dev)]
+        size = 4 if dtype == F32 else 2
+        ops.append(Op(name, hc.Reduce(kind, hc.Axes.all() if axes is None else hc.Axes.from_(axes),
+                                      accumulation_type=F32),
+                      [D(dtype, dims)], set_reduce, sets, dims[0] * dims[1] * size + out_bytes, dims[0] * dims[1],
+                      "f32" if dtype == F32 else "bf16", in_step=False))
     if want("next_copy_bf16"):
         def set_copy(i):
             src = torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev).normal_()

@@ -33,6 +33,7 @@ class OpDescC(C.Structure):
         ("keep_dimensions", C.c_uint32), ("epsilon", C.c_float), ("scale", C.c_float),
         ("count", C.c_uint64), ("largest", C.c_uint32), ("input_count", C.c_uint32),
         ("inputs", TensorDescC * MAX_INPUTS),
+        ("axes_count", C.c_uint32), ("axes", C.c_int32 * MAX_RANK),
     ]
 
 

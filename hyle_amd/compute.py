@@ -265,9 +265,35 @@ class BinaryChain:
 
 
 @dataclass(frozen=True)
+class Axes:
+    """include/hyle/compute/operation.h:232-247: every axis, or an explicit list whose entries
+    may count from the end.  Duplicates are refused when the output is inferred."""
+    values: tuple = ()
+    all_axes: bool = True
+
+    @staticmethod
+    def all() -> "Axes":
+        return Axes()
+
+    @staticmethod
+    def from_(axes) -> "Axes":  # Axes::from (src/compute_ops/operation.cc:768-789)
+        axes = tuple(int(a) for a in axes)
+        if not axes:
+            raise StatusError(StatusCode.kInvalidArgument, "explicit axis list cannot be empty")
+        if len(axes) > capi.MAX_RANK:
+            raise StatusError(StatusCode.kInvalidArgument, "axis list exceeds kMaxTensorRank")
+        if any(a < -capi.MAX_RANK or a >= capi.MAX_RANK for a in axes):
+            raise StatusError(StatusCode.kOutOfRange, "axis cannot address a supported tensor rank")
+        return Axes(axes, False)
+
+    def is_all(self) -> bool:
+        return self.all_axes
+
+
+@dataclass(frozen=True)
 class Reduce:
     kind: ReductionKind = ReductionKind.kSum
-    axis: int = -1
+    axes: Axes = Axes()
     keep_dimensions: bool = False
     accumulation_type: DataType = DataType.kUnknown
 
@@ -328,7 +354,10 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
     elif isinstance(operation, BinaryChain):
         c.op, c.kind, c.kind2 = OperationKind.kBinaryChain, int(operation.first), int(operation.second)
     elif isinstance(operation, Reduce):
-        c.op, c.kind, c.axis = OperationKind.kReduce, int(operation.kind), operation.axis
+        c.op, c.kind = OperationKind.kReduce, int(operation.kind)
+        c.axes_count = 0 if operation.axes.is_all() else len(operation.axes.values)
+        for i, axis in enumerate(operation.axes.values):
+            c.axes[i] = axis
         c.keep_dimensions, c.accumulation = int(operation.keep_dimensions), int(operation.accumulation_type)
     elif isinstance(operation, RmsNorm):
         c.op, c.epsilon, c.accumulation = OperationKind.kRmsNorm, operation.epsilon, int(operation.accumulation_type)

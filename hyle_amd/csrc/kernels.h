@@ -107,12 +107,33 @@ struct SoftmaxGeneralParams {
 hipError_t launch_softmax_general(Elem type, const SoftmaxGeneralParams &p, const void *x,
                                   const void *mask, void *y, hipStream_t stream);
 
-struct ReduceParams {
-  RowShape shape;
-  uint8_t kind = 0;  // HYLE_HIP_REDUCE_*
+// Reduce over a set of axes.  rows = results, width = elements folded into each result.
+enum class ReduceForm : uint8_t {
+  kRows,     // dense, reduced axes innermost: [rows, width]
+  kColumns,  // dense [outer, reduced, inner], inner > 1
+  kGeneral,  // byte strides and any set of axes
 };
-hipError_t launch_reduce_rows(Elem type, const ReduceParams &p, const void *x, void *y,
-                              bool vectorised, hipStream_t stream);
+struct ReduceParams {
+  uint8_t kind = 0;  // HYLE_HIP_REDUCE_*
+  ReduceForm form = ReduceForm::kGeneral;
+  uint32_t rows = 0, width = 0;
+  float divisor = 1.0f;  // the mean's count (0 for an empty reduction: the mean is NaN)
+  uint32_t outer = 1, reduced = 1, inner = 1;  // kColumns
+  // set by reduce_plan
+  uint32_t tiles = 1, tile_width = 0;          // kRows: pieces of one row
+  uint32_t segments = 1, segment_rows = 0;     // kColumns: pieces of the reduced extent
+  size_t workspace_bytes = 0;                  // f32 partial results of a two-dispatch launch
+  uint32_t dispatches = 1;
+  // kGeneral
+  int32_t rank = 0;
+  uint32_t axes = 0;  // bit a: axis a is reduced
+  uint32_t dims[kMaxRank] = {};
+  int64_t strides[kMaxRank] = {};
+  bool bytewise = false;  // strides or addresses that are not multiples of the element size
+};
+void reduce_plan(Elem type, ReduceParams *p);
+hipError_t launch_reduce(Elem type, const ReduceParams &p, const void *x, void *y, void *workspace,
+                         bool input_vector_aligned, hipStream_t stream);
 
 // TopK(count = 1): a scan dispatch leaves per-tile candidates in the workspace, a fold dispatch
 // turns them into the outputs.

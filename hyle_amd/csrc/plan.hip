@@ -200,6 +200,29 @@ hyle_hip_status normalize_axis(int32_t axis, int rank, int *out) {
   return HYLE_HIP_OK;
 }
 
+// Reduce::axes as a bit set (src/compute_ops/operation.cc:1358-1377; Axes::from,
+// src/compute_ops/operation.cc:768-789): no entries = every axis, a duplicate is refused.
+hyle_hip_status reduce_axes(const hyle_hip_op_desc &r, int rank, uint32_t *mask) {
+  *mask = 0;
+  if (r.axes_count == 0) {
+    *mask = (1u << rank) - 1u;
+    return HYLE_HIP_OK;
+  }
+  if (r.axes_count > HYLE_HIP_MAX_RANK)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "axis list exceeds kMaxTensorRank");
+  for (uint32_t i = 0; i < r.axes_count; ++i) {
+    if (r.axes[i] < -HYLE_HIP_MAX_RANK || r.axes[i] >= HYLE_HIP_MAX_RANK)
+      return fail(HYLE_HIP_OUT_OF_RANGE, "axis cannot address a supported tensor rank");
+    int axis;
+    hyle_hip_status s = normalize_axis(r.axes[i], rank, &axis);
+    if (s != HYLE_HIP_OK) return s;
+    if ((*mask >> axis) & 1u)
+      return fail(HYLE_HIP_INVALID_ARGUMENT, "Reduce axis list contains a duplicate");
+    *mask |= 1u << axis;
+  }
+  return HYLE_HIP_OK;
+}
+
 hyle_hip_status validate_accumulation(uint32_t type) {
   if (type == HYLE_HIP_DTYPE_UNKNOWN) return HYLE_HIP_OK;
   if (type > 255 || !is_numeric((uint8_t)type))
@@ -283,12 +306,12 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
       if (!is_numeric(in[0].dtype))
         return fail(HYLE_HIP_INVALID_ARGUMENT, "Reduce requires a numeric input");
       if ((s = validate_accumulation(r.accumulation)) != HYLE_HIP_OK) return s;
-      int axis;
-      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
+      uint32_t selected;
+      if ((s = reduce_axes(r, in[0].rank, &selected)) != HYLE_HIP_OK) return s;
       int64_t dims[HYLE_HIP_MAX_RANK];
       int rank = 0;
       for (int a = 0; a < in[0].rank; ++a) {
-        if (a == axis) {
+        if ((selected >> a) & 1u) {
           if (r.keep_dimensions) dims[rank++] = 1;
         } else {
           dims[rank++] = in[0].dims[a];
@@ -429,7 +452,7 @@ enum class Route : uint8_t {
   kSwigluPacked,
   kRmsNorm,
   kSoftmax,
-  kReduceRows,
+  kReduce,
   kArgmax,
   kQ8Dequant,
   kCast,
@@ -443,7 +466,7 @@ const char *route_name(Route r) {
     case Route::kSwigluPacked: return "swiglu-packed";
     case Route::kRmsNorm: return "norm-rows";
     case Route::kSoftmax: return "softmax-rows";
-    case Route::kReduceRows: return "reduce-rows";
+    case Route::kReduce: return "reduce";
     case Route::kArgmax: return "argmax-tiles";
     case Route::kQ8Dequant: return "q8_0-dequant-rows";
     case Route::kCast: return "cast-copy";
@@ -725,21 +748,64 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       return HYLE_HIP_OK;
     }
     case HYLE_HIP_OP_REDUCE: {
-      if (!to_elem(in[0].dtype, &p->elem) || !is_dense(in[0]))
-        return fail(HYLE_HIP_UNIMPLEMENTED, "Reduce requires dense plain float32/float16/bfloat16");
+      // src/compute_provider_cuda/reduction_provider.cc:40-107: plain f32/f16/bf16 with any
+      // byte strides, dense output, f32 accumulation (explicit for the narrow types), at most
+      // INT32_MAX elements on either side; an empty reduced extent still writes identities.
+      if (!to_elem(in[0].dtype, &p->elem) || !is_plain(in[0]))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Reduce requires plain float32/float16/bfloat16");
       if ((s = require_f32_accumulation(p, in[0].dtype, "Reduce")) != HYLE_HIP_OK) return s;
-      int axis;
-      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
-      if (axis != in[0].rank - 1)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "Reduce serves the last axis only");
-      if (p->input_elements[0] > kMaxElements)
+      uint32_t selected;
+      if ((s = reduce_axes(r, in[0].rank, &selected)) != HYLE_HIP_OK) return s;
+      if (p->input_elements[0] > kMaxElements || p->output_elements[0] > kMaxElements)
         return fail(HYLE_HIP_UNIMPLEMENTED, "Reduce requires at most INT32_MAX elements");
       if (p->output_elements[0] == 0) return HYLE_HIP_OK;
-      p->route = Route::kReduceRows;
-      p->reduce.shape.width = (uint32_t)in[0].dims[axis];
-      p->reduce.shape.rows = p->output_elements[0];
-      p->reduce.kind = (uint8_t)r.kind;
-      p->dispatches = 1;
+      ReduceParams &rp = p->reduce;
+      rp = ReduceParams{};
+      rp.kind = (uint8_t)r.kind;
+      rp.rows = (uint32_t)p->output_elements[0];
+      rp.width = (uint32_t)(p->input_elements[0] / p->output_elements[0]);
+      rp.divisor = (float)rp.width;
+      const int64_t size = (int64_t)dtype_size(in[0].dtype);
+      // Runs of neighbouring axes with the same fate (extent-1 axes belong to either run).
+      int groups = 0;
+      bool group_reduced[HYLE_HIP_MAX_RANK];
+      uint64_t group_extent[HYLE_HIP_MAX_RANK];
+      for (int a = 0; a < in[0].rank; ++a) {
+        if (in[0].dims[a] == 1) continue;
+        const bool reduced = ((selected >> a) & 1u) != 0;
+        if (groups != 0 && group_reduced[groups - 1] == reduced) {
+          group_extent[groups - 1] *= (uint64_t)in[0].dims[a];
+        } else {
+          group_reduced[groups] = reduced;
+          group_extent[groups++] = (uint64_t)in[0].dims[a];
+        }
+      }
+      const bool dense = is_dense(in[0]) || rp.width == 0;
+      if (dense && (groups == 0 || rp.width == 0 || (groups == 1 && group_reduced[0]) ||
+                    (groups == 2 && !group_reduced[0]))) {
+        rp.form = ReduceForm::kRows;  // "", "R", "KR"
+      } else if (dense && ((groups == 1 && !group_reduced[0]) || (groups == 2 && group_reduced[0]) ||
+                           (groups == 3 && !group_reduced[0]))) {
+        rp.form = ReduceForm::kColumns;  // "K" (nothing to fold), "RK", "KRK"
+        rp.inner = (uint32_t)group_extent[groups - 1];
+        rp.reduced = groups == 1 ? 1u : (uint32_t)group_extent[groups - 2];
+        rp.outer = groups == 3 ? (uint32_t)group_extent[0] : 1u;
+      } else {
+        rp.form = ReduceForm::kGeneral;
+        rp.rank = in[0].rank;
+        rp.axes = selected;
+        for (int a = 0; a < in[0].rank; ++a) {
+          rp.dims[a] = (uint32_t)in[0].dims[a];
+          rp.strides[a] = in[0].byte_strides[a];
+          if (in[0].dims[a] > 1 && in[0].byte_strides[a] % size != 0) rp.bytewise = true;
+        }
+        if (rp.bytewise) p->input_alignment[0] = 1;
+      }
+      reduce_plan(p->elem, &rp);
+      p->route = Route::kReduce;
+      p->dispatches = rp.dispatches;
+      p->workspace_size = rp.workspace_bytes;
+      p->workspace_alignment = rp.workspace_bytes != 0 ? 16 : 1;
       return HYLE_HIP_OK;
     }
     case HYLE_HIP_OP_TOP_K: {
@@ -969,7 +1035,16 @@ int hyle_hip_plan_alias_support(const hyle_hip_plan *plan, uint32_t output_index
 uint32_t hyle_hip_plan_dispatch_count(const hyle_hip_plan *plan) { return plan ? plan->dispatches : 0; }
 
 const char *hyle_hip_plan_route_name(const hyle_hip_plan *plan) {
-  return plan ? route_name(plan->route) : "";
+  if (plan == nullptr) return "";
+  if (plan->route == Route::kReduce) {
+    switch (plan->reduce.form) {
+      case ReduceForm::kRows: return plan->reduce.tiles > 1 ? "reduce-row-tiles" : "reduce-rows";
+      case ReduceForm::kColumns:
+        return plan->reduce.segments > 1 ? "reduce-column-segments" : "reduce-columns";
+      case ReduceForm::kGeneral: return "reduce-strided";
+    }
+  }
+  return route_name(plan->route);
 }
 
 hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *const *inputs,
@@ -1050,8 +1125,9 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
                                      stream);
       break;
     }
-    case Route::kReduceRows:
-      err = launch_reduce_rows(plan->elem, plan->reduce, inputs[0], outputs[0], vector, stream);
+    case Route::kReduce:
+      err = launch_reduce(plan->elem, plan->reduce, inputs[0], outputs[0], workspace,
+                          inputs[0] == nullptr || aligned(inputs[0], 16), stream);
       break;
     case Route::kArgmax:
       err = launch_argmax(plan->elem, plan->argmax, inputs[0], outputs[0],

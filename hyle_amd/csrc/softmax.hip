@@ -321,58 +321,6 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_general(const char *x, 
   }
 }
 
-// ---- last-axis Reduce -------------------------------------------------------------------
-enum : int { kSum = 0, kMean = 1, kMinimum = 2, kMaximum = 3 };
-
-template <int kKind> __device__ __forceinline__ float reduce_identity() {
-  return kKind == kMinimum ? INFINITY : kKind == kMaximum ? -INFINITY : 0.0f;
-}
-template <int kKind> __device__ __forceinline__ float reduce_step(float acc, float v) {
-  if constexpr (kKind == kMinimum) return min_propagate(acc, v);
-  else if constexpr (kKind == kMaximum) return max_propagate(acc, v);
-  else return acc + v;
-}
-
-template <class T, int kKind, int kLanes, bool kVector>
-__global__ __launch_bounds__(kBlockThreads) void reduce_rows(const void *x, void *y, uint32_t rows,
-                                                             uint32_t width) {
-  constexpr int kVec = Traits<T>::kVec;
-  constexpr int kRowsPerBlock = kBlockThreads / kLanes;
-  __shared__ float joint[4];
-  const uint32_t lane = threadIdx.x % kLanes;
-  const uint32_t row = blockIdx.x * kRowsPerBlock + threadIdx.x / kLanes;
-  const bool row_ok = row < rows;
-  float acc = reduce_identity<kKind>();
-  if (row_ok) {
-    if constexpr (kVector) {
-      const uint32_t vectors = width / kVec;
-      const size_t base = (size_t)row * vectors;
-      for (uint32_t vec = lane; vec < vectors; vec += kLanes) {
-        float v[kVec];
-        Traits<T>::unpack(load16_stream(x, base + vec), v);
-#pragma unroll
-        for (int j = 0; j < kVec; ++j) acc = reduce_step<kKind>(acc, v[j]);
-      }
-    } else {
-      const size_t base = (size_t)row * width;
-      for (uint32_t i = lane; i < width; i += kLanes)
-        acc = reduce_step<kKind>(acc, Traits<T>::load(x, base + i));
-    }
-  }
-  auto combine = [](LaneF32 a, LaneF32 b) { return LaneF32{reduce_step<kKind>(a.x, b.x)}; };
-  acc = group_reduce<(kLanes < kWaveLanes ? kLanes : kWaveLanes)>(LaneF32{acc}, combine).x;
-  if constexpr (kLanes > kWaveLanes) {
-    if ((threadIdx.x & (kWaveLanes - 1)) == 0) joint[threadIdx.x / kWaveLanes] = acc;
-    __syncthreads();
-    acc = reduce_step<kKind>(reduce_step<kKind>(joint[0], joint[1]),
-                             reduce_step<kKind>(joint[2], joint[3]));
-  }
-  if (row_ok && lane == 0) {
-    if constexpr (kKind == kMean) acc = width == 0 ? __builtin_nanf("") : acc / (float)width;
-    Traits<T>::store(y, row, acc);
-  }
-}
-
 // ---- host dispatch ----------------------------------------------------------------------------
 // The leading axes a mask is broadcast over: x rows r and r + period share a mask row,
 // `repeats` times.  repeats = 1 when the mask has no such axes (or there is no mask).
@@ -480,43 +428,6 @@ hipError_t run_general(const SoftmaxGeneralParams &p, const void *x, const void 
   return hipGetLastError();
 }
 
-template <class T, int kKind>
-hipError_t run_reduce_kind(const ReduceParams &p, const void *x, void *y, bool vectorised,
-                           hipStream_t s) {
-  const uint32_t rows = (uint32_t)p.shape.rows, width = p.shape.width;
-  const bool vec = vectorised && width % Traits<T>::kVec == 0;
-  const bool wide = (size_t)width * Traits<T>::kSize >= 8192;
-  if (wide) {
-    if (vec)
-      hipLaunchKernelGGL((reduce_rows<T, kKind, kBlockThreads, true>), dim3(rows),
-                         dim3(kBlockThreads), 0, s, x, y, rows, width);
-    else
-      hipLaunchKernelGGL((reduce_rows<T, kKind, kBlockThreads, false>), dim3(rows),
-                         dim3(kBlockThreads), 0, s, x, y, rows, width);
-  } else {
-    const uint32_t blocks = (rows + 3) / 4;
-    if (vec)
-      hipLaunchKernelGGL((reduce_rows<T, kKind, kWaveLanes, true>), dim3(blocks),
-                         dim3(kBlockThreads), 0, s, x, y, rows, width);
-    else
-      hipLaunchKernelGGL((reduce_rows<T, kKind, kWaveLanes, false>), dim3(blocks),
-                         dim3(kBlockThreads), 0, s, x, y, rows, width);
-  }
-  return hipGetLastError();
-}
-
-template <class T>
-hipError_t run_reduce(const ReduceParams &p, const void *x, void *y, bool vectorised,
-                      hipStream_t s) {
-  switch (p.kind) {
-    case kSum: return run_reduce_kind<T, kSum>(p, x, y, vectorised, s);
-    case kMean: return run_reduce_kind<T, kMean>(p, x, y, vectorised, s);
-    case kMinimum: return run_reduce_kind<T, kMinimum>(p, x, y, vectorised, s);
-    case kMaximum: return run_reduce_kind<T, kMaximum>(p, x, y, vectorised, s);
-  }
-  return hipErrorInvalidValue;
-}
-
 }  // namespace
 
 hipError_t launch_softmax(Elem type, const SoftmaxParams &p, const void *x, const void *mask,
@@ -538,17 +449,6 @@ hipError_t launch_softmax_general(Elem type, const SoftmaxGeneralParams &p, cons
     case Elem::kF32: return run_general<F32>(p, x, mask, y, stream);
     case Elem::kF16: return run_general<F16>(p, x, mask, y, stream);
     case Elem::kBF16: return run_general<BF16>(p, x, mask, y, stream);
-  }
-  return hipErrorInvalidValue;
-}
-
-hipError_t launch_reduce_rows(Elem type, const ReduceParams &p, const void *x, void *y,
-                              bool vectorised, hipStream_t stream) {
-  if (p.shape.rows == 0) return hipSuccess;
-  switch (type) {
-    case Elem::kF32: return run_reduce<F32>(p, x, y, vectorised, stream);
-    case Elem::kF16: return run_reduce<F16>(p, x, y, vectorised, stream);
-    case Elem::kBF16: return run_reduce<BF16>(p, x, y, vectorised, stream);
   }
   return hipErrorInvalidValue;
 }

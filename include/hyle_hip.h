@@ -1,7 +1,7 @@
 /*
  * hyle_hip.h -- C ABI of the MI355X (gfx950) compute provider for HYLE's tensor
  * hot path: broadcast Binary, Unary SiLU, GatedActivation (SwiGLU), RMSNorm,
- * row Softmax, last-axis Reduce, TopK(count = 1) and Q8_0 block dequant.
+ * row Softmax, Reduce over any set of axes, TopK(count = 1) and Q8_0 block dequant.
  *
  * The surface is what a `hyle::compute` provider for this path binds: one cold
  * "plan" per (Operation, input descriptors) pair -- the reference's
@@ -155,7 +155,7 @@ typedef struct hyle_hip_op_desc {
   uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind; Cast: output hyle_hip_dtype */
   uint32_t kind2;            /* BINARY_CHAIN: second BinaryKind; GATED: GatedInputKind;
                                 SOFTMAX: SoftmaxKind */
-  int32_t axis;              /* Softmax / TopK / Reduce axis (negative counts from the end) */
+  int32_t axis;              /* Softmax / TopK axis (negative counts from the end) */
   uint32_t mask;             /* Softmax MaskKind */
   uint32_t accumulation;     /* hyle_hip_dtype; UNKNOWN or F32 */
   uint32_t keep_dimensions;  /* Reduce */
@@ -165,6 +165,12 @@ typedef struct hyle_hip_op_desc {
   uint32_t largest;          /* TopK */
   uint32_t input_count;
   hyle_hip_tensor_desc inputs[HYLE_HIP_MAX_INPUTS];
+  /* Reduce::axes (include/hyle/compute/operation.h:232-247, 307-312): axes_count = 0 is
+   * Axes::all(); otherwise the first axes_count entries of `axes`, each possibly negative
+   * (counted from the end); a duplicate is INVALID_ARGUMENT as in the schema
+   * (src/compute_ops/operation.cc:1358-1377). */
+  uint32_t axes_count;
+  int32_t axes[HYLE_HIP_MAX_RANK];
 } hyle_hip_op_desc;
 
 typedef struct hyle_hip_context hyle_hip_context;

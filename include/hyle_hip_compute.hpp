@@ -22,6 +22,7 @@
 #include <cstring>
 #include <initializer_list>
 #include <optional>
+#include <span>
 #include <string>
 #include <utility>
 #include <variant>
@@ -44,6 +45,7 @@ public:
   static Status Ok() noexcept { return {}; }
   static Status InvalidArgument(std::string m) noexcept { return {StatusCode::InvalidArgument, std::move(m)}; }
   static Status FailedPrecondition(std::string m) noexcept { return {StatusCode::FailedPrecondition, std::move(m)}; }
+  static Status OutOfRange(std::string m) noexcept { return {StatusCode::OutOfRange, std::move(m)}; }
   static Status Unimplemented(std::string m) noexcept { return {StatusCode::Unimplemented, std::move(m)}; }
   static Status Internal(std::string m) noexcept { return {StatusCode::Internal, std::move(m)}; }
   static Status Unavailable(std::string m) noexcept { return {StatusCode::Unavailable, std::move(m)}; }
@@ -222,9 +224,36 @@ struct Copy final {};
 struct Cast final { DataType output_type = DataType::kUnknown; };
 struct Unary final { UnaryKind kind = UnaryKind::kAbs; };
 struct Binary final { BinaryKind kind = BinaryKind::kAdd; };
+// include/hyle/compute/operation.h:232-247: every axis by default, or an explicit list
+// (entries may count from the end; duplicates are refused when the output is inferred).
+class Axes final {
+public:
+  constexpr Axes() noexcept = default;
+  static Axes all() noexcept { return {}; }
+  static Result<Axes> from(std::span<const std::int32_t> axes) noexcept {
+    if (axes.empty()) return Status::InvalidArgument("explicit axis list cannot be empty");
+    if (axes.size() > HYLE_HIP_MAX_RANK) return Status::InvalidArgument("axis list exceeds kMaxTensorRank");
+    Axes result;
+    result.all_ = false;
+    result.count_ = static_cast<std::uint8_t>(axes.size());
+    for (std::size_t i = 0; i < axes.size(); ++i) {
+      if (axes[i] < -HYLE_HIP_MAX_RANK || axes[i] >= HYLE_HIP_MAX_RANK)
+        return Status::OutOfRange("axis cannot address a supported tensor rank");
+      result.values_[i] = static_cast<std::int8_t>(axes[i]);
+    }
+    return result;
+  }
+  constexpr bool is_all() const noexcept { return all_; }
+  constexpr std::span<const std::int8_t> values() const noexcept { return {values_.data(), count_}; }
+
+private:
+  std::array<std::int8_t, HYLE_HIP_MAX_RANK> values_{};
+  std::uint8_t count_ = 0;
+  bool all_ = true;
+};
 struct Reduce final {
   ReductionKind kind = ReductionKind::kSum;
-  std::int32_t axis = -1;  // the reference carries an axis list; this provider serves one axis
+  Axes axes = Axes::all();
   bool keep_dimensions = false;
   DataType accumulation_type = DataType::kUnknown;
 };
@@ -262,7 +291,9 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
     void operator()(const Unary &o) const { r.op = HYLE_HIP_OP_UNARY; r.kind = static_cast<std::uint32_t>(o.kind); }
     void operator()(const Binary &o) const { r.op = HYLE_HIP_OP_BINARY; r.kind = static_cast<std::uint32_t>(o.kind); }
     void operator()(const Reduce &o) const {
-      r.op = HYLE_HIP_OP_REDUCE; r.kind = static_cast<std::uint32_t>(o.kind); r.axis = o.axis;
+      r.op = HYLE_HIP_OP_REDUCE; r.kind = static_cast<std::uint32_t>(o.kind);
+      r.axes_count = o.axes.is_all() ? 0u : static_cast<std::uint32_t>(o.axes.values().size());
+      for (std::uint32_t i = 0; i < r.axes_count; ++i) r.axes[i] = o.axes.values()[i];
       r.keep_dimensions = o.keep_dimensions; r.accumulation = static_cast<std::uint32_t>(o.accumulation_type);
     }
     void operator()(const RmsNorm &o) const {

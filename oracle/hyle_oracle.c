@@ -634,6 +634,52 @@ void hyle_oracle_reduce_last_axis(int kind, int type, const void *src,
   }
 }
 
+/* Reduce over any set of axes of a strided tensor.  Coordinates as in
+ * src/compute_provider_cuda/reduction_kernel.cu:38-48 (the result index runs
+ * row-major over the axes that are kept, the folded index row-major over the
+ * reduced ones; byte strides, any alignment), one result per output element
+ * as in :88-113 (f32 accumulation in the order of the folded index; mean =
+ * sum / count, NaN for an empty reduction; identities 0, +inf, -inf).  The
+ * same walk is src/compute_provider_native/reduction.cc:82-111. */
+void hyle_oracle_reduce(int kind, int type, const void *src, int rank,
+                        const int64_t *dims, const int64_t *byte_strides,
+                        uint32_t axes_mask, void *dst) {
+  const unsigned char *s = (const unsigned char *)src;
+  unsigned char *d = (unsigned char *)dst;
+  const size_t w = type_size(type);
+  size_t rows = 1, width = 1;
+  for (int a = 0; a < rank; ++a) {
+    if ((axes_mask >> a) & 1u) width *= (size_t)dims[a];
+    else rows *= (size_t)dims[a];
+  }
+  for (size_t r = 0; r < rows; ++r) {
+    size_t remaining = r;
+    int64_t base = 0;
+    for (int a = rank - 1; a >= 0; --a) {
+      if ((axes_mask >> a) & 1u) continue;
+      base += (int64_t)(remaining % (size_t)dims[a]) * byte_strides[a];
+      remaining /= (size_t)dims[a];
+    }
+    const int extremum = kind == HYLE_ORACLE_MIN || kind == HYLE_ORACLE_MAX;
+    const int maximum = kind == HYLE_ORACLE_MAX;
+    float result = extremum ? (maximum ? -INFINITY : INFINITY) : 0.0f;
+    for (size_t c = 0; c < width; ++c) {
+      remaining = c;
+      int64_t offset = base;
+      for (int a = rank - 1; a >= 0; --a) {
+        if (!((axes_mask >> a) & 1u)) continue;
+        offset += (int64_t)(remaining % (size_t)dims[a]) * byte_strides[a];
+        remaining /= (size_t)dims[a];
+      }
+      const float value = load_as_f32(type, s + offset);
+      if (extremum) accumulate_extremum(maximum, value, &result);
+      else result += value;
+    }
+    if (kind == HYLE_ORACLE_MEAN) result = width == 0 ? NAN : result / (float)width;
+    store_from_f32(type, d + r * w, result);
+  }
+}
+
 /* include/hyle/simd/search.h:11-19 */
 size_t hyle_oracle_index_of_max_f32(const float *data, size_t n) {
   if (n == 0) return 0;

@@ -200,6 +200,15 @@ void hyle_oracle_softmax(int type, const void *src, void *dst,
 void hyle_oracle_reduce_last_axis(int kind, int type, const void *src,
                                   void *dst, size_t rows, size_t width);
 
+/* Reduce over the axes in `axes_mask` (bit a = axis a) of a tensor given by
+ * dims and BYTE strides of any alignment; `dst` is the dense result, one
+ * element per combination of the kept axes in row-major order
+ * (src/compute_provider_cuda/reduction_kernel.cu:38-48, 88-113;
+ * src/compute_provider_native/reduction.cc:82-111). */
+void hyle_oracle_reduce(int kind, int type, const void *src, int rank,
+                        const int64_t *dims, const int64_t *byte_strides,
+                        uint32_t axes_mask, void *dst);
+
 /* include/hyle/simd/search.h:11-19: first index of the maximum; first NaN
  * index when any NaN is present; n for an empty range. */
 size_t hyle_oracle_index_of_max_f32(const float *data, size_t n);

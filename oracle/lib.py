@@ -81,6 +81,7 @@ _iom = _sig("hyle_oracle_index_of_max_f32", _sz, _vp, _sz)
 _topk1 = _sig("hyle_oracle_topk1_f32", None, _vp, _sz, _sz, _vp, _vp)
 _q8_bf16 = _sig("hyle_oracle_q8_0_dequant_bf16", None, _vp, _sz, _sz, _sz, _vp, _vp, _vp)
 _q8_f32 = _sig("hyle_oracle_q8_0_dequant_f32", None, _vp, _sz, _sz, _sz, _vp)
+_reduce_axes = _sig("hyle_oracle_reduce", None, C.c_int, C.c_int, _vp, C.c_int, _i64p, _i64p, C.c_uint32, _vp)
 _cast = _sig("hyle_oracle_cast", C.c_int, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int, _vp)
 
 
@@ -317,6 +318,26 @@ def reduce_last_axis(kind, type_id, src):
     rows = int(np.prod(src.shape[:-1], dtype=np.int64))
     out = np.empty(src.shape[:-1], _NP[type_id])
     _reduce(kind, type_id, _ptr(src), _ptr(out), rows, width)
+    return out
+
+
+def reduce(kind, type_id, storage, dims, axes=None, byte_strides=None, keep_dimensions=False):
+    """Reduce the axes `axes` (None = all; entries may be negative) of the plain tensor held in
+    `storage` (read as bytes) with logical `dims` and `byte_strides` (dense when omitted)."""
+    dims = [int(d) for d in dims]
+    rank = len(dims)
+    if byte_strides is None:
+        byte_strides = _byte_strides(dims, np.dtype(_NP[type_id]).itemsize)
+    selected = range(rank) if axes is None else [a + rank if a < 0 else a for a in axes]
+    mask = 0
+    for a in selected:
+        mask |= 1 << a
+    shape = [1 if (mask >> a) & 1 else dims[a] for a in range(rank)]
+    if not keep_dimensions:
+        shape = [dims[a] for a in range(rank) if not (mask >> a) & 1]
+    raw = np.ascontiguousarray(storage).view(np.uint8).reshape(-1)
+    out = np.empty(shape, _NP[type_id])
+    _reduce_axes(kind, type_id, _ptr(raw), rank, _i64(dims), _i64(byte_strides), mask, _ptr(out))
     return out
 
 

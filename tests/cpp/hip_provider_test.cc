@@ -77,7 +77,7 @@ HOST_TEST(InfersOutputsLikeTheSchema) {
   REQUIRE(out.has_value());
   EXPECT((*out)[0] == dense(DataType::kBFloat16, {9, 32}));
   EXPECT(infer_output_descriptions(GatedActivation{}, {dense(DataType::kBFloat16, {9, 63})}).error().IsInvalidArgument());
-  out = infer_output_descriptions(Reduce{ReductionKind::kMaximum, -1, true}, {dense(DataType::kFloat32, {3, 9})});
+  out = infer_output_descriptions(Reduce{ReductionKind::kMaximum, *Axes::from(std::array<std::int32_t, 1>{-1}), true}, {dense(DataType::kFloat32, {3, 9})});
   REQUIRE(out.has_value());
   EXPECT((*out)[0] == dense(DataType::kFloat32, {3, 1}));
   out = infer_output_descriptions(Q8_0DequantSumSquares{}, {*TensorDesc::gguf_q8_0_weight(DataType::kBFloat16, 64, 5)});

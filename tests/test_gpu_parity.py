@@ -466,7 +466,7 @@ def test_reduce_last_axis_row_max_and_sum(tag):
         xs = host_values(x, tag)
         for kind, okind in kinds.items():
             note(f"reduce {tag} {kind.name} [{rows},{width}]")
-            (out,) = run(hc.Reduce(kind, axis=-1, accumulation_type=hc.DataType.kFloat32), to_device(xs, tag))
+            (out,) = run(hc.Reduce(kind, hc.Axes.from_([-1]), accumulation_type=hc.DataType.kFloat32), to_device(xs, tag))
             want = orc.reduce_last_axis(okind, oid, xs)
             got = to_host(out)
             if kind in (hc.ReductionKind.kMaximum, hc.ReductionKind.kMinimum):

@@ -154,9 +154,9 @@ def test_infer_softmax_reduce_topk_rules():
         hc.infer_output_descriptions(hc.Softmax(scale=float("inf")), [s])
     with pytest.raises(hc.StatusError):  # mask supplied for a no-mask operation is an arity error
         hc.infer_output_descriptions(hc.Softmax(), [s, D(DT.kBool, [64, 64])])
-    r = hc.Reduce(hc.ReductionKind.kMaximum, axis=-1)
+    r = hc.Reduce(hc.ReductionKind.kMaximum, hc.Axes.from_([-1]))
     assert hc.infer_output_descriptions(r, [s]) == [D(DT.kFloat32, [32, 64])]
-    keep = hc.Reduce(hc.ReductionKind.kSum, axis=-1, keep_dimensions=True)
+    keep = hc.Reduce(hc.ReductionKind.kSum, hc.Axes.from_([-1]), keep_dimensions=True)
     assert hc.infer_output_descriptions(keep, [s]) == [D(DT.kFloat32, [32, 64, 1])]
     logits = D(DT.kFloat32, [64, 151936])
     values, indices = hc.infer_output_descriptions(hc.TopK(), [logits])
@@ -225,7 +225,7 @@ def test_declines_are_unimplemented_and_errors_are_not():
         lambda: hc.prepare(CTX, hc.Unary(hc.UnaryKind.kAbs), D(DT.kInt32, [4])),   # integer Unary
         lambda: hc.prepare(CTX, hc.RmsNorm(accumulation_type=DT.kBFloat16), x),
         lambda: hc.prepare(CTX, hc.Softmax(accumulation_type=DT.kUnknown), x),   # half needs explicit f32
-        lambda: hc.prepare(CTX, hc.Reduce(hc.ReductionKind.kSum, axis=0, accumulation_type=DT.kFloat32), x),
+        lambda: hc.prepare(CTX, hc.Reduce(hc.ReductionKind.kSum, hc.Axes.from_([0])), x),   # half needs explicit f32
         lambda: hc.prepare(CTX, hc.TopK(count=2), x),
         lambda: hc.prepare(CTX, hc.TopK(largest=False), x),
         lambda: hc.prepare(CTX, hc.Binary(), D(DT.kInt32, [4]), D(DT.kInt32, [4])),
