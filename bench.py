@@ -256,6 +256,13 @@ def main() -> int:
                                       accumulation_type=F32),
                       [D(dtype, dims)], set_reduce, sets, dims[0] * dims[1] * size + out_bytes, dims[0] * dims[1],
                       "f32" if dtype == F32 else "bf16", in_step=False))
+    if want("next_topk64_f32"):
+        def set_topk(i):
+            logits = torch.empty((64, 151936), dtype=torch.float32, device=dev).normal_()
+            return [logits], [torch.empty((64, 64), dtype=torch.float32, device=dev),
+                              torch.empty((64, 64), dtype=torch.int32, device=dev)]
+        ops.append(Op("next_topk64_f32", hc.TopK(count=64), [D(F32, [64, 151936])], set_topk, 14,
+                      64 * 151936 * 4 + 64 * 64 * 8, 64 * 151936, "f32", in_step=False))
     if want("next_copy_bf16"):
         def set_copy(i):
             src = torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev).normal_()

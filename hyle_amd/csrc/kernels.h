@@ -147,6 +147,27 @@ size_t argmax_workspace_bytes(const ArgmaxParams &p);
 hipError_t launch_argmax(Elem type, const ArgmaxParams &p, const void *x, void *values,
                          int32_t *indices, void *workspace, bool vectorised, hipStream_t stream);
 
+// TopK(count = k) along any axis of a plain tensor: sorted tiles, then merges of k-key lists
+// through the workspace.
+struct TopKParams {
+  uint32_t rows = 0, width = 0, count = 0, inner = 1;
+  bool largest = true;
+  bool dense_last = false;  // dense tensor, axis innermost
+  bool bytewise = false;    // strides that are not multiples of the element size
+  int32_t rank = 0, axis = 0;
+  uint32_t dims[kMaxRank] = {};
+  int64_t strides[kMaxRank] = {};
+  // set by topk_plan
+  bool select = false;           // count small enough for the register-resident selection
+  uint32_t tile_elements = 0;    // elements of a row one block of the first dispatch takes
+  uint32_t tiles = 1, fan = 2, dispatches = 1;
+  size_t workspace_bytes = 0;
+};
+uint32_t topk_max_count();
+void topk_plan(TopKParams *p);
+hipError_t launch_topk(Elem type, const TopKParams &p, const void *x, void *values, int32_t *indices,
+                       void *workspace, bool input_vector_aligned, hipStream_t stream);
+
 // Q8_0 rows of k/32 blocks {f16 d; int8 qs[32]} -> bf16 [rows, k] + f32 sumsq[rows].
 struct Q8Params {
   uint64_t rows = 0;

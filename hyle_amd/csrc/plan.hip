@@ -454,6 +454,7 @@ enum class Route : uint8_t {
   kSoftmax,
   kReduce,
   kArgmax,
+  kTopK,
   kQ8Dequant,
   kCast,
 };
@@ -468,6 +469,7 @@ const char *route_name(Route r) {
     case Route::kSoftmax: return "softmax-rows";
     case Route::kReduce: return "reduce";
     case Route::kArgmax: return "argmax-tiles";
+    case Route::kTopK: return "topk-sorted-tiles";
     case Route::kQ8Dequant: return "q8_0-dequant-rows";
     case Route::kCast: return "cast-copy";
   }
@@ -508,6 +510,7 @@ struct hyle_hip_plan {
   bool softmax_mask_vector_ok = false;
   ReduceParams reduce;
   ArgmaxParams argmax;
+  TopKParams topk;
   Q8Params q8;
   CastParams cast;
   // Cast and Copy take no alias at all (AliasPolicy::kNone, src/compute_ops/operation.cc:935-957):
@@ -809,22 +812,51 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       return HYLE_HIP_OK;
     }
     case HYLE_HIP_OP_TOP_K: {
-      if (r.count != 1 || !r.largest)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK serves count = 1, largest only");
-      if (!to_elem(in[0].dtype, &p->elem) || !is_dense(in[0]))
-        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK requires dense plain float32/float16/bfloat16");
+      // include/hyle/compute/providers/cuda.h:113-117: plain rank <= 8 byte strides, dense
+      // outputs, no aliases, caller-owned workspace.
+      if (!to_elem(in[0].dtype, &p->elem) || !is_plain(in[0]))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK requires plain float32/float16/bfloat16");
       int axis;
       if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
-      if (axis != in[0].rank - 1)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK serves the last axis only");
       if (p->input_elements[0] > kMaxElements)
         return fail(HYLE_HIP_UNIMPLEMENTED, "TopK requires at most INT32_MAX elements");
       if (p->output_elements[0] == 0) return HYLE_HIP_OK;
-      p->route = Route::kArgmax;
-      argmax_plan(p->output_elements[0], (uint32_t)in[0].dims[axis], p->elem, &p->argmax);
-      p->workspace_size = argmax_workspace_bytes(p->argmax);
-      p->workspace_alignment = 16;
-      p->dispatches = 2;
+      bool innermost = is_dense(in[0]);  // dense, and nothing but extent-1 axes after the axis
+      for (int a = axis + 1; a < in[0].rank; ++a)
+        if (in[0].dims[a] != 1) innermost = false;
+      if (r.count == 1 && r.largest && innermost) {
+        // the vocabulary argmax: a scan dispatch and a fold dispatch
+        p->route = Route::kArgmax;
+        argmax_plan(p->output_elements[0], (uint32_t)in[0].dims[axis], p->elem, &p->argmax);
+        p->workspace_size = argmax_workspace_bytes(p->argmax);
+        p->workspace_alignment = 16;
+        p->dispatches = 2;
+        return HYLE_HIP_OK;
+      }
+      if (r.count > topk_max_count())
+        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK serves count <= %u", topk_max_count());
+      TopKParams &t = p->topk;
+      t = TopKParams{};
+      t.count = (uint32_t)r.count;
+      t.rows = (uint32_t)(p->output_elements[0] / r.count);
+      t.width = (uint32_t)in[0].dims[axis];
+      t.largest = r.largest != 0;
+      t.dense_last = innermost;
+      t.rank = in[0].rank;
+      t.axis = axis;
+      const int64_t size = (int64_t)dtype_size(in[0].dtype);
+      for (int a = 0; a < in[0].rank; ++a) {
+        t.dims[a] = (uint32_t)in[0].dims[a];
+        t.strides[a] = in[0].byte_strides[a];
+        if (a > axis) t.inner *= (uint32_t)in[0].dims[a];
+        if (in[0].dims[a] > 1 && in[0].byte_strides[a] % size != 0) t.bytewise = true;
+      }
+      if (t.bytewise) p->input_alignment[0] = 1;
+      topk_plan(&t);
+      p->route = Route::kTopK;
+      p->dispatches = t.dispatches;
+      p->workspace_size = t.workspace_bytes;
+      p->workspace_alignment = t.workspace_bytes != 0 ? 16 : 1;
       return HYLE_HIP_OK;
     }
     case HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ: {
@@ -1044,6 +1076,7 @@ const char *hyle_hip_plan_route_name(const hyle_hip_plan *plan) {
       case ReduceForm::kGeneral: return "reduce-strided";
     }
   }
+  if (plan->route == Route::kTopK && plan->topk.select) return "topk-select-tiles";
   return route_name(plan->route);
 }
 
@@ -1132,6 +1165,10 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
     case Route::kArgmax:
       err = launch_argmax(plan->elem, plan->argmax, inputs[0], outputs[0],
                           static_cast<int32_t *>(outputs[1]), workspace, aligned(inputs[0], 16), stream);
+      break;
+    case Route::kTopK:
+      err = launch_topk(plan->elem, plan->topk, inputs[0], outputs[0], static_cast<int32_t *>(outputs[1]),
+                        workspace, aligned(inputs[0], 16), stream);
       break;
     case Route::kQ8Dequant:
       err = launch_q8_0_dequant(plan->q8, inputs[0], outputs[0], static_cast<float *>(outputs[1]),

@@ -715,6 +715,64 @@ void hyle_oracle_topk1_f32(const float *data, size_t rows, size_t width,
   }
 }
 
+/* TopK(count = k) along one axis of a plain strided tensor.  The order is the
+ * reference's independent host ordering
+ * (tests/compute_route_vulkan/topk_test_support.h:62-76): a stable sort in which
+ * numbers precede NaNs, larger numbers come first (smaller when `largest` is 0),
+ * and equal numbers (-0 == +0) as well as NaNs keep their index order.  Values
+ * are copies of the source bits (include/hyle/compute/providers/cuda.h:113-116).
+ * Outputs are dense with the axis extent replaced by k
+ * (src/compute_ops/operation.cc:1622-1657). */
+typedef struct {
+  float value;
+  int32_t index;
+} topk_item;
+static int g_topk_largest;
+static int topk_before(const void *pa, const void *pb) {
+  const topk_item *a = (const topk_item *)pa, *b = (const topk_item *)pb;
+  const int a_nan = isnan(a->value), b_nan = isnan(b->value);
+  if (a_nan != b_nan) return a_nan ? 1 : -1;
+  if (!a_nan && a->value != b->value) {
+    const int a_first = g_topk_largest ? a->value > b->value : a->value < b->value;
+    return a_first ? -1 : 1;
+  }
+  return a->index < b->index ? -1 : (a->index > b->index ? 1 : 0);
+}
+void hyle_oracle_topk(int type, const void *src, int rank, const int64_t *dims,
+                      const int64_t *byte_strides, int axis, size_t k, int largest,
+                      void *values, int32_t *indices) {
+  const unsigned char *s = (const unsigned char *)src;
+  unsigned char *v = (unsigned char *)values;
+  const size_t w = type_size(type);
+  const size_t width = (size_t)dims[axis];
+  size_t outer = 1, inner = 1;
+  for (int a = 0; a < axis; ++a) outer *= (size_t)dims[a];
+  for (int a = axis + 1; a < rank; ++a) inner *= (size_t)dims[a];
+  topk_item *items = (topk_item *)malloc((width ? width : 1) * sizeof(topk_item));
+  g_topk_largest = largest;
+  for (size_t row = 0; row < outer * inner; ++row) {
+    size_t remaining = row;
+    int64_t base = 0;
+    for (int a = rank - 1; a >= 0; --a) {
+      if (a == axis) continue;
+      base += (int64_t)(remaining % (size_t)dims[a]) * byte_strides[a];
+      remaining /= (size_t)dims[a];
+    }
+    for (size_t i = 0; i < width; ++i) {
+      items[i].value = load_as_f32(type, s + base + (int64_t)i * byte_strides[axis]);
+      items[i].index = (int32_t)i;
+    }
+    qsort(items, width, sizeof(topk_item), topk_before);  /* a total order: index breaks ties */
+    const size_t o = row / inner, lane = row % inner;
+    for (size_t j = 0; j < k; ++j) {
+      const size_t out = (o * k + j) * inner + lane;
+      memcpy(v + out * w, s + base + (int64_t)items[j].index * byte_strides[axis], w);
+      indices[out] = items[j].index;
+    }
+  }
+  free(items);
+}
+
 /* ------------------------------------------------------------------------ */
 /* Q8_0                                                                     */
 /* ------------------------------------------------------------------------ */

@@ -209,6 +209,16 @@ void hyle_oracle_reduce(int kind, int type, const void *src, int rank,
                         const int64_t *dims, const int64_t *byte_strides,
                         uint32_t axes_mask, void *dst);
 
+/* TopK(count = k) along `axis` of a tensor given by dims and BYTE strides:
+ * numbers before NaNs, larger first (smaller first when largest == 0), equal
+ * numbers and NaNs in index order; `values` holds copies of the source bits,
+ * `indices` positions along the axis; both dense with the axis extent k
+ * (tests/compute_route_vulkan/topk_test_support.h:62-76;
+ * src/compute_ops/operation.cc:1622-1657). */
+void hyle_oracle_topk(int type, const void *src, int rank, const int64_t *dims,
+                      const int64_t *byte_strides, int axis, size_t k, int largest,
+                      void *values, int32_t *indices);
+
 /* include/hyle/simd/search.h:11-19: first index of the maximum; first NaN
  * index when any NaN is present; n for an empty range. */
 size_t hyle_oracle_index_of_max_f32(const float *data, size_t n);

@@ -82,6 +82,7 @@ _topk1 = _sig("hyle_oracle_topk1_f32", None, _vp, _sz, _sz, _vp, _vp)
 _q8_bf16 = _sig("hyle_oracle_q8_0_dequant_bf16", None, _vp, _sz, _sz, _sz, _vp, _vp, _vp)
 _q8_f32 = _sig("hyle_oracle_q8_0_dequant_f32", None, _vp, _sz, _sz, _sz, _vp)
 _reduce_axes = _sig("hyle_oracle_reduce", None, C.c_int, C.c_int, _vp, C.c_int, _i64p, _i64p, C.c_uint32, _vp)
+_topk = _sig("hyle_oracle_topk", None, C.c_int, _vp, C.c_int, _i64p, _i64p, C.c_int, _sz, C.c_int, _vp, _vp)
 _cast = _sig("hyle_oracle_cast", C.c_int, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int, _vp)
 
 
@@ -353,6 +354,22 @@ def topk1(data):
     values = np.empty(data.shape[:-1], np.float32)
     indices = np.empty(data.shape[:-1], np.int32)
     _topk1(_ptr(data), rows, width, _ptr(values), _ptr(indices))
+    return values, indices
+
+
+def topk(type_id, storage, dims, count, axis=-1, largest=True, byte_strides=None):
+    """TopK(count) along `axis` of the plain tensor held in `storage` (read as bytes) with logical
+    `dims` and `byte_strides` (dense when omitted): (values as stored bits, int32 indices)."""
+    dims = [int(d) for d in dims]
+    axis = axis + len(dims) if axis < 0 else axis
+    if byte_strides is None:
+        byte_strides = _byte_strides(dims, np.dtype(_NP[type_id]).itemsize)
+    shape = list(dims)
+    shape[axis] = int(count)
+    raw = np.ascontiguousarray(storage).view(np.uint8).reshape(-1)
+    values, indices = np.empty(shape, _NP[type_id]), np.empty(shape, np.int32)
+    _topk(type_id, _ptr(raw), len(dims), _i64(dims), _i64(byte_strides), axis, int(count), int(bool(largest)),
+          _ptr(values), _ptr(indices))
     return values, indices
 
 
