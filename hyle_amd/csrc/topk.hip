@@ -114,7 +114,9 @@ __device__ __forceinline__ void emit(const uint64_t *keys, const Addressing &a, 
     const int64_t step = a.dense_last ? kSize : a.strides[a.axis];
     const uint32_t outer = row / a.inner, position = row - outer * a.inner;
     for (uint32_t j = threadIdx.x; j < a.count; j += kBlockThreads) {
-      const uint32_t index = ~(uint32_t)keys[j];
+      // a list always holds `count` elements of the row here; the clamp only keeps a corrupted
+      // workspace from turning into a wild address
+      const uint32_t index = min(~(uint32_t)keys[j], a.width - 1);
       const uint32_t bits = load_bits<T, kBytewise>(x + base + (int64_t)index * step);
       const size_t out = ((size_t)outer * a.count + j) * a.inner + position;
       if constexpr (kSize == 4) static_cast<uint32_t *>(values)[out] = bits;
@@ -209,8 +211,18 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t *w
   return before + inclusive - v;
 }
 
+// The ordered half of a key alone: enough for nearly every comparison of the select kernel.
+__device__ __forceinline__ uint32_t ordered_value(float v, bool largest) {
+  if (v != v) return 0;
+  const uint32_t bits = v == 0.0f ? 0u : f32_bits(v);
+  const uint32_t ordered = bits ^ ((uint32_t)((int32_t)bits >> 31) | 0x80000000u);
+  return largest ? ordered : ~ordered;
+}
+
 // One block per (row, unit).  kFromLists = false: unit = a tile of 256 * kE elements of the row.
 // kFromLists = true: unit = a group of `fan` lists of `count` keys left by an earlier dispatch.
+// A thread keeps its kE keys as two words, hi (ordered value) and lo (~index; the compiler
+// recomputes it from the slot number for elements); an empty slot is hi = lo = 0.
 template <class T, int kE, bool kFromLists, bool kVector, bool kBytewise, bool kFinal>
 __global__ __launch_bounds__(kBlockThreads) void topk_select(const char *x, void *values, int32_t *indices,
                                                              const uint64_t *in_lists, uint64_t *out_lists,
@@ -218,10 +230,10 @@ __global__ __launch_bounds__(kBlockThreads) void topk_select(const char *x, void
                                                              uint32_t units_out, uint32_t largest) {
   constexpr int kSize = Traits<T>::kSize;
   constexpr int kVec = Traits<T>::kVec;
-  __shared__ uint64_t keys[kTile];
+  __shared__ uint64_t keys[kTile];  // kBlockThreads < kTile / 2: keys[kBlockThreads] is free for the bound
   __shared__ uint32_t wave_totals[kBlockThreads / kWaveLanes];
   const uint32_t row = blockIdx.x / units_out, unit = blockIdx.x - row * units_out;
-  uint64_t mine[kE];
+  uint32_t hi[kE], lo[kE];
   if constexpr (kFromLists) {
     const uint32_t first_list = unit * fan;
     const uint32_t taken = min(fan, units_in - first_list) * a.count;
@@ -229,68 +241,153 @@ __global__ __launch_bounds__(kBlockThreads) void topk_select(const char *x, void
 #pragma unroll
     for (int j = 0; j < kE; ++j) {
       const uint32_t i = threadIdx.x + j * kBlockThreads;
-      mine[j] = i < taken ? source[i] : 0;
+      const uint64_t key = source[min(i, taken - 1)];  // an unconditional load, clamped
+      hi[j] = i < taken ? (uint32_t)(key >> 32) : 0;
+      lo[j] = i < taken ? (uint32_t)key : 0;
     }
   } else {
     const uint32_t first = unit * (kBlockThreads * kE);
     const int64_t base = row_base(a, row, kSize);
     if constexpr (kVector) {
       static_assert(kE % kVec == 0, "whole vectors per thread");
+      // Every load is issued before the first key is made: addresses past the row's end are
+      // clamped to its last vector (a load inside a branch would wait for itself there).
       const u32x4 *vectors = reinterpret_cast<const u32x4 *>(x + base);
+      const uint32_t last_vector = a.width / kVec - 1;
+      u32x4 raw[kE / kVec];
+#pragma unroll
+      for (int v = 0; v < kE / kVec; ++v) {
+        const uint32_t vector = first / kVec + threadIdx.x + v * kBlockThreads;
+        raw[v] = __builtin_nontemporal_load(vectors + min(vector, last_vector));
+      }
 #pragma unroll
       for (int v = 0; v < kE / kVec; ++v) {
         const uint32_t element = first + (threadIdx.x + v * kBlockThreads) * kVec;
-        if (element < a.width) {
-          float f[kVec];
-          Traits<T>::unpack(__builtin_nontemporal_load(vectors + element / kVec), f);
+        const bool inside = element < a.width;
+        float f[kVec];
+        Traits<T>::unpack(raw[v], f);
 #pragma unroll
-          for (int j = 0; j < kVec; ++j) mine[v * kVec + j] = make_key(f[j], element + j, largest != 0);
-        } else {
-#pragma unroll
-          for (int j = 0; j < kVec; ++j) mine[v * kVec + j] = 0;
+        for (int j = 0; j < kVec; ++j) {
+          hi[v * kVec + j] = inside ? ordered_value(f[j], largest != 0) : 0;
+          lo[v * kVec + j] = inside ? ~(element + j) : 0;
         }
       }
     } else {
       const int64_t step = a.dense_last ? kSize : a.strides[a.axis];
+      const uint32_t last = a.width - 1;
+      uint32_t bits[kE];
 #pragma unroll
       for (int j = 0; j < kE; ++j) {
         const uint32_t element = first + threadIdx.x + j * kBlockThreads;
-        mine[j] = element < a.width
-                      ? make_key(bits_value<T>(load_bits<T, kBytewise>(x + base + (int64_t)element * step)),
-                                 element, largest != 0)
-                      : 0;
+        bits[j] = load_bits<T, kBytewise>(x + base + (int64_t)min(element, last) * step);
+      }
+#pragma unroll
+      for (int j = 0; j < kE; ++j) {
+        const uint32_t element = first + threadIdx.x + j * kBlockThreads;
+        const bool inside = element < a.width;
+        hi[j] = inside ? ordered_value(bits_value<T>(bits[j]), largest != 0) : 0;
+        lo[j] = inside ? ~element : 0;
       }
     }
   }
-  // A lower bound of the count-th largest key: the count-th largest of the thread maxima.
-  uint64_t best = 0;
+  auto key_of = [&](int j) { return ((uint64_t)hi[j] << 32) | lo[j]; };
+
+  // A lower bound of the count-th largest ordered value: the count-th largest of the 256 thread
+  // maxima (at least `count` keys reach it).  Each wave sorts its 64 maxima in registers (bitonic
+  // network over lane exchanges), the four sorted runs meet in LDS, and every thread finds the
+  // rank of its maximum among all 256 with three binary searches; ties rank by wave, so exactly
+  // one thread has rank count - 1.  Everything whose ordered value reaches that bound is a
+  // candidate: one 32-bit comparison per key.  A bound of 0 (fewer than `count` threads hold a
+  // number) makes every key a candidate.
+  uint32_t *maxima = reinterpret_cast<uint32_t *>(keys);
+  uint32_t best = 0;
 #pragma unroll
-  for (int j = 0; j < kE; ++j) best = mine[j] > best ? mine[j] : best;
-  keys[threadIdx.x] = best;
-  sort_descending(keys, kBlockThreads);
-  uint64_t bound = keys[a.count - 1];
-  if (bound == 0) bound = 1;  // fewer than `count` threads hold an element: take every element
+  for (int j = 0; j < kE; ++j) best = max(best, hi[j]);
+  const uint32_t lane = threadIdx.x % kWaveLanes, wave = threadIdx.x / kWaveLanes;
+#pragma unroll
+  for (uint32_t size = 2; size <= kWaveLanes; size <<= 1) {
+#pragma unroll
+    for (uint32_t stride = size >> 1; stride > 0; stride >>= 1) {
+      const uint32_t other = __shfl_xor(best, stride, kWaveLanes);
+      const bool descending = (lane & size) == 0;       // direction of this lane's run
+      const bool lower_lane = (lane & stride) == 0;     // the lane that keeps the run's front value
+      best = (lower_lane == descending) ? max(best, other) : min(best, other);
+    }
+  }
+  maxima[threadIdx.x] = best;  // four descending runs of 64
+  __syncthreads();
+  {
+    uint32_t rank = lane;  // larger values of the own run come first
+#pragma unroll
+    for (uint32_t w = 0; w < kBlockThreads / kWaveLanes; ++w) {
+      if (w == wave) continue;
+      // values of run w that precede `best`: strictly larger ones, and equal ones of earlier waves
+      const uint32_t *run = maxima + w * kWaveLanes;
+      uint32_t low = 0, high = kWaveLanes;  // first position whose value does not precede
+      while (low < high) {
+        const uint32_t mid = (low + high) >> 1;
+        const uint32_t value = run[mid];
+        const bool precedes = value > best || (value == best && w < wave);
+        if (precedes) low = mid + 1;
+        else high = mid;
+      }
+      rank += low;
+    }
+    if (rank == a.count - 1) maxima[kBlockThreads] = best;
+  }
+  __syncthreads();
+  const uint32_t bound_hi = maxima[kBlockThreads];
   __syncthreads();
   uint32_t reach = 0, total;
+  if (bound_hi != 0) {
 #pragma unroll
-  for (int j = 0; j < kE; ++j) reach += mine[j] >= bound ? 1u : 0u;
+    for (int j = 0; j < kE; ++j) reach += hi[j] >= bound_hi ? 1u : 0u;
+  } else {
+#pragma unroll
+    for (int j = 0; j < kE; ++j) reach += (hi[j] | lo[j]) != 0 ? 1u : 0u;
+  }
   uint32_t position = block_exclusive_scan(reach, wave_totals, &total);
+  uint64_t exact = 0;  // nonzero: candidates are the keys >= exact instead
   if (total > kTile) {
     // The exact count-th largest key, one bit at a time: the largest t with >= count keys >= t.
-    uint64_t exact = 0;
     for (int bit = 63; bit >= 0; --bit) {
       const uint64_t trial = exact | (1ull << bit);
       uint32_t at_least = 0, sum;
 #pragma unroll
-      for (int j = 0; j < kE; ++j) at_least += mine[j] >= trial ? 1u : 0u;
+      for (int j = 0; j < kE; ++j) at_least += key_of(j) >= trial ? 1u : 0u;
       block_exclusive_scan(at_least, wave_totals, &sum);
       if (sum >= a.count) exact = trial;
     }
-    bound = exact != 0 ? exact : 1;
+    if (exact == 0) exact = 1;
     reach = 0;
 #pragma unroll
-    for (int j = 0; j < kE; ++j) reach += mine[j] >= bound ? 1u : 0u;
+    for (int j = 0; j < kE; ++j) reach += key_of(j) >= exact ? 1u : 0u;
     position = block_exclusive_scan(reach, wave_totals, &total);  // total == count: keys are unique
+  }
+  auto candidate = [&](int j) {
+    if (exact != 0) return key_of(j) >= exact;
+    return bound_hi != 0 ? hi[j] >= bound_hi : (hi[j] | lo[j]) != 0;
+  };
+  constexpr uint32_t kRanked = kTile / 2;  // candidates in keys[0, kRanked), ranked output above
+  if (total <= kRanked / 2) {
+    // Few candidates (the usual case): place each by counting the candidates above it.
+    for (uint32_t i = threadIdx.x; i < a.count; i += kBlockThreads) keys[kRanked + i] = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kE; ++j)
+      if (candidate(j)) keys[position++] = key_of(j);
+    __syncthreads();
+    for (uint32_t i = threadIdx.x; i < total; i += kBlockThreads) {
+      const uint64_t key = keys[i];
+      uint32_t above = 0;
+#pragma unroll 8
+      for (uint32_t other = 0; other < total; ++other) above += keys[other] > key ? 1u : 0u;
+      if (above < a.count) keys[kRanked + above] = key;
+    }
+    __syncthreads();
+    emit<T, kBytewise, kFinal>(keys + kRanked, a, row, x, values, indices,
+                               out_lists + ((size_t)row * units_out + unit) * a.count);
+    return;
   }
   uint32_t sort_n = 64;
   while (sort_n < kTile && (sort_n < total || sort_n < a.count)) sort_n <<= 1;
@@ -298,7 +395,7 @@ __global__ __launch_bounds__(kBlockThreads) void topk_select(const char *x, void
   __syncthreads();
 #pragma unroll
   for (int j = 0; j < kE; ++j)
-    if (mine[j] >= bound && position < kTile) keys[position++] = mine[j];  // the guard never binds
+    if (candidate(j) && position < kTile) keys[position++] = key_of(j);  // the guard never binds
   sort_descending(keys, sort_n);
   emit<T, kBytewise, kFinal>(keys, a, row, x, values, indices,
                              out_lists + ((size_t)row * units_out + unit) * a.count);
@@ -364,7 +461,9 @@ hipError_t run(const TopKParams &p, const void *x, void *values, int32_t *indice
   const dim3 block(kBlockThreads);
   vector = vector && p.dense_last && p.width % Traits<T>::kVec == 0;
   if (p.select) {
-    if (p.tile_elements == kBlockThreads * 32)
+    if (p.tile_elements == kBlockThreads * 64)
+      select_tiles_launch<T, 64, kBytewise>(p, a, in, values, indices, lists_a, vector, s);
+    else if (p.tile_elements == kBlockThreads * 32)
       select_tiles_launch<T, 32, kBytewise>(p, a, in, values, indices, lists_a, vector, s);
     else
       select_tiles_launch<T, 8, kBytewise>(p, a, in, values, indices, lists_a, vector, s);
@@ -420,9 +519,11 @@ uint32_t topk_max_count() { return kTile / 2; }
 void topk_plan(TopKParams *p) {
   p->select = p->count <= kSelectMax;
   if (p->select) {
-    // 8192-element tiles for long rows (32 keys per thread), 2048 otherwise; merges take as many
+    // 16384- or 8192-element tiles for long rows (64 or 32 keys per thread: the per-block work of
+    // finding the bound is paid once per tile), 2048 otherwise; merges take as many
     // lists as 8192 keys hold (2048 when that already covers every tile of a row).
-    p->tile_elements = p->width > kTile ? kBlockThreads * 32 : kBlockThreads * 8;
+    p->tile_elements = p->width > 8 * kTile ? kBlockThreads * 64
+                                            : (p->width > kTile ? kBlockThreads * 32 : kBlockThreads * 8);
     p->tiles = (p->width + p->tile_elements - 1) / p->tile_elements;
     p->fan = (p->tiles * p->count <= kBlockThreads * 8 ? kBlockThreads * 8 : kBlockThreads * 32) / p->count;
   } else {

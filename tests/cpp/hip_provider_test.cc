@@ -101,7 +101,14 @@ HOST_TEST(PreparesRoutesAndDeclinesCleanly) {
   EXPECT(top->dispatch_count() == 2 && top->workspace_requirement().size > 0);
   EXPECT(top->create_invocation().error().IsInvalidArgument());  // needs its workspace
   // Declines are Unimplemented, never an error a router would have to surface.
-  EXPECT(prepare(context, TopK{.count = 4}, dense(DataType::kFloat32, {8, 128})).error().IsUnimplemented());
+  auto top4 = prepare(context, TopK{.count = 4}, dense(DataType::kFloat32, {8, 128}));
+  REQUIRE(top4.has_value());
+  EXPECT(std::string(top4->route_name()) == "topk-select-tiles" && top4->workspace_requirement().size == 0);
+  EXPECT(prepare(context, TopK{.count = 1025}, dense(DataType::kFloat32, {8, 4096})).error().IsUnimplemented());
+  auto folded = prepare(context, Reduce{ReductionKind::kSum, *Axes::from(std::array<std::int32_t, 2>{0, 2})},
+                        dense(DataType::kFloat32, {4, 5, 6}));
+  REQUIRE(folded.has_value());
+  EXPECT(std::string(folded->route_name()) == "reduce-strided");
   EXPECT(prepare(context, Unary{UnaryKind::kAbs}, dense(DataType::kInt32, {8})).error().IsUnimplemented());
   EXPECT(prepare(context, LayerNorm{1.0e-5F, DataType::kFloat16}, dense(DataType::kFloat16, {8, 64})).error().IsUnimplemented());
   EXPECT(prepare(context, Unary{UnaryKind::kTanh}, dense(DataType::kFloat32, {8})).has_value());
