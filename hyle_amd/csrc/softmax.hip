@@ -212,14 +212,20 @@ __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const vo
     const bool invalid = __builtin_fabsf(peak) == INFINITY;
 
     // ---- exponentials and their sum -----------------------------------------------------
-    float total = 0.0f;
+    // The logarithmic form keeps the maxima (exp = 1 each) out of the float sum and counts them
+    // instead: log(sum) = log1p((maxima - 1) + tail), which keeps a tail far below 1, as the
+    // reference does by leaving its one chosen maximum out
+    // (src/compute_provider_cuda/reduction_kernel.cu:178-196).
+    float total = 0.0f, maxima = 0.0f;
 #pragma unroll
     for (int k = 0; k < kVpl; ++k)
 #pragma unroll
       for (int j = 0; j < kVec; ++j) {
         const float shifted = v[k][j] - peak;
         if constexpr (kLog) {
-          total += exp_scaled(shifted);
+          const bool at_peak = shifted == 0.0f;
+          total += at_peak ? 0.0f : exp_scaled(shifted);
+          maxima += at_peak ? 1.0f : 0.0f;
           v[k][j] = shifted;
         } else {
           v[k][j] = exp_scaled(shifted);
@@ -227,12 +233,14 @@ __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const vo
         }
       }
     total = row_sum<kLanes>(total, joint_sum[i & 1]);  // = 2^32 * sum(exp)
+    // joint_max[i & 1] is free again: every wave read it before the barrier of the sum above
+    if constexpr (kLog) maxima = row_sum<kLanes>(maxima, joint_max[i & 1]);
 
     // ---- normalise and store ------------------------------------------------------------
     // softmax: e * 2^32 * (1 / (sum * 2^32)).  log-softmax: (v - max) - log(sum).
     // An undefined row gets a NaN normaliser: it turns every lane, masked zeros included,
     // into NaN without a per-element select.
-    float normaliser = kLog ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
+    float normaliser = kLog ? log1pf((maxima - 1.0f) + total * 2.3283064365386963e-10f) : 1.0f / total;
     if (invalid) normaliser = __builtin_nanf("");
 #pragma unroll
     for (int k = 0; k < kVpl; ++k) {
@@ -295,7 +303,7 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_general(const char *x, 
                                                                  float scale, int mask_kind,
                                                                  int log_form, GeneralLayout g) {
   constexpr int kWaves = kBlockThreads / kWaveLanes;
-  __shared__ float joint_max[kWaves], joint_bad[kWaves], joint_sum[kWaves];
+  __shared__ float joint_max[kWaves], joint_bad[kWaves], joint_sum[kWaves], joint_count[kWaves];
   const uint32_t outer = blockIdx.x / g.inner, inner = blockIdx.x % g.inner;
   float peak = -INFINITY, bad = 0.0f;
   for (uint32_t c = threadIdx.x; c < width; c += kBlockThreads) {
@@ -306,11 +314,17 @@ __global__ __launch_bounds__(kBlockThreads) void softmax_general(const char *x, 
   peak = row_max<kBlockThreads>(peak, joint_max);
   bad = row_max<kBlockThreads>(bad, joint_bad);
   const bool invalid = bad != 0.0f || peak == -INFINITY;
-  float total = 0.0f;
-  for (uint32_t c = threadIdx.x; c < width; c += kBlockThreads)
-    total += exp_scaled(general_value<T>(x, mask, g, outer, inner, c, scale, mask_kind) - peak);
+  float total = 0.0f, maxima = 0.0f;
+  for (uint32_t c = threadIdx.x; c < width; c += kBlockThreads) {
+    const float shifted = general_value<T>(x, mask, g, outer, inner, c, scale, mask_kind) - peak;
+    const bool counted = log_form && shifted == 0.0f;  // the logarithmic form counts its maxima
+    total += counted ? 0.0f : exp_scaled(shifted);
+    maxima += counted ? 1.0f : 0.0f;
+  }
   total = row_sum<kBlockThreads>(total, joint_sum);
-  const float normaliser = log_form ? (logf(total) - 32.0f * 0.69314718055994530942f) : 1.0f / total;
+  maxima = row_sum<kBlockThreads>(maxima, joint_count);
+  const float normaliser =
+      log_form ? log1pf((maxima - 1.0f) + total * 2.3283064365386963e-10f) : 1.0f / total;
   // every read of this row is complete: an exact input alias may now be overwritten
   __syncthreads();
   for (uint32_t c = threadIdx.x; c < width; c += kBlockThreads) {

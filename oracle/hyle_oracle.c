@@ -547,7 +547,35 @@ void hyle_oracle_softmax_f32_row(const float *src, float *dst, size_t n) {
 /* src/compute_provider_native/transformer.cc:44-57 (bool mask) and 165-191 (row
  * loop over a dense last axis); additive mask per
  * src/compute_provider_cuda/reduction_kernel.cu:130-146. */
-void hyle_oracle_softmax(int type, const void *src, void *dst,
+/* LogSoftmax of one row, src/compute_provider_cuda/reduction_kernel.cu:73-86,
+ * 148-196: the maximum is the first NaN, else the largest value at its lowest
+ * column; that one column is left out of the f32 sum of exp(v - max) so that
+ * log1p keeps small tails (the sum in the kernel's own order: strided partial
+ * sums of 256 threads, then a tree); a maximum that is not finite makes the row NaN;
+ * result (v - max) - log1p(sum). */
+void hyle_oracle_log_softmax_f32_row(const float *src, float *dst, size_t n) {
+  if (n == 0) return;
+  size_t chosen = 0;
+  for (size_t i = 1; i < n; ++i) {
+    if (isnan(src[chosen])) break;
+    if (isnan(src[i]) || src[i] > src[chosen]) chosen = i;
+  }
+  const float maximum = src[chosen];
+  /* the kernel's order: 256 threads add every 256th column, a tree joins them */
+  float partial[256];
+  for (size_t t = 0; t < 256; ++t) {
+    partial[t] = 0.0f;
+    for (size_t i = t; i < n; i += 256)
+      if (i != chosen) partial[t] += expf(src[i] - maximum);
+  }
+  for (size_t half = 128; half > 0; half >>= 1)
+    for (size_t t = 0; t < half; ++t) partial[t] += partial[t + half];
+  const float sum = partial[0];
+  const float normalizer = isfinite(maximum) ? log1pf(sum) : NAN;
+  for (size_t i = 0; i < n; ++i) dst[i] = (src[i] - maximum) - normalizer;
+}
+
+static void softmax_rows(int log_form, int type, const void *src, void *dst,
                          const int64_t *in_dims, int in_rank, float scale,
                          int mask_kind, const void *mask,
                          const int64_t *mask_dims, const int64_t *mask_strides,
@@ -579,11 +607,30 @@ void hyle_oracle_softmax(int type, const void *src, void *dst,
       }
       scratch[lane] = value;
     }
-    hyle_oracle_softmax_f32_row(scratch, scratch, width);
+    if (log_form) hyle_oracle_log_softmax_f32_row(scratch, scratch, width);
+    else hyle_oracle_softmax_f32_row(scratch, scratch, width);
     for (size_t lane = 0; lane < width; ++lane)
       store_from_f32(type, d + (r * width + lane) * w, scratch[lane]);
   }
   free(scratch);
+}
+
+void hyle_oracle_softmax(int type, const void *src, void *dst,
+                         const int64_t *in_dims, int in_rank, float scale,
+                         int mask_kind, const void *mask,
+                         const int64_t *mask_dims, const int64_t *mask_strides,
+                         int mask_rank) {
+  softmax_rows(0, type, src, dst, in_dims, in_rank, scale, mask_kind, mask, mask_dims,
+               mask_strides, mask_rank);
+}
+
+void hyle_oracle_log_softmax(int type, const void *src, void *dst,
+                             const int64_t *in_dims, int in_rank, float scale,
+                             int mask_kind, const void *mask,
+                             const int64_t *mask_dims, const int64_t *mask_strides,
+                             int mask_rank) {
+  softmax_rows(1, type, src, dst, in_dims, in_rank, scale, mask_kind, mask, mask_dims,
+               mask_strides, mask_rank);
 }
 
 /* ------------------------------------------------------------------------ */

@@ -193,6 +193,17 @@ void hyle_oracle_softmax(int type, const void *src, void *dst,
                          const int64_t *mask_dims, const int64_t *mask_strides,
                          int mask_rank);
 
+/* LogSoftmax: the same rows, masks and scale as hyle_oracle_softmax; per row
+ * (v - max) - log1p(sum of exp(v - max) over every column but the first
+ * maximum), NaN when the maximum is not finite
+ * (src/compute_provider_cuda/reduction_kernel.cu:73-86,148-196). */
+void hyle_oracle_log_softmax_f32_row(const float *src, float *dst, size_t n);
+void hyle_oracle_log_softmax(int type, const void *src, void *dst,
+                             const int64_t *in_dims, int in_rank, float scale,
+                             int mask_kind, const void *mask,
+                             const int64_t *mask_dims, const int64_t *mask_strides,
+                             int mask_rank);
+
 /* src/compute_provider_native/reduction.cc:24-47 (NaN-propagating extrema,
  * identities +-inf) and src/compute_provider_cuda/reduction_kernel.cu:92-116
  * (sum / mean, f32 accumulate, mean of an empty row is NaN).  Reduces the

@@ -76,6 +76,9 @@ _layer = _sig("hyle_oracle_layer_norm", None, C.c_int, C.c_int, _vp, _vp, _vp, _
 _softmax_row = _sig("hyle_oracle_softmax_f32_row", None, _vp, _vp, _sz)
 _softmax = _sig("hyle_oracle_softmax", None, C.c_int, _vp, _vp, _i64p, C.c_int, C.c_float,
                 C.c_int, _vp, _i64p, _i64p, C.c_int)
+_log_softmax = _sig("hyle_oracle_log_softmax", None, C.c_int, _vp, _vp, _i64p, C.c_int, C.c_float,
+                    C.c_int, _vp, _i64p, _i64p, C.c_int)
+_log_softmax_row = _sig("hyle_oracle_log_softmax_f32_row", None, _vp, _vp, _sz)
 _reduce = _sig("hyle_oracle_reduce_last_axis", None, C.c_int, C.c_int, _vp, _vp, _sz, _sz)
 _iom = _sig("hyle_oracle_index_of_max_f32", _sz, _vp, _sz)
 _topk1 = _sig("hyle_oracle_topk1_f32", None, _vp, _sz, _sz, _vp, _vp)
@@ -292,7 +295,14 @@ def softmax_f32_row(src):
     return out
 
 
-def softmax(type_id, src, scale=1.0, mask_kind=MASK_NONE, mask=None, mask_strides=None):
+def log_softmax_f32_row(src):
+    src = _c(src, np.float32)
+    out = np.empty_like(src)
+    _log_softmax_row(_ptr(src), _ptr(out), src.size)
+    return out
+
+
+def softmax(type_id, src, scale=1.0, mask_kind=MASK_NONE, mask=None, mask_strides=None, log=False):
     src = _c(src, _NP[type_id])
     out = np.empty_like(src)
     md, ms = [], []
@@ -300,8 +310,8 @@ def softmax(type_id, src, scale=1.0, mask_kind=MASK_NONE, mask=None, mask_stride
         mask = np.ascontiguousarray(mask)
         md = list(mask.shape)
         ms = mask_strides or _byte_strides(md, mask.itemsize)
-    _softmax(type_id, _ptr(src), _ptr(out), _i64(src.shape), src.ndim, float(scale),
-             mask_kind, _ptr(mask), _i64(md), _i64(ms), len(md))
+    (_log_softmax if log else _softmax)(type_id, _ptr(src), _ptr(out), _i64(src.shape), src.ndim, float(scale),
+                                        mask_kind, _ptr(mask), _i64(md), _i64(ms), len(md))
     return out
 
 
