@@ -1,7 +1,7 @@
 /*
  * hyle_hip.h -- C ABI of the MI355X (gfx950) compute provider for HYLE's tensor
  * hot path: broadcast Binary, Unary SiLU, GatedActivation (SwiGLU), RMSNorm,
- * row Softmax, Reduce over any set of axes, TopK(count = 1) and Q8_0 block dequant.
+ * row Softmax / LogSoftmax, Reduce over any set of axes, TopK and Q8_0 block dequant.
  *
  * The surface is what a `hyle::compute` provider for this path binds: one cold
  * "plan" per (Operation, input descriptors) pair -- the reference's
@@ -161,8 +161,8 @@ typedef struct hyle_hip_op_desc {
   uint32_t keep_dimensions;  /* Reduce */
   float epsilon;             /* RmsNorm, LayerNorm */
   float scale;               /* Softmax */
-  uint64_t count;            /* TopK count (only 1 is implemented) */
-  uint32_t largest;          /* TopK */
+  uint64_t count;            /* TopK count (counts above 1024 are declined) */
+  uint32_t largest;          /* TopK: 1 = largest first, 0 = smallest first */
   uint32_t input_count;
   hyle_hip_tensor_desc inputs[HYLE_HIP_MAX_INPUTS];
   /* Reduce::axes (include/hyle/compute/operation.h:232-247, 307-312): axes_count = 0 is
