@@ -48,6 +48,9 @@ def parse_args():
     p.add_argument("--op-reps", type=int, default=200, help="launches per kernel in the per-op timing loops")
     p.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     p.add_argument("--cpu-seconds", type=float, default=2.0, help="target CPU seconds per kernel sample")
+    p.add_argument("--file-stream-mib", type=int, default=0,
+                   help="also stream a temporary file of this many MiB into HBM and report the rate (PCIe-inclusive; "
+                        "never part of `value`)")
     p.add_argument("--only", default="", help="comma-separated op names: run and time just these kernels")
     p.add_argument("--copy-probe", action="store_true",
                    help="also run three plain device copies of 1 GiB (a kernel of known traffic that "
@@ -387,8 +390,47 @@ def main() -> int:
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(args, step_ops, np, torch, wl)
+    if args.file_stream_mib > 0:
+        result["file_stream"] = file_stream_rate(args.file_stream_mib, ctx, torch, dev)
     print(json.dumps(result))
     return 0
+
+
+def file_stream_rate(mib, ctx, torch, dev):
+    """File (page cache) -> pinned staging -> HBM through the pipeline of include/hyle_hip_stream.h."""
+    import tempfile
+    from hyle_amd import file_stream as fs
+    total = mib << 20
+    chunk = torch.randint(0, 256, (min(total, 64 << 20),), dtype=torch.uint8)
+    with tempfile.NamedTemporaryFile(delete=False) as handle:
+        path = handle.name
+        written = 0
+        while written < total:
+            piece = min(total - written, chunk.numel())
+            handle.write(chunk.numpy()[:piece].tobytes())
+            written += piece
+    fd = os.open(path, os.O_RDONLY)
+    try:
+        target = torch.empty(total, dtype=torch.uint8, device=dev)
+        best = {}
+        for slots, slot_mib in ((2, 1), (4, 8), (4, 32)):
+            pipeline = fs.FileResourcePipeline.create(ctx, fs.FileStreamOptions(slots, slot_mib << 20))
+            stream = torch.cuda.current_stream().cuda_stream
+            seconds = []
+            for _ in range(3):
+                torch.cuda.synchronize()
+                begin = time.perf_counter()
+                pipeline.read(fd, [fs.StreamReadRange(0, target.data_ptr(), total)], stream)
+                pipeline.wait()
+                seconds.append(time.perf_counter() - begin)
+            pipeline.close()
+            best[f"{slots}x{slot_mib}MiB"] = round(total / min(seconds) / 1e9, 2)
+        ok = bool((target[:chunk.numel()].cpu() == chunk[:min(total, chunk.numel())]).all())
+        return {"bytes": total, "unit": "GB/s", "rates": best, "bytes_identical": ok,
+                "note": "file in the page cache; pread on one thread overlapped with the copies of the other slots"}
+    finally:
+        os.close(fd)
+        os.unlink(path)
 
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script

@@ -37,6 +37,29 @@ class OpDescC(C.Structure):
     ]
 
 
+class CopyRangeC(C.Structure):  # include/hyle_hip_stream.h
+    _fields_ = [("source", C.c_void_p), ("destination", C.c_void_p), ("bytes", C.c_size_t), ("phase", C.c_uint32)]
+
+
+class CopyPhaseC(C.Structure):
+    _fields_ = [("dependency_mask", C.c_uint64), ("group_tag", C.c_uint64)]
+
+
+class FileStreamOptionsC(C.Structure):
+    _fields_ = [("in_flight_slots", C.c_uint32), ("staging_bytes_per_slot", C.c_size_t),
+                ("staging_alignment", C.c_size_t)]
+
+
+class ReadRangeC(C.Structure):
+    _fields_ = [("file_offset", C.c_uint64), ("destination", C.c_void_p), ("bytes", C.c_size_t)]
+
+
+class StreamResultC(C.Structure):
+    _fields_ = [("status", C.c_int), ("read_bytes", C.c_uint64), ("copied_bytes", C.c_uint64),
+                ("ready_ranges", C.c_uint32), ("total_ranges", C.c_uint32), ("io_calls", C.c_uint32),
+                ("native_calls", C.c_uint32), ("host_waits", C.c_uint32)]
+
+
 EXPORTS = {
     # name: (restype, argtypes)
     "hyle_hip_abi_version": (C.c_uint32, []),
@@ -56,13 +79,21 @@ EXPORTS = {
     "hyle_hip_plan_route_name": (C.c_char_p, [C.c_void_p]),
     "hyle_hip_plan_launch": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_uint32, C.POINTER(C.c_void_p),
                                        C.c_uint32, C.c_void_p, C.c_size_t, C.c_void_p]),
+    # include/hyle_hip_stream.h
+    "hyle_hip_copy_batch_submit": (C.c_int, [C.c_void_p, C.POINTER(CopyPhaseC), C.c_uint32, C.POINTER(CopyRangeC),
+                                             C.c_uint32, C.c_void_p]),
+    "hyle_hip_file_pipeline_create": (C.c_int, [C.c_void_p, C.POINTER(FileStreamOptionsC), C.POINTER(C.c_void_p)]),
+    "hyle_hip_file_pipeline_destroy": (None, [C.c_void_p]),
+    "hyle_hip_file_pipeline_read": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(ReadRangeC), C.c_uint32, C.c_void_p,
+                                              C.POINTER(StreamResultC)]),
+    "hyle_hip_file_pipeline_wait": (C.c_int, [C.c_void_p]),
 }
 
 _lib = None
 
 
 def load() -> C.CDLL:
-    """Load libhyle_hip.so and bind every symbol include/hyle_hip.h declares."""
+    """Load libhyle_hip.so and bind every symbol include/hyle_hip.h and include/hyle_hip_stream.h declare."""
     global _lib
     if _lib is not None:
         return _lib

@@ -1183,3 +1183,12 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
 }
 
 }  // extern "C"
+
+// Hooks for the other translation units of the library (file_stream.hip): the device a context
+// is bound to, and the per-thread error text behind hyle_hip_last_error.
+namespace hyle_hip {
+int context_device(const hyle_hip_context *context) { return context ? context->device : -1; }
+int record_error(int status, const char *text) {
+  return fail(static_cast<hyle_hip_status>(status), "%s", text);
+}
+}  // namespace hyle_hip

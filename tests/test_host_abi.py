@@ -27,7 +27,7 @@ CTX = hc.Context.planning_only()
 
 
 def test_library_exports_every_declared_symbol():
-    text = open(HEADER).read()
+    text = open(HEADER).read() + open(os.path.join(ROOT, "include", "hyle_hip_stream.h")).read()
     declared = set(re.findall(r"HYLE_HIP_API\s+[\w\s\*]+?\b(hyle_hip_\w+)\s*\(", text))
     assert declared, "no declarations parsed"
     lib = capi.load()
@@ -281,3 +281,18 @@ def test_cast_and_copy_inference_and_admission():
             hc.prepare(CTX, hc.Cast(dst), D(src, [8]))
         assert err.value.is_unimplemented()
     assert hc.prepare(CTX, hc.Copy(), D(DT.kFloat32, [0, 9])).dispatch_count() == 0
+
+
+def test_stream_abi_is_exported_and_validates_without_a_device():
+    from hyle_amd import capi
+    from hyle_amd import file_stream as fs
+    lib = capi.load()
+    for name in ("hyle_hip_copy_batch_submit", "hyle_hip_file_pipeline_create", "hyle_hip_file_pipeline_destroy",
+                 "hyle_hip_file_pipeline_read", "hyle_hip_file_pipeline_wait"):
+        assert hasattr(lib, name)
+    with pytest.raises(hc.StatusError) as err:     # a planning-only context binds no device
+        fs.FileResourcePipeline.create(CTX)
+    assert err.value.is_invalid_argument()
+    with pytest.raises(hc.StatusError) as err:
+        fs.submit_copy_batch(CTX, [fs.CopyPhase()], [], 0)
+    assert err.value.is_invalid_argument()
