@@ -194,6 +194,21 @@ def main() -> int:
         ops.append(Op("cfg5_q8_0_dequant_sumsq", hc.Q8_0DequantSumSquares(),
                       [hc.TensorDesc.gguf_q8_0_weight(BF, 2048, 6144)], set5, 16,
                       wl.ALGORITHMIC_BYTES["cfg5_q8_0_dequant_sumsq"], 6144 * 2048, "u8/bf16"))
+    # ---- the K-quant siblings of cfg5 (GGUF Q4_K / Q6_K), timed beside the step ------------------
+    for name, gguf, block_bytes in (("next_q4_k_dequant_sumsq", hc.GgufQuantizedType.kQ4K, 144),
+                                    ("next_q6_k_dequant_sumsq", hc.GgufQuantizedType.kQ6K, 210)):
+        if not want(name):
+            continue
+
+        def set_k(i, block_bytes=block_bytes):
+            raw = torch.randint(0, 256, (6144, 8 * block_bytes), dtype=torch.uint8)
+            fields = raw.view(6144, 8, block_bytes)      # keep the f16 scales finite
+            for at in ((1, 3) if block_bytes == 144 else (209,)):
+                fields[:, :, at] &= 0x3B
+            return [raw.to(dev)], [torch.empty((6144, 2048), dtype=torch.bfloat16, device=dev),
+                                   torch.empty(6144, dtype=torch.float32, device=dev)]
+        ops.append(Op(name, hc.GgufDequantSumSquares(), [hc.TensorDesc.gguf_weight(gguf, BF, 2048, 6144)], set_k, 16,
+                      6144 * (8 * block_bytes + 2048 * 2 + 4), 6144 * 2048, "u8/bf16", in_step=False))
     # ---- the next row of the path: Cast and Copy, timed beside the step -------------------------
     if want("next_cast_f32_to_bf16") or want("next_cast_bf16_to_f32"):
         x32 = np.random.default_rng(5).normal(0, 2, (8192, 2048)).astype(np.float32)

@@ -60,6 +60,16 @@ def _check(code: int) -> None:
 
 
 # ---- descriptors ------------------------------------------------------------------------
+class GgufQuantizedType(enum.IntEnum):  # include/hyle/compute/low_precision.h:36-41 (the decoded ones)
+    kQ4K = 1
+    kQ6K = 3
+    kQ8_0 = 4
+
+
+GGUF_BLOCKS = {GgufQuantizedType.kQ4K: (256, 144), GgufQuantizedType.kQ6K: (256, 210),
+               GgufQuantizedType.kQ8_0: (32, 34)}
+
+
 class DataType(enum.IntEnum):  # include/hyle/compute/tensor_desc.h:17-34
     kUnknown = 0
     kBool = 1
@@ -121,6 +131,19 @@ class TensorDesc:
         stride = (k // 32) * 34 if row_stride is None else int(row_stride)
         return TensorDesc(DataType(logical_type), (k, n), (34, stride), blocked=True, block_axis=0,
                           elements_per_block=32, bytes_per_block=34)
+
+    @staticmethod
+    def gguf_weight(kind: "GgufQuantizedType", logical_type: DataType, k: int, n: int,
+                    row_stride: Optional[int] = None) -> "TensorDesc":
+        """gguf_weight_description(type, logical_type, k, n) (include/hyle/compute/low_precision.h:181-186)
+        for the block formats this provider decodes: logical [K, N], physical rows of native K blocks
+        (geometry: src/compute_ops/low_precision.cc:22-29)."""
+        per_block, block_bytes = GGUF_BLOCKS[GgufQuantizedType(kind)]
+        if k <= 0 or n <= 0 or k % per_block != 0:
+            raise StatusError(capi.INVALID_ARGUMENT, "GGUF weight dimensions do not contain complete K blocks")
+        stride = (k // per_block) * block_bytes if row_stride is None else int(row_stride)
+        return TensorDesc(DataType(logical_type), (k, n), (block_bytes, stride), blocked=True, block_axis=0,
+                          elements_per_block=per_block, bytes_per_block=block_bytes)
 
     @property
     def rank(self) -> int:
@@ -337,6 +360,12 @@ class TopK:
 @dataclass(frozen=True)
 class Q8_0DequantSumSquares:
     pass
+
+
+@dataclass(frozen=True)
+class GgufDequantSumSquares(Q8_0DequantSumSquares):
+    """The same operation under its general name: Q8_0, Q4_K or Q6_K weights, told apart by the
+    block geometry of the input descriptor."""
 
 
 def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:

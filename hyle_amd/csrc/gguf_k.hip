@@ -1,0 +1,142 @@
+// GGUF Q4_K and Q6_K rows -> bf16 [rows, k] plus the f32 row sums of squares of the exact f32
+// values, the K-quant siblings of q8_0.hip.
+//
+// Geometry from the reference (src/compute_ops/low_precision.cc:22-27: 256 elements in 144 and
+// 210 bytes); the decode is ggml's dequantize_row_q4_K / dequantize_row_q6_K, restated from the
+// published block layouts (the source is not part of the reference tree):
+//   Q4_K  {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]}   y = (d * sc) * q - (dmin * m)
+//   Q6_K  {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d}  y = (d * scale) * (q - 32)
+// with separate f32 roundings for the products and the subtraction, as the source writes them.
+//
+// A block of 256 threads takes four rows at a time.  Eight super-blocks of each (at most 1680
+// bytes) are staged in LDS per step with the widest loads the row's address allows; a thread then decodes eight
+// neighbouring values from LDS bytes and stores them as one 16-byte vector.  The output (2 bytes
+// per value) is four times the input traffic, so the byte-wise LDS reads are not what bounds it.
+#include "device_common.h"
+#include "kernels.h"
+
+namespace hyle_hip {
+namespace {
+
+constexpr int kSuper = 256;                      // values per super-block
+constexpr int kChunkBlocks = kBlockThreads * 8 / kSuper;  // super-blocks decoded per step: 8
+
+__device__ __forceinline__ float lds_f16(const unsigned char *p) {
+  return f16_to_f32((uint16_t)(p[0] | ((uint16_t)p[1] << 8)));
+}
+
+// Eight values of a Q4_K block starting at position p (a multiple of 8).
+__device__ __forceinline__ void decode_q4_k(const unsigned char *blk, uint32_t p, float (&y)[8]) {
+  const float d = lds_f16(blk), dmin = lds_f16(blk + 2);
+  const unsigned char *scales = blk + 4;
+  const uint32_t sub = p / 32, within = p % 32, chunk = sub / 2;
+  uint32_t sc, m;
+  if (sub < 4) {
+    sc = scales[sub] & 63u;
+    m = scales[sub + 4] & 63u;
+  } else {
+    sc = (scales[sub + 4] & 0xFu) | ((uint32_t)(scales[sub - 4] >> 6) << 4);
+    m = (uint32_t)(scales[sub + 4] >> 4) | ((uint32_t)(scales[sub] >> 6) << 4);
+  }
+  const float step = d * (float)sc, offset = dmin * (float)m;
+  const unsigned char *q = blk + 16 + 32 * chunk + within;
+  const uint32_t shift = (sub & 1u) * 4;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = step * (float)((q[j] >> shift) & 0xFu) - offset;
+}
+
+// Eight values of a Q6_K block starting at position p (a multiple of 8).
+__device__ __forceinline__ void decode_q6_k(const unsigned char *blk, uint32_t p, float (&y)[8]) {
+  const uint32_t half = p / 128, group = (p % 128) / 32, l = p % 32;
+  const unsigned char *ql = blk + 64 * half + l + 32 * (group & 1u);
+  const unsigned char *qh = blk + 128 + 32 * half + l;
+  const int scale = (int)(int8_t)blk[192 + 8 * half + 2 * group + l / 16];
+  const float step = lds_f16(blk + 208) * (float)scale;
+  const uint32_t low_shift = (group >> 1) * 4, high_shift = group * 2;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int q = (int)(((ql[j] >> low_shift) & 0xFu) | (((qh[j] >> high_shift) & 3u) << 4)) - 32;
+    y[j] = step * (float)q;
+  }
+}
+
+// Bytes -> LDS with the widest loads the address allows (Q4_K rows of a 16-byte aligned tensor
+// always take words; Q6_K blocks are only 2-byte aligned as a rule).
+__device__ __forceinline__ void stage(unsigned char *to, const unsigned char *from, uint32_t bytes) {
+  if (((reinterpret_cast<uintptr_t>(from) | bytes) & 3u) == 0) {
+    for (uint32_t i = threadIdx.x; i < bytes / 4; i += kBlockThreads)
+      reinterpret_cast<uint32_t *>(to)[i] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(from) + i);
+  } else if (((reinterpret_cast<uintptr_t>(from) | bytes) & 1u) == 0) {
+    for (uint32_t i = threadIdx.x; i < bytes / 2; i += kBlockThreads)
+      reinterpret_cast<uint16_t *>(to)[i] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t *>(from) + i);
+  } else {
+    for (uint32_t i = threadIdx.x; i < bytes; i += kBlockThreads) to[i] = from[i];
+  }
+}
+
+// kRows rows per block: their chunks are staged together, so kRows times the bytes are in flight
+// per barrier and each thread has kRows independent decodes.
+template <int kKind, int kRows>  // 0 = Q4_K, 1 = Q6_K
+__global__ __launch_bounds__(kBlockThreads) void k_quant_rows(const unsigned char *blocks, void *out,
+                                                              float *sumsq, uint32_t rows, uint32_t k,
+                                                              uint64_t row_stride) {
+  constexpr uint32_t kBlockBytes = kKind == 0 ? 144 : 210;
+  constexpr uint32_t kSlot = (kChunkBlocks * kBlockBytes + 15) / 16 * 16;
+  __shared__ __align__(16) unsigned char staged[kRows][kSlot];
+  __shared__ float joint[kRows][kBlockThreads / kWaveLanes];
+  const uint32_t first_row = blockIdx.x * kRows;
+  const uint32_t super_blocks = k / kSuper;
+  float acc[kRows];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) acc[r] = 0.0f;
+  for (uint32_t first = 0; first < super_blocks; first += kChunkBlocks) {
+    const uint32_t count = min((uint32_t)kChunkBlocks, super_blocks - first);
+#pragma unroll
+    for (int r = 0; r < kRows; ++r) {
+      const uint32_t row = min(first_row + r, rows - 1);  // a row past the end re-reads the last one
+      stage(staged[r], blocks + (size_t)row * row_stride + (size_t)first * kBlockBytes, count * kBlockBytes);
+    }
+    __syncthreads();
+    const uint32_t local = threadIdx.x * 8;  // position within the chunk
+    if (local < count * kSuper) {
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        const unsigned char *blk = staged[r] + (local / kSuper) * kBlockBytes;
+        float y[8];
+        if constexpr (kKind == 0) decode_q4_k(blk, local % kSuper, y);
+        else decode_q6_k(blk, local % kSuper, y);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[r] += y[j] * y[j];
+        if (first_row + r < rows) {
+          const size_t element = (size_t)(first_row + r) * k + (size_t)first * kSuper + local;
+          store16_stream(out, element / 8, Traits<BF16>::pack(y));
+        }
+      }
+    }
+    __syncthreads();  // the next step overwrites the staging
+  }
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const float total = row_sum<kBlockThreads>(acc[r], joint[r]);
+    if (threadIdx.x == 0 && first_row + r < rows) sumsq[first_row + r] = total;
+  }
+}
+
+}  // namespace
+
+hipError_t launch_k_quant_dequant(const KQuantParams &p, const void *blocks, void *out, float *sumsq,
+                                  hipStream_t stream) {
+  if (p.rows == 0) return hipSuccess;
+  const unsigned char *in = static_cast<const unsigned char *>(blocks);
+  constexpr int kRows = 4;
+  const dim3 grid(((uint32_t)p.rows + kRows - 1) / kRows), block(kBlockThreads);
+  if (p.kind == 0)
+    hipLaunchKernelGGL((k_quant_rows<0, kRows>), grid, block, 0, stream, in, out, sumsq, (uint32_t)p.rows, p.k,
+                       p.row_stride);
+  else
+    hipLaunchKernelGGL((k_quant_rows<1, kRows>), grid, block, 0, stream, in, out, sumsq, (uint32_t)p.rows, p.k,
+                       p.row_stride);
+  return hipGetLastError();
+}
+
+}  // namespace hyle_hip

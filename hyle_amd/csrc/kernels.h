@@ -168,6 +168,17 @@ void topk_plan(TopKParams *p);
 hipError_t launch_topk(Elem type, const TopKParams &p, const void *x, void *values, int32_t *indices,
                        void *workspace, bool input_vector_aligned, hipStream_t stream);
 
+// GGUF Q4_K (kind 0, 144-byte blocks) / Q6_K (kind 1, 210-byte blocks) rows of k/256 blocks
+// -> bf16 [rows, k] + f32 sumsq[rows].
+struct KQuantParams {
+  uint64_t rows = 0;
+  uint32_t k = 0;
+  uint64_t row_stride = 0;  // bytes between physical rows
+  uint8_t kind = 0;
+};
+hipError_t launch_k_quant_dequant(const KQuantParams &p, const void *blocks, void *out, float *sumsq,
+                                  hipStream_t stream);
+
 // Q8_0 rows of k/32 blocks {f16 d; int8 qs[32]} -> bf16 [rows, k] + f32 sumsq[rows].
 struct Q8Params {
   uint64_t rows = 0;

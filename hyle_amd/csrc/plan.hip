@@ -426,10 +426,15 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
       if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
       // gguf_weight_description(kQ8_0, ..., k, n): logical [K, N], blocks along axis 0
       // (src/compute_ops/low_precision.cc:269-297)
-      if (in[0].storage != HYLE_HIP_STORAGE_BLOCKED || in[0].elements_per_block != 32 ||
-          in[0].bytes_per_block != 34 || in[0].rank != 2 || in[0].block_axis != 0)
+      // and the K-quant geometries of src/compute_ops/low_precision.cc:22-27
+      const bool q8_0 = in[0].elements_per_block == 32 && in[0].bytes_per_block == 34;
+      const bool q4_k = in[0].elements_per_block == 256 && in[0].bytes_per_block == 144;
+      const bool q6_k = in[0].elements_per_block == 256 && in[0].bytes_per_block == 210;
+      if (in[0].storage != HYLE_HIP_STORAGE_BLOCKED || !(q8_0 || q4_k || q6_k) || in[0].rank != 2 ||
+          in[0].block_axis != 0)
         return fail(HYLE_HIP_INVALID_ARGUMENT,
-                    "Q8_0 weight must be blocked [K, N] storage with 32-element 34-byte blocks on axis 0");
+                    "GGUF weight must be blocked [K, N] storage with Q8_0 (32 / 34), Q4_K (256 / 144) or "
+                    "Q6_K (256 / 210) blocks on axis 0");
       if (!is_floating(in[0].dtype))
         return fail(HYLE_HIP_INVALID_ARGUMENT, "GGUF weight requires a floating logical type");
       const int64_t dims0[2] = {in[0].dims[1], in[0].dims[0]};
@@ -456,6 +461,7 @@ enum class Route : uint8_t {
   kArgmax,
   kTopK,
   kQ8Dequant,
+  kKQuantDequant,
   kCast,
 };
 
@@ -471,6 +477,7 @@ const char *route_name(Route r) {
     case Route::kArgmax: return "argmax-tiles";
     case Route::kTopK: return "topk-sorted-tiles";
     case Route::kQ8Dequant: return "q8_0-dequant-rows";
+    case Route::kKQuantDequant: return "k-quant-dequant-rows";
     case Route::kCast: return "cast-copy";
   }
   return "?";
@@ -512,6 +519,7 @@ struct hyle_hip_plan {
   ArgmaxParams argmax;
   TopKParams topk;
   Q8Params q8;
+  KQuantParams kquant;
   CastParams cast;
   // Cast and Copy take no alias at all (AliasPolicy::kNone, src/compute_ops/operation.cc:935-957):
   // the bytes the input and the output occupy must not overlap.
@@ -861,14 +869,28 @@ hyle_hip_status admit(hyle_hip_plan *p) {
     }
     case HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ: {
       const int64_t k = in[0].dims[0], n = in[0].dims[1];
-      if (in[0].byte_strides[0] != 34)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "Q8_0 blocks of a row must be contiguous (34-byte block stride)");
-      if (k > 0 && n > 1 && in[0].byte_strides[1] < (k / 32) * 34)
-        return fail(HYLE_HIP_INVALID_ARGUMENT, "Q8_0 row stride is shorter than a row of blocks");
+      const int64_t per_block = in[0].elements_per_block, block_bytes = in[0].bytes_per_block;
+      if (in[0].byte_strides[0] != block_bytes)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF blocks of a row must be contiguous (block stride = block bytes)");
+      if (k > 0 && n > 1 && in[0].byte_strides[1] < (k / per_block) * block_bytes)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "GGUF row stride is shorter than a row of blocks");
       if ((uint64_t)k * (uint64_t)n > kMaxElements)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "Q8_0 dequant requires at most INT32_MAX elements");
+        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF dequant requires at most INT32_MAX elements");
       p->elem = Elem::kBF16;
       if (n == 0) return HYLE_HIP_OK;
+      if (per_block == 256) {
+        // Q4_K / Q6_K: the blocks are read at any byte address; the bf16 rows are stored as
+        // 16-byte vectors
+        p->route = Route::kKQuantDequant;
+        p->kquant.rows = (uint64_t)n;
+        p->kquant.k = (uint32_t)k;
+        p->kquant.row_stride = (uint64_t)in[0].byte_strides[1];
+        p->kquant.kind = block_bytes == 144 ? 0 : 1;
+        p->input_alignment[0] = 1;
+        p->output_alignment[0] = 16;
+        p->dispatches = 1;
+        return HYLE_HIP_OK;
+      }
       // with K == 0 the bf16 output is empty but every row still gets sumsq = 0
       p->route = Route::kQ8Dequant;
       p->q8.rows = (uint64_t)n;
@@ -1173,6 +1195,9 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
     case Route::kQ8Dequant:
       err = launch_q8_0_dequant(plan->q8, inputs[0], outputs[0], static_cast<float *>(outputs[1]),
                                 aligned(inputs[0], 16) && aligned(outputs[0], 16), stream);
+      break;
+    case Route::kKQuantDequant:
+      err = launch_k_quant_dequant(plan->kquant, inputs[0], outputs[0], static_cast<float *>(outputs[1]), stream);
       break;
     case Route::kCast:
       err = launch_cast(plan->cast, inputs[0], outputs[0], vector, stream);

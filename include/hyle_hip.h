@@ -86,7 +86,11 @@ typedef enum hyle_hip_op_kind {
   /* in0: Q8_0 blocked weight, logical [K, N], physical rows of K/32 blocks;
    * out0: bf16 [N, K] dense; out1: f32 [N] row sum of squares of the exact
    * f32 products. */
-  HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ = 0x101
+  HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ = 0x101,
+  /* The same operation under its general name: the weight may also be GGUF Q4_K (256-element,
+   * 144-byte blocks) or Q6_K (256-element, 210-byte blocks); the block geometry of in0 selects
+   * the decoder (src/compute_ops/low_precision.cc:22-29). */
+  HYLE_HIP_OP_GGUF_DEQUANT_SUMSQ = 0x101
 } hyle_hip_op_kind;
 
 /* UnaryKind (include/hyle/compute/operation.h:57-73) */

@@ -854,6 +854,96 @@ void hyle_oracle_q8_0_dequant_bf16(const void *blocks, size_t rows, size_t k,
   }
 }
 
+/* ------------------------------------------------------------------------ */
+/* Q4_K, Q6_K                                                               */
+/* ------------------------------------------------------------------------ */
+
+/* Block geometry: src/compute_ops/low_precision.cc:22-27 (256 elements in 144
+ * and 210 bytes).  The decode is ggml's (dequantize_row_q4_K / _q6_K, pinned
+ * with the other GGUF formats at ffa4e8b... in cmake/HyleDependencyLock.json
+ * and absent from the reference tree), restated from the published block
+ * layouts:
+ *   Q4_K  {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]}: eight sub-blocks of 32
+ *         with 6-bit scale sc and minimum m; y = (d * sc) * q - (dmin * m),
+ *         q the low nibbles of qs[32 c .. 32 c + 31] for sub-block 2 c and the
+ *         high nibbles for sub-block 2 c + 1;
+ *   Q6_K  {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d}: sixteen sub-blocks of
+ *         16; y = (d * scale) * (q - 32), q six bits from ql (low four) and qh
+ *         (high two).
+ * Products and the subtraction are separate f32 roundings, as the source
+ * writes them.  PARITY UNPINNED against ggml itself: no vector of its output
+ * exists in the reference tree. */
+static void q4_k_scale_min(int j, const unsigned char *q, unsigned *scale, unsigned *minimum) {
+  if (j < 4) {
+    *scale = q[j] & 63u;
+    *minimum = q[j + 4] & 63u;
+  } else {
+    *scale = (q[j + 4] & 0xFu) | ((unsigned)(q[j - 4] >> 6) << 4);
+    *minimum = (unsigned)(q[j + 4] >> 4) | ((unsigned)(q[j] >> 6) << 4);
+  }
+}
+
+static void q4_k_block_f32(const unsigned char *blk, float *y) {
+  const float d = hyle_oracle_f16_to_f32((uint16_t)(blk[0] | ((uint16_t)blk[1] << 8)));
+  const float dmin = hyle_oracle_f16_to_f32((uint16_t)(blk[2] | ((uint16_t)blk[3] << 8)));
+  const unsigned char *scales = blk + 4, *q = blk + 16;
+  for (int chunk = 0; chunk < 4; ++chunk) {
+    unsigned sc, m;
+    q4_k_scale_min(2 * chunk, scales, &sc, &m);
+    const float d1 = d * (float)sc, m1 = dmin * (float)m;
+    q4_k_scale_min(2 * chunk + 1, scales, &sc, &m);
+    const float d2 = d * (float)sc, m2 = dmin * (float)m;
+    for (int l = 0; l < 32; ++l) y[64 * chunk + l] = d1 * (float)(q[32 * chunk + l] & 0xF) - m1;
+    for (int l = 0; l < 32; ++l) y[64 * chunk + 32 + l] = d2 * (float)(q[32 * chunk + l] >> 4) - m2;
+  }
+}
+
+static void q6_k_block_f32(const unsigned char *blk, float *y) {
+  const unsigned char *ql = blk, *qh = blk + 128;
+  const int8_t *sc = (const int8_t *)(blk + 192);
+  const float d = hyle_oracle_f16_to_f32((uint16_t)(blk[208] | ((uint16_t)blk[209] << 8)));
+  for (int half = 0; half < 2; ++half) {
+    for (int l = 0; l < 32; ++l) {
+      const int is = l / 16;
+      const int q1 = (int)((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+      const int q2 = (int)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+      const int q3 = (int)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+      const int q4 = (int)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+      y[l] = d * (float)sc[is] * (float)q1;
+      y[l + 32] = d * (float)sc[is + 2] * (float)q2;
+      y[l + 64] = d * (float)sc[is + 4] * (float)q3;
+      y[l + 96] = d * (float)sc[is + 6] * (float)q4;
+    }
+    y += 128;
+    ql += 64;
+    qh += 32;
+    sc += 8;
+  }
+}
+
+/* kind: 0 = Q4_K, 1 = Q6_K.  out_f32 and out_bf16 may each be NULL. */
+void hyle_oracle_k_quant_dequant(int kind, const void *blocks, size_t rows, size_t k,
+                                 size_t row_stride_bytes, float *out_f32, uint16_t *out_bf16,
+                                 float *sumsq) {
+  const unsigned char *base = (const unsigned char *)blocks;
+  const size_t block_bytes = kind == 0 ? 144 : 210;
+  float y[256];
+  for (size_t r = 0; r < rows; ++r) {
+    float acc = 0.0f;
+    for (size_t b = 0; b < k / 256; ++b) {
+      const unsigned char *blk = base + r * row_stride_bytes + b * block_bytes;
+      if (kind == 0) q4_k_block_f32(blk, y);
+      else q6_k_block_f32(blk, y);
+      for (size_t j = 0; j < 256; ++j) {
+        if (out_f32) out_f32[r * k + b * 256 + j] = y[j];
+        if (out_bf16) out_bf16[r * k + b * 256 + j] = hyle_oracle_f32_to_bf16(y[j]);
+        acc += y[j] * y[j];
+      }
+    }
+    if (sumsq) sumsq[r] = acc;
+  }
+}
+
 void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
                                   size_t row_stride_bytes, float *out) {
   const unsigned char *base = (const unsigned char *)blocks;

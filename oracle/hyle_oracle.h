@@ -25,6 +25,12 @@
  *   - rms_norm_bf16_native tile order: "parity unpinned" at the bit level (the
  *     reference sums each 128-wide tile with a Highway vector dot whose lane
  *     order is target-dependent); pinned only to tolerance.
+ *   - cast, layer_norm, unary / gated kinds, reduce over any axes, topk,
+ *     log_softmax: pinned by the reference's scalar floor (where it holds the
+ *     function), its tests' known answers and numpy / float64 closed forms.
+ *   - k_quant_dequant (GGUF Q4_K, Q6_K): "parity unpinned" against ggml's
+ *     source, which is not in the reference tree; the restatement of the
+ *     published block layouts is checked against blocks packed field by field.
  */
 #ifndef HYLE_ORACLE_H_
 #define HYLE_ORACLE_H_
@@ -250,6 +256,15 @@ void hyle_oracle_q8_0_dequant_bf16(const void *blocks, size_t rows, size_t k,
                                    size_t row_stride_bytes, uint16_t *out,
                                    float *sumsq, float *sumsq_rounded);
 /* ggml dequantize_row_q8_0 to f32 */
+/* GGUF Q4_K (kind 0: 256 elements in 144 bytes) and Q6_K (kind 1: 256 in 210)
+ * rows -> f32 and / or bf16 [rows, k] plus the f32 row sums of squares of the
+ * exact f32 values.  Geometry from src/compute_ops/low_precision.cc:22-27; the
+ * decode is ggml's, restated from the published block layouts (the source is
+ * not in the reference tree: parity with it is unpinned). */
+void hyle_oracle_k_quant_dequant(int kind, const void *blocks, size_t rows, size_t k,
+                                 size_t row_stride_bytes, float *out_f32, uint16_t *out_bf16,
+                                 float *sumsq);
+
 void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
                                   size_t row_stride_bytes, float *out);
 

@@ -86,6 +86,7 @@ _q8_bf16 = _sig("hyle_oracle_q8_0_dequant_bf16", None, _vp, _sz, _sz, _sz, _vp, 
 _q8_f32 = _sig("hyle_oracle_q8_0_dequant_f32", None, _vp, _sz, _sz, _sz, _vp)
 _reduce_axes = _sig("hyle_oracle_reduce", None, C.c_int, C.c_int, _vp, C.c_int, _i64p, _i64p, C.c_uint32, _vp)
 _topk = _sig("hyle_oracle_topk", None, C.c_int, _vp, C.c_int, _i64p, _i64p, C.c_int, _sz, C.c_int, _vp, _vp)
+_k_quant = _sig("hyle_oracle_k_quant_dequant", None, C.c_int, _vp, _sz, _sz, _sz, _vp, _vp, _vp)
 _cast = _sig("hyle_oracle_cast", C.c_int, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int, _vp)
 
 
@@ -392,6 +393,20 @@ def q8_0_dequant_bf16(blocks: np.ndarray, rows: int, k: int, row_stride: int | N
     sumsq_rounded = np.empty(rows, np.float32)
     _q8_bf16(_ptr(blocks), rows, k, row_stride, _ptr(out), _ptr(sumsq), _ptr(sumsq_rounded))
     return out, sumsq, sumsq_rounded
+
+
+Q4_K, Q6_K = 0, 1
+K_QUANT_BLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
+
+
+def k_quant_dequant(kind: int, blocks: np.ndarray, rows: int, k: int, row_stride: int | None = None):
+    """GGUF Q4_K / Q6_K rows -> (f32 [rows, k], bf16 bits [rows, k], f32 sums of squares [rows])."""
+    blocks = _c(blocks, np.uint8)
+    row_stride = (k // 256) * K_QUANT_BLOCK_BYTES[kind] if row_stride is None else row_stride
+    wide, narrow = np.empty((rows, k), np.float32), np.empty((rows, k), np.uint16)
+    sumsq = np.empty(rows, np.float32)
+    _k_quant(kind, _ptr(blocks), rows, k, row_stride, _ptr(wide), _ptr(narrow), _ptr(sumsq))
+    return wide, narrow, sumsq
 
 
 def q8_0_dequant_f32(blocks: np.ndarray, rows: int, k: int, row_stride: int | None = None):
