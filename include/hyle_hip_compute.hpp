@@ -152,20 +152,28 @@ public:
     }
     return d;
   }
-  // gguf_weight_description(kQ8_0, type, k, n) (src/compute_ops/low_precision.cc:269-297)
-  static Result<TensorDesc> gguf_q8_0_weight(DataType logical, std::int64_t k, std::int64_t n) noexcept {
-    if (k <= 0 || n <= 0 || k % 32 != 0)
+  // gguf_weight_description(type, logical_type, k, n) (include/hyle/compute/low_precision.h:181-186;
+  // block geometry src/compute_ops/low_precision.cc:22-29) for the formats this provider decodes.
+  enum class GgufQuantizedType : std::uint8_t { kQ4K = 1, kQ6K = 3, kQ8_0 = 4 };
+  static Result<TensorDesc> gguf_weight(GgufQuantizedType type, DataType logical, std::int64_t k,
+                                        std::int64_t n) noexcept {
+    const std::int64_t per_block = type == GgufQuantizedType::kQ8_0 ? 32 : 256;
+    const std::int64_t block_bytes = type == GgufQuantizedType::kQ8_0 ? 34 : (type == GgufQuantizedType::kQ4K ? 144 : 210);
+    if (k <= 0 || n <= 0 || k % per_block != 0)
       return Status::InvalidArgument("GGUF weight dimensions do not contain complete K blocks");
     TensorDesc d;
     d.c_.dtype = static_cast<std::uint8_t>(logical);
     d.c_.rank = 2;
     d.c_.storage = HYLE_HIP_STORAGE_BLOCKED;
     d.c_.block_axis = 0;
-    d.c_.elements_per_block = 32;
-    d.c_.bytes_per_block = 34;
+    d.c_.elements_per_block = static_cast<std::uint32_t>(per_block);
+    d.c_.bytes_per_block = static_cast<std::uint32_t>(block_bytes);
     d.c_.dims[0] = k; d.c_.dims[1] = n;
-    d.c_.byte_strides[0] = 34; d.c_.byte_strides[1] = k / 32 * 34;
+    d.c_.byte_strides[0] = block_bytes; d.c_.byte_strides[1] = k / per_block * block_bytes;
     return d;
+  }
+  static Result<TensorDesc> gguf_q8_0_weight(DataType logical, std::int64_t k, std::int64_t n) noexcept {
+    return gguf_weight(GgufQuantizedType::kQ8_0, logical, k, n);
   }
   bool valid() const noexcept { return c_.dtype != 0; }
   DataType data_type() const noexcept { return static_cast<DataType>(c_.dtype); }

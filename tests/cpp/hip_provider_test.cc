@@ -80,6 +80,10 @@ HOST_TEST(InfersOutputsLikeTheSchema) {
   out = infer_output_descriptions(Reduce{ReductionKind::kMaximum, *Axes::from(std::array<std::int32_t, 1>{-1}), true}, {dense(DataType::kFloat32, {3, 9})});
   REQUIRE(out.has_value());
   EXPECT((*out)[0] == dense(DataType::kFloat32, {3, 1}));
+  out = infer_output_descriptions(Q8_0DequantSumSquares{}, {*TensorDesc::gguf_weight(TensorDesc::GgufQuantizedType::kQ6K, DataType::kBFloat16, 512, 3)});
+  REQUIRE(out.has_value() && out->size() == 2);
+  EXPECT((*out)[0] == dense(DataType::kBFloat16, {3, 512}) && (*out)[1] == dense(DataType::kFloat32, {3}));
+  EXPECT(TensorDesc::gguf_weight(TensorDesc::GgufQuantizedType::kQ4K, DataType::kBFloat16, 300, 3).error().IsInvalidArgument());
   out = infer_output_descriptions(Q8_0DequantSumSquares{}, {*TensorDesc::gguf_q8_0_weight(DataType::kBFloat16, 64, 5)});
   REQUIRE(out.has_value() && out->size() == 2);
   EXPECT((*out)[0] == dense(DataType::kBFloat16, {5, 64}) && (*out)[1] == dense(DataType::kFloat32, {5}));
