@@ -69,3 +69,66 @@ def test_captured_step_replays_bit_identically():
             for t, e in zip(outs, expected):
                 got = to_host(t)
                 assert np.array_equal(got.view(np.uint8), e.view(np.uint8))
+
+
+def test_captured_two_dispatch_routes_replay_bit_identically():
+    """The routes that pass partial results through the caller's workspace (Reduce over few long
+    rows or over columns, TopK by selection and by sorted tiles), plus Cast, LayerNorm, LogSoftmax
+    and the K-quant decoder: captured once, replayed three times, same bits as eager."""
+    ctx = context()
+    rng = np.random.default_rng(1600)
+    f32 = hc.DataType.kFloat32
+    long_rows = to_device(rng.normal(0, 1, (2, 300000)).astype(np.float32), "f32")
+    columns = to_device(rng.normal(0, 1, (70000, 8)).astype(np.float32), "f32")
+    logits = to_device(rng.normal(0, 3, (4, 40000)).astype(np.float32), "f32")
+    hidden = to_device(rng.normal(0, 1, (64, 2048)).astype(np.float32), "f32")
+    raw = torch.randint(0, 256, (32, 8 * 144), dtype=torch.uint8)
+    raw.view(32, 8, 144)[:, :, 1] &= 0x3B
+    raw.view(32, 8, 144)[:, :, 3] &= 0x3B
+    weights = raw.to(DEVICE)
+    ops = [
+        (hc.Reduce(hc.ReductionKind.kSum, hc.Axes.from_([-1])), [long_rows], None),
+        (hc.Reduce(hc.ReductionKind.kMaximum, hc.Axes.from_([0])), [columns], None),
+        (hc.TopK(count=16), [logits], None),
+        (hc.TopK(count=300, largest=False), [logits], None),
+        (hc.Cast(hc.DataType.kBFloat16), [hidden], None),
+        (hc.LayerNorm(1e-5), [hidden], None),
+        (hc.Softmax(kind=hc.SoftmaxKind.kLogSoftmax), [hidden], None),
+        (hc.GgufDequantSumSquares(), [weights],
+         [hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ4K, hc.DataType.kBFloat16, 2048, 32)]),
+    ]
+    bounds = [(tio.Bound(ctx, op, descs or [tio.desc_of(t) for t in inputs]), inputs) for op, inputs, descs in ops]
+    routes = [b.prepared.route_name() for b, _ in bounds]
+    assert routes[:4] == ["reduce-row-tiles", "reduce-column-segments", "topk-select-tiles", "topk-sorted-tiles"]
+    note("eager pass of " + ", ".join(routes))
+    eager_outs = []
+    for bound, inputs in bounds:
+        outs = bound.outputs()
+        bound.submit(inputs, outs)
+        eager_outs.append(outs)
+    torch.cuda.synchronize()
+    want = [[to_host(t).copy() for t in outs] for outs in eager_outs]
+
+    note("capture the same launches into one HIP graph")
+    graph_outs = [bound.outputs() for bound, _ in bounds]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        stream = torch.cuda.current_stream().cuda_stream
+        for (bound, inputs), outs in zip(bounds, graph_outs):
+            bound.submit(inputs, outs, stream=stream)
+    for replay in range(3):
+        note(f"graph replay {replay} of the two-dispatch routes")
+        for outs in graph_outs:
+            for t in outs:
+                t.zero_()
+        for bound, _ in bounds:                      # stale partial results must not matter
+            if bound.workspace is not None:
+                bound.workspace.fill_(0xFF if replay % 2 else 0)
+        scratch = torch.randn(1 << 20, device=DEVICE).sum().item()
+        assert np.isfinite(scratch)
+        graph.replay()
+        torch.cuda.synchronize()
+        for outs, expected in zip(graph_outs, want):
+            for t, e in zip(outs, expected):
+                got = to_host(t)
+                assert np.array_equal(got.view(np.uint8), e.view(np.uint8))
