@@ -209,6 +209,21 @@ def main() -> int:
                                    torch.empty(6144, dtype=torch.float32, device=dev)]
         ops.append(Op(name, hc.GgufDequantSumSquares(), [hc.TensorDesc.gguf_weight(gguf, BF, 2048, 6144)], set_k, 16,
                       6144 * (8 * block_bytes + 2048 * 2 + 4), 6144 * 2048, "u8/bf16", in_step=False))
+    # ---- decode-time MatMul over GGUF weights: one activation row against [K, N] ----------------
+    for name, gguf, block_bytes, n_rows, sets in (("next_matvec_q4_k_bf16_ffn", hc.GgufQuantizedType.kQ4K, 144, 6144, 80),
+                                                  ("next_matvec_q6_k_bf16_vocab", hc.GgufQuantizedType.kQ6K, 210, 151936, 3)):
+        if not want(name):
+            continue
+
+        def set_mv(i, block_bytes=block_bytes, n_rows=n_rows):
+            raw = torch.randint(0, 256, (n_rows, 8 * block_bytes), dtype=torch.uint8)
+            fields = raw.view(n_rows, 8, block_bytes)
+            for at in ((1, 3) if block_bytes == 144 else (209,)):
+                fields[:, :, at] &= 0x3B
+            x = torch.empty(2048, dtype=torch.bfloat16, device=dev).normal_()
+            return [raw.to(dev), x], [torch.empty(n_rows, dtype=torch.bfloat16, device=dev)]
+        ops.append(Op(name, hc.GgufMatVec(), [hc.TensorDesc.gguf_weight(gguf, BF, 2048, n_rows), D(BF, [2048])], set_mv,
+                      sets, n_rows * (8 * block_bytes + 2) + 2048 * 2, n_rows * 2048, "u8/bf16", in_step=False))
     # ---- the next row of the path: Cast and Copy, timed beside the step -------------------------
     if want("next_cast_f32_to_bf16") or want("next_cast_bf16_to_f32"):
         x32 = np.random.default_rng(5).normal(0, 2, (8192, 2048)).astype(np.float32)

@@ -204,6 +204,7 @@ class OperationKind(enum.IntEnum):
     kTopK = 19
     kBinaryChain = 0x100
     kQ8_0DequantSumSquares = 0x101
+    kGgufMatVec = 0x102
 
 
 class UnaryKind(enum.IntEnum):
@@ -368,6 +369,12 @@ class GgufDequantSumSquares(Q8_0DequantSumSquares):
     block geometry of the input descriptor."""
 
 
+@dataclass(frozen=True)
+class GgufMatVec:
+    """MatMul(activations, GGUF weight) for a few activation rows: inputs (weight [K, N], x [K] or
+    [M, K]); output [N] or [M, N] of x's type."""
+
+
 def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
     c = capi.OpDescC()
     c.abi_version = capi.ABI_VERSION
@@ -401,6 +408,8 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
         c.op, c.count, c.axis, c.largest = OperationKind.kTopK, operation.count, operation.axis, int(operation.largest)
     elif isinstance(operation, Q8_0DequantSumSquares):
         c.op = OperationKind.kQ8_0DequantSumSquares
+    elif isinstance(operation, GgufMatVec):
+        c.op = OperationKind.kGgufMatVec
     else:
         raise StatusError(capi.UNIMPLEMENTED, f"operation {type(operation).__name__} is not served by this provider")
     if len(inputs) > capi.MAX_INPUTS:

@@ -1,0 +1,66 @@
+// Decoders of GGUF weight blocks, eight neighbouring values at a time, from block bytes in LDS
+// (or any byte-addressable memory).  Geometry from the reference
+// (src/compute_ops/low_precision.cc:22-29: Q8_0 32 elements in 34 bytes, Q4_K 256 in 144, Q6_K 256
+// in 210); the arithmetic is ggml's dequantize_row_q8_0 / _q4_K / _q6_K, restated from the
+// published block layouts (the source is not part of the reference tree):
+//   Q8_0  {f16 d; i8 qs[32]}                              y = d * q           (exact in f32)
+//   Q4_K  {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]}    y = (d * sc) * q - (dmin * m)
+//   Q6_K  {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d}   y = (d * scale) * (q - 32)
+#pragma once
+
+#include "device_common.h"
+
+namespace hyle_hip {
+namespace {
+
+constexpr int kSuper = 256;                      // values per super-block
+
+__device__ __forceinline__ float lds_f16(const unsigned char *p) {
+  return f16_to_f32((uint16_t)(p[0] | ((uint16_t)p[1] << 8)));
+}
+
+// Eight values of a Q4_K block starting at position p (a multiple of 8).
+__device__ __forceinline__ void decode_q4_k(const unsigned char *blk, uint32_t p, float (&y)[8]) {
+  const float d = lds_f16(blk), dmin = lds_f16(blk + 2);
+  const unsigned char *scales = blk + 4;
+  const uint32_t sub = p / 32, within = p % 32, chunk = sub / 2;
+  uint32_t sc, m;
+  if (sub < 4) {
+    sc = scales[sub] & 63u;
+    m = scales[sub + 4] & 63u;
+  } else {
+    sc = (scales[sub + 4] & 0xFu) | ((uint32_t)(scales[sub - 4] >> 6) << 4);
+    m = (uint32_t)(scales[sub + 4] >> 4) | ((uint32_t)(scales[sub] >> 6) << 4);
+  }
+  const float step = d * (float)sc, offset = dmin * (float)m;
+  const unsigned char *q = blk + 16 + 32 * chunk + within;
+  const uint32_t shift = (sub & 1u) * 4;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = step * (float)((q[j] >> shift) & 0xFu) - offset;
+}
+
+// Eight values of a Q6_K block starting at position p (a multiple of 8).
+__device__ __forceinline__ void decode_q6_k(const unsigned char *blk, uint32_t p, float (&y)[8]) {
+  const uint32_t half = p / 128, group = (p % 128) / 32, l = p % 32;
+  const unsigned char *ql = blk + 64 * half + l + 32 * (group & 1u);
+  const unsigned char *qh = blk + 128 + 32 * half + l;
+  const int scale = (int)(int8_t)blk[192 + 8 * half + 2 * group + l / 16];
+  const float step = lds_f16(blk + 208) * (float)scale;
+  const uint32_t low_shift = (group >> 1) * 4, high_shift = group * 2;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int q = (int)(((ql[j] >> low_shift) & 0xFu) | (((qh[j] >> high_shift) & 3u) << 4)) - 32;
+    y[j] = step * (float)q;
+  }
+}
+
+
+// Eight values of a Q8_0 block starting at position p (a multiple of 8) of its 32.
+__device__ __forceinline__ void decode_q8_0(const unsigned char *blk, uint32_t p, float (&y)[8]) {
+  const float d = lds_f16(blk);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) y[j] = (float)(int8_t)blk[2 + p + j] * d;
+}
+
+}  // namespace
+}  // namespace hyle_hip

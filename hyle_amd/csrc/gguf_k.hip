@@ -13,52 +13,13 @@
 // neighbouring values from LDS bytes and stores them as one 16-byte vector.  The output (2 bytes
 // per value) is four times the input traffic, so the byte-wise LDS reads are not what bounds it.
 #include "device_common.h"
+#include "gguf_decode.h"
 #include "kernels.h"
 
 namespace hyle_hip {
 namespace {
 
-constexpr int kSuper = 256;                      // values per super-block
 constexpr int kChunkBlocks = kBlockThreads * 8 / kSuper;  // super-blocks decoded per step: 8
-
-__device__ __forceinline__ float lds_f16(const unsigned char *p) {
-  return f16_to_f32((uint16_t)(p[0] | ((uint16_t)p[1] << 8)));
-}
-
-// Eight values of a Q4_K block starting at position p (a multiple of 8).
-__device__ __forceinline__ void decode_q4_k(const unsigned char *blk, uint32_t p, float (&y)[8]) {
-  const float d = lds_f16(blk), dmin = lds_f16(blk + 2);
-  const unsigned char *scales = blk + 4;
-  const uint32_t sub = p / 32, within = p % 32, chunk = sub / 2;
-  uint32_t sc, m;
-  if (sub < 4) {
-    sc = scales[sub] & 63u;
-    m = scales[sub + 4] & 63u;
-  } else {
-    sc = (scales[sub + 4] & 0xFu) | ((uint32_t)(scales[sub - 4] >> 6) << 4);
-    m = (uint32_t)(scales[sub + 4] >> 4) | ((uint32_t)(scales[sub] >> 6) << 4);
-  }
-  const float step = d * (float)sc, offset = dmin * (float)m;
-  const unsigned char *q = blk + 16 + 32 * chunk + within;
-  const uint32_t shift = (sub & 1u) * 4;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) y[j] = step * (float)((q[j] >> shift) & 0xFu) - offset;
-}
-
-// Eight values of a Q6_K block starting at position p (a multiple of 8).
-__device__ __forceinline__ void decode_q6_k(const unsigned char *blk, uint32_t p, float (&y)[8]) {
-  const uint32_t half = p / 128, group = (p % 128) / 32, l = p % 32;
-  const unsigned char *ql = blk + 64 * half + l + 32 * (group & 1u);
-  const unsigned char *qh = blk + 128 + 32 * half + l;
-  const int scale = (int)(int8_t)blk[192 + 8 * half + 2 * group + l / 16];
-  const float step = lds_f16(blk + 208) * (float)scale;
-  const uint32_t low_shift = (group >> 1) * 4, high_shift = group * 2;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const int q = (int)(((ql[j] >> low_shift) & 0xFu) | (((qh[j] >> high_shift) & 3u) << 4)) - 32;
-    y[j] = step * (float)q;
-  }
-}
 
 // Bytes -> LDS with the widest loads the address allows (Q4_K rows of a 16-byte aligned tensor
 // always take words; Q6_K blocks are only 2-byte aligned as a rule).

@@ -179,6 +179,17 @@ struct KQuantParams {
 hipError_t launch_k_quant_dequant(const KQuantParams &p, const void *blocks, void *out, float *sumsq,
                                   hipStream_t stream);
 
+// y[m][n] = sum_k w[n][k] * x[m][k], w a GGUF weight (kind 0 Q4_K, 1 Q6_K, 2 Q8_0), x [m, k] dense.
+struct MatVecParams {
+  uint64_t rows = 0;        // N
+  uint32_t k = 0, m = 0;
+  uint64_t row_stride = 0;  // bytes between physical weight rows
+  uint8_t kind = 0;
+};
+size_t gguf_matvec_shared_bytes(uint32_t m, uint32_t k);
+hipError_t launch_gguf_matvec(Elem x_type, const MatVecParams &p, const void *weights, const void *x, void *y,
+                              hipStream_t stream);
+
 // Q8_0 rows of k/32 blocks {f16 d; int8 qs[32]} -> bf16 [rows, k] + f32 sumsq[rows].
 struct Q8Params {
   uint64_t rows = 0;

@@ -442,6 +442,27 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
       *out_count = 2;
       return make_dense(HYLE_HIP_DTYPE_F32, &in[0].dims[1], 1, &outs[1]);
     }
+    case HYLE_HIP_OP_GGUF_MATVEC: {
+      if ((s = expect_inputs(r, 2, 2)) != HYLE_HIP_OK) return s;
+      const bool q8_0 = in[0].elements_per_block == 32 && in[0].bytes_per_block == 34;
+      const bool q4_k = in[0].elements_per_block == 256 && in[0].bytes_per_block == 144;
+      const bool q6_k = in[0].elements_per_block == 256 && in[0].bytes_per_block == 210;
+      if (in[0].storage != HYLE_HIP_STORAGE_BLOCKED || !(q8_0 || q4_k || q6_k) || in[0].rank != 2 ||
+          in[0].block_axis != 0)
+        return fail(HYLE_HIP_INVALID_ARGUMENT,
+                    "GGUF weight must be blocked [K, N] storage with Q8_0, Q4_K or Q6_K blocks on axis 0");
+      // MatMul contraction (src/compute_ops/operation.cc, kMatMul): the last axis of the
+      // activations meets the first logical axis of the weight
+      if (!is_floating(in[1].dtype) || in[1].rank < 1 || in[1].rank > 2 ||
+          in[1].dims[in[1].rank - 1] != in[0].dims[0])
+        return fail(HYLE_HIP_INVALID_ARGUMENT,
+                    "activations must be floating [K] or [M, K] with K the weight's first logical extent");
+      int64_t dims[2];
+      int rank = 0;
+      if (in[1].rank == 2) dims[rank++] = in[1].dims[0];
+      dims[rank++] = in[0].dims[1];
+      return make_dense(in[1].dtype, dims, rank, &outs[0]);
+    }
     default:
       return fail(HYLE_HIP_UNIMPLEMENTED, "operation kind %u is not served by this provider", r.op);
   }
@@ -462,6 +483,7 @@ enum class Route : uint8_t {
   kTopK,
   kQ8Dequant,
   kKQuantDequant,
+  kGgufMatVec,
   kCast,
 };
 
@@ -478,6 +500,7 @@ const char *route_name(Route r) {
     case Route::kTopK: return "topk-sorted-tiles";
     case Route::kQ8Dequant: return "q8_0-dequant-rows";
     case Route::kKQuantDequant: return "k-quant-dequant-rows";
+    case Route::kGgufMatVec: return "gguf-matvec-rows";
     case Route::kCast: return "cast-copy";
   }
   return "?";
@@ -520,6 +543,7 @@ struct hyle_hip_plan {
   TopKParams topk;
   Q8Params q8;
   KQuantParams kquant;
+  MatVecParams matvec;
   CastParams cast;
   // Cast and Copy take no alias at all (AliasPolicy::kNone, src/compute_ops/operation.cc:935-957):
   // the bytes the input and the output occupy must not overlap.
@@ -899,6 +923,32 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }
+    case HYLE_HIP_OP_GGUF_MATVEC: {
+      const int64_t k = in[0].dims[0], n = in[0].dims[1];
+      const int64_t per_block = in[0].elements_per_block, block_bytes = in[0].bytes_per_block;
+      if (!to_elem(in[1].dtype, &p->elem) || !is_plain(in[1]) || !is_dense(in[1]))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec requires dense plain float32/float16/bfloat16 activations");
+      if (in[0].byte_strides[0] != block_bytes)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF blocks of a row must be contiguous (block stride = block bytes)");
+      if (k > 0 && n > 1 && in[0].byte_strides[1] < (k / per_block) * block_bytes)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "GGUF row stride is shorter than a row of blocks");
+      const int64_t m = in[1].rank == 2 ? in[1].dims[0] : 1;
+      if (m > 8) return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec serves at most 8 activation rows");
+      if ((uint64_t)k * (uint64_t)n > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec requires at most INT32_MAX weight elements");
+      if (gguf_matvec_shared_bytes((uint32_t)m, (uint32_t)k) > 64 * 1024)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec keeps the activations in LDS: M * K is too large");
+      if (p->output_elements[0] == 0) return HYLE_HIP_OK;
+      p->route = Route::kGgufMatVec;
+      p->matvec.rows = (uint64_t)n;
+      p->matvec.k = (uint32_t)k;
+      p->matvec.m = (uint32_t)m;
+      p->matvec.row_stride = (uint64_t)in[0].byte_strides[1];
+      p->matvec.kind = per_block == 32 ? 2 : (block_bytes == 144 ? 0 : 1);
+      p->input_alignment[0] = 1;
+      p->dispatches = 1;
+      return HYLE_HIP_OK;
+    }
     case HYLE_HIP_OP_COPY:
     case HYLE_HIP_OP_CAST: {
       // src/compute_provider_native/cast.cc:127-176,256-279 (admitted pairs, plain input, dense
@@ -1198,6 +1248,9 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
       break;
     case Route::kKQuantDequant:
       err = launch_k_quant_dequant(plan->kquant, inputs[0], outputs[0], static_cast<float *>(outputs[1]), stream);
+      break;
+    case Route::kGgufMatVec:
+      err = launch_gguf_matvec(plan->elem, plan->matvec, inputs[0], inputs[1], outputs[0], stream);
       break;
     case Route::kCast:
       err = launch_cast(plan->cast, inputs[0], outputs[0], vector, stream);

@@ -90,7 +90,13 @@ typedef enum hyle_hip_op_kind {
   /* The same operation under its general name: the weight may also be GGUF Q4_K (256-element,
    * 144-byte blocks) or Q6_K (256-element, 210-byte blocks); the block geometry of in0 selects
    * the decoder (src/compute_ops/low_precision.cc:22-29). */
-  HYLE_HIP_OP_GGUF_DEQUANT_SUMSQ = 0x101
+  HYLE_HIP_OP_GGUF_DEQUANT_SUMSQ = 0x101,
+  /* MatMul(in1, in0) for token-by-token decoding: in0 a GGUF weight (Q8_0, Q4_K, Q6_K), logical
+   * [K, N]; in1 dense f32 / f16 / bf16 activations [K] or [M, K] with M <= 8; out0 [N] or [M, N]
+   * of in1's type.  Weights are decoded exactly, products and sums are f32 (ggml, which serves
+   * this in the reference, quantises the activations to 8 bits first: its rounding is not
+   * reproduced). */
+  HYLE_HIP_OP_GGUF_MATVEC = 0x102
 } hyle_hip_op_kind;
 
 /* UnaryKind (include/hyle/compute/operation.h:57-73) */

@@ -944,6 +944,45 @@ void hyle_oracle_k_quant_dequant(int kind, const void *blocks, size_t rows, size
   }
 }
 
+/* y[m][n] = sum_k w[n][k] * x[m][k] with w the exact f32 decode of a GGUF row
+ * (kind 0 Q4_K, 1 Q6_K, 2 Q8_0) and double accumulation: the value the f32
+ * kernel is held to within its summation-order bound.  `magnitude` (optional)
+ * receives sum_k |w * x|, the scale of that bound.  This is MatMul with exact
+ * weights; ggml's 8-bit activation quantisation is not restated. */
+void hyle_oracle_gguf_matvec(int kind, const void *blocks, size_t rows, size_t k,
+                             size_t row_stride_bytes, const float *x, size_t m,
+                             double *out, double *magnitude) {
+  const unsigned char *base = (const unsigned char *)blocks;
+  float *w = (float *)malloc((k ? k : 1) * sizeof(float));
+  if (w == NULL) return;
+  for (size_t r = 0; r < rows; ++r) {
+    const unsigned char *row = base + r * row_stride_bytes;
+    if (kind == 2) {
+      for (size_t b = 0; b < k / 32; ++b) {
+        const unsigned char *blk = row + b * 34;
+        const float d = hyle_oracle_f16_to_f32((uint16_t)(blk[0] | ((uint16_t)blk[1] << 8)));
+        for (size_t j = 0; j < 32; ++j) w[b * 32 + j] = (float)(int8_t)blk[2 + j] * d;
+      }
+    } else {
+      for (size_t b = 0; b < k / 256; ++b) {
+        if (kind == 0) q4_k_block_f32(row + b * 144, w + b * 256);
+        else q6_k_block_f32(row + b * 210, w + b * 256);
+      }
+    }
+    for (size_t i = 0; i < m; ++i) {
+      double sum = 0.0, size = 0.0;
+      for (size_t j = 0; j < k; ++j) {
+        const double term = (double)w[j] * (double)x[i * k + j];
+        sum += term;
+        size += fabs(term);
+      }
+      out[i * rows + r] = sum;
+      if (magnitude) magnitude[i * rows + r] = size;
+    }
+  }
+  free(w);
+}
+
 void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
                                   size_t row_stride_bytes, float *out) {
   const unsigned char *base = (const unsigned char *)blocks;

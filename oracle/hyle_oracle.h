@@ -265,6 +265,14 @@ void hyle_oracle_k_quant_dequant(int kind, const void *blocks, size_t rows, size
                                  size_t row_stride_bytes, float *out_f32, uint16_t *out_bf16,
                                  float *sumsq);
 
+/* y[m][n] = sum_k w[n][k] * x[m][k] for GGUF rows (kind 0 Q4_K, 1 Q6_K, 2
+ * Q8_0) decoded exactly, accumulated in double; `magnitude` (optional) gets
+ * sum_k |w * x|.  MatMul with exact weights, not ggml's quantised-activation
+ * product. */
+void hyle_oracle_gguf_matvec(int kind, const void *blocks, size_t rows, size_t k,
+                             size_t row_stride_bytes, const float *x, size_t m,
+                             double *out, double *magnitude);
+
 void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
                                   size_t row_stride_bytes, float *out);
 

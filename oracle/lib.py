@@ -87,6 +87,7 @@ _q8_f32 = _sig("hyle_oracle_q8_0_dequant_f32", None, _vp, _sz, _sz, _sz, _vp)
 _reduce_axes = _sig("hyle_oracle_reduce", None, C.c_int, C.c_int, _vp, C.c_int, _i64p, _i64p, C.c_uint32, _vp)
 _topk = _sig("hyle_oracle_topk", None, C.c_int, _vp, C.c_int, _i64p, _i64p, C.c_int, _sz, C.c_int, _vp, _vp)
 _k_quant = _sig("hyle_oracle_k_quant_dequant", None, C.c_int, _vp, _sz, _sz, _sz, _vp, _vp, _vp)
+_matvec = _sig("hyle_oracle_gguf_matvec", None, C.c_int, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _vp)
 _cast = _sig("hyle_oracle_cast", C.c_int, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int, _vp)
 
 
@@ -407,6 +408,22 @@ def k_quant_dequant(kind: int, blocks: np.ndarray, rows: int, k: int, row_stride
     sumsq = np.empty(rows, np.float32)
     _k_quant(kind, _ptr(blocks), rows, k, row_stride, _ptr(wide), _ptr(narrow), _ptr(sumsq))
     return wide, narrow, sumsq
+
+
+Q8_0 = 2
+GGUF_BLOCK = {Q4_K: (256, 144), Q6_K: (256, 210), Q8_0: (32, 34)}
+
+
+def gguf_matvec(kind: int, blocks: np.ndarray, rows: int, k: int, x: np.ndarray, row_stride: int | None = None):
+    """(float64 [m, rows] products of exactly decoded rows with x [m, k] f32, float64 sums of |w x|)."""
+    blocks = _c(blocks, np.uint8)
+    x = _c(np.atleast_2d(x), np.float32)
+    per_block, block_bytes = GGUF_BLOCK[kind]
+    row_stride = (k // per_block) * block_bytes if row_stride is None else row_stride
+    out = np.empty((x.shape[0], rows), np.float64)
+    magnitude = np.empty_like(out)
+    _matvec(kind, _ptr(blocks), rows, k, row_stride, _ptr(x), x.shape[0], _ptr(out), _ptr(magnitude))
+    return out, magnitude
 
 
 def q8_0_dequant_f32(blocks: np.ndarray, rows: int, k: int, row_stride: int | None = None):
