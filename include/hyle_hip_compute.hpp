@@ -282,9 +282,14 @@ struct TopK final { std::size_t count = 1; std::int32_t axis = -1; bool largest 
 // Fused forms of this provider (custom operations on the reference side).
 struct BinaryChain final { BinaryKind first = BinaryKind::kAdd; BinaryKind second = BinaryKind::kMultiply; };
 struct Q8_0DequantSumSquares final {};
+// The same operation under its general name (Q8_0, Q4_K or Q6_K weights, told apart by the block
+// geometry of the descriptor), and MatMul(x, W) over such a weight for up to 8 activation rows
+// (inputs: weight, activations).
+using GgufDequantSumSquares = Q8_0DequantSumSquares;
+struct GgufMatVec final {};
 
 using Operation = std::variant<Copy, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
-                               Q8_0DequantSumSquares>;
+                               Q8_0DequantSumSquares, GgufMatVec>;
 
 namespace detail {
 inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *inputs, std::size_t count) noexcept {
@@ -323,6 +328,7 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
       r.op = HYLE_HIP_OP_BINARY_CHAIN; r.kind = static_cast<std::uint32_t>(o.first); r.kind2 = static_cast<std::uint32_t>(o.second);
     }
     void operator()(const Q8_0DequantSumSquares &) const { r.op = HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ; }
+    void operator()(const GgufMatVec &) const { r.op = HYLE_HIP_OP_GGUF_MATVEC; }
   };
   std::visit(Fill{r}, operation);
   r.input_count = static_cast<std::uint32_t>(count);

@@ -84,6 +84,12 @@ HOST_TEST(InfersOutputsLikeTheSchema) {
   REQUIRE(out.has_value() && out->size() == 2);
   EXPECT((*out)[0] == dense(DataType::kBFloat16, {3, 512}) && (*out)[1] == dense(DataType::kFloat32, {3}));
   EXPECT(TensorDesc::gguf_weight(TensorDesc::GgufQuantizedType::kQ4K, DataType::kBFloat16, 300, 3).error().IsInvalidArgument());
+  out = infer_output_descriptions(GgufMatVec{}, {*TensorDesc::gguf_weight(TensorDesc::GgufQuantizedType::kQ4K, DataType::kBFloat16, 512, 7),
+                                                 dense(DataType::kFloat32, {3, 512})});
+  REQUIRE(out.has_value() && out->size() == 1);
+  EXPECT((*out)[0] == dense(DataType::kFloat32, {3, 7}));
+  EXPECT(infer_output_descriptions(GgufMatVec{}, {*TensorDesc::gguf_weight(TensorDesc::GgufQuantizedType::kQ4K, DataType::kBFloat16, 512, 7),
+                                                  dense(DataType::kFloat32, {3, 256})}).error().IsInvalidArgument());
   out = infer_output_descriptions(Q8_0DequantSumSquares{}, {*TensorDesc::gguf_q8_0_weight(DataType::kBFloat16, 64, 5)});
   REQUIRE(out.has_value() && out->size() == 2);
   EXPECT((*out)[0] == dense(DataType::kBFloat16, {5, 64}) && (*out)[1] == dense(DataType::kFloat32, {5}));
