@@ -277,7 +277,7 @@ hipError_t run_kind(const ReduceParams &p, const void *x, void *y, void *workspa
         rows_launch<T, T, kKind>(x, y, p.rows, p.width, 1, p.width, p.divisor, vector, s);
       } else {
         rows_launch<T, F32, kPartial>(x, workspace, p.rows, p.width, p.tiles, p.tile_width, 1.0f, vector, s);
-        rows_launch<F32, T, kKind>(workspace, y, p.rows, p.tiles, 1, p.tiles, p.divisor, false, s);
+        rows_launch<F32, T, kKind>(workspace, y, p.rows, p.tiles, 1, p.tiles, p.divisor, p.tiles % 4 == 0, s);
       }
       break;
     }
