@@ -105,6 +105,11 @@ def main() -> int:
             self.turn = (self.turn + 1) % len(self.sets)
             self.bound.invocation.submit(on_stream, inputs, outputs)
 
+        def launch_first_set(self, on_stream):
+            """Enqueue on the first buffer set only: the operands stay in the memory-side cache."""
+            inputs, outputs = self.addresses[0]
+            self.bound.invocation.submit(on_stream, inputs, outputs)
+
     D = hc.TensorDesc.dense
     F32, BF = hc.DataType.kFloat32, hc.DataType.kBFloat16
     ops = []
@@ -381,12 +386,31 @@ def main() -> int:
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / reps
         gbps = op.credited / us / 1e3
-        per_op.append({"op": op.name, "in_step": op.in_step, "route": op.route, "dtype": op.dtype,
-                       "bytes": op.bytes, "bytes_credited": op.credited,
-                       "buffer_sets": len(op.sets), "launches": reps, "us": round(us, 3),
-                       "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                       "gelem_per_s": round(op.elements / us / 1e3, 2)})
+        entry = {"op": op.name, "in_step": op.in_step, "route": op.route, "dtype": op.dtype,
+                 "bytes": op.bytes, "bytes_credited": op.credited,
+                 "buffer_sets": len(op.sets), "launches": reps, "us": round(us, 3),
+                 "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                 "gelem_per_s": round(op.elements / us / 1e3, 2)}
         del graph
+        if op.in_step and len(op.sets) > 1:
+            # the same launches on one buffer set: operands served by the 256 MB memory-side cache
+            cached = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(cached):
+                s = torch.cuda.current_stream().cuda_stream
+                for _ in range(reps):
+                    op.launch_first_set(s)
+            cached.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            cached.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            us_cached = e0.elapsed_time(e1) * 1e3 / reps
+            entry["us_cached"] = round(us_cached, 3)
+            entry["gbps_cached"] = round(op.credited / us_cached / 1e3, 1)
+            del cached
+        per_op.append(entry)
 
     if args.copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -418,12 +442,30 @@ def main() -> int:
                      "credited_bytes": dominant.credited, "traffic": TRAFFIC.get(dominant.name)},
         "per_op": per_op,
     }
+    result["device"] = device_state(torch)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(args, step_ops, np, torch, wl)
     if args.file_stream_mib > 0:
         result["file_stream"] = file_stream_rate(args.file_stream_mib, ctx, torch, dev)
     print(json.dumps(result))
     return 0
+
+
+def device_state(torch):
+    """Name, compute units and, where the tool answers, the clocks and power state during the run."""
+    import subprocess
+    props = torch.cuda.get_device_properties(0)
+    state = {"name": props.name, "compute_units": props.multi_processor_count,
+             "memory_gib": round(props.total_memory / 2 ** 30, 1)}
+    try:
+        shown = subprocess.run(["rocm-smi", "--showclocks", "--showperflevel", "--json"], capture_output=True,
+                               text=True, timeout=20)
+        card = next(iter(json.loads(shown.stdout).values()))
+        state["rocm_smi"] = {key: value for key, value in card.items()
+                             if any(word in key.lower() for word in ("sclk", "mclk", "fclk", "performance level"))}
+    except Exception as error:  # the tool is optional: the figures stand without it
+        state["rocm_smi"] = f"unavailable ({type(error).__name__})"
+    return state
 
 
 def file_stream_rate(mib, ctx, torch, dev):
