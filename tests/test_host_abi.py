@@ -178,6 +178,19 @@ def test_infer_q8_0_descriptor():
         hc.TensorDesc.gguf_q8_0_weight(DT.kBFloat16, 2047, 8)
 
 
+def test_gguf_weight_descriptor_needs_whole_positive_blocks():
+    # src/compute_ops/low_precision.cc:277-279: K and N positive, K a whole number of blocks -- so an
+    # empty contraction (K = 0) never reaches a GGUF route
+    for kind, per_block, block_bytes in ((hc.GgufQuantizedType.kQ8_0, 32, 34), (hc.GgufQuantizedType.kQ4K, 256, 144),
+                                         (hc.GgufQuantizedType.kQ6K, 256, 210)):
+        w = hc.TensorDesc.gguf_weight(kind, DT.kBFloat16, 4 * per_block, 3)
+        assert w.byte_strides == (block_bytes, 4 * block_bytes)
+        for k, n in ((0, 3), (4 * per_block, 0), (-per_block, 3), (per_block + 1, 3)):
+            with pytest.raises(hc.StatusError) as err:
+                hc.TensorDesc.gguf_weight(kind, DT.kBFloat16, k, n)
+            assert err.value.is_invalid_argument()
+
+
 # ---------------------------------------------------------------- admission ----
 def test_routes_alias_support_and_cost_facts():
     a, b, s = D(DT.kFloat32, [4096, 2048]), D(DT.kFloat32, [2048]), D(DT.kFloat32, [1])
