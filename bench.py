@@ -452,19 +452,41 @@ def main() -> int:
 
 
 def device_state(torch):
-    """Name, compute units and, where the tool answers, the clocks and power state during the run."""
-    import subprocess
+    """Name, compute units and the clock and power state the driver shows in sysfs during the run
+    (plain file reads: no child process is started from a process that holds the GPU)."""
+    import glob
     props = torch.cuda.get_device_properties(0)
     state = {"name": props.name, "compute_units": props.multi_processor_count,
              "memory_gib": round(props.total_memory / 2 ** 30, 1)}
-    try:
-        shown = subprocess.run(["rocm-smi", "--showclocks", "--showperflevel", "--json"], capture_output=True,
-                               text=True, timeout=20)
-        card = next(iter(json.loads(shown.stdout).values()))
-        state["rocm_smi"] = {key: value for key, value in card.items()
-                             if any(word in key.lower() for word in ("sclk", "mclk", "fclk", "performance level"))}
-    except Exception as error:  # the tool is optional: the figures stand without it
-        state["rocm_smi"] = f"unavailable ({type(error).__name__})"
+
+    def active_level(path):
+        # pp_dpm_* list one level per line, the active one marked with "*"
+        with open(path) as levels:
+            marked = [line.split(":", 1)[1].replace("*", "").strip() for line in levels if "*" in line]
+        return marked[0] if marked else None
+
+    sysfs = {}
+    for card in sorted(glob.glob("/sys/class/drm/card[0-9]*/device")):
+        try:
+            with open(card + "/vendor") as vendor:
+                if vendor.read().strip() != "0x1002":
+                    continue
+            entry = {}
+            for name in ("pp_dpm_sclk", "pp_dpm_mclk", "pp_dpm_fclk"):
+                try:
+                    entry[name[len("pp_dpm_"):]] = active_level(f"{card}/{name}")
+                except OSError:
+                    pass
+            try:
+                with open(card + "/power_dpm_force_performance_level") as level:
+                    entry["performance_level"] = level.read().strip()
+            except OSError:
+                pass
+            if entry:
+                sysfs[card.split("/")[4]] = entry
+        except OSError:
+            continue
+    state["sysfs"] = sysfs if sysfs else "unavailable"
     return state
 
 

@@ -157,6 +157,244 @@ __device__ __forceinline__ void row_q8_0(const unsigned char *row, uint32_t k, c
   }
 }
 
+// ---------------------------------------------------------------------------------
+// One activation row, Q6_K, K a multiple of 2048: x in registers.
+//
+// A wave covers 2048 values of a row at a time: 16 halves of 128 values, four lanes per half.
+// Lane (half, j) owns positions l = 8 j .. 8 j + 7 of each of the half's four groups
+// (l, l + 32, l + 64, l + 96): 8 bytes of ql[64 h + l], 8 of ql[64 h + 32 + l], 8 of qh[32 h + l],
+// the half's eight scales and d.  Those positions are the same for every row, so the lane keeps
+// its 32 activations in registers and no LDS is used.  The six-bit quants are put together four
+// at a time inside a 32-bit word, as bytes holding 4 (q - 32) in two's complement (q < 64, so
+// q << 2 stays inside its byte and bit 7 is the sign after toggling it), which one converting
+// instruction per value sign-extends; the factor 1/4 goes into the group's scale.  A group's
+// sixteen values share one scale, so the lane adds up q x per group and scales the sum:
+//   y = sum over groups of (d * scale) * sum (q - 32) x
+// with f32 products and sums.  The loads of the next row are issued before the current row is
+// worked on.
+typedef uint32_t u32x2_at2 __attribute__((ext_vector_type(2), aligned(2)));
+typedef uint16_t u16_at2 __attribute__((aligned(2)));
+
+struct Q6Raw {
+  uint32_t low[2], high[2], top[2], scales[2], d;
+};
+
+// Byte offsets of a lane's share within a row, for the pass (2048 values) it works on.
+struct Q6Offsets {
+  uint32_t low, top, scales, d;
+};
+__device__ __forceinline__ Q6Offsets q6_offsets(uint32_t pass, uint32_t lane) {
+  const uint32_t half_index = pass * 16 + lane / 4, j = lane % 4;
+  const uint32_t block = (half_index / 2) * 210, half = half_index % 2;
+  return Q6Offsets{block + 64 * half + 8 * j, block + 128 + 32 * half + 8 * j, block + 192 + 8 * half, block + 208};
+}
+
+// `row` is the same for the whole wave (a scalar base), the offsets are the lane's own.
+__device__ __forceinline__ Q6Raw q6_load(const unsigned char *row, const Q6Offsets &at) {
+  const u32x2_at2 low = __builtin_nontemporal_load(reinterpret_cast<const u32x2_at2 *>(row + at.low));
+  const u32x2_at2 high = __builtin_nontemporal_load(reinterpret_cast<const u32x2_at2 *>(row + at.low + 32));
+  const u32x2_at2 top = __builtin_nontemporal_load(reinterpret_cast<const u32x2_at2 *>(row + at.top));
+  const u32x2_at2 scales = __builtin_nontemporal_load(reinterpret_cast<const u32x2_at2 *>(row + at.scales));
+  Q6Raw raw;
+  raw.low[0] = low.x, raw.low[1] = low.y;
+  raw.high[0] = high.x, raw.high[1] = high.y;
+  raw.top[0] = top.x, raw.top[1] = top.y;
+  raw.scales[0] = scales.x, raw.scales[1] = scales.y;
+  raw.d = __builtin_nontemporal_load(reinterpret_cast<const u16_at2 *>(row + at.d));
+  return raw;
+}
+
+// sum over four bytes of word (each an int8) times x[0..3], added to sum
+__device__ __forceinline__ float dot_bytes(uint32_t word, const float *x, float sum) {
+#pragma unroll
+  for (int t = 0; t < 4; ++t) sum = __builtin_fmaf((float)(int)(signed char)(word >> (8 * t)), x[t], sum);
+  return sum;
+}
+
+__device__ __forceinline__ float q6_dot(const Q6Raw &raw, const float (&x)[4][8], uint32_t j) {
+  float group[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    const uint32_t low = raw.low[w], high = raw.high[w], top = raw.top[w];
+    // bytes of 4 q: bits 2..5 from a nibble of ql, bits 6..7 from two bits of qh
+    const uint32_t q0 = ((low << 2) & 0x3C3C3C3Cu) | ((top << 6) & 0xC0C0C0C0u);
+    const uint32_t q1 = ((high << 2) & 0x3C3C3C3Cu) | ((top << 4) & 0xC0C0C0C0u);
+    const uint32_t q2 = ((low >> 2) & 0x3C3C3C3Cu) | ((top << 2) & 0xC0C0C0C0u);
+    const uint32_t q3 = ((high >> 2) & 0x3C3C3C3Cu) | (top & 0xC0C0C0C0u);
+    // toggling bit 7 subtracts 4 * 32 modulo 256: the byte is 4 (q - 32) as an int8
+    group[0] = dot_bytes(q0 ^ 0x80808080u, &x[0][4 * w], group[0]);
+    group[1] = dot_bytes(q1 ^ 0x80808080u, &x[1][4 * w], group[1]);
+    group[2] = dot_bytes(q2 ^ 0x80808080u, &x[2][4 * w], group[2]);
+    group[3] = dot_bytes(q3 ^ 0x80808080u, &x[3][4 * w], group[3]);
+  }
+  const float d = f16_to_f32((uint16_t)raw.d) * 0.25f;
+  // scales[2 g + l / 16] of this half, l / 16 = j / 2
+  float total = 0.0f;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const uint32_t word = raw.scales[g / 2] >> (16 * (g % 2) + 8 * (j / 2));
+    total = __builtin_fmaf(d * (float)(int)(signed char)word, group[g], total);
+  }
+  return total;
+}
+
+constexpr int kQ6Depth = 4;  // rows of a wave whose bytes are in flight
+
+// The grid is sized to the machine, not to the weight: wave w of W takes rows w, w + W, ...
+template <class TX, int kPasses>
+__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q6_k_single(const unsigned char *weights, const void *x,
+                                                                         void *y, uint32_t rows, uint64_t row_stride) {
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  // the wave's number as a scalar, so that row addresses are scalar too
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  const uint32_t j = lane % 4;
+  float xs[kPasses][4][8];
+  Q6Offsets at[kPasses];
+#pragma unroll
+  for (int pass = 0; pass < kPasses; ++pass) {
+    at[pass] = q6_offsets(pass, lane);
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int t = 0; t < 8; ++t)
+        xs[pass][g][t] = Traits<TX>::load(x, (size_t)pass * 2048 + (lane / 4) * 128 + 32 * g + 8 * j + t);
+  }
+  const uint32_t stride = gridDim.x * kWavesPerBlock;
+  const uint32_t first = blockIdx.x * kWavesPerBlock + wave;
+  if (first >= rows) return;
+  // A row past the end is replaced by the wave's first row: a valid address whose bytes go unused.
+  Q6Raw ring[kQ6Depth][kPasses];
+#pragma unroll
+  for (int d = 0; d < kQ6Depth; ++d) {
+    const uint64_t wanted = (uint64_t)first + (uint64_t)d * stride;
+    const uint32_t row = wanted < rows ? (uint32_t)wanted : first;
+#pragma unroll
+    for (int pass = 0; pass < kPasses; ++pass) ring[d][pass] = q6_load(weights + (size_t)row * row_stride, at[pass]);
+  }
+  for (uint64_t base = first; base < rows; base += (uint64_t)kQ6Depth * stride) {
+#pragma unroll
+    for (int d = 0; d < kQ6Depth; ++d) {
+      const uint64_t row = base + (uint64_t)d * stride;
+      if (row >= rows) break;
+      Q6Raw current[kPasses];
+#pragma unroll
+      for (int pass = 0; pass < kPasses; ++pass) current[pass] = ring[d][pass];
+      const uint64_t wanted = row + (uint64_t)kQ6Depth * stride;
+      const uint32_t following = wanted < rows ? (uint32_t)wanted : first;
+#pragma unroll
+      for (int pass = 0; pass < kPasses; ++pass)
+        ring[d][pass] = q6_load(weights + (size_t)following * row_stride, at[pass]);
+      float total = 0.0f;
+#pragma unroll
+      for (int pass = 0; pass < kPasses; ++pass) total += q6_dot(current[pass], xs[pass], j);
+      total = group_sum<kWaveLanes>(total);
+      if (lane == 0) Traits<TX>::store(y, (size_t)row, total);
+    }
+  }
+}
+
+// The same arithmetic with every cache line requested once: the wave reads a row as whole
+// 16-byte vectors (lane i takes vectors i, i + 64, ...: 1680 bytes are 105 vectors), keeps the rows
+// still in flight in registers, and hands the bytes to the lanes that decode them through a
+// region of LDS that only this wave touches.  (Reading each lane's 8-byte pieces straight from
+// memory asks for every line several times while it is still on its way, and the address unit
+// and those waits, not the arithmetic, set the time: 89 us for [2048 -> 151936].)  LDS executes
+// one wave's instructions in order, so the stores of a row and the loads that follow need no
+// barrier, and the next row is stored only after this row's loads were issued.
+template <int kPasses> struct Q6Row {
+  static constexpr int kVectors = kPasses * 105;               // 16-byte vectors in a row
+  static constexpr int kLoads = (kVectors + kWaveLanes - 1) / kWaveLanes;
+  static constexpr int kSlotBytes = kLoads * kWaveLanes * 16;  // LDS bytes of one wave
+  u32x4 v[kLoads];
+};
+
+template <int kPasses>
+__device__ __forceinline__ Q6Row<kPasses> q6_row_load(const unsigned char *row, uint32_t lane) {
+  Q6Row<kPasses> r;
+#pragma unroll
+  for (int i = 0; i < Q6Row<kPasses>::kLoads; ++i) {
+    const uint32_t wanted = lane + i * kWaveLanes;  // past the row: its last vector again (stored to LDS, never read)
+    const uint32_t vec = wanted < (uint32_t)Q6Row<kPasses>::kVectors ? wanted : Q6Row<kPasses>::kVectors - 1;
+    r.v[i] = load16_stream(row, vec);
+  }
+  return r;
+}
+
+// Eight bytes at a 2-byte aligned LDS offset, as three aligned words and two byte-wise funnel
+// shifts (an LDS read that is not naturally aligned stalls: measured, four such 8-byte reads per
+// lane made LDS the limit of the kernel).
+__device__ __forceinline__ void lds_piece(const unsigned char *slot, uint32_t offset, uint32_t (&out)[2]) {
+  const uint32_t *words = reinterpret_cast<const uint32_t *>(slot + (offset & ~3u));
+  const uint32_t w0 = words[0], w1 = words[1], w2 = words[2];
+  out[0] = __builtin_amdgcn_alignbyte(w1, w0, offset & 3u);
+  out[1] = __builtin_amdgcn_alignbyte(w2, w1, offset & 3u);
+}
+
+__device__ __forceinline__ Q6Raw q6_from_lds(const unsigned char *slot, const Q6Offsets &at) {
+  Q6Raw raw;
+  lds_piece(slot, at.low, raw.low);
+  lds_piece(slot, at.low + 32, raw.high);
+  lds_piece(slot, at.top, raw.top);
+  lds_piece(slot, at.scales, raw.scales);
+  raw.d = *reinterpret_cast<const uint16_t *>(slot + at.d);
+  return raw;
+}
+
+template <class TX, int kPasses>
+__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q6_k_lines(const unsigned char *weights, const void *x,
+                                                                        void *y, uint32_t rows, uint64_t row_stride) {
+  using Row = Q6Row<kPasses>;
+  __shared__ __align__(16) unsigned char slots[kWavesPerBlock][Row::kSlotBytes];
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  unsigned char *slot = slots[wave];
+  const uint32_t j = lane % 4;
+  float xs[kPasses][4][8];
+  Q6Offsets at[kPasses];
+#pragma unroll
+  for (int pass = 0; pass < kPasses; ++pass) {
+    at[pass] = q6_offsets(pass, lane);
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int t = 0; t < 8; ++t)
+        xs[pass][g][t] = Traits<TX>::load(x, (size_t)pass * 2048 + (lane / 4) * 128 + 32 * g + 8 * j + t);
+  }
+  const uint32_t stride = gridDim.x * kWavesPerBlock;
+  const uint32_t first = blockIdx.x * kWavesPerBlock + wave;
+  if (first >= rows) return;
+  Row ring[kQ6Depth];
+#pragma unroll
+  for (int d = 0; d < kQ6Depth; ++d) {
+    const uint64_t wanted = (uint64_t)first + (uint64_t)d * stride;
+    const uint32_t row = wanted < rows ? (uint32_t)wanted : first;
+    ring[d] = q6_row_load<kPasses>(weights + (size_t)row * row_stride, lane);
+  }
+  for (uint64_t base = first; base < rows; base += (uint64_t)kQ6Depth * stride) {
+#pragma unroll
+    for (int d = 0; d < kQ6Depth; ++d) {
+      const uint64_t row = base + (uint64_t)d * stride;
+      if (row >= rows) break;
+#pragma unroll
+      for (int i = 0; i < Row::kLoads; ++i)
+        *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = ring[d].v[i];
+      const uint64_t wanted = row + (uint64_t)kQ6Depth * stride;
+      const uint32_t following = wanted < rows ? (uint32_t)wanted : first;
+      ring[d] = q6_row_load<kPasses>(weights + (size_t)following * row_stride, lane);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      float total = 0.0f;
+#pragma unroll
+      for (int pass = 0; pass < kPasses; ++pass) total += q6_dot(q6_from_lds(slot, at[pass]), xs[pass], j);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      total = group_sum<kWaveLanes>(total);
+      if (lane == 0) Traits<TX>::store(y, (size_t)row, total);
+    }
+  }
+}
+
 template <int kKind, int kM, class TX>  // 0 = Q4_K, 1 = Q6_K, 2 = Q8_0
 __global__ __launch_bounds__(kBlockThreads) void gguf_matvec(const unsigned char *weights, const void *x, void *y,
                                                              uint32_t rows, uint32_t k, uint64_t row_stride,
@@ -199,6 +437,29 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
   const dim3 grid(((uint32_t)p.rows + rows_per_block - 1) / rows_per_block), block(kBlockThreads);
   const size_t shared = (size_t)p.m * p.k * sizeof(float);
   const unsigned char *in = static_cast<const unsigned char *>(w);
+  if constexpr (kKind == 1) {
+    // one activation row over 2048 or 4096 values per weight row, rows at even addresses
+    const bool even = ((reinterpret_cast<uintptr_t>(w) | p.row_stride) & 1u) == 0;
+    if (p.m == 1 && even && (p.k == 2048 || p.k == 4096)) {
+      // enough waves to fill the machine several times over, each walking many rows
+      const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
+      const dim3 machine(wanted < 256u * 5u ? wanted : 256u * 5u);
+      const bool lines = ((reinterpret_cast<uintptr_t>(w) | p.row_stride) & 15u) == 0;
+      if (lines && p.k == 2048)
+        hipLaunchKernelGGL((gguf_matvec_q6_k_lines<TX, 1>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
+                           p.row_stride);
+      else if (lines)
+        hipLaunchKernelGGL((gguf_matvec_q6_k_lines<TX, 2>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
+                           p.row_stride);
+      else if (p.k == 2048)
+        hipLaunchKernelGGL((gguf_matvec_q6_k_single<TX, 1>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
+                           p.row_stride);
+      else
+        hipLaunchKernelGGL((gguf_matvec_q6_k_single<TX, 2>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
+                           p.row_stride);
+      return hipGetLastError();
+    }
+  }
   if (p.m == 1)
     hipLaunchKernelGGL((gguf_matvec<kKind, 1, TX>), grid, block, shared, s, in, x, y, (uint32_t)p.rows, p.k,
                        p.row_stride, p.m, rows_per_wave);
