@@ -20,6 +20,10 @@
 //   Q8_0  8 lanes per block: lane i takes quants 4 i .. 4 i + 3.
 // Block headers (scales) are read by every lane that needs them; those loads hit the same
 // cache line.  A wave reduction leaves the row's M results.
+//
+// The one shape decoding spends most bytes on -- a single activation row against Q6_K rows of
+// 2048 or 4096 values -- has a kernel of its own further down (x in registers, rows read as
+// whole cache lines).
 #include "device_common.h"
 #include "kernels.h"
 
@@ -158,23 +162,22 @@ __device__ __forceinline__ void row_q8_0(const unsigned char *row, uint32_t k, c
 }
 
 // ---------------------------------------------------------------------------------
-// One activation row, Q6_K, K a multiple of 2048: x in registers.
+// One activation row, Q6_K, K = 2048 or 4096, rows made of whole 16-byte vectors: the
+// vocabulary projection of a decoded token.
 //
 // A wave covers 2048 values of a row at a time: 16 halves of 128 values, four lanes per half.
 // Lane (half, j) owns positions l = 8 j .. 8 j + 7 of each of the half's four groups
 // (l, l + 32, l + 64, l + 96): 8 bytes of ql[64 h + l], 8 of ql[64 h + 32 + l], 8 of qh[32 h + l],
 // the half's eight scales and d.  Those positions are the same for every row, so the lane keeps
-// its 32 activations in registers and no LDS is used.  The six-bit quants are put together four
-// at a time inside a 32-bit word, as bytes holding 4 (q - 32) in two's complement (q < 64, so
-// q << 2 stays inside its byte and bit 7 is the sign after toggling it), which one converting
-// instruction per value sign-extends; the factor 1/4 goes into the group's scale.  A group's
-// sixteen values share one scale, so the lane adds up q x per group and scales the sum:
+// its 32 activations in registers for all the rows it walks.  The six-bit quants are put
+// together four at a time inside a 32-bit word, as bytes holding 4 (q - 32) in two's complement
+// (q < 64, so q << 2 stays inside its byte, and bit 7 is the sign once the upper bit of the qh
+// field is toggled), which one converting instruction per value sign-extends; the factor 1/4
+// goes into the group's scale.  A group's sixteen values share one scale, so the lane adds up
+// (q - 32) x per group and scales the sum:
 //   y = sum over groups of (d * scale) * sum (q - 32) x
-// with f32 products and sums.  The loads of the next row are issued before the current row is
-// worked on.
-typedef uint32_t u32x2_at2 __attribute__((ext_vector_type(2), aligned(2)));
-typedef uint16_t u16_at2 __attribute__((aligned(2)));
-
+// with f32 products and sums.  About 135 vector instructions per row and lane remain, which on
+// 256 compute units is about 40 us for 151,936 rows: the kernel is bound by that arithmetic.
 struct Q6Raw {
   uint32_t low[2], high[2], top[2], scales[2], d;
 };
@@ -189,21 +192,6 @@ __device__ __forceinline__ Q6Offsets q6_offsets(uint32_t pass, uint32_t lane) {
   return Q6Offsets{block + 64 * half + 8 * j, block + 128 + 32 * half + 8 * j, block + 192 + 8 * half, block + 208};
 }
 
-// `row` is the same for the whole wave (a scalar base), the offsets are the lane's own.
-__device__ __forceinline__ Q6Raw q6_load(const unsigned char *row, const Q6Offsets &at) {
-  const u32x2_at2 low = __builtin_nontemporal_load(reinterpret_cast<const u32x2_at2 *>(row + at.low));
-  const u32x2_at2 high = __builtin_nontemporal_load(reinterpret_cast<const u32x2_at2 *>(row + at.low + 32));
-  const u32x2_at2 top = __builtin_nontemporal_load(reinterpret_cast<const u32x2_at2 *>(row + at.top));
-  const u32x2_at2 scales = __builtin_nontemporal_load(reinterpret_cast<const u32x2_at2 *>(row + at.scales));
-  Q6Raw raw;
-  raw.low[0] = low.x, raw.low[1] = low.y;
-  raw.high[0] = high.x, raw.high[1] = high.y;
-  raw.top[0] = top.x, raw.top[1] = top.y;
-  raw.scales[0] = scales.x, raw.scales[1] = scales.y;
-  raw.d = __builtin_nontemporal_load(reinterpret_cast<const u16_at2 *>(row + at.d));
-  return raw;
-}
-
 // sum over four bytes of word (each an int8) times x[0..3], added to sum
 __device__ __forceinline__ float dot_bytes(uint32_t word, const float *x, float sum) {
 #pragma unroll
@@ -215,17 +203,18 @@ __device__ __forceinline__ float q6_dot(const Q6Raw &raw, const float (&x)[4][8]
   float group[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
   for (int w = 0; w < 2; ++w) {
-    const uint32_t low = raw.low[w], high = raw.high[w], top = raw.top[w];
+    // Toggling the upper bit of every two-bit field of qh subtracts 32 from each q modulo 64;
+    // as bit 7 of a byte that holds 4 q it makes the byte 4 (q - 32) as an int8.
+    const uint32_t low = raw.low[w], high = raw.high[w], top = raw.top[w] ^ 0xAAAAAAAAu;
     // bytes of 4 q: bits 2..5 from a nibble of ql, bits 6..7 from two bits of qh
     const uint32_t q0 = ((low << 2) & 0x3C3C3C3Cu) | ((top << 6) & 0xC0C0C0C0u);
     const uint32_t q1 = ((high << 2) & 0x3C3C3C3Cu) | ((top << 4) & 0xC0C0C0C0u);
     const uint32_t q2 = ((low >> 2) & 0x3C3C3C3Cu) | ((top << 2) & 0xC0C0C0C0u);
     const uint32_t q3 = ((high >> 2) & 0x3C3C3C3Cu) | (top & 0xC0C0C0C0u);
-    // toggling bit 7 subtracts 4 * 32 modulo 256: the byte is 4 (q - 32) as an int8
-    group[0] = dot_bytes(q0 ^ 0x80808080u, &x[0][4 * w], group[0]);
-    group[1] = dot_bytes(q1 ^ 0x80808080u, &x[1][4 * w], group[1]);
-    group[2] = dot_bytes(q2 ^ 0x80808080u, &x[2][4 * w], group[2]);
-    group[3] = dot_bytes(q3 ^ 0x80808080u, &x[3][4 * w], group[3]);
+    group[0] = dot_bytes(q0, &x[0][4 * w], group[0]);
+    group[1] = dot_bytes(q1, &x[1][4 * w], group[1]);
+    group[2] = dot_bytes(q2, &x[2][4 * w], group[2]);
+    group[3] = dot_bytes(q3, &x[3][4 * w], group[3]);
   }
   const float d = f16_to_f32((uint16_t)raw.d) * 0.25f;
   // scales[2 g + l / 16] of this half, l / 16 = j / 2
@@ -240,67 +229,15 @@ __device__ __forceinline__ float q6_dot(const Q6Raw &raw, const float (&x)[4][8]
 
 constexpr int kQ6Depth = 4;  // rows of a wave whose bytes are in flight
 
-// The grid is sized to the machine, not to the weight: wave w of W takes rows w, w + W, ...
-template <class TX, int kPasses>
-__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q6_k_single(const unsigned char *weights, const void *x,
-                                                                         void *y, uint32_t rows, uint64_t row_stride) {
-  const uint32_t lane = threadIdx.x % kWaveLanes;
-  // the wave's number as a scalar, so that row addresses are scalar too
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
-  const uint32_t j = lane % 4;
-  float xs[kPasses][4][8];
-  Q6Offsets at[kPasses];
-#pragma unroll
-  for (int pass = 0; pass < kPasses; ++pass) {
-    at[pass] = q6_offsets(pass, lane);
-#pragma unroll
-    for (int g = 0; g < 4; ++g)
-#pragma unroll
-      for (int t = 0; t < 8; ++t)
-        xs[pass][g][t] = Traits<TX>::load(x, (size_t)pass * 2048 + (lane / 4) * 128 + 32 * g + 8 * j + t);
-  }
-  const uint32_t stride = gridDim.x * kWavesPerBlock;
-  const uint32_t first = blockIdx.x * kWavesPerBlock + wave;
-  if (first >= rows) return;
-  // A row past the end is replaced by the wave's first row: a valid address whose bytes go unused.
-  Q6Raw ring[kQ6Depth][kPasses];
-#pragma unroll
-  for (int d = 0; d < kQ6Depth; ++d) {
-    const uint64_t wanted = (uint64_t)first + (uint64_t)d * stride;
-    const uint32_t row = wanted < rows ? (uint32_t)wanted : first;
-#pragma unroll
-    for (int pass = 0; pass < kPasses; ++pass) ring[d][pass] = q6_load(weights + (size_t)row * row_stride, at[pass]);
-  }
-  for (uint64_t base = first; base < rows; base += (uint64_t)kQ6Depth * stride) {
-#pragma unroll
-    for (int d = 0; d < kQ6Depth; ++d) {
-      const uint64_t row = base + (uint64_t)d * stride;
-      if (row >= rows) break;
-      Q6Raw current[kPasses];
-#pragma unroll
-      for (int pass = 0; pass < kPasses; ++pass) current[pass] = ring[d][pass];
-      const uint64_t wanted = row + (uint64_t)kQ6Depth * stride;
-      const uint32_t following = wanted < rows ? (uint32_t)wanted : first;
-#pragma unroll
-      for (int pass = 0; pass < kPasses; ++pass)
-        ring[d][pass] = q6_load(weights + (size_t)following * row_stride, at[pass]);
-      float total = 0.0f;
-#pragma unroll
-      for (int pass = 0; pass < kPasses; ++pass) total += q6_dot(current[pass], xs[pass], j);
-      total = group_sum<kWaveLanes>(total);
-      if (lane == 0) Traits<TX>::store(y, (size_t)row, total);
-    }
-  }
-}
-
-// The same arithmetic with every cache line requested once: the wave reads a row as whole
-// 16-byte vectors (lane i takes vectors i, i + 64, ...: 1680 bytes are 105 vectors), keeps the rows
-// still in flight in registers, and hands the bytes to the lanes that decode them through a
-// region of LDS that only this wave touches.  (Reading each lane's 8-byte pieces straight from
-// memory asks for every line several times while it is still on its way, and the address unit
-// and those waits, not the arithmetic, set the time: 89 us for [2048 -> 151936].)  LDS executes
-// one wave's instructions in order, so the stores of a row and the loads that follow need no
-// barrier, and the next row is stored only after this row's loads were issued.
+// Every cache line is requested once: the wave reads a row as whole 16-byte vectors (lane i
+// takes vectors i, i + 64, ...: 1680 bytes are 105 vectors), keeps the four rows still in
+// flight in registers, and hands the bytes to the lanes that decode them through a region of
+// LDS that only this wave touches.  (Reading each lane's 8-byte pieces straight from memory asks
+// for every line several times while it is still on its way; the address unit and those waits
+// then set the time: 89 us for [2048 -> 151936] against 54 us.)  LDS executes one wave's
+// instructions in order, so the stores of a row and the loads that follow need no barrier, and
+// the next row is stored only after this row's loads were issued.  The grid is sized to the
+// machine, not to the weight: wave w of W takes rows w, w + W, ...
 template <int kPasses> struct Q6Row {
   static constexpr int kVectors = kPasses * 105;               // 16-byte vectors in a row
   static constexpr int kLoads = (kVectors + kWaveLanes - 1) / kWaveLanes;
@@ -371,6 +308,7 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q6_k_lines(const un
     ring[d] = q6_row_load<kPasses>(weights + (size_t)row * row_stride, lane);
   }
   for (uint64_t base = first; base < rows; base += (uint64_t)kQ6Depth * stride) {
+    float totals[kQ6Depth] = {};
 #pragma unroll
     for (int d = 0; d < kQ6Depth; ++d) {
       const uint64_t row = base + (uint64_t)d * stride;
@@ -384,14 +322,22 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q6_k_lines(const un
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      float total = 0.0f;
 #pragma unroll
-      for (int pass = 0; pass < kPasses; ++pass) total += q6_dot(q6_from_lds(slot, at[pass]), xs[pass], j);
+      for (int pass = 0; pass < kPasses; ++pass) totals[d] += q6_dot(q6_from_lds(slot, at[pass]), xs[pass], j);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-      total = group_sum<kWaveLanes>(total);
-      if (lane == 0) Traits<TX>::store(y, (size_t)row, total);
     }
+    // The four rows are summed over the wave together: two exchanges leave lane l with the sum
+    // of row l % 4 over its group of four lanes, four more add the sixteen groups.
+    static_assert(kQ6Depth == 4, "the joint reduction is written for four rows");
+    const bool odd = (lane & 1u) != 0, upper = (lane & 2u) != 0;
+    const float pair01 = (odd ? totals[1] : totals[0]) + __shfl_xor(odd ? totals[0] : totals[1], 1);
+    const float pair23 = (odd ? totals[3] : totals[2]) + __shfl_xor(odd ? totals[2] : totals[3], 1);
+    float mine = (upper ? pair23 : pair01) + __shfl_xor(upper ? pair01 : pair23, 2);
+#pragma unroll
+    for (int step = 4; step < kWaveLanes; step *= 2) mine += __shfl_xor(mine, step);
+    const uint64_t row = base + (uint64_t)lane * stride;
+    if (lane < (uint32_t)kQ6Depth && row < rows) Traits<TX>::store(y, (size_t)row, mine);
   }
 }
 
@@ -438,24 +384,17 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
   const size_t shared = (size_t)p.m * p.k * sizeof(float);
   const unsigned char *in = static_cast<const unsigned char *>(w);
   if constexpr (kKind == 1) {
-    // one activation row over 2048 or 4096 values per weight row, rows at even addresses
-    const bool even = ((reinterpret_cast<uintptr_t>(w) | p.row_stride) & 1u) == 0;
-    if (p.m == 1 && even && (p.k == 2048 || p.k == 4096)) {
+    // one activation row over 2048 or 4096 values per weight row, rows made of whole 16-byte vectors
+    const bool lines = ((reinterpret_cast<uintptr_t>(w) | p.row_stride) & 15u) == 0;
+    if (p.m == 1 && lines && (p.k == 2048 || p.k == 4096)) {
       // enough waves to fill the machine several times over, each walking many rows
       const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
       const dim3 machine(wanted < 256u * 5u ? wanted : 256u * 5u);
-      const bool lines = ((reinterpret_cast<uintptr_t>(w) | p.row_stride) & 15u) == 0;
-      if (lines && p.k == 2048)
+      if (p.k == 2048)
         hipLaunchKernelGGL((gguf_matvec_q6_k_lines<TX, 1>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
                            p.row_stride);
-      else if (lines)
-        hipLaunchKernelGGL((gguf_matvec_q6_k_lines<TX, 2>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
-                           p.row_stride);
-      else if (p.k == 2048)
-        hipLaunchKernelGGL((gguf_matvec_q6_k_single<TX, 1>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
-                           p.row_stride);
       else
-        hipLaunchKernelGGL((gguf_matvec_q6_k_single<TX, 2>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
+        hipLaunchKernelGGL((gguf_matvec_q6_k_lines<TX, 2>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
                            p.row_stride);
       return hipGetLastError();
     }

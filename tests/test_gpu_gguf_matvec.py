@@ -85,9 +85,9 @@ def test_matvec_padded_rows_and_odd_addresses(tag):
 
 @pytest.mark.parametrize("x_tag", ["f32", "bf16"])
 def test_matvec_q6_k_single_token_forms(x_tag):
-    """One activation row over 2048 or 4096 values takes the x-in-registers kernels: whole 16-byte
-    vectors through LDS when base and row stride allow, 8-byte pieces straight from memory at even
-    addresses, the general kernel at odd ones.  Enough rows that a wave walks several of them."""
+    """One activation row over 2048 or 4096 values takes the x-in-registers kernel (rows read as
+    whole 16-byte vectors and redistributed through LDS) when base and row stride are multiples of
+    16, the general kernel otherwise.  Enough rows that a wave walks several of them."""
     rng = np.random.default_rng(1703)
     for rows, k in ((21, 4096), (23001, 2048), (5200, 4096)):
         raw = weights_for("q6_k", rng, rows, k)
