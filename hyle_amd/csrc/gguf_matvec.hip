@@ -25,6 +25,7 @@
 // 2048 or 4096 values -- has a kernel of its own further down (x in registers, rows read as
 // whole cache lines).
 #include "device_common.h"
+#include "gguf_decode.h"
 #include "kernels.h"
 
 namespace hyle_hip {
@@ -255,16 +256,6 @@ __device__ __forceinline__ Q6Row<kPasses> q6_row_load(const unsigned char *row, 
     r.v[i] = load16_stream(row, vec);
   }
   return r;
-}
-
-// Eight bytes at a 2-byte aligned LDS offset, as three aligned words and two byte-wise funnel
-// shifts (an LDS read that is not naturally aligned stalls: measured, four such 8-byte reads per
-// lane made LDS the limit of the kernel).
-__device__ __forceinline__ void lds_piece(const unsigned char *slot, uint32_t offset, uint32_t (&out)[2]) {
-  const uint32_t *words = reinterpret_cast<const uint32_t *>(slot + (offset & ~3u));
-  const uint32_t w0 = words[0], w1 = words[1], w2 = words[2];
-  out[0] = __builtin_amdgcn_alignbyte(w1, w0, offset & 3u);
-  out[1] = __builtin_amdgcn_alignbyte(w2, w1, offset & 3u);
 }
 
 __device__ __forceinline__ Q6Raw q6_from_lds(const unsigned char *slot, const Q6Offsets &at) {

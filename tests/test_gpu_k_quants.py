@@ -82,6 +82,28 @@ def test_k_quant_padded_rows_and_odd_addresses(tag):
         sumsq_bar(sumsq, wide)
 
 
+@pytest.mark.parametrize("tag", ["q4_k", "q6_k"])
+def test_k_quant_whole_vector_rows(tag):
+    """K a multiple of 2048 with base and row stride multiples of 16 takes the wave-per-row kernel
+    (several spans per row, padded strides, a row count that leaves waves of the last block idle);
+    the same rows 2 bytes off take the general one."""
+    kind, _, block_bytes = KINDS[tag]
+    rng = np.random.default_rng(1503)
+    for rows, k in ((7, 2048), (13, 6144), (257, 4096)):
+        row_bytes = k // 256 * block_bytes
+        raw = finite_scales(tag, rng.integers(0, 256, (rows, row_bytes), dtype=np.uint8), block_bytes)
+        wide, want, _ = orc.k_quant_dequant(kind, raw, rows, k)
+        for pad, offset in ((0, 0), (16, 0), (48, 32), (16, 2)):
+            padded = np.zeros(offset + rows * (row_bytes + pad) + 8, np.uint8)
+            for r in range(rows):
+                start = offset + r * (row_bytes + pad)
+                padded[start:start + row_bytes] = raw[r]
+            note(f"{tag} [{rows}, {k}] rows {row_bytes + pad} bytes apart, tensor at byte {offset}")
+            got, sumsq = dequant_on_device(tag, padded, rows, k, row_stride=row_bytes + pad, offset=offset)
+            assert np.array_equal(got, want)
+            sumsq_bar(sumsq, wide)
+
+
 def test_k_quant_schema_and_benchmark_shape():
     DT = hc.DataType
     desc = hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ4K, DT.kBFloat16, 2048, 6144)
