@@ -216,6 +216,7 @@ def main() -> int:
                       6144 * (8 * block_bytes + 2048 * 2 + 4), 6144 * 2048, "u8/bf16", in_step=False))
     # ---- decode-time MatMul over GGUF weights: one activation row against [K, N] ----------------
     for name, gguf, block_bytes, n_rows, sets in (("next_matvec_q4_k_bf16_ffn", hc.GgufQuantizedType.kQ4K, 144, 6144, 80),
+                                                  ("next_matvec_q4_k_bf16_vocab", hc.GgufQuantizedType.kQ4K, 144, 151936, 4),
                                                   ("next_matvec_q6_k_bf16_vocab", hc.GgufQuantizedType.kQ6K, 210, 151936, 3)):
         if not want(name):
             continue

@@ -84,17 +84,18 @@ def test_matvec_padded_rows_and_odd_addresses(tag):
 
 
 @pytest.mark.parametrize("x_tag", ["f32", "bf16"])
-def test_matvec_q6_k_single_token_forms(x_tag):
-    """One activation row over 2048 or 4096 values takes the x-in-registers kernel (rows read as
-    whole 16-byte vectors and redistributed through LDS) when base and row stride are multiples of
-    16, the general kernel otherwise.  Enough rows that a wave walks several of them."""
+@pytest.mark.parametrize("tag", ["q4_k", "q6_k"])
+def test_matvec_single_token_forms(tag, x_tag):
+    """One activation row over 2048 or 4096 values of a K-quant takes the x-in-registers kernel
+    (rows read as whole 16-byte vectors and redistributed through LDS) when base and row stride
+    are multiples of 16, the general kernel otherwise.  Enough rows that a wave walks several."""
     rng = np.random.default_rng(1703)
     for rows, k in ((21, 4096), (23001, 2048), (5200, 4096)):
-        raw = weights_for("q6_k", rng, rows, k)
-        note(f"matvec q6_k single token rows {rows} k {k} x {x_tag}")
-        check("q6_k", x_tag, raw, rows, k, rng.normal(0, 1, k).astype(np.float32))
+        raw = weights_for(tag, rng, rows, k)
+        note(f"matvec {tag} single token rows {rows} k {k} x {x_tag}")
+        check(tag, x_tag, raw, rows, k, rng.normal(0, 1, k).astype(np.float32))
     rows, k = 300, 2048
-    raw = weights_for("q6_k", rng, rows, k)
+    raw = weights_for(tag, rng, rows, k)
     row_bytes = raw.shape[1]
     x = rng.normal(0, 1, k).astype(np.float32)
     for pad, offset in ((16, 0), (32, 16), (2, 0), (6, 2), (16, 4), (3, 0), (0, 1)):
@@ -102,8 +103,8 @@ def test_matvec_q6_k_single_token_forms(x_tag):
         for r in range(rows):
             start = offset + r * (row_bytes + pad)
             padded[start:start + row_bytes] = raw[r]
-        note(f"matvec q6_k single token rows {row_bytes + pad} bytes apart, tensor at byte {offset}")
-        check("q6_k", x_tag, padded, rows, k, x, row_stride=row_bytes + pad, offset=offset)
+        note(f"matvec {tag} single token rows {row_bytes + pad} bytes apart, tensor at byte {offset}")
+        check(tag, x_tag, padded, rows, k, x, row_stride=row_bytes + pad, offset=offset)
 
 
 def test_matvec_schema_admission_and_decode_shape():
