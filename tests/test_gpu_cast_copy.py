@@ -210,3 +210,28 @@ def test_cast_benchmark_shapes_bit_exact():
     note("copy bf16 [8192, 6144]: byte-identical")
     big = rng.integers(0, 1 << 16, (8192, 6144), dtype=np.uint32).astype(np.uint16)
     assert np.array_equal(cast_on_device(DT.kBFloat16, DT.kBFloat16, big, [8192, 6144]), big)
+
+
+@pytest.mark.parametrize("narrow", [DT.kBFloat16, DT.kFloat16])
+def test_cast_norm_cast_is_one_narrow_rms_norm(narrow):
+    """The decoder graph wraps every RMSNorm in two casts (src/compute_models/graph_builder.cc:492-499):
+    narrow -> f32, RMSNorm with an f32 scale, f32 -> narrow.  RMSNorm over the narrow tensor with the
+    same f32 scale is that chain in one launch: the widening is exact, the arithmetic is the same
+    f32 arithmetic, and the one rounding at the end is the closing cast.  The two differ only in the
+    order the row's squares are added (the kernels split a row over lanes differently), so: equal
+    within one unit in the last place, and equal bit for bit nearly everywhere."""
+    from gpu_support import assert_narrow_ulp
+    torch_type = torch.bfloat16 if narrow == DT.kBFloat16 else torch.float16
+    generator = torch.Generator(device="cpu").manual_seed(1900)
+    for rows, width in ((8192, 2048), (33, 4096), (7, 1000)):
+        x = (torch.randn(rows, width, generator=generator) * 3.0).to(torch_type).to(DEVICE)
+        w = (1.0 + 0.1 * torch.randn(width, generator=generator)).to(DEVICE)
+        note(f"cast + rms_norm + cast against one rms_norm, {narrow.name} [{rows}, {width}]")
+        (wide,) = run(hc.Cast(DT.kFloat32), x)
+        (normed,) = run(hc.RmsNorm(epsilon=1e-6), wide, w)
+        (chain,) = run(hc.Cast(narrow), normed)
+        (single,) = run(hc.RmsNorm(epsilon=1e-6), x, w)
+        got = single.view(torch.int16).cpu().numpy().view(np.uint16)
+        want = chain.view(torch.int16).cpu().numpy().view(np.uint16)
+        differing = assert_narrow_ulp(got, want, "bf16" if narrow == DT.kBFloat16 else "f16")
+        assert differing <= got.size // 1000
