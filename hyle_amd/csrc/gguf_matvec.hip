@@ -163,11 +163,11 @@ __device__ __forceinline__ void row_q8_0(const unsigned char *row, uint32_t k, c
 }
 
 // ---------------------------------------------------------------------------------
-// One activation row against Q4_K or Q6_K rows of 2048 or 4096 values made of whole 16-byte
-// vectors: the projections of a decoded token.
+// One activation row against Q4_K, Q6_K or Q8_0 rows of 2048 or 4096 values made of whole
+// 16-byte vectors: the projections of a decoded token.
 //
 // Every cache line is requested once: the wave reads a row as whole 16-byte vectors (lane i
-// takes vectors i, i + 64, ...: 2048 values are 72 or 105 vectors), keeps the four rows still in
+// takes vectors i, i + 64, ...: 2048 values are 72, 105 or 136 vectors), keeps the four rows still in
 // flight in registers, and hands the bytes to the lanes that decode them through a region of
 // LDS that only this wave touches.  (Reading each lane's pieces straight from memory asks for
 // every line several times while it is still on its way; the address unit and those waits then
@@ -181,6 +181,7 @@ __device__ __forceinline__ void row_q8_0(const unsigned char *row, uint32_t k, c
 // stay in registers.  Values that share a scale are summed against x first and scaled once:
 //   Q6_K  y = sum over groups of (d * scale) * sum (q - 32) x
 //   Q4_K  y = sum over sub-blocks of (d * sc) * sum q x - (dmin * m) * sum x
+//   Q8_0  y = sum over blocks of d * sum q x
 // with f32 products and sums (the sums of x are per lane and computed once).  About 135 vector
 // instructions per row and lane remain for Q6_K, which on 256 compute units is about 40 us for
 // 151,936 rows: the kernels are bound by that arithmetic.
@@ -333,6 +334,35 @@ template <> struct Lines<0> {
   }
 };
 
+// Q8_0.  2048 values are 64 blocks of 34 bytes {f16 d; i8 q[32]}: one block per lane.  Blocks
+// are 2-byte aligned, so the 32 quants are taken from nine aligned words with a per-lane funnel
+// shift; each byte is already the int8 the converting instruction wants.
+template <> struct Lines<2> {
+  static constexpr int kPassVectors = 136;
+  struct Lane {
+    uint32_t block, words, shift;
+  };
+  static __device__ __forceinline__ Lane lane_of(uint32_t pass, uint32_t lane) {
+    const uint32_t block = pass * 2176 + 34 * lane, quants = block + 2;
+    return Lane{block, quants & ~3u, quants & 3u};
+  }
+  static __device__ __forceinline__ uint32_t position(uint32_t pass, uint32_t lane, uint32_t e) {
+    return pass * 2048 + 32 * lane + e;
+  }
+  static __device__ __forceinline__ float dot(const unsigned char *slot, const Lane &at, const float (&x)[32],
+                                              const float (&)[4]) {
+    const uint32_t *words = reinterpret_cast<const uint32_t *>(slot + at.words);
+    uint32_t w[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) w[i] = words[i];
+    const float d = f16_to_f32(*reinterpret_cast<const uint16_t *>(slot + at.block));
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum = dot_signed_bytes(__builtin_amdgcn_alignbyte(w[i + 1], w[i], at.shift), &x[4 * i], sum);
+    return d * sum;
+  }
+};
+
 constexpr int kLinesDepth = 4;  // rows of a wave whose bytes are in flight
 
 template <int kKind, int kPasses> struct LinesRow {
@@ -463,7 +493,7 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
   const dim3 grid(((uint32_t)p.rows + rows_per_block - 1) / rows_per_block), block(kBlockThreads);
   const size_t shared = (size_t)p.m * p.k * sizeof(float);
   const unsigned char *in = static_cast<const unsigned char *>(w);
-  if constexpr (kKind == 0 || kKind == 1) {
+  {
     // one activation row over 2048 or 4096 values per weight row, rows made of whole 16-byte vectors
     const bool lines = ((reinterpret_cast<uintptr_t>(w) | p.row_stride) & 15u) == 0;
     if (p.m == 1 && lines && (p.k == 2048 || p.k == 4096)) {

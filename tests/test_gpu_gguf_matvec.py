@@ -84,9 +84,9 @@ def test_matvec_padded_rows_and_odd_addresses(tag):
 
 
 @pytest.mark.parametrize("x_tag", ["f32", "bf16"])
-@pytest.mark.parametrize("tag", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("tag", ["q4_k", "q6_k", "q8_0"])
 def test_matvec_single_token_forms(tag, x_tag):
-    """One activation row over 2048 or 4096 values of a K-quant takes the x-in-registers kernel
+    """One activation row over 2048 or 4096 values takes the x-in-registers kernel
     (rows read as whole 16-byte vectors and redistributed through LDS) when base and row stride
     are multiples of 16, the general kernel otherwise.  Enough rows that a wave walks several."""
     rng = np.random.default_rng(1703)
