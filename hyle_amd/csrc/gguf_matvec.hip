@@ -451,6 +451,102 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_lines(const unsigne
   }
 }
 
+// Longer rows (K = 2048 n, up to 10240 or 12288): the same walk over spans of 2048 values, with the
+// activations as f32 in LDS instead of registers.  They are laid out [span][e / 4][lane][e % 4], so
+// that a lane fetches its 32 values of a span with eight 16-byte reads that are contiguous across
+// the wave; Q4_K's per-lane sums of x sit beside them.  A wave walks the spans of its rows one
+// after another, four spans in flight, and closes a row with a wave reduction.
+template <int kKind, class TX>
+__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_lines_long(const unsigned char *weights, const void *x,
+                                                                        void *y, uint32_t rows, uint64_t row_stride,
+                                                                        uint32_t spans) {
+  using Row = LinesRow<kKind, 1>;
+  using Kind = Lines<kKind>;
+  constexpr uint32_t kSpanBytes = Kind::kPassVectors * 16;
+  __shared__ __align__(16) unsigned char slots[kWavesPerBlock][Row::kSlotBytes];
+  extern __shared__ __align__(16) float staged[];  // x: spans * 2048 floats, then the sums: spans * 256
+  float *sums = staged + (size_t)spans * 2048;
+  for (uint32_t i = threadIdx.x; i < spans * 2048; i += kBlockThreads) {
+    const uint32_t span = i / 2048, quad = (i % 2048) / 256, lane = (i / 4) % kWaveLanes, e = 4 * quad + i % 4;
+    staged[i] = Traits<TX>::load(x, Kind::position(span, lane, e));
+  }
+  __syncthreads();
+  if constexpr (kKind == 0) {
+    for (uint32_t i = threadIdx.x; i < spans * 256; i += kBlockThreads) {
+      const uint32_t span = i / 256, lane = (i / 4) % kWaveLanes, part = i % 4;
+      float sum = 0.0f;
+      for (uint32_t t = 0; t < 8; ++t) {
+        const uint32_t e = 8 * part + t;
+        sum += staged[((span * 8 + e / 4) * kWaveLanes + lane) * 4 + e % 4];
+      }
+      sums[i] = sum;
+    }
+    __syncthreads();
+  }
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  unsigned char *slot = slots[wave];
+  const typename Kind::Lane at = Kind::lane_of(0, lane);
+  const uint32_t stride = gridDim.x * kWavesPerBlock;
+  const uint32_t first = blockIdx.x * kWavesPerBlock + wave;
+  if (first >= rows) return;  // no barrier follows
+  const uint32_t own_rows = (rows - first + stride - 1) / stride;
+  const uint64_t segments = (uint64_t)own_rows * spans;
+  // the stream of loads runs kLinesDepth segments ahead of the stream of decodes
+  uint32_t load_row = first, load_span = 0;
+  uint64_t loaded = 0;
+  auto next_load = [&]() {
+    // past the wave's last segment: its first row again, a valid address whose bytes go unused
+    const bool live = loaded < segments;
+    const unsigned char *source = weights + (size_t)(live ? load_row : first) * row_stride +
+                                  (size_t)(live ? load_span : 0u) * kSpanBytes;
+    ++loaded;
+    if (++load_span == spans) {
+      load_span = 0;
+      load_row += stride;
+    }
+    return Row::load(source, lane);
+  };
+  Row ring[kLinesDepth];
+#pragma unroll
+  for (int d = 0; d < kLinesDepth; ++d) ring[d] = next_load();
+  uint32_t row = first, span = 0;
+  float total = 0.0f;
+  for (uint64_t done = 0; done < segments; done += kLinesDepth) {
+#pragma unroll
+    for (int d = 0; d < kLinesDepth; ++d) {
+      if (done + d >= segments) break;
+#pragma unroll
+      for (int i = 0; i < Row::kLoads; ++i)
+        *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = ring[d].v[i];
+      ring[d] = next_load();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      float xs[32], xsum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int quad = 0; quad < 8; ++quad) {
+        const float4 v = *reinterpret_cast<const float4 *>(staged + ((size_t)(span * 8 + quad) * kWaveLanes + lane) * 4);
+        xs[4 * quad] = v.x, xs[4 * quad + 1] = v.y, xs[4 * quad + 2] = v.z, xs[4 * quad + 3] = v.w;
+      }
+      if constexpr (kKind == 0) {
+        const float4 v = *reinterpret_cast<const float4 *>(sums + ((size_t)span * kWaveLanes + lane) * 4);
+        xsum[0] = v.x, xsum[1] = v.y, xsum[2] = v.z, xsum[3] = v.w;
+      }
+      total += Kind::dot(slot, at, xs, xsum);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (++span == spans) {
+        const float whole = group_sum<kWaveLanes>(total);
+        if (lane == 0) Traits<TX>::store(y, (size_t)row, whole);
+        total = 0.0f;
+        span = 0;
+        row += stride;
+      }
+    }
+  }
+}
+
 template <int kKind, int kM, class TX>  // 0 = Q4_K, 1 = Q6_K, 2 = Q8_0
 __global__ __launch_bounds__(kBlockThreads) void gguf_matvec(const unsigned char *weights, const void *x, void *y,
                                                              uint32_t rows, uint32_t k, uint64_t row_stride,
@@ -506,6 +602,17 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
       else
         hipLaunchKernelGGL((gguf_matvec_lines<kKind, TX, 2>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
                            p.row_stride);
+      return hipGetLastError();
+    }
+    // longer rows: x in LDS, as long as it fits in a block's 64 KiB beside the waves' row buffers
+    const size_t staged = (size_t)(p.k / 2048) * (2048 + (kKind == 0 ? 256 : 0)) * sizeof(float);
+    const size_t parked = (size_t)kWavesPerBlock * LinesRow<kKind, 1>::kSlotBytes;
+    if (p.m == 1 && lines && p.k % 2048 == 0 && p.k > 4096 && staged + parked <= 64 * 1024) {
+      const uint32_t spans = p.k / 2048;
+      const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
+      const dim3 machine(wanted < 256u * 3u ? wanted : 256u * 3u);
+      hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX>), machine, block, staged, s, in, x, y, (uint32_t)p.rows,
+                         p.row_stride, spans);
       return hipGetLastError();
     }
   }

@@ -107,6 +107,19 @@ def test_matvec_single_token_forms(tag, x_tag):
         check(tag, x_tag, padded, rows, k, x, row_stride=row_bytes + pad, offset=offset)
 
 
+@pytest.mark.parametrize("x_tag", ["f32", "bf16"])
+@pytest.mark.parametrize("tag", ["q4_k", "q6_k", "q8_0"])
+def test_matvec_single_token_long_rows(tag, x_tag):
+    """One activation row over 6144 to 12288 values (whole 2048-value spans): activations in LDS,
+    a wave walks the spans of its rows.  Row counts around the number of waves of the grid, and
+    one past the LDS limit that falls back to the general kernel."""
+    rng = np.random.default_rng(1704)
+    for rows, k in ((2048, 6144), (3, 8192), (3100, 10240), (37, 12288)):
+        raw = weights_for(tag, rng, rows, k)
+        note(f"matvec {tag} long rows {rows} k {k} x {x_tag}")
+        check(tag, x_tag, raw, rows, k, rng.normal(0, 1, k).astype(np.float32))
+
+
 def test_matvec_schema_admission_and_decode_shape():
     D, DT = hc.TensorDesc.dense, hc.DataType
     w = hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ4K, DT.kBFloat16, 2048, 6144)
