@@ -21,9 +21,12 @@
 // Block headers (scales) are read by every lane that needs them; those loads hit the same
 // cache line.  A wave reduction leaves the row's M results.
 //
-// The one shape decoding spends most bytes on -- a single activation row against Q6_K rows of
-// 2048 or 4096 values -- has a kernel of its own further down (x in registers, rows read as
-// whole cache lines).
+// The shapes decoding spends its bytes on -- a single activation row against rows of 2048 n
+// values made of whole 16-byte vectors -- have kernels of their own further down (rows read as
+// whole cache lines, x in registers or LDS).  Those factor the scale out of each group of values
+// that share it, y = sum of scale * (sum of q x): the same real number as the sum over exactly
+// decoded weights, with different f32 roundings; every form is held to 1e-5 * sum |w x| of the
+// exact product.
 #include "device_common.h"
 #include "gguf_decode.h"
 #include "kernels.h"
