@@ -218,6 +218,7 @@ def main() -> int:
     for name, gguf, block_bytes, k, n_rows, sets in (
             ("next_matvec_q4_k_bf16_ffn", hc.GgufQuantizedType.kQ4K, 144, 2048, 6144, 80),
             ("next_matvec_q4_k_bf16_ffn_down", hc.GgufQuantizedType.kQ4K, 144, 6144, 2048, 80),
+            ("next_matvec_q4_k_bf16_k4096", hc.GgufQuantizedType.kQ4K, 144, 4096, 14336, 16),
             ("next_matvec_q4_k_bf16_vocab", hc.GgufQuantizedType.kQ4K, 144, 2048, 151936, 4),
             ("next_matvec_q6_k_bf16_vocab", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3),
             ("next_matvec_q8_0_bf16_vocab", hc.GgufQuantizedType.kQ8_0, 34, 2048, 151936, 3)):

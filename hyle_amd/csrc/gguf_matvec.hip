@@ -166,8 +166,8 @@ __device__ __forceinline__ void row_q8_0(const unsigned char *row, uint32_t k, c
 }
 
 // ---------------------------------------------------------------------------------
-// One activation row against Q4_K, Q6_K or Q8_0 rows of 2048 or 4096 values made of whole
-// 16-byte vectors: the projections of a decoded token.
+// One activation row against Q4_K, Q6_K or Q8_0 rows of 2048 values made of whole 16-byte
+// vectors (longer rows: the variant further down): the projections of a decoded token.
 //
 // Every cache line is requested once: the wave reads a row as whole 16-byte vectors (lane i
 // takes vectors i, i + 64, ...: 2048 values are 72, 105 or 136 vectors), keeps the four rows still in
@@ -454,7 +454,7 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_lines(const unsigne
   }
 }
 
-// Longer rows (K = 2048 n, up to 10240 or 12288): the same walk over spans of 2048 values, with the
+// Longer rows (K = 2048 n from 4096 up to 10240 or 12288): the same walk over spans of 2048 values, with the
 // activations as f32 in LDS instead of registers.  They are laid out [span][e / 4][lane][e % 4], so
 // that a lane fetches its 32 values of a span with eight 16-byte reads that are contiguous across
 // the wave; Q4_K's per-lane sums of x sit beside them.  A wave walks the spans of its rows one
@@ -593,24 +593,22 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
   const size_t shared = (size_t)p.m * p.k * sizeof(float);
   const unsigned char *in = static_cast<const unsigned char *>(w);
   {
-    // one activation row over 2048 or 4096 values per weight row, rows made of whole 16-byte vectors
+    // one activation row over rows of 2048 n values made of whole 16-byte vectors
     const bool lines = ((reinterpret_cast<uintptr_t>(w) | p.row_stride) & 15u) == 0;
-    if (p.m == 1 && lines && (p.k == 2048 || p.k == 4096)) {
+    if (p.m == 1 && lines && p.k == 2048) {
       // enough waves to fill the machine several times over, each walking many rows
       const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
       const dim3 machine(wanted < 256u * 5u ? wanted : 256u * 5u);
-      if (p.k == 2048)
-        hipLaunchKernelGGL((gguf_matvec_lines<kKind, TX, 1>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
-                           p.row_stride);
-      else
-        hipLaunchKernelGGL((gguf_matvec_lines<kKind, TX, 2>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
-                           p.row_stride);
+      hipLaunchKernelGGL((gguf_matvec_lines<kKind, TX, 1>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
+                         p.row_stride);
       return hipGetLastError();
     }
     // longer rows: x in LDS, as long as it fits in a block's 64 KiB beside the waves' row buffers
+    // (for K = 4096 this measured slightly faster than 64 activations in registers: 13.8 against
+    // 14.4 us for Q4_K [4096 -> 14336])
     const size_t staged = (size_t)(p.k / 2048) * (2048 + (kKind == 0 ? 256 : 0)) * sizeof(float);
     const size_t parked = (size_t)kWavesPerBlock * LinesRow<kKind, 1>::kSlotBytes;
-    if (p.m == 1 && lines && p.k % 2048 == 0 && p.k > 4096 && staged + parked <= 64 * 1024) {
+    if (p.m == 1 && lines && p.k % 2048 == 0 && p.k > 2048 && staged + parked <= 64 * 1024) {
       const uint32_t spans = p.k / 2048;
       const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
       const dim3 machine(wanted < 256u * 3u ? wanted : 256u * 3u);
