@@ -239,6 +239,20 @@ hyle_hip_status expect_inputs(const hyle_hip_op_desc &r, uint32_t low, uint32_t 
   return HYLE_HIP_OK;
 }
 
+// gguf_weight_description(type, ..., k, n): logical [K, N], native blocks along axis 0
+// (src/compute_ops/low_precision.cc:269-297), for the block geometries this provider decodes
+// (src/compute_ops/low_precision.cc:22-29).
+hyle_hip_status expect_gguf_weight(const Desc &w) {
+  const bool q8_0 = w.elements_per_block == 32 && w.bytes_per_block == 34;
+  const bool q4_k = w.elements_per_block == 256 && w.bytes_per_block == 144;
+  const bool q6_k = w.elements_per_block == 256 && w.bytes_per_block == 210;
+  if (w.storage != HYLE_HIP_STORAGE_BLOCKED || !(q8_0 || q4_k || q6_k) || w.rank != 2 || w.block_axis != 0)
+    return fail(HYLE_HIP_INVALID_ARGUMENT,
+                "GGUF weight must be blocked [K, N] storage with Q8_0 (32 / 34), Q4_K (256 / 144) or "
+                "Q6_K (256 / 210) blocks on axis 0");
+  return HYLE_HIP_OK;
+}
+
 hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count) {
   if (r.abi_version != HYLE_HIP_ABI_VERSION)
     return fail(HYLE_HIP_INVALID_ARGUMENT, "hyle_hip_op_desc ABI version %u is not %u", r.abi_version,
@@ -424,17 +438,7 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
     }
     case HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ: {
       if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
-      // gguf_weight_description(kQ8_0, ..., k, n): logical [K, N], blocks along axis 0
-      // (src/compute_ops/low_precision.cc:269-297)
-      // and the K-quant geometries of src/compute_ops/low_precision.cc:22-27
-      const bool q8_0 = in[0].elements_per_block == 32 && in[0].bytes_per_block == 34;
-      const bool q4_k = in[0].elements_per_block == 256 && in[0].bytes_per_block == 144;
-      const bool q6_k = in[0].elements_per_block == 256 && in[0].bytes_per_block == 210;
-      if (in[0].storage != HYLE_HIP_STORAGE_BLOCKED || !(q8_0 || q4_k || q6_k) || in[0].rank != 2 ||
-          in[0].block_axis != 0)
-        return fail(HYLE_HIP_INVALID_ARGUMENT,
-                    "GGUF weight must be blocked [K, N] storage with Q8_0 (32 / 34), Q4_K (256 / 144) or "
-                    "Q6_K (256 / 210) blocks on axis 0");
+      if ((s = expect_gguf_weight(in[0])) != HYLE_HIP_OK) return s;
       if (!is_floating(in[0].dtype))
         return fail(HYLE_HIP_INVALID_ARGUMENT, "GGUF weight requires a floating logical type");
       const int64_t dims0[2] = {in[0].dims[1], in[0].dims[0]};
@@ -444,13 +448,7 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
     }
     case HYLE_HIP_OP_GGUF_MATVEC: {
       if ((s = expect_inputs(r, 2, 2)) != HYLE_HIP_OK) return s;
-      const bool q8_0 = in[0].elements_per_block == 32 && in[0].bytes_per_block == 34;
-      const bool q4_k = in[0].elements_per_block == 256 && in[0].bytes_per_block == 144;
-      const bool q6_k = in[0].elements_per_block == 256 && in[0].bytes_per_block == 210;
-      if (in[0].storage != HYLE_HIP_STORAGE_BLOCKED || !(q8_0 || q4_k || q6_k) || in[0].rank != 2 ||
-          in[0].block_axis != 0)
-        return fail(HYLE_HIP_INVALID_ARGUMENT,
-                    "GGUF weight must be blocked [K, N] storage with Q8_0, Q4_K or Q6_K blocks on axis 0");
+      if ((s = expect_gguf_weight(in[0])) != HYLE_HIP_OK) return s;
       // MatMul contraction (src/compute_ops/operation.cc, kMatMul): the last axis of the
       // activations meets the first logical axis of the weight
       if (!is_floating(in[1].dtype) || in[1].rank < 1 || in[1].rank > 2 ||
@@ -646,6 +644,20 @@ hyle_hip_status require_f32_accumulation(const hyle_hip_plan *p, uint8_t input_d
   if (acc == HYLE_HIP_DTYPE_F32) return HYLE_HIP_OK;
   if (acc == HYLE_HIP_DTYPE_UNKNOWN && input_dtype == HYLE_HIP_DTYPE_F32) return HYLE_HIP_OK;
   return fail(HYLE_HIP_UNIMPLEMENTED, "%s supports float32 accumulation (explicit for half inputs)", op);
+}
+
+// Physical layout of a GGUF weight the kernels walk: the blocks of a row one after another, rows
+// at least a row of blocks apart, at most INT32_MAX values.
+hyle_hip_status admit_gguf_rows(const Desc &w) {
+  const int64_t k = w.dims[0], n = w.dims[1];
+  const int64_t per_block = w.elements_per_block, block_bytes = w.bytes_per_block;
+  if (w.byte_strides[0] != block_bytes)
+    return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF blocks of a row must be contiguous (block stride = block bytes)");
+  if (k > 0 && n > 1 && w.byte_strides[1] < (k / per_block) * block_bytes)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "GGUF row stride is shorter than a row of blocks");
+  if ((uint64_t)k * (uint64_t)n > kMaxElements)
+    return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF weights of at most INT32_MAX values are served");
+  return HYLE_HIP_OK;
 }
 
 hyle_hip_status admit(hyle_hip_plan *p) {
@@ -894,12 +906,7 @@ hyle_hip_status admit(hyle_hip_plan *p) {
     case HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ: {
       const int64_t k = in[0].dims[0], n = in[0].dims[1];
       const int64_t per_block = in[0].elements_per_block, block_bytes = in[0].bytes_per_block;
-      if (in[0].byte_strides[0] != block_bytes)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF blocks of a row must be contiguous (block stride = block bytes)");
-      if (k > 0 && n > 1 && in[0].byte_strides[1] < (k / per_block) * block_bytes)
-        return fail(HYLE_HIP_INVALID_ARGUMENT, "GGUF row stride is shorter than a row of blocks");
-      if ((uint64_t)k * (uint64_t)n > kMaxElements)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF dequant requires at most INT32_MAX elements");
+      if ((s = admit_gguf_rows(in[0])) != HYLE_HIP_OK) return s;
       p->elem = Elem::kBF16;
       if (n == 0) return HYLE_HIP_OK;
       if (per_block == 256) {
@@ -928,14 +935,9 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       const int64_t per_block = in[0].elements_per_block, block_bytes = in[0].bytes_per_block;
       if (!to_elem(in[1].dtype, &p->elem) || !is_plain(in[1]) || !is_dense(in[1]))
         return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec requires dense plain float32/float16/bfloat16 activations");
-      if (in[0].byte_strides[0] != block_bytes)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF blocks of a row must be contiguous (block stride = block bytes)");
-      if (k > 0 && n > 1 && in[0].byte_strides[1] < (k / per_block) * block_bytes)
-        return fail(HYLE_HIP_INVALID_ARGUMENT, "GGUF row stride is shorter than a row of blocks");
+      if ((s = admit_gguf_rows(in[0])) != HYLE_HIP_OK) return s;
       const int64_t m = in[1].rank == 2 ? in[1].dims[0] : 1;
       if (m > 8) return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec serves at most 8 activation rows");
-      if ((uint64_t)k * (uint64_t)n > kMaxElements)
-        return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec requires at most INT32_MAX weight elements");
       if (gguf_matvec_shared_bytes((uint32_t)m, (uint32_t)k) > 64 * 1024)
         return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec keeps the activations in LDS: M * K is too large");
       if (p->output_elements[0] == 0) return HYLE_HIP_OK;
