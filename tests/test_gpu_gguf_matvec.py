@@ -120,6 +120,18 @@ def test_matvec_single_token_long_rows(tag, x_tag):
         check(tag, x_tag, raw, rows, k, rng.normal(0, 1, k).astype(np.float32))
 
 
+@pytest.mark.parametrize("tag", ["q4_k", "q6_k", "q8_0"])
+def test_matvec_single_token_few_rows(tag):
+    """Fewer rows than a wave keeps in flight, and row counts around a block's four waves."""
+    rng = np.random.default_rng(1705)
+    for k in (2048, 4096):
+        x = rng.normal(0, 1, k).astype(np.float32)
+        for rows in (1, 2, 3, 4, 5, 7, 9):
+            raw = weights_for(tag, rng, rows, k)
+            note(f"matvec {tag} single token rows {rows} k {k}")
+            check(tag, "f32", raw, rows, k, x)
+
+
 def test_matvec_schema_admission_and_decode_shape():
     D, DT = hc.TensorDesc.dense, hc.DataType
     w = hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ4K, DT.kBFloat16, 2048, 6144)
