@@ -596,9 +596,11 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
     // one activation row over rows of 2048 n values made of whole 16-byte vectors
     const bool lines = ((reinterpret_cast<uintptr_t>(w) | p.row_stride) & 15u) == 0;
     if (p.m == 1 && lines && p.k == 2048) {
-      // enough waves to fill the machine several times over, each walking many rows
       const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
-      const dim3 machine(wanted < 256u * 5u ? wanted : 256u * 5u);
+      // three blocks per compute unit measured best (Q4_K [2048 -> 6144] 4.9 us and [2048 -> 151936]
+      // 45.9 us, against 6.4 and 47.7 us with five; counts that are not a multiple of the 256
+      // compute units leave some of them a block short and are slower)
+      const dim3 machine(wanted < 256u * 3u ? wanted : 256u * 3u);
       hipLaunchKernelGGL((gguf_matvec_lines<kKind, TX, 1>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
                          p.row_stride);
       return hipGetLastError();
