@@ -10,12 +10,13 @@
 // against NaN) go to the lower index.  The value output carries the original
 // storage bits of the winner.
 //
-// Measured on MI355X over logits[64, 151936] f32: a tile of 256 lanes x 2
-// vectors scans at about 5.2 TB/s, larger tiles are slower (4 vectors 4.2 TB/s,
-// 8 vectors 1.3 TB/s); folding inside the scan kernel with device-scope atomics
-// (a packed key, or a last-block ticket) costs 5 to 13 us, and a device-wide
-// fence writes back and invalidates a whole L2 (100 us), so the fold is a second,
-// tiny dispatch (about 2 us including the dependent launch).
+// Measured on MI355X over logits[64, 151936] f32: a lane that holds all the vectors
+// of its tile in registers at once scans at about 5.2 TB/s with 2 vectors and slower
+// with more (4 vectors 4.2 TB/s, 8 vectors 1.3 TB/s), so a lane walks a longer tile
+// two vectors at a time; folding inside the scan kernel with device-scope atomics
+// (a packed key, or a last-block ticket) costs 5 to 13 us, and a device-wide fence
+// writes back and invalidates a whole L2 (100 us), so the fold is a second, tiny
+// dispatch (2 to 4 us including the dependent launch).
 #include "device_common.h"
 #include "kernels.h"
 
@@ -39,64 +40,65 @@ __device__ __forceinline__ void consider(LaneArg &best, float value, int32_t ind
   if (better) best = LaneArg{value, index};
 }
 
-constexpr int kTileVectorsPerLane = 2;
+constexpr int kVectorsInFlight = 2;  // loads a lane issues before it compares
 
-// One block per (row, tile).  A lane issues all of its loads before it compares.
+// One block per (row, tile).  A lane walks its tile two vectors at a time: both loads are issued
+// (from clamped, always valid addresses) before either is compared.
 template <class T, bool kVector>
 __global__ __launch_bounds__(kBlockThreads) void argmax_tiles(const void *x, Candidate *partial,
                                                               uint32_t width, uint32_t tiles,
                                                               uint32_t tile_elems) {
   constexpr int kVec = Traits<T>::kVec;
-  constexpr int kVpl = kTileVectorsPerLane;
+  constexpr int kVpl = kVectorsInFlight;
   __shared__ LaneArg joint[kBlockThreads / kWaveLanes];
   const uint32_t row = blockIdx.x / tiles, tile = blockIdx.x % tiles;
   const uint32_t begin = tile * tile_elems;
   const uint32_t end = begin + tile_elems < width ? begin + tile_elems : width;
   LaneArg best{0.0f, -1};
   if constexpr (kVector) {
-    // width % kVec == 0 and tile_elems == kVpl * kBlockThreads * kVec: whole vectors only
+    // width % kVec == 0 and tile_elems % kVec == 0: whole vectors only
     const size_t row_vec = (size_t)row * (width / kVec);
-    const uint32_t vec_end = end / kVec;
-    const uint32_t first = begin / kVec + threadIdx.x;
-    u32x4 raw[kVpl];
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) {
-      const uint32_t vec = first + k * kBlockThreads;
-      if (vec < vec_end) raw[k] = load16_stream(x, row_vec + vec);
-    }
+    const uint32_t vec_begin = begin / kVec, vec_end = end / kVec;
     // Common case first: the greatest number above -inf, found with one compare per element
-    // (a NaN never passes "greater than"; the first of equal values stays).  `slot` is the
-    // position inside the lane's own vectors.
+    // (a NaN never passes "greater than"; the first of equal values stays: a lane meets its
+    // elements in increasing index order, and a vector read twice because its address was
+    // clamped cannot win against itself).
     float top = -INFINITY;
-    int slot = -1;
+    uint32_t top_vec = 0, top_at = 0;
+    bool found = false;
+    for (uint32_t base = vec_begin + threadIdx.x; base < vec_end; base += kVpl * kBlockThreads) {
+      u32x4 raw[kVpl];
+      uint32_t vec[kVpl];
 #pragma unroll
-    for (int k = 0; k < kVpl; ++k) {
-      const uint32_t vec = first + k * kBlockThreads;
-      if (vec < vec_end) {
+      for (int k = 0; k < kVpl; ++k) {
+        const uint32_t wanted = base + k * kBlockThreads;
+        vec[k] = wanted < vec_end ? wanted : vec_end - 1;
+        raw[k] = load16_stream(x, row_vec + vec[k]);
+      }
+#pragma unroll
+      for (int k = 0; k < kVpl; ++k) loads_issued(raw[k]);
+#pragma unroll
+      for (int k = 0; k < kVpl; ++k) {
         float a[kVec];
         Traits<T>::unpack(raw[k], a);
 #pragma unroll
         for (int j = 0; j < kVec; ++j) {
           const bool greater = a[j] > top;
           top = greater ? a[j] : top;
-          slot = greater ? k * kVec + j : slot;
+          top_vec = greater ? vec[k] : top_vec;
+          top_at = greater ? (uint32_t)j : top_at;
+          found = found || greater;
         }
       }
     }
-    if (slot >= 0) {
-      best = LaneArg{top, (int32_t)((first + (slot / kVec) * kBlockThreads) * kVec + slot % kVec)};
+    if (found) {
+      best = LaneArg{top, (int32_t)(top_vec * kVec + top_at)};
     } else {
       // nothing but -inf and NaN in this lane's share: apply the full ordering
-#pragma unroll
-      for (int k = 0; k < kVpl; ++k) {
-        const uint32_t vec = first + k * kBlockThreads;
-        if (vec < vec_end) {
-          float a[kVec];
-          Traits<T>::unpack(raw[k], a);
-#pragma unroll
-          for (int j = 0; j < kVec; ++j) consider(best, a[j], (int32_t)(vec * kVec + j));
-        }
-      }
+      const size_t base = (size_t)row * width;
+      for (uint32_t v = vec_begin + threadIdx.x; v < vec_end; v += kBlockThreads)
+        for (uint32_t j = 0; j < (uint32_t)kVec; ++j)
+          consider(best, Traits<T>::load(x, base + (size_t)v * kVec + j), (int32_t)(v * kVec + j));
     }
   } else {
     const size_t base = (size_t)row * width;
@@ -146,8 +148,7 @@ hipError_t run(const ArgmaxParams &p, const void *x, void *values, int32_t *indi
                bool vectorised, hipStream_t s) {
   const uint32_t rows = (uint32_t)p.shape.rows, width = p.shape.width;
   auto *partial = static_cast<Candidate *>(workspace);
-  const bool vec = vectorised && width % Traits<T>::kVec == 0 &&
-                   p.tile_elems == (uint32_t)(kTileVectorsPerLane * kBlockThreads * Traits<T>::kVec);
+  const bool vec = vectorised && width % Traits<T>::kVec == 0 && p.tile_elems % Traits<T>::kVec == 0;
   if (vec)
     hipLaunchKernelGGL((argmax_tiles<T, true>), dim3(rows * p.tiles), dim3(kBlockThreads), 0, s, x,
                        partial, width, p.tiles, p.tile_elems);
@@ -164,12 +165,24 @@ hipError_t run(const ArgmaxParams &p, const void *x, void *values, int32_t *indi
 
 }  // namespace
 
-// A tile is what one block holds in registers at once: 256 lanes x 2 vectors (2048 f32 or
-// 4096 narrow elements).  64 rows of 151936 logits become 4800 blocks.
+// Tiles are cut so that rows x tiles is about four blocks of 256 threads per compute unit:
+// measured on MI355X over logits[64, 151936] f32, scan and fold together take 11.4 us with 1024
+// blocks, 11.8 with 768 or 1536, 12.3 with 2048, 13.3 with 512 and 12.9-14.0 with 3072-8192 (four
+// vectors in flight instead of two: 11.2-12.0 us over the same range).  64 rows of 151936 logits
+// become 64 x 16 blocks of 9496 elements; 1024 rows or more are one block each.  A tile is a
+// whole number of 16-byte vectors and never shorter than one pass of the block.
 void argmax_plan(uint64_t rows, uint32_t width, Elem type, ArgmaxParams *p) {
   p->shape.rows = rows;
   p->shape.width = width;
-  p->tile_elems = (uint32_t)(kTileVectorsPerLane * kBlockThreads * elem_vec(type));
+  const uint32_t vec = (uint32_t)elem_vec(type);
+  const uint32_t pass = (uint32_t)(kVectorsInFlight * kBlockThreads) * vec;  // elements of one pass
+  const uint64_t blocks = 4u * 256u;
+  uint64_t wanted = rows == 0 ? 1 : (blocks + rows / 2) / rows;
+  wanted = wanted < 1 ? 1 : wanted;
+  const uint32_t row_vectors = (width + vec - 1) / vec;
+  uint32_t tile_vectors = (uint32_t)((row_vectors + wanted - 1) / wanted);
+  if (tile_vectors * vec < pass) tile_vectors = pass / vec;
+  p->tile_elems = tile_vectors * vec;
   p->tiles = width == 0 ? 1 : (width + p->tile_elems - 1) / p->tile_elems;
 }
 
