@@ -70,7 +70,7 @@ __global__ __launch_bounds__(kBlockThreads) void k_quant_rows(const unsigned cha
         if constexpr (kKind == 0) decode_q4_k(blk, local % kSuper, y);
         else decode_q6_k(blk, local % kSuper, y);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[r] += y[j] * y[j];
+        for (int j = 0; j < 8; ++j) acc[r] = __builtin_fmaf(y[j], y[j], acc[r]);
         if (first_row + r < rows) {
           const size_t element = (size_t)(first_row + r) * k + (size_t)first * kSuper + local;
           store16_stream(out, element / 8, Traits<BF16>::pack(y));
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kBlockThreads) void k_quant_lines(const unsigned ch
       if constexpr (kKind == 0) decode_q4_k_words(slot, (p / kSuper) * kBlockBytes, p % kSuper, y);
       else decode_q6_k_words(slot, (p / kSuper) * kBlockBytes, p % kSuper, y);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) squares += y[j] * y[j];
+      for (int j = 0; j < 8; ++j) squares = __builtin_fmaf(y[j], y[j], squares);
       store16_stream(out, ((size_t)row * k + (size_t)step * kSpan + p) / 8, Traits<BF16>::pack(y));
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
