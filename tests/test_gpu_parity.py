@@ -523,6 +523,37 @@ def test_argmax_widths_against_oracle(tag):
         assert np.array_equal(got_values, want_values)
 
 
+@pytest.mark.parametrize("tag", ["f32", "bf16", "f16"])
+def test_argmax_tiles_walked_in_several_steps(tag):
+    """64 rows of 40000: sixteen tiles per row, each walked in more than one step with a ragged
+    last step.  Rows of nothing but NaN, nothing but -inf, one number late among NaNs, one finite
+    value among -inf, and exact ties across tiles take the full ordering as well as the fast one."""
+    rng = np.random.default_rng(112)
+    rows, width = 64, 40000
+    x = rng.integers(-30, 30, (rows, width)).astype(np.float32)
+    x[1, :] = np.nan
+    x[2, :] = -np.inf
+    x[3, :] = np.nan
+    x[3, 39990] = -5.0
+    x[4, :] = -np.inf
+    x[4, 12345] = -60000.0         # finite in every storage type
+    x[5, :] = 7.0                    # the same value everywhere: index 0
+    x[6, :] = -np.inf
+    x[6, 20000:] = np.nan            # -inf before NaN: index 0
+    x[7, :] = np.nan
+    x[7, 39999] = -np.inf            # a number (even -inf) beats every NaN
+    note(f"argmax {tag} [{rows},{width}] special rows over walked tiles")
+    xs = host_values(x, tag)
+    values, indices = run(hc.TopK(), to_device(xs, tag))
+    xf = x if tag == "f32" else orc.to_f32(TYPES[tag][1], xs)
+    want_values, want_indices = orc.topk1(xf)
+    assert np.array_equal(to_host(indices)[:, 0], want_indices)
+    assert want_indices[[1, 2, 3, 4, 5, 6, 7]].tolist() == [0, 0, 39990, 12345, 0, 0, 39999]
+    got_values = to_host(values)[:, 0]
+    got_values = got_values if tag == "f32" else orc.to_f32(TYPES[tag][1], got_values)
+    assert np.array_equal(got_values, want_values, equal_nan=True)
+
+
 def test_config4_argmax_full_shape_bit_exact():
     note("cfg4 argmax logits[64,151936] with planted ties")
     logits = wl.config4_argmax()
