@@ -200,7 +200,7 @@ __device__ __forceinline__ float dot_signed_bytes(uint32_t word, const float *x,
 // to the mask that made it: it would otherwise extract every nibble with a bit-field
 // instruction of its own before converting, two instructions per value instead of one.
 __device__ __forceinline__ float dot_bytes(uint32_t word, const float *x, float sum) {
-  asm volatile("" : "+v"(word));
+  asm("" : "+v"(word));
 #pragma unroll
   for (int t = 0; t < 4; ++t) sum = __builtin_fmaf((float)((word >> (8 * t)) & 0xFFu), x[t], sum);
   return sum;
@@ -454,33 +454,38 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_lines(const unsigne
   }
 }
 
-// Longer rows (K = 2048 n from 4096 up to 10240 or 12288): the same walk over spans of 2048 values, with the
+// Longer rows (K = 2048 n from 4096 up to 10240 or 12288) and two to eight activation rows (any
+// K = 2048 n whose activations fit): the same walk over spans of 2048 values, with the
 // activations as f32 in LDS instead of registers.  They are laid out [span][e / 4][lane][e % 4], so
 // that a lane fetches its 32 values of a span with eight 16-byte reads that are contiguous across
 // the wave; Q4_K's per-lane sums of x sit beside them.  A wave walks the spans of its rows one
 // after another, four spans in flight, and closes a row with a wave reduction.
-template <int kKind, class TX>
+template <int kKind, class TX, int kM>
 __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_lines_long(const unsigned char *weights, const void *x,
                                                                         void *y, uint32_t rows, uint64_t row_stride,
-                                                                        uint32_t spans) {
+                                                                        uint32_t spans, uint32_t m) {
   using Row = LinesRow<kKind, 1>;
   using Kind = Lines<kKind>;
   constexpr uint32_t kSpanBytes = Kind::kPassVectors * 16;
   __shared__ __align__(16) unsigned char slots[kWavesPerBlock][Row::kSlotBytes];
-  extern __shared__ __align__(16) float staged[];  // x: spans * 2048 floats, then the sums: spans * 256
-  float *sums = staged + (size_t)spans * 2048;
-  for (uint32_t i = threadIdx.x; i < spans * 2048; i += kBlockThreads) {
-    const uint32_t span = i / 2048, quad = (i % 2048) / 256, lane = (i / 4) % kWaveLanes, e = 4 * quad + i % 4;
-    staged[i] = Traits<TX>::load(x, Kind::position(span, lane, e));
+  // x: m rows of spans * 2048 floats (an activation row after the other), then their sums: m * spans * 256
+  extern __shared__ __align__(16) float staged[];
+  const uint32_t k = spans * 2048;
+  float *sums = staged + (size_t)m * k;
+  for (uint32_t r = 0; r < m; ++r) {
+    for (uint32_t i = threadIdx.x; i < k; i += kBlockThreads) {
+      const uint32_t span = i / 2048, quad = (i % 2048) / 256, lane = (i / 4) % kWaveLanes, e = 4 * quad + i % 4;
+      staged[(size_t)r * k + i] = Traits<TX>::load(x, (size_t)r * k + Kind::position(span, lane, e));
+    }
   }
   __syncthreads();
   if constexpr (kKind == 0) {
-    for (uint32_t i = threadIdx.x; i < spans * 256; i += kBlockThreads) {
-      const uint32_t span = i / 256, lane = (i / 4) % kWaveLanes, part = i % 4;
+    for (uint32_t i = threadIdx.x; i < m * spans * 256; i += kBlockThreads) {
+      const uint32_t group = i / 256, lane = (i / 4) % kWaveLanes, part = i % 4;  // group = r * spans + span
       float sum = 0.0f;
       for (uint32_t t = 0; t < 8; ++t) {
         const uint32_t e = 8 * part + t;
-        sum += staged[((span * 8 + e / 4) * kWaveLanes + lane) * 4 + e % 4];
+        sum += staged[((group * 8 + e / 4) * kWaveLanes + lane) * 4 + e % 4];
       }
       sums[i] = sum;
     }
@@ -514,7 +519,7 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_lines_long(const un
 #pragma unroll
   for (int d = 0; d < kLinesDepth; ++d) ring[d] = next_load();
   uint32_t row = first, span = 0;
-  float total = 0.0f;
+  float totals[kM] = {};
   for (uint64_t done = 0; done < segments; done += kLinesDepth) {
 #pragma unroll
     for (int d = 0; d < kLinesDepth; ++d) {
@@ -526,23 +531,34 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_lines_long(const un
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      float xs[32], xsum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      // One call per activation row: the span's bytes are decoded by the same expressions each
+      // time, which the compiler works out once and multiplies against every row of x.
 #pragma unroll
-      for (int quad = 0; quad < 8; ++quad) {
-        const float4 v = *reinterpret_cast<const float4 *>(staged + ((size_t)(span * 8 + quad) * kWaveLanes + lane) * 4);
-        xs[4 * quad] = v.x, xs[4 * quad + 1] = v.y, xs[4 * quad + 2] = v.z, xs[4 * quad + 3] = v.w;
+      // (No branch around a call, or the sharing is lost: a row of x past the last one is
+      // the last one again, worked on and never stored.)
+      for (int r = 0; r < kM; ++r) {
+        const uint32_t group = ((uint32_t)r < m ? (uint32_t)r : m - 1) * spans + span;
+        float xs[32], xsum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int quad = 0; quad < 8; ++quad) {
+          const float4 v = *reinterpret_cast<const float4 *>(staged + ((size_t)(group * 8 + quad) * kWaveLanes + lane) * 4);
+          xs[4 * quad] = v.x, xs[4 * quad + 1] = v.y, xs[4 * quad + 2] = v.z, xs[4 * quad + 3] = v.w;
+        }
+        if constexpr (kKind == 0) {
+          const float4 v = *reinterpret_cast<const float4 *>(sums + ((size_t)group * kWaveLanes + lane) * 4);
+          xsum[0] = v.x, xsum[1] = v.y, xsum[2] = v.z, xsum[3] = v.w;
+        }
+        totals[r] += Kind::dot(slot, at, xs, xsum);
       }
-      if constexpr (kKind == 0) {
-        const float4 v = *reinterpret_cast<const float4 *>(sums + ((size_t)span * kWaveLanes + lane) * 4);
-        xsum[0] = v.x, xsum[1] = v.y, xsum[2] = v.z, xsum[3] = v.w;
-      }
-      total += Kind::dot(slot, at, xs, xsum);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       if (++span == spans) {
-        const float whole = group_sum<kWaveLanes>(total);
-        if (lane == 0) Traits<TX>::store(y, (size_t)row, whole);
-        total = 0.0f;
+#pragma unroll
+        for (int r = 0; r < kM; ++r) {
+          const float whole = group_sum<kWaveLanes>(totals[r]);
+          if (lane == 0 && (uint32_t)r < m) Traits<TX>::store(y, (size_t)r * rows + row, whole);
+          totals[r] = 0.0f;
+        }
         span = 0;
         row += stride;
       }
@@ -608,14 +624,24 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
     // longer rows: x in LDS, as long as it fits in a block's 64 KiB beside the waves' row buffers
     // (for K = 4096 this measured slightly faster than 64 activations in registers: 13.8 against
     // 14.4 us for Q4_K [4096 -> 14336])
-    const size_t staged = (size_t)(p.k / 2048) * (2048 + (kKind == 0 ? 256 : 0)) * sizeof(float);
+    const size_t staged = (size_t)p.m * (p.k / 2048) * (2048 + (kKind == 0 ? 256 : 0)) * sizeof(float);
     const size_t parked = (size_t)kWavesPerBlock * LinesRow<kKind, 1>::kSlotBytes;
-    if (p.m == 1 && lines && p.k % 2048 == 0 && p.k > 2048 && staged + parked <= 64 * 1024) {
+    if (lines && p.k % 2048 == 0 && (p.k > 2048 || p.m > 1) && staged + parked <= 64 * 1024) {
       const uint32_t spans = p.k / 2048;
       const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
       const dim3 machine(wanted < 256u * 3u ? wanted : 256u * 3u);
-      hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX>), machine, block, staged, s, in, x, y, (uint32_t)p.rows,
-                         p.row_stride, spans);
+      if (p.m == 1)
+        hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 1>), machine, block, staged, s, in, x, y,
+                           (uint32_t)p.rows, p.row_stride, spans, p.m);
+      else if (p.m == 2)
+        hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 2>), machine, block, staged, s, in, x, y,
+                           (uint32_t)p.rows, p.row_stride, spans, p.m);
+      else if (p.m <= 4)
+        hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 4>), machine, block, staged, s, in, x, y,
+                           (uint32_t)p.rows, p.row_stride, spans, p.m);
+      else
+        hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 8>), machine, block, staged, s, in, x, y,
+                           (uint32_t)p.rows, p.row_stride, spans, p.m);
       return hipGetLastError();
     }
   }

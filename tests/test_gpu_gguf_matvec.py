@@ -132,6 +132,20 @@ def test_matvec_single_token_few_rows(tag):
             check(tag, "f32", raw, rows, k, x)
 
 
+@pytest.mark.parametrize("x_tag", ["f32", "bf16"])
+@pytest.mark.parametrize("tag", ["q4_k", "q6_k", "q8_0"])
+def test_matvec_few_tokens_whole_spans(tag, x_tag):
+    """Two to eight activation rows over rows of 2048 n values: each span is decoded once and
+    multiplied against every activation row held in LDS; what does not fit there (eight rows of
+    2048) takes the general kernel."""
+    rng = np.random.default_rng(1706)
+    for rows, k, m in ((300, 2048, 2), (3100, 2048, 4), (77, 2048, 6), (50, 4096, 3), (33, 6144, 2), (20, 2048, 8),
+                       (1, 2048, 5)):
+        raw = weights_for(tag, rng, rows, k)
+        note(f"matvec {tag} x {x_tag} rows {rows} k {k} m {m}")
+        check(tag, x_tag, raw, rows, k, rng.normal(0, 1, (m, k)).astype(np.float32))
+
+
 def test_matvec_schema_admission_and_decode_shape():
     D, DT = hc.TensorDesc.dense, hc.DataType
     w = hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ4K, DT.kBFloat16, 2048, 6144)
