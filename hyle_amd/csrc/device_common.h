@@ -25,18 +25,6 @@ struct BF16 {};
 __device__ __forceinline__ float bits_f32(uint32_t u) { return __uint_as_float(u); }
 __device__ __forceinline__ uint32_t f32_bits(float f) { return __float_as_uint(f); }
 
-// Multiply in which a zero operand gives +0 whatever the other operand is (even
-// infinity or NaN); every other case is the IEEE product.
-// The s_nop is part of the instruction's contract here: a result of the transcendental unit
-// (v_exp, v_rcp, v_rsq ...) needs one wait state before an ordinary VALU instruction reads it.
-// The compiler inserts that wait for its own instructions but does not look inside inline
-// assembly, so an operand that comes straight from exp2 / rcp would be read too early.
-__device__ __forceinline__ float mul_zero_wins(float a, float b) {
-  float r;
-  asm("s_nop 0\n\tv_mul_legacy_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
-  return r;
-}
-
 // f32 -> bf16 with the gfx950 converter (v_cvt_pk_bf16_f32).  It was compared on the
 // device with the reference rule of include/hyle/simd/dtype.h:114-121 (RN-even, NaN keeps
 // its upper payload and gains the quiet bit) over all 2^32 f32 patterns: identical.

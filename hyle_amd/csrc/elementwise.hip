@@ -57,14 +57,19 @@ __device__ __forceinline__ float silu_exact(float x) {
 // 1e-6 relative).  exp(-x) is carried scaled by 2^-32 so that it stays finite
 // down to x = -110, where silu(x) itself underflows every storage type:
 //   sigmoid = 2^-32 / (exp(-x) * 2^-32 + 2^-32).
-// The final product uses the "zero wins" multiply so that silu(-inf) is +0 as
-// in the reference rather than -inf * 0.
+// The final product is the ordinary one, so a sigmoid that underflowed to zero gives -0 for a
+// negative x, as x * sigmoid(x) does in the reference; only x = -inf is singled out (+0 there,
+// src/simd/math/activations.cc:44-47, instead of -inf * 0).
+__device__ __forceinline__ float times_or_zero_at_minus_inf(float x, float factor) {
+  const float product = x * factor;
+  return x == -INFINITY ? 0.0f : product;
+}
 __device__ __forceinline__ float silu_fast(float x) {
   constexpr float kNegLog2e = -1.44269504088896340736f;
   constexpr float kTwoM32 = 2.3283064365386963e-10f;
   const float scaled = __builtin_amdgcn_exp2f(__builtin_fmaf(x, kNegLog2e, -32.0f));
   const float sigmoid = __builtin_amdgcn_rcpf(scaled + kTwoM32) * kTwoM32;
-  return mul_zero_wins(x, sigmoid);
+  return times_or_zero_at_minus_inf(x, sigmoid);
 }
 
 template <class T> __device__ __forceinline__ float silu_for(float x) {
@@ -113,7 +118,7 @@ __device__ __forceinline__ float sigmoid_fast(float x) {
 // 0.5 * (1 + tanh(u)) = sigmoid(2u): the tanh form of GELU without the cancelling 1 + tanh.
 __device__ __forceinline__ float gelu_tanh_fast(float x) {
   const float inner = 0.79788456080286535588f * x * __builtin_fmaf(0.044715f, x * x, 1.0f);
-  return mul_zero_wins(x, sigmoid_fast(2.0f * inner));
+  return times_or_zero_at_minus_inf(x, sigmoid_fast(2.0f * inner));
 }
 // 1 - erf(z) for z >= 0 is poly(t) * exp(-z^2), t = 1 / (1 + p z) (Abramowitz and Stegun
 // 7.1.26, absolute error 1.5e-7); the negative side of 1 + erf is that product itself.
@@ -124,9 +129,9 @@ __device__ __forceinline__ float gelu_erf_fast(float x) {
   poly = __builtin_fmaf(t, poly, 1.421413741f);
   poly = __builtin_fmaf(t, poly, -0.284496736f);
   poly = __builtin_fmaf(t, poly, 0.254829592f);
-  const float tail = mul_zero_wins(poly * t, __builtin_amdgcn_exp2f(-1.44269504088896340736f * z * z));
+  const float tail = (poly * t) * __builtin_amdgcn_exp2f(-1.44269504088896340736f * z * z);
   const float one_plus_erf = x < 0.0f ? tail : 2.0f - tail;
-  return mul_zero_wins(x, 0.5f * one_plus_erf);
+  return times_or_zero_at_minus_inf(x, 0.5f * one_plus_erf);
 }
 template <class T> __device__ __forceinline__ float sigmoid_for(float x) {
   if constexpr (Traits<T>::kSize == 4) return sigmoid_exact(x);

@@ -93,10 +93,16 @@ def narrow_is_nan(bits: np.ndarray, tag: str) -> np.ndarray:
 
 
 def assert_narrow_ulp(got: np.ndarray, want: np.ndarray, tag: str, ulps: int = 1) -> int:
-    """Narrow float bit patterns within `ulps` units in the last place; NaN matches NaN.
+    """Narrow float bit patterns within `ulps` units in the last place; NaN matches NaN; where
+    both are zeros they must be the same zero (+0 and -0 are zero units apart but not equal).
     Returns how many elements differ at all."""
     g_nan, w_nan = narrow_is_nan(got, tag), narrow_is_nan(want, tag)
     assert np.array_equal(g_nan, w_nan), "NaN positions differ"
+    zeros = ((got & 0x7FFF) == 0) & ((want & 0x7FFF) == 0) & (got != want)
+    if zeros.any():
+        at = tuple(np.argwhere(zeros)[0])
+        raise AssertionError(f"{int(zeros.sum())} zeros of the wrong sign, first at {at}: "
+                             f"got {got[at]:#06x} want {want[at]:#06x}")
     diff = np.abs(ordered16(got) - ordered16(want))
     diff[w_nan] = 0
     worst = int(diff.max()) if diff.size else 0
