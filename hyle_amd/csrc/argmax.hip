@@ -114,31 +114,36 @@ __global__ __launch_bounds__(kBlockThreads) void argmax_tiles(const void *x, Can
   }
 }
 
-// One wave per row folds that row's candidates.
-template <class T>
+// kGroup adjacent lanes fold one row's candidates: 16 when a row has at most 16 tiles (four rows
+// per wave), a whole wave otherwise.  The candidate carries the winning element widened exactly,
+// so the value output is narrowed back from it without a second, dependent read of the row;
+// only a NaN winner (a row of nothing but NaN) is fetched again, for its payload bits.
+template <class T, int kGroup>
 __global__ __launch_bounds__(kBlockThreads) void argmax_finish(const void *x, const Candidate *partial,
                                                                void *values, int32_t *indices,
                                                                uint32_t rows, uint32_t width,
                                                                uint32_t tiles) {
-  const uint32_t row = blockIdx.x * (kBlockThreads / kWaveLanes) + threadIdx.x / kWaveLanes;
-  const uint32_t lane = threadIdx.x & (kWaveLanes - 1);
+  const uint32_t row = blockIdx.x * (kBlockThreads / kGroup) + threadIdx.x / kGroup;
+  const uint32_t lane = threadIdx.x % kGroup;
   LaneArg best{0.0f, -1};
   if (row < rows) {
-    for (uint32_t t = lane; t < tiles; t += kWaveLanes) {
+    for (uint32_t t = lane; t < tiles; t += kGroup) {
       const Candidate c = partial[(size_t)row * tiles + t];
       best = arg_best(best, LaneArg{c.value, c.index});
     }
   }
-  best = wave_best(best);
+  best = group_reduce<kGroup>(best, [](LaneArg a, LaneArg b) { return arg_best(a, b); });
   if (row < rows && lane == 0) {
     indices[row] = best.index;
     if (values != nullptr) {
-      // copy the winner's storage bits untouched
-      const size_t at = (size_t)row * width + (uint32_t)best.index;
-      if constexpr (Traits<T>::kSize == 4)
-        static_cast<uint32_t *>(values)[row] = static_cast<const uint32_t *>(x)[at];
-      else
-        static_cast<uint16_t *>(values)[row] = static_cast<const uint16_t *>(x)[at];
+      if constexpr (Traits<T>::kSize == 4) {
+        static_cast<uint32_t *>(values)[row] = f32_bits(best.value);
+      } else if (best.value != best.value) {
+        static_cast<uint16_t *>(values)[row] =
+            static_cast<const uint16_t *>(x)[(size_t)row * width + (uint32_t)best.index];
+      } else {
+        Traits<T>::store(values, row, best.value);
+      }
     }
   }
 }
@@ -157,9 +162,15 @@ hipError_t run(const ArgmaxParams &p, const void *x, void *values, int32_t *indi
                        partial, width, p.tiles, p.tile_elems);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
-  constexpr int kRowsPerBlock = kBlockThreads / kWaveLanes;
-  hipLaunchKernelGGL((argmax_finish<T>), dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock),
-                     dim3(kBlockThreads), 0, s, x, partial, values, indices, rows, width, p.tiles);
+  if (p.tiles <= 16) {
+    constexpr int kRowsPerBlock = kBlockThreads / 16;
+    hipLaunchKernelGGL((argmax_finish<T, 16>), dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock),
+                       dim3(kBlockThreads), 0, s, x, partial, values, indices, rows, width, p.tiles);
+  } else {
+    constexpr int kRowsPerBlock = kBlockThreads / kWaveLanes;
+    hipLaunchKernelGGL((argmax_finish<T, kWaveLanes>), dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock),
+                       dim3(kBlockThreads), 0, s, x, partial, values, indices, rows, width, p.tiles);
+  }
   return hipGetLastError();
 }
 

@@ -47,10 +47,25 @@ __device__ __forceinline__ float bf16_hi(uint32_t w) { return bits_f32(w & 0xFFF
 __device__ __forceinline__ float f16_to_f32(uint16_t h) {
   return (float)__builtin_bit_cast(_Float16, h);
 }
+// The value is made opaque before it is narrowed: left alone, the compiler fuses a preceding
+// multiply by a widened f16 into v_fma_mixlo_f16 (a * b + 0), and that +0 addend turns a
+// product of -0 into +0.
 __device__ __forceinline__ uint16_t f32_to_f16(float f) {
+  asm("" : "+v"(f));
   const uint16_t h = __builtin_bit_cast(uint16_t, (_Float16)f);
   const uint16_t nan = (uint16_t)(((f32_bits(f) >> 16) & 0x8000u) | 0x7FFFu);
   return (f != f) ? nan : h;
+}
+
+// Two values narrowed by one v_cvt_pk_f16_f32, under the same rules as f32_to_f16.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  asm("" : "+v"(lo), "+v"(hi));
+  const f32x2 in = {lo, hi};
+  const uint32_t pair = __builtin_bit_cast(uint32_t, __builtin_convertvector(in, f16x2));
+  const uint32_t nans = ((f32_bits(lo) >> 16) & 0x8000u) | (f32_bits(hi) & 0x80000000u) | 0x7FFF7FFFu;
+  const uint32_t take = (lo != lo ? 0x0000FFFFu : 0u) | (hi != hi ? 0xFFFF0000u : 0u);
+  return (pair & ~take) | (nans & take);
 }
 
 // ---- per-type traits: element size, elements per 16-byte vector, scalar and
@@ -118,10 +133,8 @@ template <> struct Traits<F16> {
   }
   static __device__ __forceinline__ u32x4 pack(const float (&v)[8]) {
     u32x4 w;
-    w.x = (uint32_t)f32_to_f16(v[0]) | ((uint32_t)f32_to_f16(v[1]) << 16);
-    w.y = (uint32_t)f32_to_f16(v[2]) | ((uint32_t)f32_to_f16(v[3]) << 16);
-    w.z = (uint32_t)f32_to_f16(v[4]) | ((uint32_t)f32_to_f16(v[5]) << 16);
-    w.w = (uint32_t)f32_to_f16(v[6]) | ((uint32_t)f32_to_f16(v[7]) << 16);
+    w.x = pack_f16x2(v[0], v[1]); w.y = pack_f16x2(v[2], v[3]);
+    w.z = pack_f16x2(v[4], v[5]); w.w = pack_f16x2(v[6], v[7]);
     return w;
   }
 };

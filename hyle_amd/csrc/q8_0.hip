@@ -8,11 +8,17 @@
 // an 8-bit by 11-bit significand product, exact in f32, so the bf16 store is one
 // RN-even rounding and the result is bit-identical on every implementation.
 //
-// Blocks are only 2-byte aligned, so a wave stages its rows in LDS with 16-byte
-// global loads and re-slices them with 2-byte LDS reads; output leaves as
-// 16-byte bf16x8 stores.  Each row's sum of squares of the exact products is
-// reduced with a wave64 butterfly.
+// Blocks are only 2-byte aligned, so a wave parks its row in LDS with 16-byte global loads
+// (every cache line requested once) and re-slices it there; output leaves as 16-byte bf16x8
+// stores, 1 KiB of consecutive bf16 per store instruction of a wave.  Each row's sum of squares
+// of the exact products is reduced with a wave64 butterfly.
+//
+// Three kernels: rows of K = 2048 n values made of whole 16-byte vectors take one wave per row
+// with a region of LDS that only this wave touches and no block barrier (q8_0_lines: aligned
+// 32-bit LDS words joined by byte-wise funnel shifts); other rows of whole vectors stage
+// block-wide with 2-byte LDS reads (q8_0_rows); anything else reads bytes (q8_0_rows_bytes).
 #include "device_common.h"
+#include "gguf_decode.h"
 #include "kernels.h"
 
 namespace hyle_hip {
@@ -74,6 +80,73 @@ __global__ __launch_bounds__(kWaves *kWaveLanes) void q8_0_rows(const char *bloc
   }
 }
 
+// Rows of K = 2048 n values, whole 16-byte vectors, 16-byte aligned: one wave per row, no barrier.
+// A span of 2048 values is 64 blocks = 2176 bytes = 136 vectors: two per lane and a third for
+// the first eight lanes (the others repeat the span's last vector, one request for all of them);
+// plain loads: the non-temporal hint costs 10 % here, while the stores keep it.
+// The vectors are parked in LDS that only this wave touches (LDS executes one wave's
+// instructions in order); lane l then decodes output vectors l, l + 64, l + 128, l + 192 of
+// the span: eight quants at a 2-byte aligned offset come out of three aligned words and two
+// funnel shifts, the block's scale out of one 16-bit read.  The next span's loads are in flight
+// while this one is decoded.
+template <int kWaves>
+__global__ __launch_bounds__(kWaves *kWaveLanes) void q8_0_lines(const unsigned char *blocks, void *out,
+                                                                float *sumsq, uint32_t rows, uint32_t k,
+                                                                uint64_t row_stride) {
+  constexpr uint32_t kSpan = 2048;
+  constexpr uint32_t kVectors = kSpan / kBlockElems * kBlockBytes / 16;  // 136
+  constexpr int kLoads = (kVectors + kWaveLanes - 1) / kWaveLanes;       // 3
+  __shared__ __align__(16) unsigned char slots[kWaves][kLoads * kWaveLanes * 16];
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  const uint32_t row = blockIdx.x * kWaves + wave;
+  if (row >= rows) return;
+  unsigned char *slot = slots[wave];
+  const unsigned char *source = blocks + (size_t)row * row_stride;
+  const uint32_t steps = k / kSpan;
+  uint32_t vec[kLoads];
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) {
+    const uint32_t wanted = lane + i * kWaveLanes;
+    vec[i] = wanted < kVectors ? wanted : kVectors - 1;
+  }
+  u32x4 raw[kLoads];
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) raw[i] = load16(source, vec[i]);
+  float squares = 0.0f;
+  for (uint32_t step = 0; step < steps; ++step) {
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = raw[i];
+    if (step + 1 < steps) {  // uniform across the wave
+#pragma unroll
+      for (int i = 0; i < kLoads; ++i) raw[i] = load16(source, (size_t)(step + 1) * kVectors + vec[i]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (uint32_t i = 0; i < kSpan / (kWaveLanes * 8); ++i) {
+      const uint32_t j = i * kWaveLanes + lane;  // output vector of the span: block j / 4, quants 8 (j % 4) ..
+      const uint32_t block_offset = (j / 4) * kBlockBytes;
+      const float d = f16_to_f32(*reinterpret_cast<const uint16_t *>(slot + block_offset));
+      uint32_t q[2];
+      lds_piece(slot, block_offset + 2 + 8 * (j % 4), q);
+      float y[8];
+#pragma unroll
+      for (int w = 0; w < 2; ++w)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) y[4 * w + t] = (float)(int)(signed char)(q[w] >> (8 * t)) * d;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) squares = __builtin_fmaf(y[e], y[e], squares);
+      store16_stream(out, ((size_t)row * k + (size_t)step * kSpan) / 8 + j, Traits<BF16>::pack(y));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  squares = group_sum<kWaveLanes>(squares);
+  if (lane == 0) sumsq[row] = squares;
+}
+
 // Any k (multiple of 32), any stride or alignment: one wave per row, byte loads.
 __global__ __launch_bounds__(kBlockThreads) void q8_0_rows_bytes(const uint8_t *blocks, uint16_t *out,
                                                                  float *sumsq, uint32_t rows,
@@ -117,6 +190,16 @@ hipError_t launch_q8_0_dequant(const Q8Params &p, const void *blocks, void *out,
   const uint32_t row_bytes = p.k / kBlockElems * kBlockBytes;
   const bool fast = vectorised && row_bytes != 0 && row_bytes % 16 == 0 &&
                     p.row_stride % 16 == 0 && row_bytes <= kMaxRowBytes;
+  if (fast && p.k % 2048 == 0) {
+    // Measured on MI355X for W[6144 x 2048] (38.6 MB of traffic, buffers rotated): 6.7 us with
+    // plain loads and non-temporal stores; 7.4 us with non-temporal loads too; 8.6 / 10.5 us with
+    // plain stores; a wave that walks several rows with the next row in flight 7.3 - 9.3 us; the
+    // block-staged kernel below 7.1 us.
+    constexpr int kWaves = 4;
+    hipLaunchKernelGGL((q8_0_lines<kWaves>), dim3((rows + kWaves - 1) / kWaves), dim3(kWaves * kWaveLanes), 0, stream,
+                       static_cast<const unsigned char *>(blocks), out, sumsq, rows, p.k, p.row_stride);
+    return hipGetLastError();
+  }
   if (fast) {
     // Measured on MI355X for W[6144 x 2048]: 2, 4 or 8 waves per block with one row per wave
     // all take about 8 us; two or four rows per wave are slower (9 to 13 us).
