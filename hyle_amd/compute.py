@@ -506,6 +506,10 @@ class PreparedOperation:
             raise StatusError(capi.INVALID_ARGUMENT, "workspace is smaller than the plan requires")
         return OperationInvocation(self, workspace, workspace_size)
 
+    def create_invocation_without_workspace(self) -> "OperationInvocation":
+        """An invocation for `submit_without_workspace` only."""
+        return OperationInvocation(self, 0, 0)
+
     def close(self) -> None:
         if self._handle:
             capi.load().hyle_hip_plan_destroy(self._handle)
@@ -534,6 +538,17 @@ class OperationInvocation:
         _check(capi.load().hyle_hip_plan_launch(
             self._prepared._handle, self._in, len(inputs), self._out, len(outputs),
             self._workspace, self._workspace_size, stream))
+
+    def submit_without_workspace(self, stream: int, inputs: Sequence[int], outputs: Sequence[int]) -> None:
+        """The same launch through hyle_hip_plan_launch_static: the route's workspace is the
+        library's per-device scratch array, nothing is allocated.  Calls that may overlap on
+        one device race on that array."""
+        for i, p in enumerate(inputs):
+            self._in[i] = p
+        for i, p in enumerate(outputs):
+            self._out[i] = p
+        _check(capi.load().hyle_hip_plan_launch_static(
+            self._prepared._handle, self._in, len(inputs), self._out, len(outputs), stream))
 
 
 def prepare(context: Context, operation, *inputs: TensorDesc,

@@ -9,6 +9,7 @@
 #include <cstdio>
 #include <cstring>
 #include <limits>
+#include <mutex>
 #include <new>
 
 #include "../../include/hyle_hip.h"
@@ -511,6 +512,7 @@ constexpr uint64_t kMaxElements = (uint64_t)std::numeric_limits<int32_t>::max();
 struct hyle_hip_context {
   int device = 0;
   int compute_units = 0;
+  void *static_scratch = nullptr;  // this device's copy of `scratch` (hyle_hip_plan_launch_static)
 };
 
 struct hyle_hip_plan {
@@ -1008,6 +1010,49 @@ bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) &
 }  // namespace
 
 // ---------------------------------------------------------------------------------
+// Device scratch of hyle_hip_plan_launch_static: the workspace of the two-dispatch routes for
+// callers that cannot allocate.  Every device the library runs on holds its own copy of the
+// array at its own address until the process ends.  In host code the array's name is only a
+// stand-in for the symbol, never a device address: the address is looked up once per device,
+// with that device current, and only that pointer is handed to kernels.
+// ---------------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = HYLE_HIP_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_address[kMaxDevices] = {};
+
+// The address of `scratch` on `device`, resolved on first use.  The calling thread's current
+// device is left as it was.
+hyle_hip_status static_scratch_address(int device, void **address) {
+  *address = nullptr;
+  if (device < 0 || device >= kMaxDevices)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "device %d is outside the %d devices the scratch table holds", device,
+                kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_address[device] == nullptr) {
+    int previous = 0;
+    hipError_t err = hipGetDevice(&previous);
+    if (err != hipSuccess) return hip_fail(err, "hipGetDevice");
+    if (previous != device && (err = hipSetDevice(device)) != hipSuccess) return hip_fail(err, "hipSetDevice");
+    void *found = nullptr;
+    err = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+    if (previous != device) (void)hipSetDevice(previous);
+    if (err != hipSuccess) return hip_fail(err, "hipGetSymbolAddress(scratch)");
+    if (found == nullptr || !aligned(found, 256))
+      return fail(HYLE_HIP_INTERNAL, "device scratch has no usable address on device %d", device);
+    g_scratch_address[device] = found;
+  }
+  *address = g_scratch_address[device];
+  return HYLE_HIP_OK;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------
 // C ABI
 // ---------------------------------------------------------------------------------
 extern "C" {
@@ -1051,6 +1096,11 @@ hyle_hip_status hyle_hip_context_create(int device, hyle_hip_context **context) 
   if (ctx == nullptr) return fail(HYLE_HIP_RESOURCE_EXHAUSTED, "out of host memory");
   ctx->device = device;
   ctx->compute_units = props.multiProcessorCount;
+  const hyle_hip_status scratch_status = static_scratch_address(device, &ctx->static_scratch);
+  if (scratch_status != HYLE_HIP_OK) {
+    delete ctx;
+    return scratch_status;
+  }
   *context = ctx;
   return HYLE_HIP_OK;
 }
@@ -1260,6 +1310,29 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
   }
   if (err != hipSuccess) return hip_fail(err, "kernel launch");
   return HYLE_HIP_OK;
+}
+
+size_t hyle_hip_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+hyle_hip_status hyle_hip_plan_launch_static(const hyle_hip_plan *plan, const void *const *inputs,
+                                            uint32_t input_count, void *const *outputs, uint32_t output_count,
+                                            void *stream_handle) {
+  if (plan == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "plan is null");
+  if (plan->workspace_size > kStaticScratchBytes)
+    return fail(HYLE_HIP_RESOURCE_EXHAUSTED,
+                "the plan needs %zu bytes of workspace; the device scratch of hyle_hip_plan_launch_static holds %zu: "
+                "use hyle_hip_plan_launch with a caller-owned workspace",
+                plan->workspace_size, kStaticScratchBytes);
+  void *workspace = nullptr;
+  if (plan->workspace_size != 0) {
+    if (plan->context == nullptr || plan->context->static_scratch == nullptr)
+      return fail(HYLE_HIP_FAILED_PRECONDITION, "plan was built without a device context");
+    workspace = plan->context->static_scratch;
+  }
+  // Every route writes the part of the workspace it later reads, so nothing has to start at
+  // zero; the last call's contents are simply overwritten.
+  return hyle_hip_plan_launch(plan, inputs, input_count, outputs, output_count, workspace,
+                              plan->workspace_size, stream_handle);
 }
 
 }  // extern "C"

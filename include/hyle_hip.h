@@ -36,6 +36,8 @@ extern "C" {
 #define HYLE_HIP_MAX_INPUTS 4
 #define HYLE_HIP_MAX_OUTPUTS 2
 #define HYLE_HIP_ABI_VERSION 1u
+/* Device scratch behind hyle_hip_plan_launch_static, per device. */
+#define HYLE_HIP_STATIC_SCRATCH_BYTES (4u * 1024u * 1024u)
 
 /* hyle::StatusCode.  UNIMPLEMENTED from plan_create is a clean decline (the
  * caller tries its next provider, src/compute/operation.cc:1259-1266); every
@@ -244,6 +246,24 @@ HYLE_HIP_API hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan,
                                                   void *const *outputs, uint32_t output_count,
                                                   void *workspace, size_t workspace_size,
                                                   void *stream);
+
+/* hyle_hip_plan_launch for callers that cannot allocate device memory and have no workspace to
+ * pass: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
+ * has no counterpart in the reference, whose callers always own the workspace
+ * (ProviderPrepared::workspace).  The workspace of the two-dispatch routes (TopK, tiled Reduce)
+ * is a file-scope device array of HYLE_HIP_STATIC_SCRATCH_BYTES that every device holds from
+ * the first context on it until the process ends; its address is looked up once per device in
+ * hyle_hip_context_create.  Nothing is allocated or freed here.  A plan whose workspace exceeds
+ * the array is refused with RESOURCE_EXHAUSTED.  All calls on one device share the one array:
+ * calls that may overlap on a device (different streams, different threads) race, so serialise
+ * them on one stream or use hyle_hip_plan_launch with separate workspaces.  Results are those of
+ * hyle_hip_plan_launch bit for bit. */
+HYLE_HIP_API hyle_hip_status hyle_hip_plan_launch_static(const hyle_hip_plan *plan,
+                                                         const void *const *inputs, uint32_t input_count,
+                                                         void *const *outputs, uint32_t output_count,
+                                                         void *stream);
+/* Size of that array: the largest hyle_hip_plan_workspace a plan may need to be served. */
+HYLE_HIP_API size_t hyle_hip_static_scratch_bytes(void);
 
 /* Text of the last non-OK status returned on the calling thread. */
 HYLE_HIP_API const char *hyle_hip_last_error(void);
