@@ -87,8 +87,11 @@ def main() -> int:
         """One kernel of the step: a prepared operation plus `sets` rotating buffer sets."""
 
         def __init__(self, name, operation, descs, make_set, sets, algorithmic_bytes, elements, dtype,
-                     credited_bytes=None, in_step=True):
+                     credited_bytes=None, in_step=True, ceiling=None):
             self.name, self.bytes, self.elements, self.dtype = name, algorithmic_bytes, elements, dtype
+            # name of the plain kernel (a copy or a read-only scan of about the same traffic, timed in
+            # this run) whose GB/s is the practical ceiling for a launch of this size
+            self.ceiling = ceiling
             # Bytes the kernel is credited with: the algorithmic bytes, minus loads it provably
             # does not need and does not issue (no bandwidth is claimed for bytes never moved).
             self.credited = algorithmic_bytes if credited_bytes is None else credited_bytes
@@ -128,7 +131,8 @@ def main() -> int:
             return [da, db, ds], [torch.empty_like(da)]
         ops.append(Op("cfg1_broadcast_add_mul_f32", hc.BinaryChain(BK.kAdd, BK.kMultiply),
                       [D(F32, [4096, 2048]), D(F32, [2048]), D(F32, [1])], set1, 10,
-                      wl.ALGORITHMIC_BYTES["cfg1_broadcast_add_mul_f32"], 4096 * 2048, "f32"))
+                      wl.ALGORITHMIC_BYTES["cfg1_broadcast_add_mul_f32"], 4096 * 2048, "f32",
+                      ceiling="ceiling_copy_67mb"))
     # ---- cfg2 ---------------------------------------------------------------------------
     if want("cfg2_rmsnorm_bf16"):
         x, w = wl.config2()
@@ -138,7 +142,7 @@ def main() -> int:
             dx = bf16(np.roll(x, i, axis=0))
             return [dx, dw], [torch.empty_like(dx)]
         ops.append(Op("cfg2_rmsnorm_bf16", hc.RmsNorm(epsilon=1e-6), [D(BF, [8192, 2048]), D(BF, [2048])], set2, 10,
-                      wl.ALGORITHMIC_BYTES["cfg2_rmsnorm_bf16"], 8192 * 2048, "bf16"))
+                      wl.ALGORITHMIC_BYTES["cfg2_rmsnorm_bf16"], 8192 * 2048, "bf16", ceiling="ceiling_copy_67mb"))
     # ---- cfg3 ---------------------------------------------------------------------------
     if want("cfg3_swiglu_bf16"):
         gate, up = wl.config3_swiglu()
@@ -159,9 +163,10 @@ def main() -> int:
                       set3r, 10, wl.ALGORITHMIC_BYTES["cfg3_residual_add_bf16"], 8192 * 2048, "bf16"))
     # ---- cfg4 ---------------------------------------------------------------------------
     if want("cfg4_softmax_f32_causal"):
-        gen = torch.Generator(device=dev).manual_seed(3)
-        big = torch.randn((32, 4096, 4096), generator=gen, device=dev, dtype=torch.float32).mul_(3.0)
-        causal = torch.ones((4096, 4096), dtype=torch.bool, device=dev).tril_()
+        s4_host, mask_host = wl.config4_softmax()  # seed 3: the bytes the parity test and the CPU leg use
+        big = torch.from_numpy(s4_host).to(dev)
+        causal = torch.from_numpy(mask_host).to(dev).view(torch.bool)
+        del s4_host, mask_host
         big_out = torch.empty_like(big)
         # Under the Boolean mask the kernel does not load a 16-byte vector of S whose four
         # elements are all masked (they cannot influence the result), so row q reads q // 4 + 1
@@ -187,7 +192,7 @@ def main() -> int:
             return [dl], [torch.empty((64, 1), dtype=torch.float32, device=dev),
                           torch.empty((64, 1), dtype=torch.int32, device=dev)]
         ops.append(Op("cfg4_argmax_f32", hc.TopK(), [D(F32, [64, 151936])], set4a, 16,
-                      wl.ALGORITHMIC_BYTES["cfg4_argmax_f32"], 64 * 151936, "f32"))
+                      wl.ALGORITHMIC_BYTES["cfg4_argmax_f32"], 64 * 151936, "f32", ceiling="ceiling_scan_38mb"))
     # ---- cfg5 ---------------------------------------------------------------------------
     if want("cfg5_q8_0_dequant_sumsq"):
         blocks = wl.config5()
@@ -198,7 +203,7 @@ def main() -> int:
                            torch.empty(6144, dtype=torch.float32, device=dev)]
         ops.append(Op("cfg5_q8_0_dequant_sumsq", hc.Q8_0DequantSumSquares(),
                       [hc.TensorDesc.gguf_q8_0_weight(BF, 2048, 6144)], set5, 16,
-                      wl.ALGORITHMIC_BYTES["cfg5_q8_0_dequant_sumsq"], 6144 * 2048, "u8/bf16"))
+                      wl.ALGORITHMIC_BYTES["cfg5_q8_0_dequant_sumsq"], 6144 * 2048, "u8/bf16", ceiling="ceiling_copy_38mb"))
     # ---- the K-quant siblings of cfg5 (GGUF Q4_K / Q6_K), timed beside the step ------------------
     for name, gguf, block_bytes in (("next_q4_k_dequant_sumsq", hc.GgufQuantizedType.kQ4K, 144),
                                     ("next_q6_k_dequant_sumsq", hc.GgufQuantizedType.kQ6K, 210)):
@@ -314,6 +319,35 @@ def main() -> int:
             return [src], [torch.empty_like(src)]
         ops.append(Op("next_copy_bf16", hc.Copy(), [D(BF, [8192, 6144])], set_copy, 3,
                       8192 * 6144 * 4, 8192 * 6144, "bf16", in_step=False))
+    # ---- practical ceilings for launches of 38 / 67 MB: a plain copy and a plain read-only scan (a
+    # row maximum, one wave per row, one dispatch) of the traffic of the step's small shapes, through
+    # the same C ABI and rotated the same way.  Kernels of this size run for 6 - 12 us, of which the
+    # start and the drain of the launch are a fixed part no kernel avoids; `frac_of_ceiling` of a
+    # small op is its GB/s over the GB/s of the plain kernel named in `ceiling`.
+    ceiling_lines = (
+        ("ceiling_copy_38mb", "copy", BF, torch.bfloat16, [4712, 2048], 16),
+        ("ceiling_copy_67mb", "copy", F32, torch.float32, [4096, 2048], 10),
+        ("ceiling_scan_38mb", "scan", F32, torch.float32, [9496, 1024], 16),
+        ("ceiling_scan_67mb", "scan", F32, torch.float32, [16384, 1024], 10),
+    )
+    needed = {o.ceiling for o in ops if o.ceiling}
+    for name, form, dtype, torch_dtype, dims, sets in ceiling_lines:
+        if not (want(name) if wanted else True) and name not in needed:
+            continue
+        size = 4 if dtype == F32 else 2
+        if form == "copy":
+            def set_plain(i, dims=dims, torch_dtype=torch_dtype):
+                src = torch.empty(dims, dtype=torch_dtype, device=dev).normal_()
+                return [src], [torch.empty_like(src)]
+            ops.append(Op(name, hc.Copy(), [D(dtype, dims)], set_plain, sets, 2 * dims[0] * dims[1] * size,
+                          dims[0] * dims[1], "bf16" if dtype == BF else "f32", in_step=False))
+        else:
+            def set_plain(i, dims=dims, torch_dtype=torch_dtype):
+                src = torch.empty(dims, dtype=torch_dtype, device=dev).normal_()
+                return [src], [torch.empty(dims[:1], dtype=torch_dtype, device=dev)]
+            ops.append(Op(name, hc.Reduce(hc.ReductionKind.kMaximum, hc.Axes.from_([-1]), accumulation_type=F32),
+                          [D(dtype, dims)], set_plain, sets, dims[0] * dims[1] * size + dims[0] * size,
+                          dims[0] * dims[1], "f32", in_step=False))
     if not any(o.in_step for o in ops):
         print("no kernel of the step selected", file=sys.stderr)
         return 2
@@ -418,6 +452,14 @@ def main() -> int:
             entry["gbps_cached"] = round(op.credited / us_cached / 1e3, 1)
             del cached
         per_op.append(entry)
+
+    by_name = {entry["op"]: entry for entry in per_op}
+    for op in ops:
+        if op.ceiling and op.ceiling in by_name:
+            entry, plain = by_name[op.name], by_name[op.ceiling]
+            entry["ceiling"] = op.ceiling
+            entry["ceiling_gbps"] = plain["gbps"]
+            entry["frac_of_ceiling"] = round(entry["gbps"] / plain["gbps"], 4)
 
     if args.copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -661,6 +703,8 @@ def cpu_baseline(args, ops, np, torch, wl):
     step_bytes = sum(o.bytes for o in ops)
     return {"value": round(step_bytes / total_seconds_full / 1e9, 3), "unit": "GB/s", "cores": cores,
             "kind": "port",
+            "build": "oracle/hyle_oracle.c, gcc -O3 -march=x86-64-v3 -ffp-contract=off (AVX2 + FMA, not "
+                     "-march=native: the library is built before it travels to this host)",
             "sample": "row subsets of the same seeded inputs, per-kernel time scaled to the full shape; " + "; ".join(samples)}
 
 

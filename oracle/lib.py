@@ -297,6 +297,26 @@ def softmax_f32_row(src):
     return out
 
 
+def softmax_bool_f32_rows(src, mask, threads=1):
+    """Row softmax of dense f32 [rows, cols] under a Boolean mask [mask_rows, cols] (row r uses
+    mask row r % mask_rows), rows fanned out over `threads` host threads (the C loop releases
+    the interpreter lock)."""
+    from concurrent.futures import ThreadPoolExecutor
+    src = _c(src, np.float32)
+    mask = _c(mask, np.uint8)
+    rows, cols = src.shape
+    out = np.empty_like(src)
+    fn = _lib.hyle_oracle_rows_softmax_bool_f32
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t]
+    threads = max(1, min(threads, rows))
+    edges = [rows * t // threads for t in range(threads + 1)]
+    with ThreadPoolExecutor(max_workers=threads) as pool:
+        list(pool.map(lambda t: fn(_ptr(src), _ptr(mask), _ptr(out), cols, mask.shape[0], edges[t], edges[t + 1]),
+                      range(threads)))
+    return out
+
+
 def log_softmax_f32_row(src):
     src = _c(src, np.float32)
     out = np.empty_like(src)
