@@ -575,6 +575,29 @@ void hyle_oracle_log_softmax_f32_row(const float *src, float *dst, size_t n) {
   for (size_t i = 0; i < n; ++i) dst[i] = (src[i] - maximum) - normalizer;
 }
 
+/* LogSoftmax of one row as the reference's scalar floor writes it
+ * (src/simd/math/activations.cc:320-336): the same row validity rule as softmax
+ * (any NaN, any +inf or nothing above -inf: the whole row is a quiet NaN), the
+ * sum of expf(v - max) in double, shift = max + (float)log(sum), result
+ * v - shift. */
+void hyle_oracle_log_softmax_floor_f32_row(const float *src, float *dst, size_t n) {
+  if (n == 0) return;
+  float maximum = -INFINITY;
+  int valid = 1;
+  for (size_t i = 0; i < n && valid; ++i) {
+    if (isnan(src[i]) || src[i] == INFINITY) valid = 0;
+    else if (src[i] > maximum) maximum = src[i];
+  }
+  if (!valid || !isfinite(maximum)) {
+    for (size_t i = 0; i < n; ++i) dst[i] = NAN;
+    return;
+  }
+  double sum = 0.0;
+  for (size_t i = 0; i < n; ++i) sum += (double)expf(src[i] - maximum);
+  const float shift = maximum + (float)log(sum);
+  for (size_t i = 0; i < n; ++i) dst[i] = src[i] - shift;
+}
+
 static void softmax_rows(int log_form, int type, const void *src, void *dst,
                          const int64_t *in_dims, int in_rank, float scale,
                          int mask_kind, const void *mask,

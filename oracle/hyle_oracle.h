@@ -25,9 +25,12 @@
  *   - rms_norm_bf16_native tile order: "parity unpinned" at the bit level (the
  *     reference sums each 128-wide tile with a Highway vector dot whose lane
  *     order is target-dependent); pinned only to tolerance.
- *   - cast, layer_norm, unary / gated kinds, reduce over any axes, topk,
- *     log_softmax: pinned by the reference's scalar floor (where it holds the
- *     function), its tests' known answers and numpy / float64 closed forms.
+ *   - cast, layer_norm, unary / gated kinds, reduce over any axes, topk:
+ *     pinned by the reference's scalar floor (where it holds the function),
+ *     its tests' known answers and numpy / float64 closed forms.
+ *   - log_softmax: the floor's form (log_softmax_floor) is pinned bit-exact
+ *     against oracle/_ref and golden vectors; the log1p form the GPU kernel
+ *     follows is held to it at the reference's own bound.
  *   - k_quant_dequant (GGUF Q4_K, Q6_K): "parity unpinned" against ggml's
  *     source, which is not in the reference tree; the restatement of the
  *     published block layouts is checked against blocks packed field by field.
@@ -204,6 +207,11 @@ void hyle_oracle_softmax(int type, const void *src, void *dst,
  * maximum), NaN when the maximum is not finite
  * (src/compute_provider_cuda/reduction_kernel.cu:73-86,148-196). */
 void hyle_oracle_log_softmax_f32_row(const float *src, float *dst, size_t n);
+/* The same row in the scalar floor's own form (double sum, one log, one shift;
+ * src/simd/math/activations.cc:320-336), pinned bit for bit against the floor
+ * compiled from the reference's sources; hyle_oracle_log_softmax_f32_row is
+ * held to it at the reference's bound (4e-6 relative + 2e-7). */
+void hyle_oracle_log_softmax_floor_f32_row(const float *src, float *dst, size_t n);
 void hyle_oracle_log_softmax(int type, const void *src, void *dst,
                              const int64_t *in_dims, int in_rank, float scale,
                              int mask_kind, const void *mask,

@@ -79,6 +79,7 @@ _softmax = _sig("hyle_oracle_softmax", None, C.c_int, _vp, _vp, _i64p, C.c_int, 
 _log_softmax = _sig("hyle_oracle_log_softmax", None, C.c_int, _vp, _vp, _i64p, C.c_int, C.c_float,
                     C.c_int, _vp, _i64p, _i64p, C.c_int)
 _log_softmax_row = _sig("hyle_oracle_log_softmax_f32_row", None, _vp, _vp, _sz)
+_log_softmax_floor_row = _sig("hyle_oracle_log_softmax_floor_f32_row", None, _vp, _vp, _sz)
 _reduce = _sig("hyle_oracle_reduce_last_axis", None, C.c_int, C.c_int, _vp, _vp, _sz, _sz)
 _iom = _sig("hyle_oracle_index_of_max_f32", _sz, _vp, _sz)
 _topk1 = _sig("hyle_oracle_topk1_f32", None, _vp, _sz, _sz, _vp, _vp)
@@ -321,6 +322,14 @@ def log_softmax_f32_row(src):
     src = _c(src, np.float32)
     out = np.empty_like(src)
     _log_softmax_row(_ptr(src), _ptr(out), src.size)
+    return out
+
+
+def log_softmax_floor_f32_row(src):
+    """The scalar floor's own form of LogSoftmax (double sum, one log, one shift)."""
+    src = _c(src, np.float32)
+    out = np.empty_like(src)
+    _log_softmax_floor_row(_ptr(src), _ptr(out), src.size)
     return out
 
 

@@ -110,3 +110,10 @@ def softmax_f32(src: np.ndarray) -> np.ndarray:
     out = np.empty_like(src)
     _fn("ref_softmax_f32", None, _vp, _vp, _sz)(_p(src), _p(out), src.size)
     return out
+
+
+def log_softmax_f32(src: np.ndarray) -> np.ndarray:
+    src = np.ascontiguousarray(src, np.float32)
+    out = np.empty_like(src)
+    _fn("ref_log_softmax_f32", None, _vp, _vp, _sz)(_p(src), _p(out), src.size)
+    return out

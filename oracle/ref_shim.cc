@@ -142,5 +142,8 @@ void ref_layer_norm_bf16(const std::uint16_t *src, const std::uint16_t *scale, c
 void ref_softmax_f32(const float *src, float *dst, std::size_t n) {
   hd::softmax_f32_scalar(src, dst, n);
 }
+void ref_log_softmax_f32(const float *src, float *dst, std::size_t n) {
+  hd::log_softmax_f32_scalar(src, dst, n);
+}
 
 }  // extern "C"

@@ -135,6 +135,25 @@ def main() -> None:
     out["geglu_bf16"] = ref.gated("geglu", 2, out["more_x_bf16"], out["more_u_bf16"])
     out["geglu_tanh_bf16"] = ref.gated("geglu_tanh", 2, out["more_x_bf16"], out["more_u_bf16"])
 
+    # log-softmax rows of the floor (drawn last, see above)
+    for n in (1, 7, 8, 9, 257, 4096):
+        row = rng.normal(0, 3, n).astype(np.float32)
+        out[f"log_softmax_x_{n}"] = row
+        out[f"log_softmax_y_{n}"] = ref.log_softmax_f32(row)
+    masked = rng.normal(0, 3, 512).astype(np.float32)
+    masked[rng.random(512) < 0.5] = -np.inf
+    out["log_softmax_x_masked"] = masked
+    out["log_softmax_y_masked_words"] = ref.log_softmax_f32(masked).view(np.uint32)
+    wide = rng.uniform(-120, 40, 300).astype(np.float32)
+    out["log_softmax_x_wide"] = wide
+    out["log_softmax_y_wide_words"] = ref.log_softmax_f32(wide).view(np.uint32)
+    for width in (129, 8193):   # tests/compute_provider_cuda/tensor_test.cc:1168-1199: near-one tails
+        tails = np.full((3, width), -20.0, np.float32)
+        tails[0, width - 1] = 0
+        tails[1, 0] = tails[1, width - 1] = 0
+        tails[2, :] = 0
+        out[f"log_softmax_y_tails_{width}"] = np.stack([ref.log_softmax_f32(r) for r in tails])
+
     np.savez_compressed(OUT, **out)
     print(f"wrote {OUT}: {os.path.getsize(OUT)} bytes, {len(out)} arrays")
 

@@ -117,3 +117,16 @@ def test_log_softmax_other_axes_views_and_undefined_rows():
     got = to_host(out)
     log_bar(got, orc.softmax(orc.F32, rows, log=True), "f32")
     assert np.isneginf(got[0, 1]) and np.isneginf(got[0, 3]) and np.isnan(got[1:]).all()
+
+
+def test_log_softmax_against_the_scalar_floor_golden_rows():
+    """The floor's own outputs (src/simd/math/activations.cc:320-336, committed as data) at the
+    reference's bound for this operator."""
+    import os
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "scalar_floor_vectors.npz"))
+    cases = [(gold[f"log_softmax_x_{n}"], gold[f"log_softmax_y_{n}"]) for n in (1, 7, 8, 9, 257, 4096)]
+    cases.append((gold["log_softmax_x_masked"], gold["log_softmax_y_masked_words"].view(np.float32)))
+    for x, want in cases:
+        note(f"log-softmax floor golden row n={x.size}")
+        (out,) = run(hc.Softmax(kind=LOG), to_device(x[None, :], "f32"))
+        log_bar(to_host(out)[0], want, "f32")

@@ -72,3 +72,86 @@ def test_closed_form_masks_and_undefined_rows():
     assert np.all(np.isnan(got[1])) and np.all(np.isnan(got[2])) and not np.any(np.isnan(got[0]))
     assert np.all(np.isnan(orc.log_softmax_f32_row(np.array([-np.inf, -np.inf], np.float32))))
     assert orc.log_softmax_f32_row(np.array([3.0], np.float32)).tolist() == [0.0]
+
+
+# ---- the scalar floor's own form (src/simd/math/activations.cc:320-336) ----------------------
+import os
+
+import pytest
+
+from oracle import ref
+
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "scalar_floor_vectors.npz"))
+needs_ref = pytest.mark.skipif(not ref.available(), reason="oracle/_ref not built (no reference tree)")
+TAIL_WIDTHS = (129, 8193)
+
+
+def same_bits_or_nan(got, want):
+    got, want = np.asarray(got, np.float32), np.asarray(want, np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got.view(np.uint32)[~nan], want.view(np.uint32)[~nan])
+
+
+def tail_rows(width):
+    x = np.full((3, width), -20.0, np.float32)
+    x[0, width - 1] = 0
+    x[1, 0] = x[1, width - 1] = 0
+    x[2, :] = 0
+    return x
+
+
+def test_floor_form_golden_bit_exact():
+    for n in (1, 7, 8, 9, 257, 4096):
+        same_bits_or_nan(orc.log_softmax_floor_f32_row(GOLD[f"log_softmax_x_{n}"]), GOLD[f"log_softmax_y_{n}"])
+    same_bits_or_nan(orc.log_softmax_floor_f32_row(GOLD["log_softmax_x_masked"]),
+                     GOLD["log_softmax_y_masked_words"].view(np.float32))
+    same_bits_or_nan(orc.log_softmax_floor_f32_row(GOLD["log_softmax_x_wide"]),
+                     GOLD["log_softmax_y_wide_words"].view(np.float32))
+    for width in TAIL_WIDTHS:
+        for row, want in zip(tail_rows(width), GOLD[f"log_softmax_y_tails_{width}"]):
+            same_bits_or_nan(orc.log_softmax_floor_f32_row(row), want)
+
+
+@needs_ref
+def test_floor_form_live_bit_exact_and_invalid_rows():
+    rng = np.random.default_rng(83)
+    for n in (1, 2, 3, 31, 64, 1000, 5000):
+        for spread in (0.5, 3.0, 30.0):
+            row = rng.normal(0, spread, n).astype(np.float32)
+            same_bits_or_nan(orc.log_softmax_floor_f32_row(row), ref.log_softmax_f32(row))
+            row[rng.random(n) < 0.3] = -np.inf
+            same_bits_or_nan(orc.log_softmax_floor_f32_row(row), ref.log_softmax_f32(row))
+    for bad in ([1.0, np.nan, 2.0], [1.0, np.inf], [-np.inf, -np.inf], [np.nan]):
+        row = np.array(bad, np.float32)
+        got = orc.log_softmax_floor_f32_row(row)
+        assert np.all(np.isnan(got)) and np.all(np.isnan(ref.log_softmax_f32(row)))
+
+
+def test_log1p_form_is_held_to_the_floor_form_at_the_reference_bound():
+    """The kernel's form (maximum left out of an f32 sum, log1p) against the floor's form (double
+    sum, log): 4e-6 relative + 2e-7, the bound of the reference's own LogSoftmax checks
+    (tests/compute_provider_cuda/tensor_test.cc:75-84, 1168-1199); the same rows are invalid."""
+    rng = np.random.default_rng(84)
+    rows = [GOLD[f"log_softmax_x_{n}"] for n in (1, 7, 8, 9, 257, 4096)]
+    rows += [GOLD["log_softmax_x_masked"], GOLD["log_softmax_x_wide"]]
+    rows += [r for width in TAIL_WIDTHS for r in tail_rows(width)]
+    rows += [rng.normal(0, s, n).astype(np.float32) for n in (5, 300, 4096, 20000) for s in (0.1, 4.0)]
+    for row in rows:
+        floor = orc.log_softmax_floor_f32_row(row).astype(np.float64)
+        form = orc.log_softmax_f32_row(row).astype(np.float64)
+        finite = np.isfinite(floor)
+        assert np.array_equal(np.isneginf(floor), np.isneginf(form))
+        assert np.all(np.abs(form[finite] - floor[finite]) <= np.abs(floor[finite]) * 4e-6 + 2e-7)
+    # Rows of large magnitude: the floor rounds max + log(sum) to f32 at the magnitude of the
+    # maximum (half a unit of 139 is 8e-6), which the log1p form does not; there the two agree
+    # to the same relative bound taken on the largest operand of that subtraction.
+    for n in (5, 300, 4096, 20000):
+        row = rng.normal(0, 40.0, n).astype(np.float32)
+        floor = orc.log_softmax_floor_f32_row(row).astype(np.float64)
+        form = orc.log_softmax_f32_row(row).astype(np.float64)
+        scale = np.maximum(np.abs(floor), float(np.abs(row).max()))
+        assert np.all(np.abs(form - floor) <= scale * 4e-6 + 2e-7)
+    for bad in ([1.0, np.nan, 2.0], [1.0, np.inf], [-np.inf, -np.inf], [np.nan]):
+        row = np.array(bad, np.float32)
+        assert np.all(np.isnan(orc.log_softmax_floor_f32_row(row))) and np.all(np.isnan(orc.log_softmax_f32_row(row)))
