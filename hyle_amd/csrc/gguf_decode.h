@@ -2,7 +2,9 @@
 // (or any byte-addressable memory).  Geometry from the reference
 // (src/compute_ops/low_precision.cc:22-29: Q8_0 32 elements in 34 bytes, Q4_K 256 in 144, Q6_K 256
 // in 210); the arithmetic is ggml's dequantize_row_q8_0 / _q4_K / _q6_K, restated from the
-// published block layouts (the source is not part of the reference tree):
+// published block layouts, checked against the two readings of these formats the reference
+// tree holds (third_party/ggml_q4k_apple/ggml_q4k_apple.h:9-38;
+// tests/compute_models/qwen27_original_nextn_reference.h:74-86,262-287):
 //   Q8_0  {f16 d; i8 qs[32]}                              y = d * q           (exact in f32)
 //   Q4_K  {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]}    y = (d * sc) * q - (dmin * m)
 //   Q6_K  {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d}   y = (d * scale) * (q - 32)

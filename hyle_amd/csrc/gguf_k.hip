@@ -3,7 +3,9 @@
 //
 // Geometry from the reference (src/compute_ops/low_precision.cc:22-27: 256 elements in 144 and
 // 210 bytes); the decode is ggml's dequantize_row_q4_K / dequantize_row_q6_K, restated from the
-// published block layouts (the source is not part of the reference tree):
+// published block layouts, checked against the two readings of these formats the reference
+// tree holds (third_party/ggml_q4k_apple/ggml_q4k_apple.h:9-38;
+// tests/compute_models/qwen27_original_nextn_reference.h:74-86,262-287):
 //   Q4_K  {f16 d; f16 dmin; u8 scales[12]; u8 qs[128]}   y = (d * sc) * q - (dmin * m)
 //   Q6_K  {u8 ql[128]; u8 qh[64]; i8 scales[16]; f16 d}  y = (d * scale) * (q - 32)
 // with separate f32 roundings for the products and the subtraction, as the source writes them.

@@ -31,9 +31,12 @@
  *   - log_softmax: the floor's form (log_softmax_floor) is pinned bit-exact
  *     against oracle/_ref and golden vectors; the log1p form the GPU kernel
  *     follows is held to it at the reference's own bound.
- *   - k_quant_dequant (GGUF Q4_K, Q6_K): "parity unpinned" against ggml's
- *     source, which is not in the reference tree; the restatement of the
- *     published block layouts is checked against blocks packed field by field.
+ *   - k_quant_dequant (GGUF Q4_K, Q6_K) and q8_0 decode: ggml's source is not
+ *     in the reference tree, but two independent readings of the formats are
+ *     (third_party/ggml_q4k_apple/ggml_q4k_apple.h:9-38; the element values of
+ *     tests/compute_models/qwen27_original_nextn_reference.h:74-86,262-287):
+ *     pinned bit for bit against both over random raw bytes, and against
+ *     blocks packed field by field.
  */
 #ifndef HYLE_ORACLE_H_
 #define HYLE_ORACLE_H_

@@ -1,6 +1,6 @@
 """The oracle's Q4_K / Q6_K decode against blocks built field by field in the packing direction
-(tests/k_quant_support.py).  ggml itself is not in the reference tree: these tests pin the index
-conventions and the arithmetic order of the restatement, not ggml's source."""
+(tests/k_quant_support.py), and against the two independent readings of these formats that the
+reference tree holds (ggml's own source is not in it)."""
 from __future__ import annotations
 
 import numpy as np
@@ -56,3 +56,76 @@ def test_random_blocks_rows_and_strides():
         padded[:, :raw.shape[1]] = raw
         again, _, _ = orc.k_quant_dequant(kind, padded, 5, 768, row_stride=padded.shape[1])
         assert np.array_equal(again, want)
+
+
+# ---- the reference's own independent decoders, restated array-wise over raw random bytes --------
+# The reference tree holds two readings of these formats that do not go through ggml's code:
+#   third_party/ggml_q4k_apple/ggml_q4k_apple.h:9-38  Q4_K as array operations (the ggml
+#       dequantize_row_q4_K / get_scale_min_k4 sequence);
+#   tests/compute_models/qwen27_original_nextn_reference.h:74-86 (q4_scale, q6_code), 119-127
+#       (Q4_K group), 262-287 (expect_embedding: the bit-exact value each decoded element must have).
+def random_raw_rows(rng, rows, blocks, size, scale_bytes):
+    raw = rng.integers(0, 256, (rows, blocks, size), dtype=np.uint8)
+    for at in scale_bytes:                    # keep the f16 fields finite (exponent below 31)
+        raw[:, :, at] &= 0x3B
+    return raw
+
+
+def f16_field(raw, at):
+    return (raw[..., at].astype(np.uint16) | (raw[..., at + 1].astype(np.uint16) << 8)).view(np.float16).astype(np.float32)
+
+
+def rn_multiply(a, b):                        # one binary32 rounding of the exact product
+    return (np.asarray(a, np.float64) * np.asarray(b, np.float64)).astype(np.float32)
+
+
+def test_q4_k_against_the_array_form_in_the_reference_tree():
+    rng = np.random.default_rng(1401)
+    raw = random_raw_rows(rng, 6, 3, 144, (1, 3))
+    field = raw.astype(np.uint32)
+    scale_lo, min_lo, high = field[..., 4:8], field[..., 8:12], field[..., 12:16]
+    scales = np.concatenate([scale_lo & 63, (high & 15) | ((scale_lo >> 6) << 4)], axis=-1)
+    mins = np.concatenate([min_lo & 63, (high >> 4) | ((min_lo >> 6) << 4)], axis=-1)
+    q = field[..., 16:144].reshape(6, 3, 4, 32)
+    codes = np.stack([q & 15, q >> 4], axis=-2).reshape(6, 3, 8, 32)
+    d = f16_field(raw, 0)[..., None] * scales.astype(np.float32)
+    minimum = f16_field(raw, 2)[..., None] * mins.astype(np.float32)
+    want = (d[..., None] * codes.astype(np.float32)).astype(np.float32) - minimum[..., None]
+    wide, _, _ = orc.k_quant_dequant(orc.Q4_K, raw.reshape(6, -1), 6, 768)
+    assert np.array_equal(wide.view(np.uint32), want.reshape(6, 768).astype(np.float32).view(np.uint32))
+
+
+def test_q4_k_q6_k_q8_0_against_the_reference_tests_embedding_expectations():
+    rng = np.random.default_rng(1402)
+    column = np.arange(256)
+    # Q6_K: code from its low nibble and two high bits; value = RN(RN(d * scale16) * code)
+    raw = random_raw_rows(rng, 5, 2, 210, (209,))
+    half, within = column // 128, column % 128
+    lane, quarter = within % 32, within // 32
+    low = raw[..., half * 64 + lane + (quarter % 2) * 32].astype(np.int32)
+    top = raw[..., 128 + half * 32 + lane].astype(np.int32)
+    code = (((low >> np.where(quarter >= 2, 4, 0)) & 15) | (((top >> (quarter * 2)) & 3) << 4)) - 32
+    scale16 = raw[..., 192 + column // 16].view(np.int8).astype(np.float32)
+    want = rn_multiply(rn_multiply(f16_field(raw, 208)[..., None], scale16), code.astype(np.float32))
+    wide, _, _ = orc.k_quant_dequant(orc.Q6_K, raw.reshape(5, -1), 5, 512)
+    assert np.array_equal(wide.view(np.uint32), want.reshape(5, 512).view(np.uint32))
+    # Q4_K: float(d * (q * scale) + dmin * (-minimum)), the sum taken in double
+    raw = random_raw_rows(rng, 5, 2, 144, (1, 3))
+    group = column // 32
+    b = raw.astype(np.int32)
+    first = group < 4
+    g_hi = np.where(first, 4, group)          # keeps the indices below in range for groups 0..3
+    scale = np.where(first, b[..., 4 + np.minimum(group, 3)] & 63,
+                     (b[..., 8 + g_hi] & 15) | ((b[..., g_hi] >> 6) << 4))
+    minimum = np.where(first, b[..., 8 + np.minimum(group, 3)] & 63,
+                       (b[..., 8 + g_hi] >> 4) | ((b[..., 4 + g_hi] >> 6) << 4))
+    q = (b[..., 16 + (group // 2) * 32 + column % 32] >> np.where(group % 2 == 1, 4, 0)) & 15
+    d, dmin = f16_field(raw, 0).astype(np.float64)[..., None], f16_field(raw, 2).astype(np.float64)[..., None]
+    want = (d * (q * scale) + dmin * (-minimum)).astype(np.float32)
+    wide, _, _ = orc.k_quant_dequant(orc.Q4_K, raw.reshape(5, -1), 5, 512)
+    assert np.array_equal(wide.view(np.uint32), want.reshape(5, 512).view(np.uint32))
+    # Q8_0: RN(d * code), exact
+    raw = random_raw_rows(rng, 4, 8, 34, (1,))
+    want = rn_multiply(f16_field(raw, 0)[..., None], raw[..., 2:].view(np.int8).astype(np.float32))
+    got = orc.q8_0_dequant_f32(raw.reshape(4, -1), 4, 256)
+    assert np.array_equal(got.view(np.uint32), want.reshape(4, 256).view(np.uint32))
