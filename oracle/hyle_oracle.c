@@ -1006,6 +1006,184 @@ void hyle_oracle_gguf_matvec(int kind, const void *blocks, size_t rows, size_t k
   free(w);
 }
 
+/* ------------------------------------------------------------------------ */
+/* MatMul over a GGUF weight the way the reference's ggml CPU route computes  */
+/* it: the activation row is quantised to 8-bit blocks first, block dot      */
+/* products are integers, scales are applied in f32.  ggml's source is not    */
+/* in the reference tree; the reference's tests restate its activation        */
+/* codecs and the product they accept, and that restatement is followed here: */
+/*   tests/compute_models/dspark_original_shared_reference.h:147-185 (Q8_0    */
+/*     activation block, the AVX form), 219-262 (Q8_0 x Q8_0 centre + bound); */
+/*   tests/compute_models/qwen27_original_nextn_reference.h:74-86 (scales,    */
+/*     six-bit codes), 94-130 (weight groups), 144-167 (Q8_K activation       */
+/*     block), 193-257 (centre + bound).                                      */
+/* ------------------------------------------------------------------------ */
+static float rn_divide(float a, float b) { return (float)((double)a / (double)b); }
+static float rn_multiply(float a, float b) { return (float)((double)a * (double)b); }
+
+/* Q8_0 activation blocks of 32: scale = f16(RN(max / 127)) widened again,
+ * code = nearest-even integer of RN(x * RN(127 / max)). */
+void hyle_oracle_quantize_q8_0(const float *x, size_t k, int8_t *codes, float *scales) {
+  for (size_t b = 0; b < k / 32; ++b) {
+    const float *v = x + 32 * b;
+    float maximum = 0.0f;
+    for (int i = 0; i < 32; ++i) maximum = fabsf(v[i]) > maximum ? fabsf(v[i]) : maximum;
+    if (maximum == 0.0f) {
+      scales[b] = 0.0f;
+      memset(codes + 32 * b, 0, 32);
+      continue;
+    }
+    const float divisor = rn_divide(maximum, 127.0f);
+    scales[b] = hyle_oracle_f16_to_f32(hyle_oracle_f32_to_f16(divisor));
+    const float reciprocal = rn_divide(127.0f, maximum);
+    for (int i = 0; i < 32; ++i)
+      codes[32 * b + i] = (int8_t)nearbyint((double)rn_multiply(v[i], reciprocal));
+  }
+}
+
+/* Q8_K activation blocks of 256: the first element of largest magnitude, sign
+ * kept, gives inverse = RN(-127 / max); code = min(127, nearest-even integer
+ * of RN(x * inverse)); the stored f32 scale is RN(1 / inverse). */
+void hyle_oracle_quantize_q8_k(const float *x, size_t k, int8_t *codes, float *scales) {
+  for (size_t b = 0; b < k / 256; ++b) {
+    const float *v = x + 256 * b;
+    float maximum = 0.0f, absolute = 0.0f;
+    for (int i = 0; i < 256; ++i)
+      if (fabsf(v[i]) > absolute) {
+        absolute = fabsf(v[i]);
+        maximum = v[i];
+      }
+    if (absolute == 0.0f) {
+      scales[b] = 0.0f;
+      memset(codes + 256 * b, 0, 256);
+      continue;
+    }
+    const float inverse = rn_divide(-127.0f, maximum);
+    scales[b] = rn_divide(1.0f, inverse);
+    for (int i = 0; i < 256; ++i) {
+      const int code = (int)nearbyint((double)rn_multiply(v[i], inverse));
+      codes[256 * b + i] = (int8_t)(code > 127 ? 127 : code);
+    }
+  }
+}
+
+typedef struct {
+  double plain, correction;
+} compensated_sum;
+static void compensated_add(compensated_sum *s, double term) {
+  const double next = s->plain + term;
+  s->correction += fabs(s->plain) >= fabs(term) ? (s->plain - next) + term : (term - next) + s->plain;
+  s->plain = next;
+}
+static double next_up(double v) { return nextafter(v, INFINITY); }
+static double gamma_bound(size_t count, double unit) {
+  const double product = (double)count * unit;
+  return next_up(product / (1.0 - product));
+}
+
+/* One 32-wide group of a weight row: value_i = scale * codes[i] + minimum * offsets[i]. */
+typedef struct {
+  double scale, minimum;
+  int codes[32], offsets[32];
+} weight_group;
+
+static weight_group gguf_weight_group(int kind, const unsigned char *row, size_t group) {
+  weight_group g;
+  memset(&g, 0, sizeof g);
+  if (kind == 2) {
+    const unsigned char *blk = row + group * 34;
+    g.scale = hyle_oracle_f16_to_f32((uint16_t)(blk[0] | ((uint16_t)blk[1] << 8)));
+    for (int i = 0; i < 32; ++i) g.codes[i] = (int8_t)blk[2 + i];
+    return g;
+  }
+  const size_t local = group % 8;
+  if (kind == 1) {
+    const unsigned char *blk = row + (group / 8) * 210;
+    g.scale = hyle_oracle_f16_to_f32((uint16_t)(blk[208] | ((uint16_t)blk[209] << 8)));
+    for (int i = 0; i < 32; ++i) {
+      const size_t column = local * 32 + (size_t)i;
+      const size_t half = column / 128, within = column % 128, lane = within % 32, quarter = within / 32;
+      const unsigned low = blk[half * 64 + lane + (quarter % 2) * 32], high = blk[128 + half * 32 + lane];
+      const int code = (int)(((low >> (quarter >= 2 ? 4 : 0)) & 15u) | (((high >> (quarter * 2)) & 3u) << 4)) - 32;
+      g.codes[i] = code * (int)(int8_t)blk[192 + column / 16];
+    }
+    return g;
+  }
+  const unsigned char *blk = row + (group / 8) * 144;
+  g.scale = hyle_oracle_f16_to_f32((uint16_t)(blk[0] | ((uint16_t)blk[1] << 8)));
+  g.minimum = hyle_oracle_f16_to_f32((uint16_t)(blk[2] | ((uint16_t)blk[3] << 8)));
+  int scale, minimum;
+  if (local < 4) {
+    scale = blk[4 + local] & 63;
+    minimum = blk[8 + local] & 63;
+  } else {
+    scale = (blk[8 + local] & 15) | ((blk[local] >> 6) << 4);
+    minimum = (blk[8 + local] >> 4) | ((blk[4 + local] >> 6) << 4);
+  }
+  for (int i = 0; i < 32; ++i) {
+    g.codes[i] = (int)((blk[16 + (local / 2) * 32 + i] >> (local % 2 ? 4 : 0)) & 15) * scale;
+    g.offsets[i] = -minimum;
+  }
+  return g;
+}
+
+/* centre[i * rows + r]: the exact value of sum over groups of
+ * w.scale * a.scale * (w.codes . a.codes) + w.minimum * a.scale * (w.offsets . a.codes)
+ * (every term exact in double, compensated sum); bound[...]: the distance from
+ * it the reference's test accepts of the native result,
+ * gamma(k / 4 + 65, 2^-24) * sum |terms| plus the centre's own f64 error. */
+void hyle_oracle_gguf_matvec_q8(int kind, const void *blocks, size_t rows, size_t k,
+                                size_t row_stride_bytes, const float *x, size_t m,
+                                double *centre, double *bound) {
+  const size_t groups = k / 32;
+  int8_t *codes = (int8_t *)malloc(k ? k : 1);
+  float *scales = (float *)malloc((groups ? groups : 1) * sizeof(float));
+  if (codes == NULL || scales == NULL) {
+    free(codes);
+    free(scales);
+    return;
+  }
+  const double g32 = gamma_bound(k / 4 + 65, 0x1p-24), g64 = gamma_bound(2 * groups + 2, 0x1p-53);
+  for (size_t i = 0; i < m; ++i) {
+    if (kind == 2) {
+      hyle_oracle_quantize_q8_0(x + i * k, k, codes, scales);
+    } else {  /* one f32 scale per 256: spread over the eight groups it covers */
+      hyle_oracle_quantize_q8_k(x + i * k, k, codes, scales);
+      for (size_t g = groups; g-- > 0;) scales[g] = scales[g / 8];
+    }
+    for (size_t r = 0; r < rows; ++r) {
+      const unsigned char *row = (const unsigned char *)blocks + r * row_stride_bytes;
+      compensated_sum sum = {0.0, 0.0};
+      double absolute = 0.0;
+      for (size_t g = 0; g < groups; ++g) {
+        const weight_group w = gguf_weight_group(kind, row, g);
+        const double a_scale = scales[g];
+        const int8_t *a = codes + 32 * g;
+        for (int part = 0; part < 2; ++part) {
+          const double scale = part == 0 ? w.scale : w.minimum;
+          const int *c = part == 0 ? w.codes : w.offsets;
+          if (scale == 0.0) continue;
+          long dot = 0, size = 0;
+          for (int j = 0; j < 32; ++j) {
+            dot += (long)c[j] * a[j];
+            size += labs((long)c[j]) * labs((long)a[j]);
+          }
+          compensated_add(&sum, scale * a_scale * (double)dot);
+          absolute = next_up(absolute + next_up(fabs(scale) * next_up(fabs(a_scale) * (double)size)));
+        }
+      }
+      const double value = sum.plain + sum.correction;
+      centre[i * rows + r] = value;
+      if (bound) {
+        const double own = next_up(next_up(fabs(value - sum.plain)) + next_up(g64 * absolute));
+        bound[i * rows + r] = next_up(next_up(g32 * absolute) + own);
+      }
+    }
+  }
+  free(codes);
+  free(scales);
+}
+
 void hyle_oracle_q8_0_dequant_f32(const void *blocks, size_t rows, size_t k,
                                   size_t row_stride_bytes, float *out) {
   const unsigned char *base = (const unsigned char *)blocks;

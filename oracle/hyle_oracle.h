@@ -266,6 +266,20 @@ void hyle_oracle_topk1_f32(const float *data, size_t rows, size_t width,
 void hyle_oracle_q8_0_dequant_bf16(const void *blocks, size_t rows, size_t k,
                                    size_t row_stride_bytes, uint16_t *out,
                                    float *sumsq, float *sumsq_rounded);
+/* MatMul over a GGUF weight as the reference's ggml CPU route computes it: 8-bit
+ * activation blocks (Q8_0 blocks of 32 for a Q8_0 weight, Q8_K blocks of 256 for
+ * Q4_K / Q6_K), integer block dot products, f32 scales.  Restated from the
+ * reference's own tests, which hold the activation codecs and the value and
+ * bound they accept of the native result
+ * (tests/compute_models/dspark_original_shared_reference.h:147-185,219-262;
+ * tests/compute_models/qwen27_original_nextn_reference.h:74-130,144-167,193-257).
+ * kind: 0 = Q4_K, 1 = Q6_K, 2 = Q8_0.  x is [m, k] f32; centre and bound are
+ * [m, rows].  scales: k / 32 (Q8_0) or k / 256 (Q8_K) floats. */
+void hyle_oracle_quantize_q8_0(const float *x, size_t k, int8_t *codes, float *scales);
+void hyle_oracle_quantize_q8_k(const float *x, size_t k, int8_t *codes, float *scales);
+void hyle_oracle_gguf_matvec_q8(int kind, const void *blocks, size_t rows, size_t k,
+                                size_t row_stride_bytes, const float *x, size_t m,
+                                double *centre, double *bound);
 /* ggml dequantize_row_q8_0 to f32 */
 /* GGUF Q4_K (kind 0: 256 elements in 144 bytes) and Q6_K (kind 1: 256 in 210)
  * rows -> f32 and / or bf16 [rows, k] plus the f32 row sums of squares of the

@@ -455,6 +455,41 @@ def gguf_matvec(kind: int, blocks: np.ndarray, rows: int, k: int, x: np.ndarray,
     return out, magnitude
 
 
+def quantize_q8_0(x: np.ndarray):
+    """ggml's Q8_0 activation blocks (AVX form): (int8 codes [k], f32 scales [k / 32], each an f16 value)."""
+    x = _c(x, np.float32).reshape(-1)
+    codes, scales = np.empty(x.size, np.int8), np.empty(x.size // 32, np.float32)
+    fn = _lib.hyle_oracle_quantize_q8_0
+    fn.restype, fn.argtypes = None, [_vp, _sz, _vp, _vp]
+    fn(_ptr(x), x.size, _ptr(codes), _ptr(scales))
+    return codes, scales
+
+
+def quantize_q8_k(x: np.ndarray):
+    """ggml's Q8_K activation blocks: (int8 codes [k], f32 scales [k / 256])."""
+    x = _c(x, np.float32).reshape(-1)
+    codes, scales = np.empty(x.size, np.int8), np.empty(x.size // 256, np.float32)
+    fn = _lib.hyle_oracle_quantize_q8_k
+    fn.restype, fn.argtypes = None, [_vp, _sz, _vp, _vp]
+    fn(_ptr(x), x.size, _ptr(codes), _ptr(scales))
+    return codes, scales
+
+
+def gguf_matvec_q8(kind: int, blocks: np.ndarray, rows: int, k: int, x: np.ndarray, row_stride: int | None = None):
+    """MatMul with 8-bit activation blocks, as the reference's ggml CPU route computes it:
+    (float64 centre [m, rows], float64 bound [m, rows] the reference's tests accept around it)."""
+    blocks = _c(blocks, np.uint8)
+    x = _c(np.atleast_2d(x), np.float32)
+    per_block, block_bytes = GGUF_BLOCK[kind]
+    row_stride = (k // per_block) * block_bytes if row_stride is None else row_stride
+    centre = np.empty((x.shape[0], rows), np.float64)
+    bound = np.empty_like(centre)
+    fn = _lib.hyle_oracle_gguf_matvec_q8
+    fn.restype, fn.argtypes = None, [C.c_int, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _vp]
+    fn(kind, _ptr(blocks), rows, k, row_stride, _ptr(x), x.shape[0], _ptr(centre), _ptr(bound))
+    return centre, bound
+
+
 def q8_0_dequant_f32(blocks: np.ndarray, rows: int, k: int, row_stride: int | None = None):
     blocks = _c(blocks, np.uint8)
     row_stride = (k // 32) * 34 if row_stride is None else row_stride
