@@ -220,14 +220,23 @@ def main() -> int:
         ops.append(Op(name, hc.GgufDequantSumSquares(), [hc.TensorDesc.gguf_weight(gguf, BF, 2048, 6144)], set_k, 16,
                       6144 * (8 * block_bytes + 2048 * 2 + 4), 6144 * 2048, "u8/bf16", in_step=False))
     # ---- decode-time MatMul over GGUF weights: one activation row against [K, N] ----------------
-    for name, gguf, block_bytes, k, n_rows, sets, m in (
-            ("next_matvec_q4_k_bf16_ffn", hc.GgufQuantizedType.kQ4K, 144, 2048, 6144, 80, 1),
-            ("next_matvec_q4_k_bf16_ffn_down", hc.GgufQuantizedType.kQ4K, 144, 6144, 2048, 80, 1),
-            ("next_matvec_q4_k_bf16_k4096", hc.GgufQuantizedType.kQ4K, 144, 4096, 14336, 16, 1),
-            ("next_matvec_q4_k_bf16_vocab", hc.GgufQuantizedType.kQ4K, 144, 2048, 151936, 4, 1),
-            ("next_matvec_q6_k_bf16_vocab", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 1),
-            ("next_matvec_q6_k_bf16_vocab_4_tokens", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 4),
-            ("next_matvec_q8_0_bf16_vocab", hc.GgufQuantizedType.kQ8_0, 34, 2048, 151936, 3, 1)):
+    EXACT, GGML_Q8 = hc.ActivationArithmetic.kExact, hc.ActivationArithmetic.kGgmlQ8
+    for name, gguf, block_bytes, k, n_rows, sets, m, arithmetic in (
+            ("next_matvec_q4_k_bf16_ffn", hc.GgufQuantizedType.kQ4K, 144, 2048, 6144, 80, 1, EXACT),
+            ("next_matvec_q4_k_bf16_ffn_down", hc.GgufQuantizedType.kQ4K, 144, 6144, 2048, 80, 1, EXACT),
+            ("next_matvec_q4_k_bf16_k4096", hc.GgufQuantizedType.kQ4K, 144, 4096, 14336, 16, 1, EXACT),
+            ("next_matvec_q4_k_bf16_vocab", hc.GgufQuantizedType.kQ4K, 144, 2048, 151936, 4, 1, EXACT),
+            ("next_matvec_q6_k_bf16_vocab", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 1, EXACT),
+            ("next_matvec_q6_k_bf16_vocab_4_tokens", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 4, EXACT),
+            ("next_matvec_q8_0_bf16_vocab", hc.GgufQuantizedType.kQ8_0, 34, 2048, 151936, 3, 1, EXACT),
+            # the same products as the reference's ggml route computes them: 8-bit activation blocks, integer dots
+            ("next_matvec_ggml_q8_q4_k_ffn", hc.GgufQuantizedType.kQ4K, 144, 2048, 6144, 80, 1, GGML_Q8),
+            ("next_matvec_ggml_q8_q4_k_ffn_down", hc.GgufQuantizedType.kQ4K, 144, 6144, 2048, 80, 1, GGML_Q8),
+            ("next_matvec_ggml_q8_q4_k_vocab", hc.GgufQuantizedType.kQ4K, 144, 2048, 151936, 4, 1, GGML_Q8),
+            ("next_matvec_ggml_q8_q6_k_vocab", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 1, GGML_Q8),
+            ("next_matvec_ggml_q8_q6_k_vocab_4_tokens", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 4, GGML_Q8),
+            ("next_matvec_ggml_q8_q6_k_vocab_8_tokens", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 8, GGML_Q8),
+            ("next_matvec_ggml_q8_q8_0_vocab", hc.GgufQuantizedType.kQ8_0, 34, 2048, 151936, 3, 1, GGML_Q8)):
         if not want(name):
             continue
         per_row = k // (32 if block_bytes == 34 else 256)   # blocks in a row of k values
@@ -239,7 +248,7 @@ def main() -> int:
                 fields[:, :, at] &= 0x3B
             x = torch.empty([k] if m == 1 else [m, k], dtype=torch.bfloat16, device=dev).normal_()
             return [raw.to(dev), x], [torch.empty([n_rows] if m == 1 else [m, n_rows], dtype=torch.bfloat16, device=dev)]
-        ops.append(Op(name, hc.GgufMatVec(), [hc.TensorDesc.gguf_weight(gguf, BF, k, n_rows), D(BF, [k] if m == 1 else [m, k])],
+        ops.append(Op(name, hc.GgufMatVec(arithmetic), [hc.TensorDesc.gguf_weight(gguf, BF, k, n_rows), D(BF, [k] if m == 1 else [m, k])],
                       set_mv, sets, n_rows * (per_row * block_bytes + 2 * m) + m * k * 2, m * n_rows * k, "u8/bf16", in_step=False))
     # ---- the next row of the path: Cast and Copy, timed beside the step -------------------------
     if want("next_cast_f32_to_bf16") or want("next_cast_bf16_to_f32"):

@@ -369,10 +369,19 @@ class GgufDequantSumSquares(Q8_0DequantSumSquares):
     block geometry of the input descriptor."""
 
 
+class ActivationArithmetic(enum.IntEnum):
+    """How GgufMatVec treats the activations: kExact multiplies exactly decoded weights by them in
+    f32; kGgmlQ8 first quantises them to ggml's 8-bit blocks and takes integer block dot products,
+    which is what the reference's ggml CPU route computes."""
+    kExact = 0
+    kGgmlQ8 = 1
+
+
 @dataclass(frozen=True)
 class GgufMatVec:
     """MatMul(activations, GGUF weight) for a few activation rows: inputs (weight [K, N], x [K] or
     [M, K]); output [N] or [M, N] of x's type."""
+    activations: ActivationArithmetic = ActivationArithmetic.kExact
 
 
 def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
@@ -409,7 +418,7 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
     elif isinstance(operation, Q8_0DequantSumSquares):
         c.op = OperationKind.kQ8_0DequantSumSquares
     elif isinstance(operation, GgufMatVec):
-        c.op = OperationKind.kGgufMatVec
+        c.op, c.kind2 = OperationKind.kGgufMatVec, int(operation.activations)
     else:
         raise StatusError(capi.UNIMPLEMENTED, f"operation {type(operation).__name__} is not served by this provider")
     if len(inputs) > capi.MAX_INPUTS:

@@ -1,0 +1,435 @@
+// y[m][n] = MatMul(x, W) for a GGUF weight (Q8_0, Q4_K, Q6_K; logical [K, N]) and a few activation
+// rows, computed the way the reference's ggml CPU route computes it: each activation row is first
+// quantised to 8-bit blocks (Q8_0 blocks of 32 for a Q8_0 weight, Q8_K blocks of 256 for Q4_K and
+// Q6_K), block dot products are integers, and the scales are applied in f32.
+//
+// ggml's source is not in the reference tree.  The arithmetic follows the restatement the
+// reference's own tests hold of it:
+//   Q8_0 activation block   scale = f16(RN(max / 127)), code = RNE(RN(x * RN(127 / max)))
+//       (tests/compute_models/dspark_original_shared_reference.h:147-185, the AVX form)
+//   Q8_K activation block   the first element of largest magnitude, sign kept, gives
+//       inverse = RN(-127 / max); code = min(127, RNE(RN(x * inverse))); scale = RN(1 / inverse)
+//       (tests/compute_models/qwen27_original_nextn_reference.h:144-167)
+//   product                 sum over 32-wide groups of w.scale * a.scale * (w.codes . a.codes)
+//       [+ w.minimum * a.scale * (w.offsets . a.codes) for Q4_K], integer dots
+//       (tests/compute_models/qwen27_original_nextn_reference.h:94-130, 216-244)
+// The integer parts are exact here; the f32 products and sums differ from ggml's only in their
+// order, which the reference's tests allow for with gamma(K / 4 + 65, 2^-24) * sum |terms|.
+//
+// Rows are read exactly as in gguf_matvec.hip (whole 16-byte vectors through wave-private LDS,
+// four spans of 2048 values in flight per wave, gguf_lines.h).  The activation codes of a lane's
+// 32 positions are eight 32-bit words per activation row, so a weight word of four quants meets
+// them in one v_dot4c_i32_i8, and decoding a span once serves every activation row:
+//   Q6_K  four quants are assembled per word as int8 bytes 4 (q - 32); a 16-value group's dot is
+//         multiplied by its int8 scale as an integer; one conversion and (d / 4) * a.scale close
+//         the half block
+//   Q4_K  nibbles are already bytes 0..15; sc * dot and m * (sum of activation codes) stay
+//         integers; d * a.scale and dmin * a.scale close the sub-blocks
+//   Q8_0  the bytes are the int8 quants; d * a.scale closes the block
+#include "device_common.h"
+#include "gguf_decode.h"
+#include "gguf_lines.h"
+#include "kernels.h"
+
+namespace hyle_hip {
+namespace {
+
+// a * b + c for factors that fit 24 signed bits (v_mad_i32_i24; a full 32-bit multiply is four
+// times slower)
+__device__ __forceinline__ int mad24(int a, int b, int c) { return __mul24(a, b) + c; }
+
+__device__ __forceinline__ int dot4(uint32_t weights, uint32_t codes, int sum) {
+  return __builtin_amdgcn_sdot4((int)weights, (int)codes, sum, false);
+}
+
+// The element of largest magnitude of a block spread over kLanes adjacent lanes; among equal
+// magnitudes the one at the lowest position of the row wins (ggml walks the block in order and
+// replaces its candidate only on a strictly larger magnitude).
+struct LaneMax {
+  float magnitude, value;
+  uint32_t position;
+  template <int kCtrl> __device__ __forceinline__ LaneMax moved() const {
+    return {dpp_move<kCtrl>(magnitude), dpp_move<kCtrl>(value), (uint32_t)dpp_move<kCtrl>((int)position)};
+  }
+  __device__ __forceinline__ LaneMax shuffled_xor(int mask) const {
+    return {__shfl_xor(magnitude, mask, kWaveLanes), __shfl_xor(value, mask, kWaveLanes),
+            (uint32_t)__shfl_xor((int)position, mask, kWaveLanes)};
+  }
+};
+__device__ __forceinline__ LaneMax first_largest(LaneMax a, LaneMax b) {
+  if (a.magnitude != b.magnitude) return a.magnitude > b.magnitude ? a : b;
+  return a.position <= b.position ? a : b;
+}
+template <int kLanes> __device__ __forceinline__ LaneMax block_largest(LaneMax mine) {
+  if constexpr (kLanes == 1) return mine;
+  else return group_reduce<kLanes>(mine, [](LaneMax a, LaneMax b) { return first_largest(a, b); });
+}
+
+__device__ __forceinline__ uint32_t code_of(float scaled) {
+  int code = (int)__builtin_rintf(scaled);  // nearest, ties to even
+  code = code > 127 ? 127 : code;
+  return (uint32_t)code & 0xFFu;
+}
+
+// What a lane holds of one activation row for one span of 2048 values: the codes of its 32
+// positions (word e / 4, byte e % 4), the scale of the activation block(s) they belong to and,
+// for Q4_K, the sums of the codes of its four runs of eight.
+struct LaneCodes {
+  uint32_t codes[8];
+  float scale[2];
+  int sums[4];
+};
+
+// Quantises the lane's share of span `span` of the activation row at `x` (k values of type TX).
+// Every lane of a wave calls it; lanes that share an activation block agree on its scale through
+// a cross-lane maximum.
+template <int kKind, class TX>
+__device__ __forceinline__ LaneCodes quantise_span(const void *x, size_t row_offset, uint32_t span, uint32_t lane) {
+  using Kind = Lines<kKind>;
+  float values[32];
+#pragma unroll
+  for (int e = 0; e < 32; ++e) values[e] = Traits<TX>::load(x, row_offset + Kind::position(span, lane, e));
+  LaneCodes out;
+  // Q8_0: the lane's 32 values are one block.  Q6_K: eight lanes share a block of 256.
+  // Q4_K: the lane's values 0..15 and 16..31 belong to two blocks of 256, sixteen lanes each.
+  constexpr int kParts = kKind == 0 ? 2 : 1;
+  constexpr int kPartValues = 32 / kParts;
+  constexpr int kLanesPerBlock = kKind == 0 ? 16 : (kKind == 1 ? 8 : 1);
+#pragma unroll
+  for (int part = 0; part < kParts; ++part) {
+    LaneMax mine{0.0f, 0.0f, 0u};
+#pragma unroll
+    for (int t = 0; t < kPartValues; ++t) {  // positions rise with e, so ">" keeps the first
+      const int e = part * kPartValues + t;
+      const float magnitude = __builtin_fabsf(values[e]);
+      if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], Kind::position(span, lane, e)};
+    }
+    if (mine.magnitude == 0.0f) mine.position = 0xFFFFFFFFu;  // no candidate: any lane with one goes first
+    const LaneMax top = block_largest<kLanesPerBlock>(mine);
+    float factor = 0.0f, stored = 0.0f;
+    if (top.magnitude != 0.0f) {
+      if constexpr (kKind == 2) {
+        stored = f16_to_f32(f32_to_f16(top.magnitude / 127.0f));
+        factor = 127.0f / top.magnitude;
+      } else {
+        factor = -127.0f / top.value;
+        stored = 1.0f / factor;
+      }
+    }
+    out.scale[part] = stored;
+#pragma unroll
+    for (int w = 0; w < kPartValues / 4; ++w) {
+      uint32_t word = 0;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) word |= code_of(values[part * kPartValues + 4 * w + t] * factor) << (8 * t);
+      out.codes[part * (kPartValues / 4) + w] = top.magnitude != 0.0f ? word : 0u;
+    }
+  }
+  if constexpr (kParts == 1) out.scale[1] = out.scale[0];
+#pragma unroll
+  for (int run = 0; run < 4; ++run)
+    out.sums[run] = dot4(0x01010101u, out.codes[2 * run], dot4(0x01010101u, out.codes[2 * run + 1], 0));
+  return out;
+}
+
+// The span's bytes decoded once into words of four int8 quants, then met with each activation row.
+template <int kKind> struct SpanDot;
+
+template <> struct SpanDot<1> {  // Q6_K
+  uint32_t q[4][2];
+  int scale[4];
+  float step;  // d / 4
+  __device__ __forceinline__ void decode(const unsigned char *slot, const Lines<1>::Lane &at) {
+    uint32_t lows[2], highs[2], tops[2], scales[2];
+    lds_piece(slot, at.low, lows);
+    lds_piece(slot, at.low + 32, highs);
+    lds_piece(slot, at.top, tops);
+    lds_piece(slot, at.scales, scales);
+    step = f16_to_f32(*reinterpret_cast<const uint16_t *>(slot + at.d)) * 0.25f;
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const uint32_t low = lows[w], high = highs[w], top = tops[w] ^ 0xAAAAAAAAu;
+      q[0][w] = ((low << 2) & 0x3C3C3C3Cu) | ((top << 6) & 0xC0C0C0C0u);
+      q[1][w] = ((high << 2) & 0x3C3C3C3Cu) | ((top << 4) & 0xC0C0C0C0u);
+      q[2][w] = ((low >> 2) & 0x3C3C3C3Cu) | ((top << 2) & 0xC0C0C0C0u);
+      q[3][w] = ((high >> 2) & 0x3C3C3C3Cu) | (top & 0xC0C0C0C0u);
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      scale[g] = (int)(signed char)(scales[g / 2] >> (16 * (g % 2) + 8 * (at.j / 2)));
+  }
+  __device__ __forceinline__ float against(const LaneCodes &a) const {
+    int total = 0;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) total = mad24(scale[g], dot4(q[g][0], a.codes[2 * g], dot4(q[g][1], a.codes[2 * g + 1], 0)), total);
+    return (step * a.scale[0]) * (float)total;
+  }
+};
+
+// Sums of kCount values over the wave, jointly: log2(kCount) exchange steps halve the values a
+// lane carries (lane l ends with value l % kCount summed over its group of kCount lanes), the
+// remaining steps add the groups.  Every lane with l % kCount == i returns the total of v[i].
+template <int kCount> __device__ __forceinline__ float joint_sum(float (&v)[kCount], uint32_t lane) {
+  static_assert(kCount == 1 || kCount == 2 || kCount == 4 || kCount == 8, "joint sums of 1, 2, 4 or 8 values");
+  int live = kCount;
+#pragma unroll
+  for (int step = 1; step < kCount; step *= 2) {
+    const bool upper = (lane & (uint32_t)step) != 0;
+    live /= 2;
+#pragma unroll
+    for (int i = 0; i < live; ++i) {
+      const float keep = upper ? v[2 * i + 1] : v[2 * i], give = upper ? v[2 * i] : v[2 * i + 1];
+      v[i] = keep + __shfl_xor(give, step, kWaveLanes);
+    }
+  }
+  float mine = v[0];
+#pragma unroll
+  for (int step = kCount; step < kWaveLanes; step *= 2) mine += __shfl_xor(mine, step, kWaveLanes);
+  return mine;
+}
+
+template <> struct SpanDot<0> {  // Q4_K
+  uint32_t low[2][2], high[2][2];
+  int sc_low[2], sc_high[2], m_low[2], m_high[2];
+  float d[2], dmin[2];
+  __device__ __forceinline__ void decode(const unsigned char *slot, const Lines<0>::Lane &at) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const u32x4 head = *reinterpret_cast<const u32x4 *>(slot + at.header[i]);
+      const uint32_t s0 = head.y, s1 = head.z, s2 = head.w;
+      d[i] = f16_to_f32((uint16_t)head.x);
+      dmin[i] = f16_to_f32((uint16_t)(head.x >> 16));
+      // lane u of the block's sixteen works out sc (u < 8) or m (u >= 8) of sub-block u % 8
+      const uint32_t own = at.minimum ? s1 : s0;
+      const int bits = (int)((((at.main_in_s2 ? s2 : own) >> at.main_shift) & at.main_mask) |
+                             (((own >> at.top_shift) & at.top_mask) << 4));
+      sc_low[i] = __shfl(bits, at.source);
+      sc_high[i] = __shfl(bits, at.source + 1);
+      m_low[i] = __shfl(bits, at.source + 8);
+      m_high[i] = __shfl(bits, at.source + 9);
+      const uint32_t *words = reinterpret_cast<const uint32_t *>(slot + at.quants[i]);
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        low[i][w] = words[w] & 0x0F0F0F0Fu;
+        high[i][w] = (words[w] >> 4) & 0x0F0F0F0Fu;
+      }
+    }
+  }
+  __device__ __forceinline__ float against(const LaneCodes &a) const {
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int lows = dot4(low[i][0], a.codes[4 * i], dot4(low[i][1], a.codes[4 * i + 1], 0));
+      const int highs = dot4(high[i][0], a.codes[4 * i + 2], dot4(high[i][1], a.codes[4 * i + 3], 0));
+      const int scaled = mad24(sc_low[i], lows, __mul24(sc_high[i], highs));
+      const int minima = mad24(m_low[i], a.sums[2 * i], __mul24(m_high[i], a.sums[2 * i + 1]));
+      total += a.scale[i] * (d[i] * (float)scaled - dmin[i] * (float)minima);
+    }
+    return total;
+  }
+};
+
+template <> struct SpanDot<2> {  // Q8_0
+  uint32_t q[8];
+  float d;
+  __device__ __forceinline__ void decode(const unsigned char *slot, const Lines<2>::Lane &at) {
+    const uint32_t *words = reinterpret_cast<const uint32_t *>(slot + at.words);
+    uint32_t w[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) w[i] = words[i];
+    d = f16_to_f32(*reinterpret_cast<const uint16_t *>(slot + at.block));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[i] = __builtin_amdgcn_alignbyte(w[i + 1], w[i], at.shift);
+  }
+  __device__ __forceinline__ float against(const LaneCodes &a) const {
+    int total = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) total = dot4(q[i], a.codes[i], total);
+    return (d * a.scale[0]) * (float)total;
+  }
+};
+
+// LDS of a block: for every (activation row, span) the 64 lanes' LaneCodes, stored as
+// [word][lane] so that a wave reads each word of its lanes from consecutive banks.
+constexpr uint32_t kCodeWords = 8 + 2 + 4;  // codes, scales, sums
+__device__ __forceinline__ void park(uint32_t *staged, uint32_t pair, uint32_t lane, const LaneCodes &c) {
+  uint32_t *at = staged + (size_t)pair * kCodeWords * kWaveLanes + lane;
+#pragma unroll
+  for (int w = 0; w < 8; ++w) at[w * kWaveLanes] = c.codes[w];
+  at[8 * kWaveLanes] = f32_bits(c.scale[0]);
+  at[9 * kWaveLanes] = f32_bits(c.scale[1]);
+#pragma unroll
+  for (int w = 0; w < 4; ++w) at[(10 + w) * kWaveLanes] = (uint32_t)c.sums[w];
+}
+__device__ __forceinline__ LaneCodes fetch(const uint32_t *staged, uint32_t pair, uint32_t lane) {
+  const uint32_t *at = staged + (size_t)pair * kCodeWords * kWaveLanes + lane;
+  LaneCodes c;
+#pragma unroll
+  for (int w = 0; w < 8; ++w) c.codes[w] = at[w * kWaveLanes];
+  c.scale[0] = bits_f32(at[8 * kWaveLanes]);
+  c.scale[1] = bits_f32(at[9 * kWaveLanes]);
+#pragma unroll
+  for (int w = 0; w < 4; ++w) c.sums[w] = (int)at[(10 + w) * kWaveLanes];
+  return c;
+}
+
+// kM activation rows (rows past m repeat the last one and are not stored); kRegisters: one span
+// per row (K = 2048), the lane's codes live in registers for the whole kernel.
+template <int kKind, class TX, int kM, bool kRegisters>
+__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_lines(const unsigned char *weights, const void *x,
+                                                                      void *y, uint32_t rows, uint64_t row_stride,
+                                                                      uint32_t spans, uint32_t m) {
+  using Row = LinesRow<kKind, 1>;
+  using Kind = Lines<kKind>;
+  constexpr uint32_t kSpanBytes = Kind::kPassVectors * 16;
+  __shared__ __align__(16) unsigned char slots[kWavesPerBlock][Row::kSlotBytes];
+  extern __shared__ __align__(16) uint32_t staged[];  // [m * spans][kCodeWords][64]
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  const uint32_t k = spans * 2048;
+  // every wave quantises its share of the (activation row, span) pairs; the block then shares them
+  for (uint32_t pair = wave; pair < m * spans; pair += kWavesPerBlock)
+    park(staged, pair, lane, quantise_span<kKind, TX>(x, (size_t)(pair / spans) * k, pair % spans, lane));
+  __syncthreads();
+  LaneCodes held[kRegisters ? kM : 1];
+  if constexpr (kRegisters) {
+#pragma unroll
+    for (int r = 0; r < kM; ++r) held[r] = fetch(staged, (uint32_t)r < m ? (uint32_t)r : m - 1, lane);
+  }
+  unsigned char *slot = slots[wave];
+  const typename Kind::Lane at = Kind::lane_of(0, lane);
+  const uint32_t stride = gridDim.x * kWavesPerBlock;
+  const uint32_t first = blockIdx.x * kWavesPerBlock + wave;
+  if (first >= rows) return;  // no barrier follows
+  const uint32_t own_rows = (rows - first + stride - 1) / stride;
+  const uint64_t segments = (uint64_t)own_rows * spans;
+  // the stream of loads runs kLinesDepth segments ahead of the stream of decodes
+  uint32_t load_row = first, load_span = 0;
+  uint64_t loaded = 0;
+  auto next_load = [&]() {
+    // past the wave's last segment: its first row again, a valid address whose bytes go unused
+    const bool live = loaded < segments;
+    const unsigned char *source = weights + (size_t)(live ? load_row : first) * row_stride +
+                                  (size_t)(live ? load_span : 0u) * kSpanBytes;
+    ++loaded;
+    if (++load_span == spans) {
+      load_span = 0;
+      load_row += stride;
+    }
+    return Row::load(source, lane);
+  };
+  Row ring[kLinesDepth];
+#pragma unroll
+  for (int d = 0; d < kLinesDepth; ++d) ring[d] = next_load();
+  uint32_t row = first, span = 0;
+  float totals[kM] = {};
+  // value b * kM + r of a batch is activation row r against the batch's b-th weight row
+  constexpr int kBatch = kM >= 4 ? 1 : 4 / kM;
+  float pending[kBatch * kM] = {};
+  int filled = 0;
+  auto flush = [&](uint32_t first_row, int count) {
+    const float mine = joint_sum<kBatch * kM>(pending, lane);
+    const uint32_t b = (lane % (uint32_t)(kBatch * kM)) / (uint32_t)kM, r = lane % (uint32_t)kM;
+    if (lane < (uint32_t)(kBatch * kM) && (int)b < count && r < m)
+      Traits<TX>::store(y, (size_t)r * rows + first_row + b * stride, mine);
+#pragma unroll
+    for (int i = 0; i < kBatch * kM; ++i) pending[i] = 0.0f;
+  };
+  for (uint64_t done = 0; done < segments; done += kLinesDepth) {
+#pragma unroll
+    for (int d = 0; d < kLinesDepth; ++d) {
+      if (done + d >= segments) break;
+#pragma unroll
+      for (int i = 0; i < Row::kLoads; ++i)
+        *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = ring[d].v[i];
+      ring[d] = next_load();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      SpanDot<kKind> decoded;
+      decoded.decode(slot, at);
+#pragma unroll
+      for (int r = 0; r < kM; ++r) {
+        if constexpr (kRegisters) {
+          totals[r] += decoded.against(held[r]);
+        } else {
+          const uint32_t pair = ((uint32_t)r < m ? (uint32_t)r : m - 1) * spans + span;
+          totals[r] += decoded.against(fetch(staged, pair, lane));
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (++span == spans) {
+        // the row is complete: park its kM totals; kBatch rows are summed over the wave together
+#pragma unroll
+        for (int r = 0; r < kM; ++r) {
+          pending[filled * kM + r] = totals[r];
+          totals[r] = 0.0f;
+        }
+        span = 0;
+        row += stride;
+        if (++filled == kBatch) {
+          flush(row - (uint32_t)kBatch * stride, filled);
+          filled = 0;
+        }
+      }
+    }
+  }
+  if (filled != 0) flush(row - (uint32_t)filled * stride, filled);
+}
+
+template <int kKind, class TX, int kM>
+hipError_t run_registers(const MatVecParams &p, const void *w, const void *x, void *y, uint32_t spans, dim3 grid,
+                         size_t shared, hipStream_t s) {
+  const unsigned char *in = static_cast<const unsigned char *>(w);
+  if (spans == 1)
+    hipLaunchKernelGGL((gguf_matvec_q8_lines<kKind, TX, kM, true>), grid, dim3(kBlockThreads), shared, s, in, x, y,
+                       (uint32_t)p.rows, p.row_stride, spans, p.m);
+  else
+    hipLaunchKernelGGL((gguf_matvec_q8_lines<kKind, TX, kM, false>), grid, dim3(kBlockThreads), shared, s, in, x, y,
+                       (uint32_t)p.rows, p.row_stride, spans, p.m);
+  return hipGetLastError();
+}
+
+template <int kKind, class TX>
+hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, int compute_units, hipStream_t s) {
+  const uint32_t spans = p.k / 2048;
+  const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
+  const uint32_t machine = (uint32_t)(compute_units > 0 ? compute_units : 256) * 3u;  // three blocks per compute unit
+  const dim3 grid(wanted < machine ? wanted : machine);
+  const size_t shared = gguf_matvec_q8_shared_bytes(p.m, p.k);
+  if (p.m == 1) return run_registers<kKind, TX, 1>(p, w, x, y, spans, grid, shared, s);
+  if (p.m == 2) return run_registers<kKind, TX, 2>(p, w, x, y, spans, grid, shared, s);
+  if (p.m <= 4) return run_registers<kKind, TX, 4>(p, w, x, y, spans, grid, shared, s);
+  return run_registers<kKind, TX, 8>(p, w, x, y, spans, grid, shared, s);
+}
+
+template <class TX>
+hipError_t run_kind(const MatVecParams &p, const void *w, const void *x, void *y, int compute_units, hipStream_t s) {
+  switch (p.kind) {
+    case 0: return run_m<0, TX>(p, w, x, y, compute_units, s);
+    case 1: return run_m<1, TX>(p, w, x, y, compute_units, s);
+    default: return run_m<2, TX>(p, w, x, y, compute_units, s);
+  }
+}
+
+}  // namespace
+
+size_t gguf_matvec_q8_shared_bytes(uint32_t m, uint32_t k) {
+  return (size_t)m * (k / 2048) * kCodeWords * kWaveLanes * sizeof(uint32_t);
+}
+
+// Needs K = 2048 n, rows made of whole 16-byte vectors at a 16-byte aligned address, M <= 8 and
+// gguf_matvec_q8_shared_bytes(m, k) + 12 KiB within a block's 64 KiB (the plan checks all four).
+hipError_t launch_gguf_matvec_q8(Elem x_type, const MatVecParams &p, const void *weights, const void *x, void *y,
+                                 int compute_units, hipStream_t stream) {
+  if (p.rows == 0 || p.m == 0) return hipSuccess;
+  switch (x_type) {
+    case Elem::kF32: return run_kind<F32>(p, weights, x, y, compute_units, stream);
+    case Elem::kF16: return run_kind<F16>(p, weights, x, y, compute_units, stream);
+    case Elem::kBF16: return run_kind<BF16>(p, weights, x, y, compute_units, stream);
+  }
+  return hipErrorInvalidValue;
+}
+
+}  // namespace hyle_hip

@@ -185,8 +185,13 @@ struct MatVecParams {
   uint32_t k = 0, m = 0;
   uint64_t row_stride = 0;  // bytes between physical weight rows
   uint8_t kind = 0;
+  uint8_t codec = 0;        // HYLE_HIP_ACTIVATIONS_*: 0 exact f32 activations, 1 ggml's 8-bit activation blocks
 };
 size_t gguf_matvec_shared_bytes(uint32_t m, uint32_t k);
+// The 8-bit activation route: K = 2048 n, rows of whole 16-byte vectors, M <= 8.
+size_t gguf_matvec_q8_shared_bytes(uint32_t m, uint32_t k);
+hipError_t launch_gguf_matvec_q8(Elem x_type, const MatVecParams &p, const void *weights, const void *x, void *y,
+                                 int compute_units, hipStream_t stream);
 hipError_t launch_gguf_matvec(Elem x_type, const MatVecParams &p, const void *weights, const void *x, void *y,
                               hipStream_t stream);
 

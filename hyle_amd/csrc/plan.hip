@@ -450,6 +450,8 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
     case HYLE_HIP_OP_GGUF_MATVEC: {
       if ((s = expect_inputs(r, 2, 2)) != HYLE_HIP_OK) return s;
       if ((s = expect_gguf_weight(in[0])) != HYLE_HIP_OK) return s;
+      if (r.kind2 > HYLE_HIP_ACTIVATIONS_GGML_Q8)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "GGUF matvec activation mode is invalid");
       // MatMul contraction (src/compute_ops/operation.cc, kMatMul): the last axis of the
       // activations meets the first logical axis of the weight
       if (!is_floating(in[1].dtype) || in[1].rank < 1 || in[1].rank > 2 ||
@@ -940,16 +942,27 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       if ((s = admit_gguf_rows(in[0])) != HYLE_HIP_OK) return s;
       const int64_t m = in[1].rank == 2 ? in[1].dims[0] : 1;
       if (m > 8) return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec serves at most 8 activation rows");
-      if (gguf_matvec_shared_bytes((uint32_t)m, (uint32_t)k) > 64 * 1024)
+      if (r.kind2 == HYLE_HIP_ACTIVATIONS_GGML_Q8) {
+        // whole spans of 2048 values in rows of whole 16-byte vectors; the codes of every
+        // activation row sit in LDS beside the waves' row buffers (12 KiB)
+        if (k % 2048 != 0 || in[0].byte_strides[1] % 16 != 0)
+          return fail(HYLE_HIP_UNIMPLEMENTED,
+                      "GGUF matvec with 8-bit activation blocks serves K = 2048 n and 16-byte aligned rows");
+        if (gguf_matvec_q8_shared_bytes((uint32_t)m, (uint32_t)k) + 12 * 1024 > 64 * 1024)
+          return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec keeps the activation codes in LDS: M * K is too large");
+        p->input_alignment[0] = 16;
+      } else if (gguf_matvec_shared_bytes((uint32_t)m, (uint32_t)k) > 64 * 1024) {
         return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec keeps the activations in LDS: M * K is too large");
+      }
       if (p->output_elements[0] == 0) return HYLE_HIP_OK;
       p->route = Route::kGgufMatVec;
+      p->matvec.codec = (uint8_t)r.kind2;
       p->matvec.rows = (uint64_t)n;
       p->matvec.k = (uint32_t)k;
       p->matvec.m = (uint32_t)m;
       p->matvec.row_stride = (uint64_t)in[0].byte_strides[1];
       p->matvec.kind = per_block == 32 ? 2 : (block_bytes == 144 ? 0 : 1);
-      p->input_alignment[0] = 1;
+      if (r.kind2 != HYLE_HIP_ACTIVATIONS_GGML_Q8) p->input_alignment[0] = 1;
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }
@@ -1302,7 +1315,11 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
       err = launch_k_quant_dequant(plan->kquant, inputs[0], outputs[0], static_cast<float *>(outputs[1]), stream);
       break;
     case Route::kGgufMatVec:
-      err = launch_gguf_matvec(plan->elem, plan->matvec, inputs[0], inputs[1], outputs[0], stream);
+      if (plan->matvec.codec == HYLE_HIP_ACTIVATIONS_GGML_Q8)
+        err = launch_gguf_matvec_q8(plan->elem, plan->matvec, inputs[0], inputs[1], outputs[0],
+                                    plan->context->compute_units, stream);
+      else
+        err = launch_gguf_matvec(plan->elem, plan->matvec, inputs[0], inputs[1], outputs[0], stream);
       break;
     case Route::kCast:
       err = launch_cast(plan->cast, inputs[0], outputs[0], vector, stream);

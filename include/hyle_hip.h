@@ -95,9 +95,12 @@ typedef enum hyle_hip_op_kind {
   HYLE_HIP_OP_GGUF_DEQUANT_SUMSQ = 0x101,
   /* MatMul(in1, in0) for token-by-token decoding: in0 a GGUF weight (Q8_0, Q4_K, Q6_K), logical
    * [K, N]; in1 dense f32 / f16 / bf16 activations [K] or [M, K] with M <= 8; out0 [N] or [M, N]
-   * of in1's type.  Weights are decoded exactly, products and sums are f32 (ggml, which serves
-   * this in the reference, quantises the activations to 8 bits first: its rounding is not
-   * reproduced). */
+   * of in1's type.  kind2 selects the arithmetic (HYLE_HIP_ACTIVATIONS_*): EXACT decodes the
+   * weights exactly and multiplies in f32; GGML_Q8 is what the reference's ggml CPU route
+   * computes: the activations are first quantised to ggml's 8-bit blocks (Q8_0 blocks for a Q8_0
+   * weight, Q8_K blocks for Q4_K / Q6_K) and the block dot products are integers
+   * (tests/compute_models/qwen27_original_nextn_reference.h:94-167,193-257 holds that
+   * arithmetic and the bound the reference accepts of it). */
   HYLE_HIP_OP_GGUF_MATVEC = 0x102
 } hyle_hip_op_kind;
 
@@ -140,6 +143,9 @@ enum { HYLE_HIP_GATED_PACKED_HALVES = 0, HYLE_HIP_GATED_SEPARATE = 1 };
 enum { HYLE_HIP_SOFTMAX = 0, HYLE_HIP_LOG_SOFTMAX = 1 };
 enum { HYLE_HIP_MASK_NONE = 0, HYLE_HIP_MASK_ADDITIVE = 1, HYLE_HIP_MASK_BOOLEAN = 2 };
 
+/* GGUF_MATVEC kind2 */
+enum { HYLE_HIP_ACTIVATIONS_EXACT = 0, HYLE_HIP_ACTIVATIONS_GGML_Q8 = 1 };
+
 /* StorageFormatKind (include/hyle/compute/tensor_desc.h:77-81) */
 enum { HYLE_HIP_STORAGE_PLAIN = 0, HYLE_HIP_STORAGE_BLOCKED = 1 };
 
@@ -166,7 +172,7 @@ typedef struct hyle_hip_op_desc {
   uint32_t op;               /* hyle_hip_op_kind */
   uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind; Cast: output hyle_hip_dtype */
   uint32_t kind2;            /* BINARY_CHAIN: second BinaryKind; GATED: GatedInputKind;
-                                SOFTMAX: SoftmaxKind */
+                                SOFTMAX: SoftmaxKind; GGUF_MATVEC: HYLE_HIP_ACTIVATIONS_* */
   int32_t axis;              /* Softmax / TopK axis (negative counts from the end) */
   uint32_t mask;             /* Softmax MaskKind */
   uint32_t accumulation;     /* hyle_hip_dtype; UNKNOWN or F32 */
