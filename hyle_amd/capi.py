@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(HERE, "libhyle_hip.so")
 MAX_RANK, MAX_INPUTS, MAX_OUTPUTS, ABI_VERSION = 8, 4, 2, 1
 
 # hyle_hip_status
-OK, INVALID_ARGUMENT, RESOURCE_EXHAUSTED, FAILED_PRECONDITION = 0, 3, 8, 9
+OK, CANCELLED, INVALID_ARGUMENT, RESOURCE_EXHAUSTED, FAILED_PRECONDITION = 0, 1, 3, 8, 9
 OUT_OF_RANGE, UNIMPLEMENTED, INTERNAL, UNAVAILABLE = 11, 12, 13, 14
 
 
@@ -57,7 +57,28 @@ class ReadRangeC(C.Structure):
 class StreamResultC(C.Structure):
     _fields_ = [("status", C.c_int), ("read_bytes", C.c_uint64), ("copied_bytes", C.c_uint64),
                 ("ready_ranges", C.c_uint32), ("total_ranges", C.c_uint32), ("io_calls", C.c_uint32),
-                ("native_calls", C.c_uint32), ("host_waits", C.c_uint32)]
+                ("native_calls", C.c_uint32), ("host_waits", C.c_uint32),
+                ("written_bytes", C.c_uint64), ("complete", C.c_uint32)]
+
+
+class WriteRangeC(C.Structure):
+    _fields_ = [("source", C.c_void_p), ("file_offset", C.c_uint64), ("bytes", C.c_size_t)]
+
+
+class DevicePropertiesC(C.Structure):  # include/hyle_hip_backend.h
+    _fields_ = [("ordinal", C.c_int32), ("compute_units", C.c_int32), ("total_memory_bytes", C.c_uint64),
+                ("unified_memory", C.c_uint32), ("asynchronous_queues", C.c_uint32),
+                ("name", C.c_char * 128), ("architecture", C.c_char * 64)]
+
+
+class MemoryPropertiesC(C.Structure):
+    _fields_ = [("flags", C.c_uint32), ("kind", C.c_uint32), ("minimum_alignment", C.c_size_t),
+                ("maximum_allocation", C.c_size_t)]
+
+
+class MemoryStatsC(C.Structure):
+    _fields_ = [("used_bytes", C.c_size_t), ("peak_bytes", C.c_size_t), ("live_allocations", C.c_uint64),
+                ("total_allocations", C.c_uint64)]
 
 
 EXPORTS = {
@@ -90,13 +111,48 @@ EXPORTS = {
     "hyle_hip_file_pipeline_read": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(ReadRangeC), C.c_uint32, C.c_void_p,
                                               C.POINTER(StreamResultC)]),
     "hyle_hip_file_pipeline_wait": (C.c_int, [C.c_void_p]),
+    "hyle_hip_file_pipeline_write": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(WriteRangeC), C.c_uint32, C.c_void_p,
+                                               C.POINTER(StreamResultC)]),
+    "hyle_hip_file_pipeline_submit_read": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(ReadRangeC), C.c_uint32, C.c_void_p,
+                                                     C.POINTER(C.c_void_p)]),
+    "hyle_hip_file_pipeline_submit_write": (C.c_int, [C.c_void_p, C.c_int, C.POINTER(WriteRangeC), C.c_uint32,
+                                                      C.c_void_p, C.POINTER(C.c_void_p)]),
+    "hyle_hip_stream_ticket_result": (C.c_int, [C.c_void_p, C.POINTER(StreamResultC)]),
+    "hyle_hip_stream_ticket_wait": (C.c_int, [C.c_void_p, C.POINTER(StreamResultC)]),
+    "hyle_hip_stream_ticket_request_cancel": (None, [C.c_void_p]),
+    "hyle_hip_stream_ticket_release": (None, [C.c_void_p]),
+    # include/hyle_hip_backend.h
+    "hyle_hip_backend_device_count": (C.c_int, [C.POINTER(C.c_size_t)]),
+    "hyle_hip_backend_device_properties": (C.c_int, [C.c_size_t, C.POINTER(DevicePropertiesC)]),
+    "hyle_hip_memory_resource_create": (C.c_int, [C.c_void_p, C.c_uint32, C.POINTER(C.c_void_p)]),
+    "hyle_hip_memory_resource_destroy": (None, [C.c_void_p]),
+    "hyle_hip_memory_resource_properties": (C.c_int, [C.c_void_p, C.POINTER(MemoryPropertiesC)]),
+    "hyle_hip_memory_allocate": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, C.POINTER(C.c_void_p)]),
+    "hyle_hip_memory_deallocate": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "hyle_hip_memory_resource_stats": (C.c_int, [C.c_void_p, C.POINTER(MemoryStatsC)]),
+    "hyle_hip_backend_validate_resource": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "hyle_hip_queue_create": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "hyle_hip_queue_destroy": (None, [C.c_void_p]),
+    "hyle_hip_queue_stream": (C.c_void_p, [C.c_void_p]),
+    "hyle_hip_queue_reserve_completions": (C.c_int, [C.c_void_p, C.c_size_t]),
+    "hyle_hip_queue_begin_sequence": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p)]),
+    "hyle_hip_queue_finish_sequence": (C.c_void_p, [C.c_void_p, C.c_void_p, C.c_int, C.c_int]),
+    "hyle_hip_completion_poll": (C.c_int, [C.c_void_p, C.POINTER(C.c_int)]),
+    "hyle_hip_completion_wait": (C.c_int, [C.c_void_p]),
+    "hyle_hip_completion_release": (None, [C.c_void_p]),
+    "hyle_hip_queue_wait_completion": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "hyle_hip_queue_copy_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
+    "hyle_hip_queue_fill_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint8, C.c_size_t]),
+    "hyle_hip_queue_drain": (C.c_int, [C.c_void_p]),
+    "hyle_hip_context_drain": (C.c_int, [C.c_void_p]),
 }
 
 _lib = None
 
 
 def load() -> C.CDLL:
-    """Load libhyle_hip.so and bind every symbol include/hyle_hip.h and include/hyle_hip_stream.h declare."""
+    """Load libhyle_hip.so and bind every symbol that include/hyle_hip.h, include/hyle_hip_stream.h and
+    include/hyle_hip_backend.h declare."""
     global _lib
     if _lib is not None:
         return _lib

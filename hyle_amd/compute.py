@@ -26,6 +26,7 @@ from . import capi
 # ---- status ---------------------------------------------------------------------------
 class StatusCode(enum.IntEnum):  # include/hyle/error/status.h:18-38
     kOk = 0
+    kCancelled = 1
     kInvalidArgument = 3
     kResourceExhausted = 8
     kFailedPrecondition = 9

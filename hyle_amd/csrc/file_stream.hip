@@ -1,17 +1,23 @@
 // file_stream.hip -- the C ABI of include/hyle_hip_stream.h: a stream-ordered batch of copies
 // (the copy endpoint a route gives the reference's file streamer,
-// src/compute_stream_cuda/file_stream.cc:8-21) and a staging loop that reads file ranges into
-// pinned slots and copies each filled slot to its device destinations
-// (the slot discipline of src/compute_stream/file_stream.cc: a slot is refilled only after the
-// copies that read it have finished).  Host code only.
+// src/compute_stream_cuda/file_stream.cc:8-21) and a staging loop in both directions: file
+// ranges read into pinned slots and copied to their device destinations, device ranges copied
+// into pinned slots and written to a file (the slot discipline of
+// src/compute_stream/file_stream.cc: a slot is reused only after the copies that touch it have
+// finished), on the caller's thread or behind a ticket, with cooperative cancellation at slot
+// boundaries.  Host code only.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cerrno>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
 #include <new>
+#include <thread>
+#include <type_traits>
 #include <unistd.h>
+#include <vector>
 
 #include "../../include/hyle_hip_stream.h"
 
@@ -51,6 +57,7 @@ struct hyle_hip_file_pipeline {
   size_t slot_bytes = 0;
   Slot slots[kMaxSlots];
   uint32_t next_slot = 0;
+  std::atomic<bool> busy{false};  // a request (on the caller's thread or behind a ticket) is running
 };
 
 extern "C" {
@@ -146,39 +153,48 @@ void hyle_hip_file_pipeline_destroy(hyle_hip_file_pipeline *p) {
   delete p;
 }
 
-hyle_hip_status hyle_hip_file_pipeline_read(hyle_hip_file_pipeline *p, int fd, const hyle_hip_read_range *ranges,
-                                            uint32_t range_count, void *stream_handle,
-                                            hyle_hip_stream_result *result) {
-  hyle_hip_stream_result local{};
-  hyle_hip_stream_result &out = result ? *result : local;
-  out = hyle_hip_stream_result{};
-  out.total_ranges = range_count;
-  auto finish = [&](hyle_hip_status status) {
-    out.status = status;
-    return status;
-  };
-  if (p == nullptr) return finish(fail(HYLE_HIP_INVALID_ARGUMENT, "pipeline is null"));
-  if (fd < 0) return finish(fail(HYLE_HIP_INVALID_ARGUMENT, "file descriptor is invalid"));
-  if (range_count != 0 && ranges == nullptr) return finish(fail(HYLE_HIP_INVALID_ARGUMENT, "ranges are null"));
-  for (uint32_t r = 0; r < range_count; ++r)
-    if (ranges[r].bytes != 0 && ranges[r].destination == nullptr)
-      return finish(fail(HYLE_HIP_INVALID_ARGUMENT, "range %u has no destination", r));
-  hipError_t err = hipSetDevice(p->device);
-  if (err != hipSuccess) return finish(hip_fail(err, "hipSetDevice"));
-  hipStream_t stream = static_cast<hipStream_t>(stream_handle);
+}  // extern "C"
 
-  // Ranges are packed into a slot back to back (several small ranges share one, a large one
-  // takes many in turn); a slot goes to the device as soon as it is full or the ranges end.
+namespace {
+
+// Marks the slot as read by copies still in flight; if the event cannot be recorded the
+// stream is drained instead, so that the slot is never refilled or freed under a copy.
+void seal_slot(Slot &slot, hipStream_t stream) {
+  if (hipEventRecord(slot.drained, stream) == hipSuccess) {
+    slot.in_flight = true;
+  } else {
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize(stream);
+    slot.in_flight = false;
+  }
+}
+
+hyle_hip_status wait_slot(Slot &slot, hyle_hip_stream_result &out) {
+  if (!slot.in_flight) return HYLE_HIP_OK;
+  ++out.host_waits;
+  const hipError_t err = hipEventSynchronize(slot.drained);
+  if (err != hipSuccess) return hip_fail(err, "hipEventSynchronize");
+  slot.in_flight = false;
+  return HYLE_HIP_OK;
+}
+
+bool cancelled(const std::atomic<bool> *cancel) { return cancel != nullptr && cancel->load(std::memory_order_relaxed); }
+
+// file -> pinned slots -> device.  Ranges are packed into a slot back to back (several small
+// ranges share one, a large one takes many in turn); a slot goes to the device as soon as it is
+// full or the ranges end.  `out` is updated as the work proceeds, so another thread may read
+// the progress; a cancellation request is honoured before each slot is filled.
+hyle_hip_status run_read(hyle_hip_file_pipeline *p, int fd, const hyle_hip_read_range *ranges, uint32_t range_count,
+                         hipStream_t stream, hyle_hip_stream_result &out, const std::atomic<bool> *cancel) {
+  hipError_t err = hipSetDevice(p->device);
+  if (err != hipSuccess) return hip_fail(err, "hipSetDevice");
   uint32_t r = 0;
   size_t done_in_range = 0;
   while (r < range_count) {
+    if (cancelled(cancel)) return fail(HYLE_HIP_CANCELLED, "the read was cancelled");
     Slot &slot = p->slots[p->next_slot];
-    if (slot.in_flight) {
-      ++out.host_waits;
-      err = hipEventSynchronize(slot.drained);
-      if (err != hipSuccess) return finish(hip_fail(err, "hipEventSynchronize"));
-      slot.in_flight = false;
-    }
+    hyle_hip_status status = wait_slot(slot, out);
+    if (status != HYLE_HIP_OK) return status;
     size_t used = 0;
     bool enqueued = false;
     while (r < range_count && used < p->slot_bytes) {
@@ -198,18 +214,22 @@ hyle_hip_status hyle_hip_file_pipeline_read(hyle_hip_file_pipeline *p, int fd, c
         if (n < 0 && errno == EINTR) continue;
         if (n <= 0) {
           // what was read so far still goes nowhere: the range is incomplete
-          if (enqueued && hipEventRecord(slot.drained, stream) == hipSuccess) slot.in_flight = true;
+          const int saved = errno;
+          if (enqueued) seal_slot(slot, stream);
           out.read_bytes += got;
-          return finish(n == 0 ? fail(HYLE_HIP_OUT_OF_RANGE, "end of file inside range %u at offset %llu", r,
-                                      (unsigned long long)(ranges[r].file_offset + done_in_range + got))
-                               : fail(HYLE_HIP_INTERNAL, "pread: %s", strerror(errno)));
+          return n == 0 ? fail(HYLE_HIP_OUT_OF_RANGE, "end of file inside range %u at offset %llu", r,
+                               (unsigned long long)(ranges[r].file_offset + done_in_range + got))
+                        : fail(HYLE_HIP_INTERNAL, "pread: %s", strerror(saved));
         }
         got += (size_t)n;
       }
       out.read_bytes += piece;
       err = hipMemcpyAsync(static_cast<unsigned char *>(ranges[r].destination) + done_in_range, slot.bytes + used,
                            piece, hipMemcpyHostToDevice, stream);
-      if (err != hipSuccess) return finish(hip_fail(err, "hipMemcpyAsync"));
+      if (err != hipSuccess) {
+        if (enqueued) seal_slot(slot, stream);  // earlier pieces of this slot are still being read
+        return hip_fail(err, "hipMemcpyAsync");
+      }
       enqueued = true;
       ++out.native_calls;
       out.copied_bytes += piece;
@@ -217,13 +237,271 @@ hyle_hip_status hyle_hip_file_pipeline_read(hyle_hip_file_pipeline *p, int fd, c
       done_in_range += piece;
     }
     if (enqueued) {
-      err = hipEventRecord(slot.drained, stream);
-      if (err != hipSuccess) return finish(hip_fail(err, "hipEventRecord"));
-      slot.in_flight = true;
+      seal_slot(slot, stream);
       p->next_slot = (p->next_slot + 1) % p->slot_count;
     }
   }
-  return finish(HYLE_HIP_OK);
+  return HYLE_HIP_OK;
+}
+
+// device -> pinned slots -> file.  Up to slot_count pieces are on their way from the device
+// while the oldest one is written to the file; pieces leave in range order.
+hyle_hip_status run_write(hyle_hip_file_pipeline *p, int fd, const hyle_hip_write_range *ranges, uint32_t range_count,
+                          hipStream_t stream, hyle_hip_stream_result &out, const std::atomic<bool> *cancel) {
+  hipError_t err = hipSetDevice(p->device);
+  if (err != hipSuccess) return hip_fail(err, "hipSetDevice");
+  hyle_hip_status status = HYLE_HIP_OK;
+  for (uint32_t s = 0; s < p->slot_count; ++s)  // leftovers of an earlier read
+    if ((status = wait_slot(p->slots[s], out)) != HYLE_HIP_OK) return status;
+  struct Piece {
+    uint32_t range;
+    uint64_t file_offset;
+    size_t bytes;
+    bool closes_range;
+  };
+  Piece in_slot[kMaxSlots];
+  uint32_t head = 0, filled = 0;  // slots [head, head + filled) hold pieces on their way, oldest first
+  uint32_t r = 0;
+  size_t done_in_range = 0;
+  auto retire_oldest = [&]() -> hyle_hip_status {
+    Slot &slot = p->slots[head];
+    const Piece piece = in_slot[head];
+    hyle_hip_status waited = wait_slot(slot, out);
+    if (waited != HYLE_HIP_OK) return waited;
+    size_t put = 0;
+    while (put < piece.bytes) {
+      const ssize_t n = pwrite(fd, slot.bytes + put, piece.bytes - put, (off_t)(piece.file_offset + put));
+      ++out.io_calls;
+      if (n < 0 && errno == EINTR) continue;
+      if (n <= 0) {
+        out.written_bytes += put;
+        return fail(HYLE_HIP_INTERNAL, "pwrite at offset %llu: %s", (unsigned long long)(piece.file_offset + put),
+                    n == 0 ? "no progress" : strerror(errno));
+      }
+      put += (size_t)n;
+    }
+    out.written_bytes += piece.bytes;
+    if (piece.closes_range) ++out.ready_ranges;
+    head = (head + 1) % p->slot_count;
+    --filled;
+    return HYLE_HIP_OK;
+  };
+  auto drain_in_flight = [&]() {  // on an error exit: no copy may still write into a slot
+    for (uint32_t s = 0; s < p->slot_count; ++s)
+      if (p->slots[s].in_flight && hipEventSynchronize(p->slots[s].drained) == hipSuccess) p->slots[s].in_flight = false;
+  };
+  while (r < range_count || filled != 0) {
+    if (cancelled(cancel)) {
+      drain_in_flight();
+      return fail(HYLE_HIP_CANCELLED, "the write was cancelled");
+    }
+    while (r < range_count && ranges[r].bytes == done_in_range) {  // empty or finished ranges
+      if (ranges[r].bytes == 0) ++out.ready_ranges;
+      ++r;
+      done_in_range = 0;
+    }
+    if (r < range_count && filled < p->slot_count) {
+      const uint32_t at = (head + filled) % p->slot_count;
+      Slot &slot = p->slots[at];
+      const size_t left = ranges[r].bytes - done_in_range;
+      const size_t piece = left < p->slot_bytes ? left : p->slot_bytes;
+      err = hipMemcpyAsync(slot.bytes, static_cast<const unsigned char *>(ranges[r].source) + done_in_range, piece,
+                           hipMemcpyDeviceToHost, stream);
+      if (err != hipSuccess) {
+        drain_in_flight();
+        return hip_fail(err, "hipMemcpyAsync");
+      }
+      seal_slot(slot, stream);
+      ++out.native_calls;
+      out.copied_bytes += piece;
+      in_slot[at] = Piece{r, ranges[r].file_offset + done_in_range, piece, piece == left};
+      ++filled;
+      done_in_range += piece;
+      continue;
+    }
+    if (filled != 0 && (status = retire_oldest()) != HYLE_HIP_OK) {
+      drain_in_flight();
+      return status;
+    }
+  }
+  p->next_slot = 0;
+  return HYLE_HIP_OK;
+}
+
+hyle_hip_status check_request(hyle_hip_file_pipeline *p, int fd, const void *ranges, uint32_t range_count) {
+  if (p == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "pipeline is null");
+  if (fd < 0) return fail(HYLE_HIP_INVALID_ARGUMENT, "file descriptor is invalid");
+  if (range_count != 0 && ranges == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "ranges are null");
+  return HYLE_HIP_OK;
+}
+hyle_hip_status check_ranges(const hyle_hip_read_range *ranges, uint32_t range_count) {
+  for (uint32_t r = 0; r < range_count; ++r)
+    if (ranges[r].bytes != 0 && ranges[r].destination == nullptr)
+      return fail(HYLE_HIP_INVALID_ARGUMENT, "range %u has no destination", r);
+  return HYLE_HIP_OK;
+}
+hyle_hip_status check_ranges(const hyle_hip_write_range *ranges, uint32_t range_count) {
+  for (uint32_t r = 0; r < range_count; ++r)
+    if (ranges[r].bytes != 0 && ranges[r].source == nullptr)
+      return fail(HYLE_HIP_INVALID_ARGUMENT, "range %u has no source", r);
+  return HYLE_HIP_OK;
+}
+
+// One request at a time per pipeline.
+bool claim(hyle_hip_file_pipeline *p) {
+  bool idle = false;
+  return p->busy.compare_exchange_strong(idle, true);
+}
+
+}  // namespace
+
+// A request running on a thread of its own.  `result` is written by that thread only, in
+// whole fields; readers take a snapshot that may be a moment old.
+struct hyle_hip_stream_ticket {
+  hyle_hip_file_pipeline *pipeline = nullptr;
+  std::thread worker;
+  std::atomic<bool> cancel{false};
+  std::atomic<bool> ended{false};
+  hyle_hip_stream_result result{};
+  std::vector<hyle_hip_read_range> reads;
+  std::vector<hyle_hip_write_range> writes;
+  char error_text[320] = "";
+  int fd = -1;
+  hipStream_t stream = nullptr;
+  bool is_write = false;
+};
+
+namespace {
+
+void ticket_main(hyle_hip_stream_ticket *t) {
+  hyle_hip_status status;
+  if (t->is_write)
+    status = run_write(t->pipeline, t->fd, t->writes.data(), (uint32_t)t->writes.size(), t->stream, t->result, &t->cancel);
+  else
+    status = run_read(t->pipeline, t->fd, t->reads.data(), (uint32_t)t->reads.size(), t->stream, t->result, &t->cancel);
+  if (status == HYLE_HIP_OK && !t->is_write) status = hyle_hip_file_pipeline_wait(t->pipeline);  // the copies too
+  std::snprintf(t->error_text, sizeof t->error_text, "%s", hyle_hip_last_error());  // this thread's text
+  t->result.status = status;
+  t->result.complete = 1;
+  t->pipeline->busy.store(false);
+  t->ended.store(true, std::memory_order_release);
+}
+
+template <class Range>
+hyle_hip_status submit(hyle_hip_file_pipeline *p, int fd, const Range *ranges, uint32_t range_count, void *stream,
+                       hyle_hip_stream_ticket **out, bool is_write) {
+  if (out == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "ticket output is null");
+  *out = nullptr;
+  hyle_hip_status status = check_request(p, fd, ranges, range_count);
+  if (status == HYLE_HIP_OK) status = check_ranges(ranges, range_count);
+  if (status != HYLE_HIP_OK) return status;
+  auto *t = new (std::nothrow) hyle_hip_stream_ticket();
+  if (t == nullptr) return fail(HYLE_HIP_RESOURCE_EXHAUSTED, "out of host memory");
+  if (!claim(p)) {
+    delete t;
+    return fail(HYLE_HIP_FAILED_PRECONDITION, "the pipeline is running another request");
+  }
+  t->pipeline = p;
+  t->fd = fd;
+  t->stream = static_cast<hipStream_t>(stream);
+  t->is_write = is_write;
+  t->result.total_ranges = range_count;
+  try {
+    if constexpr (std::is_same<Range, hyle_hip_write_range>::value) t->writes.assign(ranges, ranges + range_count);
+    else t->reads.assign(ranges, ranges + range_count);
+    t->worker = std::thread(ticket_main, t);
+  } catch (...) {
+    p->busy.store(false);
+    delete t;
+    return fail(HYLE_HIP_RESOURCE_EXHAUSTED, "the request's thread could not be started");
+  }
+  *out = t;
+  return HYLE_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+hyle_hip_status hyle_hip_file_pipeline_read(hyle_hip_file_pipeline *p, int fd, const hyle_hip_read_range *ranges,
+                                            uint32_t range_count, void *stream_handle,
+                                            hyle_hip_stream_result *result) {
+  hyle_hip_stream_result local{};
+  hyle_hip_stream_result &out = result ? *result : local;
+  out = hyle_hip_stream_result{};
+  out.total_ranges = range_count;
+  hyle_hip_status status = check_request(p, fd, ranges, range_count);
+  if (status == HYLE_HIP_OK) status = check_ranges(ranges, range_count);
+  if (status == HYLE_HIP_OK && !claim(p))
+    status = fail(HYLE_HIP_FAILED_PRECONDITION, "the pipeline is running another request");
+  else if (status == HYLE_HIP_OK) {
+    status = run_read(p, fd, ranges, range_count, static_cast<hipStream_t>(stream_handle), out, nullptr);
+    p->busy.store(false);
+  }
+  out.status = status;
+  out.complete = 1;
+  return status;
+}
+
+hyle_hip_status hyle_hip_file_pipeline_write(hyle_hip_file_pipeline *p, int fd, const hyle_hip_write_range *ranges,
+                                             uint32_t range_count, void *stream_handle,
+                                             hyle_hip_stream_result *result) {
+  hyle_hip_stream_result local{};
+  hyle_hip_stream_result &out = result ? *result : local;
+  out = hyle_hip_stream_result{};
+  out.total_ranges = range_count;
+  hyle_hip_status status = check_request(p, fd, ranges, range_count);
+  if (status == HYLE_HIP_OK) status = check_ranges(ranges, range_count);
+  if (status == HYLE_HIP_OK && !claim(p))
+    status = fail(HYLE_HIP_FAILED_PRECONDITION, "the pipeline is running another request");
+  else if (status == HYLE_HIP_OK) {
+    status = run_write(p, fd, ranges, range_count, static_cast<hipStream_t>(stream_handle), out, nullptr);
+    p->busy.store(false);
+  }
+  out.status = status;
+  out.complete = 1;
+  return status;
+}
+
+hyle_hip_status hyle_hip_file_pipeline_submit_read(hyle_hip_file_pipeline *p, int fd, const hyle_hip_read_range *ranges,
+                                                   uint32_t range_count, void *stream, hyle_hip_stream_ticket **ticket) {
+  return submit(p, fd, ranges, range_count, stream, ticket, false);
+}
+
+hyle_hip_status hyle_hip_file_pipeline_submit_write(hyle_hip_file_pipeline *p, int fd,
+                                                    const hyle_hip_write_range *ranges, uint32_t range_count,
+                                                    void *stream, hyle_hip_stream_ticket **ticket) {
+  return submit(p, fd, ranges, range_count, stream, ticket, true);
+}
+
+hyle_hip_status hyle_hip_stream_ticket_result(hyle_hip_stream_ticket *ticket, hyle_hip_stream_result *result) {
+  if (ticket == nullptr || result == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "null argument");
+  const bool ended = ticket->ended.load(std::memory_order_acquire);
+  *result = ticket->result;
+  if (!ended) {  // a snapshot of a running request: its status is not known yet
+    result->status = HYLE_HIP_OK;
+    result->complete = 0;
+  }
+  return HYLE_HIP_OK;
+}
+
+hyle_hip_status hyle_hip_stream_ticket_wait(hyle_hip_stream_ticket *ticket, hyle_hip_stream_result *result) {
+  if (ticket == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "ticket is null");
+  if (ticket->worker.joinable()) ticket->worker.join();
+  if (result != nullptr) *result = ticket->result;
+  if (ticket->result.status != HYLE_HIP_OK) return fail(ticket->result.status, "%s", ticket->error_text);
+  return HYLE_HIP_OK;
+}
+
+void hyle_hip_stream_ticket_request_cancel(hyle_hip_stream_ticket *ticket) {
+  if (ticket != nullptr) ticket->cancel.store(true, std::memory_order_relaxed);
+}
+
+void hyle_hip_stream_ticket_release(hyle_hip_stream_ticket *ticket) {
+  if (ticket == nullptr) return;
+  ticket->cancel.store(true, std::memory_order_relaxed);
+  if (ticket->worker.joinable()) ticket->worker.join();
+  delete ticket;
 }
 
 }  // extern "C"

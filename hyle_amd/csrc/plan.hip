@@ -1077,6 +1077,7 @@ const char *hyle_hip_last_error(void) { return g_error; }
 const char *hyle_hip_status_name(hyle_hip_status status) {
   switch (status) {
     case HYLE_HIP_OK: return "OK";
+    case HYLE_HIP_CANCELLED: return "CANCELLED";
     case HYLE_HIP_INVALID_ARGUMENT: return "INVALID_ARGUMENT";
     case HYLE_HIP_RESOURCE_EXHAUSTED: return "RESOURCE_EXHAUSTED";
     case HYLE_HIP_FAILED_PRECONDITION: return "FAILED_PRECONDITION";

@@ -35,6 +35,55 @@ class StreamResult:  # include/hyle/compute/file_stream.h:111-118
     io_calls: int
     native_calls: int
     host_waits: int
+    written_bytes: int = 0
+    complete: int = 0
+
+
+@dataclass(frozen=True)
+class StreamWriteRange:  # include/hyle/compute/file_stream.h:92-105 (StreamWriteRange::ready)
+    source: int  # device address
+    file_offset: int
+    bytes: int
+
+
+class StreamTicket:
+    """include/hyle/compute/file_stream.h:158-180: a request running on a thread of the pipeline."""
+
+    def __init__(self, handle: int):
+        self._handle: Optional[int] = handle
+
+    @staticmethod
+    def _snapshot(c_result) -> StreamResult:
+        return StreamResult(*[getattr(c_result, name) for name, _ in capi.StreamResultC._fields_])
+
+    def result(self) -> StreamResult:
+        c_result = capi.StreamResultC()
+        _check(capi.load().hyle_hip_stream_ticket_result(self._handle, C.byref(c_result)))
+        return self._snapshot(c_result)
+
+    def wait(self) -> StreamResult:
+        """Blocks until the request has ended; raises StatusError if it failed or was cancelled
+        (`last_result` keeps the progress)."""
+        c_result = capi.StreamResultC()
+        code = capi.load().hyle_hip_stream_ticket_wait(self._handle, C.byref(c_result))
+        self.last_result = self._snapshot(c_result)
+        if code != capi.OK:
+            raise StatusError(code, capi.last_error())
+        return self.last_result
+
+    def request_cancel(self) -> None:
+        capi.load().hyle_hip_stream_ticket_request_cancel(self._handle)
+
+    def close(self) -> None:
+        if self._handle:
+            capi.load().hyle_hip_stream_ticket_release(self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 @dataclass(frozen=True)
@@ -85,6 +134,34 @@ class FileResourcePipeline:
         if code != capi.OK:
             raise StatusError(code, capi.last_error())
         return self.last_result
+
+    def write(self, fd: int, ranges: Sequence["StreamWriteRange"], stream: int) -> StreamResult:
+        """Device ranges to the file; returns when the last byte is written."""
+        c_ranges = (capi.WriteRangeC * max(len(ranges), 1))(*[capi.WriteRangeC(r.source, r.file_offset, r.bytes)
+                                                              for r in ranges])
+        c_result = capi.StreamResultC()
+        code = capi.load().hyle_hip_file_pipeline_write(self._handle, fd, c_ranges, len(ranges), stream,
+                                                        C.byref(c_result))
+        self.last_result = StreamResult(*[getattr(c_result, name) for name, _ in capi.StreamResultC._fields_])
+        if code != capi.OK:
+            raise StatusError(code, capi.last_error())
+        return self.last_result
+
+    def submit_read(self, fd: int, ranges: Sequence[StreamReadRange], stream: int) -> "StreamTicket":
+        c_ranges = (capi.ReadRangeC * max(len(ranges), 1))(*[capi.ReadRangeC(r.file_offset, r.destination, r.bytes)
+                                                             for r in ranges])
+        handle = C.c_void_p()
+        _check(capi.load().hyle_hip_file_pipeline_submit_read(self._handle, fd, c_ranges, len(ranges), stream,
+                                                              C.byref(handle)))
+        return StreamTicket(handle.value)
+
+    def submit_write(self, fd: int, ranges: Sequence["StreamWriteRange"], stream: int) -> "StreamTicket":
+        c_ranges = (capi.WriteRangeC * max(len(ranges), 1))(*[capi.WriteRangeC(r.source, r.file_offset, r.bytes)
+                                                              for r in ranges])
+        handle = C.c_void_p()
+        _check(capi.load().hyle_hip_file_pipeline_submit_write(self._handle, fd, c_ranges, len(ranges), stream,
+                                                               C.byref(handle)))
+        return StreamTicket(handle.value)
 
     def wait(self) -> None:
         _check(capi.load().hyle_hip_file_pipeline_wait(self._handle))

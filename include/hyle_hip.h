@@ -44,6 +44,7 @@ extern "C" {
  * other non-OK code is an error. */
 typedef enum hyle_hip_status {
   HYLE_HIP_OK = 0,
+  HYLE_HIP_CANCELLED = 1, /* a file-pipeline request that was asked to stop (hyle_hip_stream.h) */
   HYLE_HIP_INVALID_ARGUMENT = 3,
   HYLE_HIP_RESOURCE_EXHAUSTED = 8,
   HYLE_HIP_FAILED_PRECONDITION = 9,

@@ -10,10 +10,12 @@
  * (src/compute_stream_cuda/file_stream.cc:8-21 over CopyBatchProgram /
  * CopyBatchInvocation, include/hyle/compute/batch_transfer.h:30-140).  This
  * header is the HIP counterpart of the endpoint (hyle_hip_copy_batch_submit)
- * plus a small, synchronous-IO staging loop over it (hyle_hip_file_pipeline_*)
- * for callers that do not run the reference's streamer.  Leases, tickets,
- * cancellation and the write direction of the reference's streamer are not
- * part of this surface.
+ * plus a staging loop over it (hyle_hip_file_pipeline_*) for callers that do not
+ * run the reference's streamer: both directions (file -> device and device ->
+ * file), run on the calling thread or behind a ticket on a thread of the
+ * pipeline, with cooperative cancellation at slot boundaries and the progress
+ * made so far reported either way.  The reference's leases, budgets and ready
+ * groups are its streamer's own and are not part of this surface.
  */
 #ifndef HYLE_HIP_STREAM_H_
 #define HYLE_HIP_STREAM_H_
@@ -82,9 +84,20 @@ typedef struct hyle_hip_stream_result {
   uint32_t io_calls;     /* pread calls */
   uint32_t native_calls; /* device copies enqueued */
   uint32_t host_waits;   /* waits for a staging slot still in flight */
+  uint64_t written_bytes; /* bytes written to the file (write direction) */
+  uint32_t complete;      /* 1 once the request has ended, successfully or not */
 } hyle_hip_stream_result;
 
+/* StreamWriteRange::ready (include/hyle/compute/file_stream.h:92-105): `bytes` at the
+ * device address `source` go to `file_offset` of the file. */
+typedef struct hyle_hip_write_range {
+  const void *source;
+  uint64_t file_offset;
+  size_t bytes;
+} hyle_hip_write_range;
+
 typedef struct hyle_hip_file_pipeline hyle_hip_file_pipeline;
+typedef struct hyle_hip_stream_ticket hyle_hip_stream_ticket;
 
 /* cuda::create_file_pipeline (src/compute_stream_cuda/file_stream.cc:8-21):
  * binds the context's device and allocates the pinned staging slots. */
@@ -108,6 +121,46 @@ HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_read(hyle_hip_file_pipeline 
 /* StreamTicket::wait (include/hyle/compute/file_stream.h:171): block until
  * every copy this pipeline enqueued has finished. */
 HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_wait(hyle_hip_file_pipeline *pipeline);
+
+/* The write direction (FileResourcePipeline::write, include/hyle/compute/file_stream.h:205-206;
+ * src/compute_stream/file_stream.cc:519-560): every range goes from device memory through
+ * the pinned slots to the open file `fd` (pwrite).  The device-to-host copies are
+ * enqueued on `stream`, so they are ordered after whatever produced the data there;
+ * the copy of one slot overlaps the file write of another.  Returns when the last byte
+ * has been written.  A short write or an IO error is INTERNAL. */
+HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_write(hyle_hip_file_pipeline *pipeline, int fd,
+                                                          const hyle_hip_write_range *ranges,
+                                                          uint32_t range_count, void *stream,
+                                                          hyle_hip_stream_result *result);
+
+/* StreamTicket (include/hyle/compute/file_stream.h:158-180; FileResourcePipeline::read and
+ * ::write return one, :203-206): the same two requests
+ * run on a thread of the pipeline; the call returns at once with a ticket.  One request
+ * (with or without a ticket) runs on a pipeline at a time: a second one is
+ * FAILED_PRECONDITION.  The ranges are copied; the file must stay open and the device
+ * memory alive until the ticket has ended. */
+HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_submit_read(hyle_hip_file_pipeline *pipeline, int fd,
+                                                                const hyle_hip_read_range *ranges,
+                                                                uint32_t range_count, void *stream,
+                                                                hyle_hip_stream_ticket **ticket);
+HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_submit_write(hyle_hip_file_pipeline *pipeline, int fd,
+                                                                 const hyle_hip_write_range *ranges,
+                                                                 uint32_t range_count, void *stream,
+                                                                 hyle_hip_stream_ticket **ticket);
+/* StreamTicket::result: the progress so far, without waiting (`complete` says whether the
+ * request has ended). */
+HYLE_HIP_API hyle_hip_status hyle_hip_stream_ticket_result(hyle_hip_stream_ticket *ticket,
+                                                           hyle_hip_stream_result *result);
+/* StreamTicket::wait: block until the request has ended and, for a read, until its copies
+ * have finished on the device; returns the request's status. */
+HYLE_HIP_API hyle_hip_status hyle_hip_stream_ticket_wait(hyle_hip_stream_ticket *ticket,
+                                                         hyle_hip_stream_result *result);
+/* StreamTicket::request_cancel: cooperative, honoured at the next slot boundary; the
+ * request then ends with HYLE_HIP_CANCELLED (1) and the progress it had made.  Work
+ * already enqueued on the device is not recalled. */
+HYLE_HIP_API void hyle_hip_stream_ticket_request_cancel(hyle_hip_stream_ticket *ticket);
+/* Waits for the request to end (after asking it to cancel) and frees the ticket. */
+HYLE_HIP_API void hyle_hip_stream_ticket_release(hyle_hip_stream_ticket *ticket);
 
 #ifdef __cplusplus
 }

@@ -27,7 +27,8 @@ CTX = hc.Context.planning_only()
 
 
 def test_library_exports_every_declared_symbol():
-    text = open(HEADER).read() + open(os.path.join(ROOT, "include", "hyle_hip_stream.h")).read()
+    text = "".join(open(os.path.join(ROOT, "include", name)).read()
+                   for name in ("hyle_hip.h", "hyle_hip_stream.h", "hyle_hip_backend.h"))
     declared = set(re.findall(r"HYLE_HIP_API\s+[\w\s\*]+?\b(hyle_hip_\w+)\s*\(", text))
     assert declared, "no declarations parsed"
     lib = capi.load()
@@ -309,3 +310,24 @@ def test_stream_abi_is_exported_and_validates_without_a_device():
     with pytest.raises(hc.StatusError) as err:
         fs.submit_copy_batch(CTX, [fs.CopyPhase()], [], 0)
     assert err.value.is_invalid_argument()
+
+
+def test_backend_and_stream_calls_reject_bad_arguments_without_a_device():
+    """include/hyle_hip_backend.h, include/hyle_hip_stream.h: argument errors are reported before
+    anything touches a device."""
+    lib = capi.load()
+    count = C.c_size_t(99)
+    assert lib.hyle_hip_backend_device_count(C.byref(count)) in (capi.OK, capi.UNAVAILABLE)
+    assert lib.hyle_hip_backend_device_count(None) == capi.INVALID_ARGUMENT
+    handle = C.c_void_p()
+    assert lib.hyle_hip_memory_resource_create(None, 0, C.byref(handle)) == capi.INVALID_ARGUMENT
+    assert lib.hyle_hip_queue_create(None, None, C.byref(handle)) == capi.INVALID_ARGUMENT
+    assert lib.hyle_hip_queue_begin_sequence(None, C.byref(handle)) == capi.INVALID_ARGUMENT
+    assert lib.hyle_hip_queue_copy_async(None, None, None, None, None, 16) == capi.INVALID_ARGUMENT
+    assert lib.hyle_hip_completion_wait(None) == capi.INVALID_ARGUMENT
+    assert lib.hyle_hip_file_pipeline_write(None, 0, None, 0, None, None) == capi.INVALID_ARGUMENT
+    assert lib.hyle_hip_file_pipeline_submit_read(None, 0, None, 0, None, C.byref(handle)) == capi.INVALID_ARGUMENT
+    assert lib.hyle_hip_stream_ticket_wait(None, None) == capi.INVALID_ARGUMENT
+    lib.hyle_hip_stream_ticket_release(None)
+    lib.hyle_hip_completion_release(None)
+    assert lib.hyle_hip_status_name(capi.CANCELLED) == b"CANCELLED"
