@@ -154,11 +154,13 @@ struct TopKParams {
   bool largest = true;
   bool dense_last = false;  // dense tensor, axis innermost
   bool bytewise = false;    // strides that are not multiples of the element size
+  bool integer = false;     // int32 elements (the Elem passed to launch_topk is then ignored)
   int32_t rank = 0, axis = 0;
   uint32_t dims[kMaxRank] = {};
   int64_t strides[kMaxRank] = {};
   // set by topk_plan
   bool select = false;           // count small enough for the register-resident selection
+  bool runs = false;             // count above 1024: whole sorted tiles merged as runs, two at a time
   uint32_t tile_elements = 0;    // elements of a row one block of the first dispatch takes
   uint32_t tiles = 1, fan = 2, dispatches = 1;
   size_t workspace_bytes = 0;

@@ -862,8 +862,9 @@ hyle_hip_status admit(hyle_hip_plan *p) {
     case HYLE_HIP_OP_TOP_K: {
       // include/hyle/compute/providers/cuda.h:113-117: plain rank <= 8 byte strides, dense
       // outputs, no aliases, caller-owned workspace.
-      if (!to_elem(in[0].dtype, &p->elem) || !is_plain(in[0]))
-        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK requires plain float32/float16/bfloat16");
+      const bool integer = in[0].dtype == HYLE_HIP_DTYPE_I32;
+      if ((!integer && !to_elem(in[0].dtype, &p->elem)) || !is_plain(in[0]))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK requires plain float32/float16/bfloat16/int32");
       int axis;
       if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
       if (p->input_elements[0] > kMaxElements)
@@ -872,7 +873,7 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       bool innermost = is_dense(in[0]);  // dense, and nothing but extent-1 axes after the axis
       for (int a = axis + 1; a < in[0].rank; ++a)
         if (in[0].dims[a] != 1) innermost = false;
-      if (r.count == 1 && r.largest && innermost) {
+      if (r.count == 1 && r.largest && innermost && !integer) {
         // the vocabulary argmax: a scan dispatch and a fold dispatch
         p->route = Route::kArgmax;
         argmax_plan(p->output_elements[0], (uint32_t)in[0].dims[axis], p->elem, &p->argmax);
@@ -881,10 +882,9 @@ hyle_hip_status admit(hyle_hip_plan *p) {
         p->dispatches = 2;
         return HYLE_HIP_OK;
       }
-      if (r.count > topk_max_count())
-        return fail(HYLE_HIP_UNIMPLEMENTED, "TopK serves count <= %u", topk_max_count());
       TopKParams &t = p->topk;
       t = TopKParams{};
+      t.integer = integer;
       t.count = (uint32_t)r.count;
       t.rows = (uint32_t)(p->output_elements[0] / r.count);
       t.width = (uint32_t)in[0].dims[axis];

@@ -21,6 +21,7 @@
 // little more than k -- go to LDS to be sorted.  When more than 2048 keys reach it (ordered
 // data can do that) the exact k-th key is found bit by bit with block-wide counts instead.
 #include <algorithm>
+#include <type_traits>
 
 #include "device_common.h"
 #include "kernels.h"
@@ -51,9 +52,20 @@ __device__ __forceinline__ int64_t row_base(const Addressing &a, uint32_t row, u
   return base;
 }
 
+// Element types: the three float storage types and int32 (include/hyle/compute/providers/cuda.h:108-121).
+struct I32 {};
+template <class T> struct KeyTraits {
+  static constexpr int kSize = Traits<T>::kSize;
+  static constexpr int kVec = Traits<T>::kVec;
+};
+template <> struct KeyTraits<I32> {
+  static constexpr int kSize = 4;
+  static constexpr int kVec = 4;
+};
+
 template <class T, bool kBytewise>
 __device__ __forceinline__ uint32_t load_bits(const char *p) {
-  constexpr int kSize = Traits<T>::kSize;
+  constexpr int kSize = KeyTraits<T>::kSize;
   if constexpr (kBytewise) {
     uint32_t bits = 0;
 #pragma unroll
@@ -66,22 +78,43 @@ __device__ __forceinline__ uint32_t load_bits(const char *p) {
   }
 }
 template <class T> __device__ __forceinline__ float bits_value(uint32_t bits) {
-  if constexpr (Traits<T>::kSize == 4) return bits_f32(bits);
+  if constexpr (KeyTraits<T>::kSize == 4) return bits_f32(bits);
   else {
     const uint16_t narrow = (uint16_t)bits;
     return Traits<T>::load(&narrow, 0);
   }
 }
 
-// Larger key = better.  NaN keys (ordered part 0) sit below every number; 0 is no element.
-__device__ __forceinline__ uint64_t make_key(float v, uint32_t index, bool largest) {
-  uint32_t ordered = 0;
-  if (v == v) {
-    const uint32_t bits = v == 0.0f ? 0u : f32_bits(v);
-    ordered = (bits & 0x80000000u) ? ~bits : (bits ^ 0x80000000u);
-    if (!largest) ordered = ~ordered;
+// The ordered half of a key from an element's storage bits: larger = better.  A NaN is 0 and
+// sits below every number; -0 and +0 are one value.  int32 orders as a signed integer.
+__device__ __forceinline__ uint32_t ordered_value(float v, bool largest) {
+  if (v != v) return 0;
+  const uint32_t bits = v == 0.0f ? 0u : f32_bits(v);
+  const uint32_t ordered = bits ^ ((uint32_t)((int32_t)bits >> 31) | 0x80000000u);
+  return largest ? ordered : ~ordered;
+}
+template <class T> __device__ __forceinline__ uint32_t ordered_bits(uint32_t bits, bool largest) {
+  if constexpr (std::is_same<T, I32>::value) {
+    const uint32_t ordered = bits ^ 0x80000000u;
+    return largest ? ordered : ~ordered;
+  } else {
+    return ordered_value(bits_value<T>(bits), largest);
   }
-  return ((uint64_t)ordered << 32) | (uint32_t)~index;
+}
+// The storage bits of the kVec elements of a 16-byte vector.
+template <class T> __device__ __forceinline__ void vector_bits(u32x4 raw, uint32_t (&bits)[KeyTraits<T>::kVec]) {
+  const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+  if constexpr (KeyTraits<T>::kSize == 4) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) bits[j] = words[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) bits[j] = (words[j / 2] >> (16 * (j % 2))) & 0xFFFFu;
+  }
+}
+// A whole key: 0 is no element.
+template <class T> __device__ __forceinline__ uint64_t make_key(uint32_t bits, uint32_t index, bool largest) {
+  return ((uint64_t)ordered_bits<T>(bits, largest) << 32) | (uint32_t)~index;
 }
 
 // Descending bitonic sort of keys[0 .. n), n a power of two <= kTile; every thread of the block.
@@ -108,7 +141,7 @@ __device__ __forceinline__ void sort_descending(uint64_t *keys, uint32_t n) {
 template <class T, bool kBytewise, bool kFinal>
 __device__ __forceinline__ void emit(const uint64_t *keys, const Addressing &a, uint32_t row,
                                      const char *x, void *values, int32_t *indices, uint64_t *list) {
-  constexpr int kSize = Traits<T>::kSize;
+  constexpr int kSize = KeyTraits<T>::kSize;
   if constexpr (kFinal) {
     const int64_t base = row_base(a, row, kSize);
     const int64_t step = a.dense_last ? kSize : a.strides[a.axis];
@@ -133,8 +166,8 @@ template <class T, bool kVector, bool kBytewise, bool kFinal>
 __global__ __launch_bounds__(kBlockThreads) void topk_tiles(const char *x, void *values, int32_t *indices,
                                                             uint64_t *lists, Addressing a, uint32_t tiles,
                                                             uint32_t sort_n, uint32_t largest) {
-  constexpr int kSize = Traits<T>::kSize;
-  constexpr int kVec = Traits<T>::kVec;
+  constexpr int kSize = KeyTraits<T>::kSize;
+  constexpr int kVec = KeyTraits<T>::kVec;
   __shared__ uint64_t keys[kTile];
   const uint32_t row = blockIdx.x / tiles, tile = blockIdx.x - row * tiles;
   const uint32_t first = tile * kTile;
@@ -145,10 +178,10 @@ __global__ __launch_bounds__(kBlockThreads) void topk_tiles(const char *x, void 
     for (uint32_t v = threadIdx.x; v < sort_n / kVec; v += kBlockThreads) {
       const uint32_t element = first + v * kVec;
       if (element < a.width) {
-        float f[kVec];
-        Traits<T>::unpack(__builtin_nontemporal_load(vectors + element / kVec), f);
+        uint32_t bits[kVec];
+        vector_bits<T>(__builtin_nontemporal_load(vectors + element / kVec), bits);
 #pragma unroll
-        for (int j = 0; j < kVec; ++j) keys[v * kVec + j] = make_key(f[j], element + j, largest != 0);
+        for (int j = 0; j < kVec; ++j) keys[v * kVec + j] = make_key<T>(bits[j], element + j, largest != 0);
       } else {
 #pragma unroll
         for (int j = 0; j < kVec; ++j) keys[v * kVec + j] = 0;
@@ -159,8 +192,7 @@ __global__ __launch_bounds__(kBlockThreads) void topk_tiles(const char *x, void 
     for (uint32_t i = threadIdx.x; i < sort_n; i += kBlockThreads) {
       const uint32_t element = first + i;
       keys[i] = element < a.width
-                    ? make_key(bits_value<T>(load_bits<T, kBytewise>(x + base + (int64_t)element * step)),
-                               element, largest != 0)
+                    ? make_key<T>(load_bits<T, kBytewise>(x + base + (int64_t)element * step), element, largest != 0)
                     : 0;
     }
   }
@@ -184,6 +216,75 @@ __global__ __launch_bounds__(kBlockThreads) void topk_merge(const char *x, void 
   sort_descending(keys, sort_n);
   emit<T, kBytewise, kFinal>(keys, a, row, x, values, indices,
                              out_lists + ((size_t)row * lists_out + group) * a.count);
+}
+
+// ---- counts above kTile / 2: whole sorted tiles, merged two runs at a time -------------------
+// A run is a descending list of keys padded with zeros (no element) to a whole number of tiles.
+// One block writes kTile keys of the merged run: a binary search along its diagonal (merge path)
+// finds how many of the keys before its window come from each input run; the two windows, the
+// second one reversed, form a bitonic sequence of 2 * kTile keys that one bitonic merge puts in
+// order; its first half is the block's output.
+__global__ __launch_bounds__(kBlockThreads) void topk_merge_runs(const uint64_t *in, uint64_t *out, uint32_t runs_in,
+                                                                uint32_t run_in_keys, uint32_t runs_out,
+                                                                uint32_t run_out_keys) {
+  __shared__ uint64_t keys[2 * kTile];
+  __shared__ uint32_t split;
+  const uint32_t chunks = run_out_keys / kTile;
+  const uint32_t chunk = blockIdx.x % chunks, run = (blockIdx.x / chunks) % runs_out, row = blockIdx.x / (chunks * runs_out);
+  const uint64_t *a = in + ((size_t)row * runs_in + 2 * run) * run_in_keys;
+  const bool paired = 2 * run + 1 < runs_in;
+  const uint64_t *b = a + run_in_keys;  // read only when paired
+  const uint32_t length_a = run_in_keys, length_b = paired ? run_in_keys : 0;
+  const uint32_t diagonal = chunk * kTile;
+  if (threadIdx.x == 0) {
+    uint32_t low = diagonal > length_b ? diagonal - length_b : 0, high = diagonal < length_a ? diagonal : length_a;
+    while (low < high) {
+      const uint32_t mid = (low + high) / 2;  // mid keys of a and diagonal - mid of b before the window?
+      if (a[mid] > b[diagonal - mid - 1]) low = mid + 1;  // a[mid] outranks the last key taken from b: take more of a
+      else high = mid;
+    }
+    split = low;
+  }
+  __syncthreads();
+  const uint32_t from_a = split, from_b = diagonal - split;
+  for (uint32_t i = threadIdx.x; i < kTile; i += kBlockThreads) {
+    keys[i] = from_a + i < length_a ? a[from_a + i] : 0;
+    keys[2 * kTile - 1 - i] = from_b + i < length_b ? b[from_b + i] : 0;
+  }
+  for (uint32_t stride = kTile; stride > 0; stride >>= 1) {
+    __syncthreads();
+    for (uint32_t pair = threadIdx.x; pair < kTile; pair += kBlockThreads) {
+      const uint32_t lo = 2 * pair - (pair & (stride - 1)), hi = lo + stride;
+      const uint64_t first = keys[lo], second = keys[hi];
+      if (first < second) {
+        keys[lo] = second;
+        keys[hi] = first;
+      }
+    }
+  }
+  __syncthreads();
+  uint64_t *target = out + ((size_t)row * runs_out + run) * run_out_keys + diagonal;
+  for (uint32_t i = threadIdx.x; i < kTile; i += kBlockThreads) target[i] = keys[i];
+}
+
+// The first `count` keys of every row's single run -> the two outputs.
+template <class T, bool kBytewise>
+__global__ __launch_bounds__(kBlockThreads) void topk_emit_run(const char *x, void *values, int32_t *indices,
+                                                              const uint64_t *runs, Addressing a, uint32_t run_keys,
+                                                              uint32_t blocks_per_row) {
+  constexpr int kSize = KeyTraits<T>::kSize;
+  const uint32_t row = blockIdx.x / blocks_per_row;
+  const uint32_t j = (blockIdx.x % blocks_per_row) * kBlockThreads + threadIdx.x;
+  if (j >= a.count) return;
+  const int64_t base = row_base(a, row, kSize);
+  const int64_t step = a.dense_last ? kSize : a.strides[a.axis];
+  const uint32_t outer = row / a.inner, position = row - outer * a.inner;
+  const uint32_t index = min(~(uint32_t)runs[(size_t)row * run_keys + j], a.width - 1);
+  const uint32_t bits = load_bits<T, kBytewise>(x + base + (int64_t)index * step);
+  const size_t at = ((size_t)outer * a.count + j) * a.inner + position;
+  if constexpr (kSize == 4) static_cast<uint32_t *>(values)[at] = bits;
+  else static_cast<uint16_t *>(values)[at] = (uint16_t)bits;
+  indices[at] = (int32_t)index;
 }
 
 constexpr uint32_t kSelectMax = kBlockThreads;  // largest count the select route serves
@@ -211,14 +312,6 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t v, uint32_t *w
   return before + inclusive - v;
 }
 
-// The ordered half of a key alone: enough for nearly every comparison of the select kernel.
-__device__ __forceinline__ uint32_t ordered_value(float v, bool largest) {
-  if (v != v) return 0;
-  const uint32_t bits = v == 0.0f ? 0u : f32_bits(v);
-  const uint32_t ordered = bits ^ ((uint32_t)((int32_t)bits >> 31) | 0x80000000u);
-  return largest ? ordered : ~ordered;
-}
-
 // One block per (row, unit).  kFromLists = false: unit = a tile of 256 * kE elements of the row.
 // kFromLists = true: unit = a group of `fan` lists of `count` keys left by an earlier dispatch.
 // A thread keeps its kE keys as two words, hi (ordered value) and lo (~index; the compiler
@@ -228,8 +321,8 @@ __global__ __launch_bounds__(kBlockThreads) void topk_select(const char *x, void
                                                              const uint64_t *in_lists, uint64_t *out_lists,
                                                              Addressing a, uint32_t units_in, uint32_t fan,
                                                              uint32_t units_out, uint32_t largest) {
-  constexpr int kSize = Traits<T>::kSize;
-  constexpr int kVec = Traits<T>::kVec;
+  constexpr int kSize = KeyTraits<T>::kSize;
+  constexpr int kVec = KeyTraits<T>::kVec;
   __shared__ uint64_t keys[kTile];  // kBlockThreads < kTile / 2: keys[kBlockThreads] is free for the bound
   __shared__ uint32_t wave_totals[kBlockThreads / kWaveLanes];
   const uint32_t row = blockIdx.x / units_out, unit = blockIdx.x - row * units_out;
@@ -264,11 +357,11 @@ __global__ __launch_bounds__(kBlockThreads) void topk_select(const char *x, void
       for (int v = 0; v < kE / kVec; ++v) {
         const uint32_t element = first + (threadIdx.x + v * kBlockThreads) * kVec;
         const bool inside = element < a.width;
-        float f[kVec];
-        Traits<T>::unpack(raw[v], f);
+        uint32_t bits[kVec];
+        vector_bits<T>(raw[v], bits);
 #pragma unroll
         for (int j = 0; j < kVec; ++j) {
-          hi[v * kVec + j] = inside ? ordered_value(f[j], largest != 0) : 0;
+          hi[v * kVec + j] = inside ? ordered_bits<T>(bits[j], largest != 0) : 0;
           lo[v * kVec + j] = inside ? ~(element + j) : 0;
         }
       }
@@ -285,7 +378,7 @@ __global__ __launch_bounds__(kBlockThreads) void topk_select(const char *x, void
       for (int j = 0; j < kE; ++j) {
         const uint32_t element = first + threadIdx.x + j * kBlockThreads;
         const bool inside = element < a.width;
-        hi[j] = inside ? ordered_value(bits_value<T>(bits[j]), largest != 0) : 0;
+        hi[j] = inside ? ordered_bits<T>(bits[j], largest != 0) : 0;
         lo[j] = inside ? ~element : 0;
       }
     }
@@ -459,7 +552,7 @@ hipError_t run(const TopKParams &p, const void *x, void *values, int32_t *indice
   const uint32_t largest = p.largest ? 1u : 0u;
   const uint32_t tile_n = pow2_at_least(std::min(p.width, kTile), 64);
   const dim3 block(kBlockThreads);
-  vector = vector && p.dense_last && p.width % Traits<T>::kVec == 0;
+  vector = vector && p.dense_last && p.width % KeyTraits<T>::kVec == 0;
   if (p.select) {
     if (p.tile_elements == kBlockThreads * 64)
       select_tiles_launch<T, 64, kBytewise>(p, a, in, values, indices, lists_a, vector, s);
@@ -478,6 +571,32 @@ hipError_t run(const TopKParams &p, const void *x, void *values, int32_t *indice
       std::swap(from, to);
       lists = out;
     }
+    return hipGetLastError();
+  }
+  if (p.runs && p.tiles > 1) {
+    // whole tiles sorted (every key kept), then runs merged in pairs until one is left per row
+    Addressing whole = a;
+    whole.count = kTile;
+    uint64_t *from = lists_a, *to = lists_a + (size_t)p.rows * p.tiles * kTile;
+    if (vector)
+      hipLaunchKernelGGL((topk_tiles<T, true, false, false>), dim3(p.rows * p.tiles), block, 0, s, in, values, indices,
+                         from, whole, p.tiles, kTile, largest);
+    else
+      hipLaunchKernelGGL((topk_tiles<T, false, kBytewise, false>), dim3(p.rows * p.tiles), block, 0, s, in, values,
+                         indices, from, whole, p.tiles, kTile, largest);
+    const uint32_t limit = (p.count + kTile - 1) / kTile * kTile;  // no run needs more keys than this
+    uint32_t runs = p.tiles, run_keys = kTile;
+    while (runs > 1) {
+      const uint32_t runs_out = (runs + 1) / 2, out_keys = std::min(2 * run_keys, limit);
+      hipLaunchKernelGGL(topk_merge_runs, dim3(p.rows * runs_out * (out_keys / kTile)), block, 0, s, from, to, runs,
+                         run_keys, runs_out, out_keys);
+      std::swap(from, to);
+      runs = runs_out;
+      run_keys = out_keys;
+    }
+    const uint32_t blocks_per_row = (p.count + kBlockThreads - 1) / kBlockThreads;
+    hipLaunchKernelGGL((topk_emit_run<T, kBytewise>), dim3(p.rows * blocks_per_row), block, 0, s, in, values, indices,
+                       from, a, run_keys, blocks_per_row);
     return hipGetLastError();
   }
   if (p.tiles == 1) {
@@ -514,7 +633,7 @@ hipError_t run(const TopKParams &p, const void *x, void *values, int32_t *indice
 
 }  // namespace
 
-uint32_t topk_max_count() { return kTile / 2; }
+uint32_t topk_max_count() { return kTile / 2; }  // above it: sorted runs merged in pairs
 
 void topk_plan(TopKParams *p) {
   p->select = p->count <= kSelectMax;
@@ -529,10 +648,18 @@ void topk_plan(TopKParams *p) {
   } else {
     p->tile_elements = kTile;
     p->tiles = (p->width + kTile - 1) / kTile;
-    p->fan = kTile / p->count;  // >= 2 for count <= kTile / 2
+    p->runs = p->count > kTile / 2;
+    p->fan = p->runs ? 2 : kTile / p->count;  // >= 2 for count <= kTile / 2
   }
   p->dispatches = 1;
   p->workspace_bytes = 0;
+  if (p->runs && p->tiles > 1) {
+    // sorted tiles, merges of pairs of runs, one dispatch for the outputs; two buffers of whole tiles
+    for (uint32_t runs = p->tiles; runs > 1; runs = (runs + 1) / 2) ++p->dispatches;
+    ++p->dispatches;
+    p->workspace_bytes = 2 * (size_t)p->rows * p->tiles * kTile * sizeof(uint64_t);
+    return;
+  }
   if (p->tiles > 1) {
     uint32_t lists = p->tiles;
     while (lists > 1) {
@@ -548,6 +675,9 @@ void topk_plan(TopKParams *p) {
 hipError_t launch_topk(Elem type, const TopKParams &p, const void *x, void *values, int32_t *indices,
                        void *workspace, bool input_vector_aligned, hipStream_t stream) {
   if (p.rows == 0 || p.count == 0) return hipSuccess;
+  if (p.integer)
+    return p.bytewise ? run<I32, true>(p, x, values, indices, workspace, false, stream)
+                      : run<I32, false>(p, x, values, indices, workspace, input_vector_aligned, stream);
   switch (type) {
     case Elem::kF32:
       return p.bytewise ? run<F32, true>(p, x, values, indices, workspace, false, stream)

@@ -180,7 +180,7 @@ typedef struct hyle_hip_op_desc {
   uint32_t keep_dimensions;  /* Reduce */
   float epsilon;             /* RmsNorm, LayerNorm */
   float scale;               /* Softmax */
-  uint64_t count;            /* TopK count (counts above 1024 are declined) */
+  uint64_t count;            /* TopK count */
   uint32_t largest;          /* TopK: 1 = largest first, 0 = smallest first */
   uint32_t input_count;
   hyle_hip_tensor_desc inputs[HYLE_HIP_MAX_INPUTS];

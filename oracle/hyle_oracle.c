@@ -88,7 +88,7 @@ uint16_t hyle_oracle_f32_to_bf16(float f) {
 }
 
 static inline size_t type_size(int type) {
-  return type == HYLE_ORACLE_F32 ? 4u : 2u;
+  return type == HYLE_ORACLE_F32 || type == HYLE_ORACLE_I32 ? 4u : 2u;
 }
 
 /* src/compute_provider_native/numeric.h:13-47 (decode / encode / load / store) */
@@ -794,7 +794,7 @@ void hyle_oracle_topk1_f32(const float *data, size_t rows, size_t width,
  * Outputs are dense with the axis extent replaced by k
  * (src/compute_ops/operation.cc:1622-1657). */
 typedef struct {
-  float value;
+  double value;  /* a float widened exactly, or an int32 */
   int32_t index;
 } topk_item;
 static int g_topk_largest;
@@ -829,7 +829,14 @@ void hyle_oracle_topk(int type, const void *src, int rank, const int64_t *dims,
       remaining /= (size_t)dims[a];
     }
     for (size_t i = 0; i < width; ++i) {
-      items[i].value = load_as_f32(type, s + base + (int64_t)i * byte_strides[axis]);
+      const unsigned char *at = s + base + (int64_t)i * byte_strides[axis];
+      if (type == HYLE_ORACLE_I32) {
+        int32_t whole;
+        memcpy(&whole, at, sizeof whole);
+        items[i].value = (double)whole;
+      } else {
+        items[i].value = (double)load_as_f32(type, at);
+      }
       items[i].index = (int32_t)i;
     }
     qsort(items, width, sizeof(topk_item), topk_before);  /* a total order: index breaks ties */

@@ -114,7 +114,9 @@ HOST_TEST(PreparesRoutesAndDeclinesCleanly) {
   auto top4 = prepare(context, TopK{.count = 4}, dense(DataType::kFloat32, {8, 128}));
   REQUIRE(top4.has_value());
   EXPECT(std::string(top4->route_name()) == "topk-select-tiles" && top4->workspace_requirement().size == 0);
-  EXPECT(prepare(context, TopK{.count = 1025}, dense(DataType::kFloat32, {8, 4096})).error().IsUnimplemented());
+  EXPECT(prepare(context, TopK{.count = 1025}, dense(DataType::kFloat32, {8, 4096})).has_value());
+  EXPECT(prepare(context, TopK{.count = 3}, dense(DataType::kInt32, {8, 4096})).has_value());
+  EXPECT(prepare(context, TopK{.count = 3}, dense(DataType::kUInt8, {8, 4096})).error().IsUnimplemented());
   auto folded = prepare(context, Reduce{ReductionKind::kSum, *Axes::from(std::array<std::int32_t, 2>{0, 2})},
                         dense(DataType::kFloat32, {4, 5, 6}));
   REQUIRE(folded.has_value());

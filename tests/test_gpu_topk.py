@@ -143,11 +143,10 @@ def test_topk_schema_and_admission():
         hc.infer_output_descriptions(hc.TopK(count=5001), [x])
     assert err.value.is_out_of_range()
     with pytest.raises(hc.StatusError) as err:
-        hc.prepare(context(), hc.TopK(count=1025), x)
+        hc.prepare(context(), hc.TopK(count=2), D(DT.kUInt8, [4, 50]))
     assert err.value.is_unimplemented()
-    with pytest.raises(hc.StatusError) as err:
-        hc.prepare(context(), hc.TopK(count=2), D(DT.kInt32, [4, 50]))
-    assert err.value.is_unimplemented()
+    assert hc.prepare(context(), hc.TopK(count=1025), x).route_name() == "topk-sorted-tiles"
+    assert hc.prepare(context(), hc.TopK(count=1), D(DT.kInt32, [4, 5000])).route_name() == "topk-select-tiles"
     wide = hc.prepare(context(), hc.TopK(count=8), x)
     assert wide.route_name() == "topk-select-tiles" and wide.workspace_requirement().size == 0
     assert hc.prepare(context(), hc.TopK(count=8), D(DT.kFloat32, [4, 50000])).workspace_requirement().size > 0
@@ -157,3 +156,45 @@ def test_topk_schema_and_admission():
     note("topk count 0 writes nothing")
     values, indices = run(hc.TopK(count=0), torch.zeros((3, 9), device=DEVICE))
     assert list(values.shape) == [3, 0] and list(indices.shape) == [3, 0]
+
+
+def test_topk_counts_above_1024_merge_sorted_runs():
+    """Counts the selection and single-tile sorts do not reach: whole sorted tiles, merged as runs."""
+    rng = np.random.default_rng(1170)
+    for tag, dims, counts in (("f32", [3, 5000], (1025, 2048, 3000, 5000)), ("bf16", [2, 70001], (1500, 4097)),
+                              ("f32", [1, 300000], (2049, 20000)), ("f16", [5, 2049], (2049,)),
+                              ("f32", [2, 4100, 3], (4000,))):
+        stored = tied_values(rng, dims, tag)
+        axis = 1 if len(dims) == 3 else -1
+        for count in counts:
+            for largest in (True, False):
+                note(f"topk runs {tag} {dims} count {count} largest {largest}")
+                outputs = run(hc.TopK(count=count, axis=axis, largest=largest), to_device(stored, tag))
+                check(tag, stored, dims, count, axis, largest, outputs)
+    note("topk runs: distinct values, every key kept")
+    x = rng.permutation(40000).astype(np.float32).reshape(2, 20000)
+    values, indices = run(hc.TopK(count=20000), to_device(x, "f32"))
+    assert np.array_equal(to_host(values), -np.sort(-x, axis=1))
+    assert np.array_equal(np.take_along_axis(x, to_host(indices).astype(np.int64), 1), to_host(values))
+
+
+def test_topk_int32_keys():
+    """include/hyle/compute/providers/cuda.h:108-121 admits I32: signed integer order, lowest index
+    among equals, the extremes included."""
+    rng = np.random.default_rng(1171)
+    cases = (([4, 37], -1, (1, 5, 37)), ([3, 5000], -1, (1, 64, 300, 2000)), ([6, 9, 16], 1, (4,)), ([2, 70001], -1, (64, 1000)))
+    for dims, axis, counts in cases:
+        x = rng.integers(-50, 51, dims).astype(np.int32)                 # ties everywhere
+        flat = x.reshape(-1)
+        flat[rng.integers(0, flat.size, 5)] = np.iinfo(np.int32).min
+        flat[rng.integers(0, flat.size, 5)] = np.iinfo(np.int32).max
+        flat[rng.integers(0, flat.size, 7)] = rng.integers(-2**31, 2**31, 7)   # beyond what a float tells apart
+        for count in counts:
+            for largest in (True, False):
+                note(f"topk int32 {dims} axis {axis} count {count} largest {largest}")
+                values, indices = run(hc.TopK(count=count, axis=axis, largest=largest), torch.from_numpy(x).to(DEVICE))
+                want_values, want_indices = orc.topk(orc.I32, x, dims, count, axis, largest)
+                assert np.array_equal(to_host(indices), want_indices)
+                assert np.array_equal(to_host(values), want_values)
+                order = np.argsort(-x.astype(np.int64) if largest else x.astype(np.int64), axis=axis, kind="stable")
+                assert np.array_equal(np.take(order, range(count), axis=axis), want_indices)   # the oracle against numpy
