@@ -328,6 +328,19 @@ def main() -> int:
             return [src], [torch.empty_like(src)]
         ops.append(Op("next_copy_bf16", hc.Copy(), [D(BF, [8192, 6144])], set_copy, 3,
                       8192 * 6144 * 4, 8192 * 6144, "bf16", in_step=False))
+    if want("next_fill_bf16"):
+        def set_fill(i):
+            return [], [torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev)]
+        ops.append(Op("next_fill_bf16", hc.Fill((8192, 6144), BF, hc.ScalarValue.of(BF, 1.0)), [], set_fill, 3,
+                      8192 * 6144 * 2, 8192 * 6144, "bf16", in_step=False))
+    if want("next_select_bf16"):
+        # the masked residual: Bool mask, a full branch, a rank-0 zero (1 + 2 bytes read, 2 written per element)
+        def set_select(i):
+            mask = torch.empty((8192, 6144), dtype=torch.uint8, device=dev).random_(0, 2)
+            src = torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev).normal_()
+            return [mask, src, torch.zeros((), dtype=torch.bfloat16, device=dev)], [torch.empty_like(src)]
+        ops.append(Op("next_select_bf16", hc.Select(), [D(hc.DataType.kBool, [8192, 6144]), D(BF, [8192, 6144]), D(BF, [])],
+                      set_select, 3, 8192 * 6144 * 5, 8192 * 6144, "bf16", in_step=False))
     # ---- practical ceilings for launches of 38 / 67 MB: a plain copy and a plain read-only scan (a
     # row maximum, one wave per row, one dispatch) of the traffic of the step's small shapes, through
     # the same C ABI and rotated the same way.  Kernels of this size run for 6 - 12 us, of which the

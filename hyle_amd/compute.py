@@ -194,9 +194,11 @@ class TensorDesc:
 # ---- operations (include/hyle/compute/operation.h) -----------------------------------------
 class OperationKind(enum.IntEnum):
     kCopy = 2
+    kFill = 3
     kCast = 4
     kUnary = 5
     kBinary = 6
+    kSelect = 7
     kReduce = 8
     kRmsNorm = 9
     kLayerNorm = 10
@@ -265,6 +267,52 @@ class MaskKind(enum.IntEnum):
 @dataclass(frozen=True)
 class Copy:
     """Materialise any plain tensor (dense or strided) as a dense tensor of the same type."""
+
+
+@dataclass(frozen=True)
+class ScalarValue:
+    """Exact scalar payload of Fill (include/hyle/compute/operation.h:187-230): a type and the
+    element's bit pattern."""
+    data_type: DataType = DataType.kUnknown
+    bits: int = 0
+
+    @staticmethod
+    def of(data_type: DataType, value) -> "ScalarValue":
+        """The pattern the reference's typed constructors store; float16 / bfloat16 patterns
+        (from_bits there) are the nearest-even narrowing of `value`."""
+        import numpy as np
+        if data_type == DataType.kBool:
+            return ScalarValue(data_type, 1 if value else 0)
+        if data_type == DataType.kFloat32:
+            return ScalarValue(data_type, int(np.array(value, np.float32).view(np.uint32)))
+        if data_type == DataType.kFloat16:
+            return ScalarValue(data_type, int(np.array(value, np.float16).view(np.uint16)))
+        if data_type == DataType.kBFloat16:
+            word = int(np.array(value, np.float32).view(np.uint32))
+            if (word & 0x7FFFFFFF) > 0x7F800000:
+                return ScalarValue(data_type, (word >> 16) | 0x40)
+            return ScalarValue(data_type, ((word + 0x7FFF + ((word >> 16) & 1)) >> 16) & 0xFFFF)
+        size = data_type_size(data_type)
+        if size == 0:
+            raise StatusError(capi.INVALID_ARGUMENT, "Fill requires a valid shape and exactly typed scalar")
+        return ScalarValue(data_type, int(value) & ((1 << (8 * size)) - 1))
+
+    @staticmethod
+    def from_bits(data_type: DataType, bits: int) -> "ScalarValue":
+        return ScalarValue(data_type, bits)
+
+
+@dataclass(frozen=True)
+class Fill:
+    """No inputs: a dense tensor of `output_shape` whose every element is `value`."""
+    output_shape: tuple = ()
+    output_type: DataType = DataType.kUnknown
+    value: ScalarValue = ScalarValue()
+
+
+@dataclass(frozen=True)
+class Select:
+    """Inputs (condition Bool, first, second) broadcast together; first where the condition holds."""
 
 
 @dataclass(frozen=True)
@@ -393,6 +441,18 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
         c.op = OperationKind.kCopy
     elif isinstance(operation, Cast):
         c.op, c.kind = OperationKind.kCast, int(operation.output_type)
+    elif isinstance(operation, Fill):
+        # the scalar's type travels as the output type: they must agree (operation.cc:1263-1275)
+        shape = tuple(operation.output_shape)
+        if (operation.value.data_type != operation.output_type or len(shape) > capi.MAX_RANK
+                or any(d < 0 for d in shape) or inputs):
+            raise StatusError(capi.INVALID_ARGUMENT, "Fill requires a valid shape and exactly typed scalar")
+        c.op, c.kind, c.count = OperationKind.kFill, int(operation.output_type), operation.value.bits
+        c.inputs[0].rank = len(shape)
+        for i, d in enumerate(shape):
+            c.inputs[0].dims[i] = d
+    elif isinstance(operation, Select):
+        c.op = OperationKind.kSelect
     elif isinstance(operation, Unary):
         c.op, c.kind = OperationKind.kUnary, int(operation.kind)
     elif isinstance(operation, Binary):

@@ -221,4 +221,27 @@ struct CastParams {
 hipError_t launch_cast(const CastParams &p, const void *in, void *out, bool vectorised,
                        hipStream_t stream);
 
+// Fill: `elements` elements of `size` bytes (1, 2 or 4) set to the low bytes of `bits`.
+struct FillParams {
+  uint64_t elements = 0;
+  uint32_t bits = 0;
+  uint8_t size = 4;
+};
+hipError_t launch_fill(const FillParams &p, void *out, hipStream_t stream);
+
+// Select(condition Bool, first, second) -> dense output of `size`-byte elements.  flat: every
+// operand is dense and either as long as the output or one element (scalar[i]); otherwise byte
+// strides per output axis (0 where an operand is broadcast).
+struct SelectParams {
+  uint64_t elements = 0;
+  uint8_t size = 4;
+  bool flat = false;
+  bool scalar[3] = {false, false, false};
+  int32_t rank = 0;
+  uint32_t dims[kMaxRank] = {};
+  int64_t strides[3][kMaxRank] = {};
+};
+hipError_t launch_select(const SelectParams &p, const void *condition, const void *first, const void *second, void *out,
+                         bool vector_aligned, hipStream_t stream);
+
 }  // namespace hyle_hip

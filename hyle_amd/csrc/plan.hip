@@ -274,6 +274,27 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
         return fail(HYLE_HIP_UNIMPLEMENTED, "Copy handles plain dense/strided storage");
       return make_dense(in[0].dtype, in[0].dims, in[0].rank, &outs[0]);
     }
+    case HYLE_HIP_OP_FILL: {  // src/compute_ops/operation.cc:1263-1275
+      // no inputs: inputs[0] carries Fill::output_shape (rank, dims), kind the output type, which
+      // is also the scalar's type (the two are one field here, so they cannot differ)
+      if ((s = expect_inputs(r, 0, 0)) != HYLE_HIP_OK) return s;
+      const Desc &shape = r.inputs[0];
+      bool valid = shape.rank <= HYLE_HIP_MAX_RANK && r.kind <= 255 && dtype_size((uint8_t)r.kind) != 0;
+      for (int i = 0; valid && i < shape.rank; ++i) valid = shape.dims[i] >= 0;
+      if (!valid) return fail(HYLE_HIP_INVALID_ARGUMENT, "Fill requires a valid shape and exactly typed scalar");
+      return make_dense((uint8_t)r.kind, shape.dims, shape.rank, &outs[0]);
+    }
+    case HYLE_HIP_OP_SELECT: {  // src/compute_ops/operation.cc:1309-1330
+      if ((s = expect_inputs(r, 3, 3)) != HYLE_HIP_OK) return s;
+      if (in[0].dtype != HYLE_HIP_DTYPE_BOOL || in[1].dtype != in[2].dtype)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Select requires Bool condition and equal branch types");
+      int64_t branches[HYLE_HIP_MAX_RANK], dims[HYLE_HIP_MAX_RANK];
+      int branch_rank, rank;
+      if ((s = broadcast_shape(in[1].dims, in[1].rank, in[2].dims, in[2].rank, branches, &branch_rank)) != HYLE_HIP_OK)
+        return s;
+      if ((s = broadcast_shape(in[0].dims, in[0].rank, branches, branch_rank, dims, &rank)) != HYLE_HIP_OK) return s;
+      return make_dense(in[1].dtype, dims, rank, &outs[0]);
+    }
     case HYLE_HIP_OP_CAST: {  // src/compute_ops/operation.cc:1276-1285
       if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
       if (r.kind > 255 || dtype_size((uint8_t)r.kind) == 0 || !is_plain(in[0]))
@@ -486,6 +507,8 @@ enum class Route : uint8_t {
   kKQuantDequant,
   kGgufMatVec,
   kCast,
+  kFill,
+  kSelect,
 };
 
 const char *route_name(Route r) {
@@ -503,6 +526,8 @@ const char *route_name(Route r) {
     case Route::kKQuantDequant: return "k-quant-dequant-rows";
     case Route::kGgufMatVec: return "gguf-matvec-rows";
     case Route::kCast: return "cast-copy";
+    case Route::kFill: return "fill-pattern";
+    case Route::kSelect: return "select";
   }
   return "?";
 }
@@ -547,6 +572,8 @@ struct hyle_hip_plan {
   KQuantParams kquant;
   MatVecParams matvec;
   CastParams cast;
+  FillParams fill;
+  SelectParams select;
   // Cast and Copy take no alias at all (AliasPolicy::kNone, src/compute_ops/operation.cc:935-957):
   // the bytes the input and the output occupy must not overlap.
   uint64_t no_overlap_input_bytes = 0, no_overlap_output_bytes = 0;
@@ -966,6 +993,57 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }
+    case HYLE_HIP_OP_FILL: {
+      // storage only: the scalar's bits go to every element (src/compute_provider_cuda/
+      // tensor_provider.cc:85-98, tensor_kernel.cu:190-193)
+      const uint64_t n = p->output_elements[0];
+      if (n > kMaxElements) return fail(HYLE_HIP_UNIMPLEMENTED, "Fill output exceeds INT32_MAX elements");
+      if (n == 0) return HYLE_HIP_OK;
+      const size_t size = dtype_size(out.dtype);
+      if (size < 8 && (r.count >> (8 * size)) != 0)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Fill scalar bits do not fit the output type");
+      p->route = Route::kFill;
+      p->dispatches = 1;
+      p->fill.elements = n;
+      p->fill.bits = (uint32_t)r.count;
+      p->fill.size = (uint8_t)size;
+      return HYLE_HIP_OK;
+    }
+    case HYLE_HIP_OP_SELECT: {
+      // storage only, plain operands broadcast to a dense output (src/compute_provider_cuda/
+      // tensor_provider.cc:85-90,119-121,176-195; tensor_kernel.cu:194-198)
+      for (int i = 0; i < 3; ++i)
+        if (!is_plain(in[i])) return fail(HYLE_HIP_UNIMPLEMENTED, "Select requires plain storage");
+      const uint64_t n = p->output_elements[0];
+      if (n > kMaxElements) return fail(HYLE_HIP_UNIMPLEMENTED, "Select output exceeds INT32_MAX elements");
+      if (n == 0) return HYLE_HIP_OK;
+      // a branch whose descriptor is the output's may be written in place; the condition may not
+      for (int i = 1; i < 3; ++i)
+        if (same_desc(in[i], out)) p->alias_inputs[0] |= (uint8_t)(1u << i);
+      SelectParams &sel = p->select;
+      sel.elements = n;
+      sel.size = (uint8_t)dtype_size(out.dtype);
+      sel.flat = true;
+      for (int i = 0; i < 3; ++i) {
+        uint32_t period = 0;
+        sel.flat = sel.flat && suffix_period(in[i], out, n, &period) && period <= 1;
+        sel.scalar[i] = period == 1;
+      }
+      sel.rank = out.rank;
+      for (int a = 0; a < out.rank; ++a) sel.dims[a] = (uint32_t)out.dims[a];
+      for (int i = 0; i < 3; ++i) {
+        for (int rev = 0; rev < out.rank; ++rev) {
+          int64_t stride = 0;
+          if (rev < in[i].rank && in[i].dims[in[i].rank - 1 - rev] != 1) stride = in[i].byte_strides[in[i].rank - 1 - rev];
+          sel.strides[i][out.rank - 1 - rev] = stride;
+        }
+        // the strided kernel gathers bytes, so byte strides need not keep elements aligned
+        if (!sel.flat) p->input_alignment[i] = 1;
+      }
+      p->route = Route::kSelect;
+      p->dispatches = 1;
+      return HYLE_HIP_OK;
+    }
     case HYLE_HIP_OP_COPY:
     case HYLE_HIP_OP_CAST: {
       // src/compute_provider_native/cast.cc:127-176,256-279 (admitted pairs, plain input, dense
@@ -1227,7 +1305,7 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
   if (plan->route == Route::kNoOp) return HYLE_HIP_OK;  // zero elements: storage is never touched
   if (plan->context == nullptr)
     return fail(HYLE_HIP_FAILED_PRECONDITION, "plan was built without a device context");
-  if (inputs == nullptr || outputs == nullptr)
+  if ((inputs == nullptr && input_count != 0) || outputs == nullptr)
     return fail(HYLE_HIP_INVALID_ARGUMENT, "binding arrays are null");
   bool vector = true;
   for (uint32_t i = 0; i < input_count; ++i) {
@@ -1324,6 +1402,12 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
       break;
     case Route::kCast:
       err = launch_cast(plan->cast, inputs[0], outputs[0], vector, stream);
+      break;
+    case Route::kFill:
+      err = launch_fill(plan->fill, outputs[0], stream);
+      break;
+    case Route::kSelect:
+      err = launch_select(plan->select, inputs[0], inputs[1], inputs[2], outputs[0], vector, stream);
       break;
   }
   if (err != hipSuccess) return hip_fail(err, "kernel launch");

@@ -1,0 +1,186 @@
+// Fill and Select: the storage-only members of the reference's elementwise kernel family
+// (src/compute_provider_cuda/tensor_kernel.cu:168-199: Fill writes the scalar's bits to every
+// element, Select takes the second input where the Bool condition byte is non-zero and the third
+// elsewhere).  Elements are moved as 1-, 2- or 4-byte patterns whatever their type.
+#include "device_common.h"
+#include "kernels.h"
+
+namespace hyle_hip {
+namespace {
+
+// `pattern` is the element repeated to 32 bits; the output is element-aligned, so the pattern
+// reads the same at every address the element size divides.
+__global__ __launch_bounds__(kBlockThreads) void fill_pattern(unsigned char *out, uint64_t bytes, uint32_t pattern) {
+  const uint64_t lead = (16 - (reinterpret_cast<uintptr_t>(out) & 15u)) & 15u;
+  const uint64_t head = lead < bytes ? lead : bytes;
+  const uint64_t vectors = (bytes - head) / 16, tail_first = head + vectors * 16;
+  const uint64_t thread = (uint64_t)blockIdx.x * kBlockThreads + threadIdx.x, threads = (uint64_t)gridDim.x * kBlockThreads;
+  u32x4 word;
+  word.x = word.y = word.z = word.w = pattern;
+  for (uint64_t v = thread; v < vectors; v += threads) store16_stream(out + head, v, word);
+  auto byte_at = [&](uint64_t i) {  // the pattern byte that belongs at address out + i
+    return (unsigned char)(pattern >> (8 * ((reinterpret_cast<uintptr_t>(out) + i) & 3u)));
+  };
+  if (thread < head) out[thread] = byte_at(thread);
+  if (thread < bytes - tail_first) out[tail_first + thread] = byte_at(tail_first + thread);
+}
+
+// Operands of the flat Select kernel: as long as the output (period 0) or one element (period 1).
+struct SelectFlat {
+  const unsigned char *condition, *first, *second;
+  uint32_t condition_scalar, first_scalar, second_scalar;
+};
+
+// One 16-byte output vector per step: kVec = 16 / kSize elements, their condition bytes read as
+// one 4-, 8- or 16-byte word.  Requires 16-byte aligned full operands and elements % kVec == 0
+// for the vector part; the tail goes element by element.
+template <int kSize>
+__global__ __launch_bounds__(kBlockThreads) void select_flat(SelectFlat p, unsigned char *out, uint32_t vectors,
+                                                             uint32_t elements) {
+  constexpr int kVec = 16 / kSize;
+  const uint32_t thread = blockIdx.x * kBlockThreads + threadIdx.x, threads = gridDim.x * kBlockThreads;
+  auto element = [&](const unsigned char *base, uint32_t scalar, uint32_t index) -> uint32_t {
+    const unsigned char *at = base + (size_t)(scalar ? 0u : index) * kSize;
+    if constexpr (kSize == 4) return *reinterpret_cast<const uint32_t *>(at);
+    else if constexpr (kSize == 2) return *reinterpret_cast<const uint16_t *>(at);
+    else return *at;
+  };
+  const uint32_t splat_first = p.first_scalar ? element(p.first, 1, 0) : 0, splat_second = p.second_scalar ? element(p.second, 1, 0) : 0;
+  const bool whole = p.condition_scalar ? p.condition[0] != 0 : false;
+  for (uint32_t v = thread; v < vectors; v += threads) {
+    unsigned char take[kVec];
+    if (p.condition_scalar) {
+#pragma unroll
+      for (int j = 0; j < kVec; ++j) take[j] = whole;
+    } else if constexpr (kVec == 4) {
+      const uint32_t c = *reinterpret_cast<const uint32_t *>(p.condition + (size_t)v * 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) take[j] = ((c >> (8 * j)) & 0xFFu) != 0;
+    } else if constexpr (kVec == 8) {
+      const uint2 c = *reinterpret_cast<const uint2 *>(p.condition + (size_t)v * 8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) take[j] = (((j < 4 ? c.x : c.y) >> (8 * (j % 4))) & 0xFFu) != 0;
+    } else {
+      const u32x4 c = load16(p.condition, v);
+      const uint32_t words[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+      for (int j = 0; j < 16; ++j) take[j] = ((words[j / 4] >> (8 * (j % 4))) & 0xFFu) != 0;
+    }
+    auto vector_of = [&](const unsigned char *base, uint32_t scalar, uint32_t splat, uint32_t (&e)[kVec]) {
+      if (scalar) {
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) e[j] = splat;
+        return;
+      }
+      const u32x4 raw = load16_stream(base, v);
+      const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < kVec; ++j) {
+        if constexpr (kSize == 4) e[j] = words[j];
+        else if constexpr (kSize == 2) e[j] = (words[j / 2] >> (16 * (j % 2))) & 0xFFFFu;
+        else e[j] = (words[j / 4] >> (8 * (j % 4))) & 0xFFu;
+      }
+    };
+    uint32_t a[kVec], b[kVec];
+    vector_of(p.first, p.first_scalar, splat_first, a);
+    vector_of(p.second, p.second_scalar, splat_second, b);
+    uint32_t words[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < kVec; ++j) {
+      const uint32_t chosen = take[j] ? a[j] : b[j];
+      if constexpr (kSize == 4) words[j] = chosen;
+      else if constexpr (kSize == 2) words[j / 2] |= chosen << (16 * (j % 2));
+      else words[j / 4] |= chosen << (8 * (j % 4));
+    }
+    u32x4 result;
+    result.x = words[0], result.y = words[1], result.z = words[2], result.w = words[3];
+    store16_stream(out, v, result);
+  }
+  // elements past the last whole vector
+  const uint32_t e = vectors * kVec + thread;
+  if (e < elements) {
+    const bool take = (p.condition_scalar ? p.condition[0] : p.condition[e]) != 0;
+    const uint32_t chosen = take ? element(p.first, p.first_scalar, e) : element(p.second, p.second_scalar, e);
+    if constexpr (kSize == 4) reinterpret_cast<uint32_t *>(out)[e] = chosen;
+    else if constexpr (kSize == 2) reinterpret_cast<uint16_t *>(out)[e] = (uint16_t)chosen;
+    else out[e] = (unsigned char)chosen;
+  }
+}
+
+struct SelectLayout {
+  int32_t rank;
+  uint32_t dims[kMaxRank];
+  int64_t strides[3][kMaxRank];
+};
+
+// Any byte strides (0 on broadcast axes), elements gathered bytewise.
+template <int kSize>
+__global__ __launch_bounds__(kBlockThreads) void select_general(const unsigned char *condition, const unsigned char *first,
+                                                                const unsigned char *second, unsigned char *out,
+                                                                uint64_t elements, SelectLayout layout) {
+  const uint64_t e = (uint64_t)blockIdx.x * kBlockThreads + threadIdx.x;
+  if (e >= elements) return;
+  uint64_t rest = e;
+  int64_t off[3] = {0, 0, 0};
+  for (int axis = layout.rank - 1; axis >= 0; --axis) {
+    const uint32_t extent = layout.dims[axis];
+    const uint64_t coordinate = rest % extent;
+    rest /= extent;
+#pragma unroll
+    for (int i = 0; i < 3; ++i) off[i] += (int64_t)coordinate * layout.strides[i][axis];
+  }
+  const unsigned char *source = condition[off[0]] != 0 ? first + off[1] : second + off[2];
+#pragma unroll
+  for (int b = 0; b < kSize; ++b) out[e * kSize + b] = source[b];
+}
+
+}  // namespace
+
+hipError_t launch_fill(const FillParams &p, void *out, hipStream_t stream) {
+  if (p.elements == 0) return hipSuccess;
+  uint32_t pattern = p.bits;
+  if (p.size == 1) pattern = (p.bits & 0xFFu) * 0x01010101u;
+  else if (p.size == 2) pattern = (p.bits & 0xFFFFu) * 0x00010001u;
+  const uint64_t bytes = p.elements * p.size;
+  uint64_t blocks = (bytes / 16 + kBlockThreads) / kBlockThreads;
+  blocks = blocks > 2048 ? 2048 : blocks;
+  hipLaunchKernelGGL(fill_pattern, dim3((uint32_t)blocks), dim3(kBlockThreads), 0, stream,
+                     static_cast<unsigned char *>(out), bytes, pattern);
+  return hipGetLastError();
+}
+
+hipError_t launch_select(const SelectParams &p, const void *condition, const void *first, const void *second, void *out,
+                         bool vector_aligned, hipStream_t stream) {
+  if (p.elements == 0) return hipSuccess;
+  const unsigned char *c = static_cast<const unsigned char *>(condition);
+  const unsigned char *a = static_cast<const unsigned char *>(first), *b = static_cast<const unsigned char *>(second);
+  unsigned char *o = static_cast<unsigned char *>(out);
+  if (p.flat && vector_aligned) {
+    const SelectFlat flat{c, a, b, p.scalar[0] ? 1u : 0u, p.scalar[1] ? 1u : 0u, p.scalar[2] ? 1u : 0u};
+    const uint32_t vec = 16u / p.size, vectors = (uint32_t)(p.elements / vec);
+    uint64_t blocks = ((uint64_t)vectors + kBlockThreads) / kBlockThreads;
+    blocks = blocks < 1 ? 1 : (blocks > 8192 ? 8192 : blocks);
+    const dim3 grid((uint32_t)blocks), block(kBlockThreads);
+    switch (p.size) {
+      case 1: hipLaunchKernelGGL((select_flat<1>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
+      case 2: hipLaunchKernelGGL((select_flat<2>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
+      default: hipLaunchKernelGGL((select_flat<4>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
+    }
+    return hipGetLastError();
+  }
+  SelectLayout layout{};
+  layout.rank = p.rank;
+  for (int i = 0; i < kMaxRank; ++i) {
+    layout.dims[i] = p.dims[i];
+    for (int k = 0; k < 3; ++k) layout.strides[k][i] = p.strides[k][i];
+  }
+  const dim3 grid((uint32_t)((p.elements + kBlockThreads - 1) / kBlockThreads)), block(kBlockThreads);
+  switch (p.size) {
+    case 1: hipLaunchKernelGGL((select_general<1>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
+    case 2: hipLaunchKernelGGL((select_general<2>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
+    default: hipLaunchKernelGGL((select_general<4>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
+  }
+  return hipGetLastError();
+}
+
+}  // namespace hyle_hip

@@ -64,7 +64,7 @@ def run(context: hc.Context, operation, *inputs: torch.Tensor, outputs: Optional
         descs: Optional[Sequence[hc.TensorDesc]] = None):
     """prepare + create_invocation + submit on torch's current stream; returns the outputs."""
     descs = list(descs) if descs is not None else [desc_of(t) for t in inputs]
-    bound = Bound(context, operation, descs, device=inputs[0].device)
+    bound = Bound(context, operation, descs, device=inputs[0].device if inputs else "cuda:0")
     outs = list(outputs) if outputs is not None else bound.outputs()
     bound.submit(inputs, outs)
     # the workspace must outlive the enqueued kernels

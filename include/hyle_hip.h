@@ -71,9 +71,17 @@ typedef enum hyle_hip_op_kind {
    * (f32/f16/bf16 among each other, int32 -> f32, Bool <-> float; equal types copy).
    * Neither takes an alias: input and output bytes must not overlap. */
   HYLE_HIP_OP_COPY = 2,
+  /* Fill (include/hyle/compute/operation.h: struct Fill): no inputs (input_count = 0).  The
+   * output shape is the rank and dims of inputs[0] (its other fields are ignored), `kind` the
+   * output hyle_hip_dtype, which is also the scalar's type, and `count` ScalarValue::bits():
+   * the element's bit pattern in the low bytes. */
+  HYLE_HIP_OP_FILL = 3,
   HYLE_HIP_OP_CAST = 4,
   HYLE_HIP_OP_UNARY = 5,
   HYLE_HIP_OP_BINARY = 6,
+  /* Select: inputs (condition Bool, first, second), the three broadcast together; the output
+   * holds `first` where the condition byte is non-zero and `second` elsewhere, bit for bit. */
+  HYLE_HIP_OP_SELECT = 7,
   HYLE_HIP_OP_REDUCE = 8,
   HYLE_HIP_OP_RMS_NORM = 9,
   /* in0 [.., n], optional scale [n], optional bias [n] (bias only with a scale) */
@@ -171,7 +179,7 @@ typedef struct hyle_hip_tensor_desc {
 typedef struct hyle_hip_op_desc {
   uint32_t abi_version;      /* HYLE_HIP_ABI_VERSION */
   uint32_t op;               /* hyle_hip_op_kind */
-  uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind; Cast: output hyle_hip_dtype */
+  uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind; Cast, Fill: output hyle_hip_dtype */
   uint32_t kind2;            /* BINARY_CHAIN: second BinaryKind; GATED: GatedInputKind;
                                 SOFTMAX: SoftmaxKind; GGUF_MATVEC: HYLE_HIP_ACTIVATIONS_* */
   int32_t axis;              /* Softmax / TopK axis (negative counts from the end) */
@@ -180,7 +188,7 @@ typedef struct hyle_hip_op_desc {
   uint32_t keep_dimensions;  /* Reduce */
   float epsilon;             /* RmsNorm, LayerNorm */
   float scale;               /* Softmax */
-  uint64_t count;            /* TopK count */
+  uint64_t count;            /* TopK count; Fill: the scalar's bits */
   uint32_t largest;          /* TopK: 1 = largest first, 0 = smallest first */
   uint32_t input_count;
   hyle_hip_tensor_desc inputs[HYLE_HIP_MAX_INPUTS];

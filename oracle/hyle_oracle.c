@@ -1302,6 +1302,38 @@ int hyle_oracle_cast(int src_type, int dst_type, const void *src,
   return 0;
 }
 
+/* src/compute_provider_cuda/tensor_kernel.cu:190-193: every element takes the
+ * scalar's bits (ScalarValue::bits, include/hyle/compute/operation.h:187-230). */
+void hyle_oracle_fill(size_t width, uint64_t bits, size_t n, void *dst) {
+  unsigned char *d = (unsigned char *)dst;
+  for (size_t i = 0; i < n; ++i)
+    for (size_t b = 0; b < width; ++b)
+      d[i * width + b] = (unsigned char)(bits >> (8 * b));
+}
+
+/* src/compute_provider_cuda/tensor_kernel.cu:194-198 with the operand offsets of
+ * tensor_provider.cc:176-189 (an operand axis of extent 1, or one the operand
+ * lacks, contributes nothing): the condition byte picks the branch, whose
+ * `width` bytes are kept as they are. */
+void hyle_oracle_select(size_t width, const void *condition,
+                        const int64_t *condition_dims, const int64_t *condition_strides, int condition_rank,
+                        const void *first, const int64_t *first_dims, const int64_t *first_strides, int first_rank,
+                        const void *second, const int64_t *second_dims, const int64_t *second_strides, int second_rank,
+                        const int64_t *out_dims, int out_rank, void *dst) {
+  const size_t n = element_count(out_dims, out_rank);
+  unsigned char *d = (unsigned char *)dst;
+  for (size_t i = 0; i < n; ++i) {
+    const unsigned char mask = ((const unsigned char *)condition)[hyle_oracle_broadcast_byte_offset(
+        condition_dims, condition_strides, condition_rank, out_dims, out_rank, i)];
+    const unsigned char *from =
+        mask != 0 ? (const unsigned char *)first + hyle_oracle_broadcast_byte_offset(
+                                                      first_dims, first_strides, first_rank, out_dims, out_rank, i)
+                  : (const unsigned char *)second + hyle_oracle_broadcast_byte_offset(
+                                                       second_dims, second_strides, second_rank, out_dims, out_rank, i);
+    memcpy(d + i * width, from, width);
+  }
+}
+
 /* ------------------------------------------------------------------------ */
 /* CPU baseline legs (row ranges, dense loops)                              */
 /* ------------------------------------------------------------------------ */

@@ -313,6 +313,20 @@ int hyle_oracle_cast(int src_type, int dst_type, const void *src,
                      const int64_t *dims, const int64_t *strides, int rank,
                      void *dst);
 
+/* ---- Fill / Select ------------------------------------------------------ */
+/* Storage-only members of the reference's elementwise kernel family
+ * (src/compute_provider_cuda/tensor_kernel.cu:168-199): Fill writes the low
+ * `width` bytes of the scalar's bits to each of n elements; Select broadcasts a
+ * Bool condition and two branches of `width`-byte elements (dims + byte strides
+ * each) to the dense out_dims and keeps the first branch's bytes where the
+ * condition byte is non-zero, the second's elsewhere. */
+void hyle_oracle_fill(size_t width, uint64_t bits, size_t n, void *dst);
+void hyle_oracle_select(size_t width, const void *condition,
+                        const int64_t *condition_dims, const int64_t *condition_strides, int condition_rank,
+                        const void *first, const int64_t *first_dims, const int64_t *first_strides, int first_rank,
+                        const void *second, const int64_t *second_dims, const int64_t *second_strides, int second_rank,
+                        const int64_t *out_dims, int out_rank, void *dst);
+
 /* ---- CPU baseline legs ---------------------------------------------------
  * The same arithmetic as above in the loop shapes the reference's CPU provider
  * runs (dense rows, no per-element offset walk), over a contiguous row range

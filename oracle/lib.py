@@ -89,6 +89,9 @@ _reduce_axes = _sig("hyle_oracle_reduce", None, C.c_int, C.c_int, _vp, C.c_int, 
 _topk = _sig("hyle_oracle_topk", None, C.c_int, _vp, C.c_int, _i64p, _i64p, C.c_int, _sz, C.c_int, _vp, _vp)
 _k_quant = _sig("hyle_oracle_k_quant_dequant", None, C.c_int, _vp, _sz, _sz, _sz, _vp, _vp, _vp)
 _matvec = _sig("hyle_oracle_gguf_matvec", None, C.c_int, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _vp)
+_fill = _sig("hyle_oracle_fill", None, C.c_size_t, C.c_uint64, C.c_size_t, _vp)
+_select = _sig("hyle_oracle_select", None, C.c_size_t, _vp, _i64p, _i64p, C.c_int, _vp, _i64p, _i64p, C.c_int,
+               _vp, _i64p, _i64p, C.c_int, _i64p, C.c_int, _vp)
 _cast = _sig("hyle_oracle_cast", C.c_int, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int, _vp)
 
 
@@ -513,4 +516,30 @@ def cast(src_type: int, dst_type: int, storage: np.ndarray, dims, byte_strides=N
     out = np.empty(dims, _NP[dst_type])
     if _cast(src_type, dst_type, _ptr(raw), _i64(dims), _i64(byte_strides), len(dims), _ptr(out)) != 0:
         raise ValueError("the reference does not define this Cast pair")
+    return out
+
+
+# ---- Fill / Select ----------------------------------------------------------
+def fill(type_id: int, dims, bits: int) -> np.ndarray:
+    """A dense array of `dims` whose every element has the bit pattern `bits`."""
+    out = np.empty([int(d) for d in dims], _NP[type_id])
+    _fill(out.dtype.itemsize, int(bits), out.size, _ptr(out))
+    return out
+
+
+def select(type_id: int, condition, first, second) -> np.ndarray:
+    """Select over operands given as (storage, dims, byte_strides) triples (byte_strides None =
+    dense); the condition's elements are single bytes.  Returns the dense result."""
+    def operand(triple, width):
+        storage, dims, strides = triple
+        dims = [int(d) for d in dims]
+        if strides is None:
+            strides = _byte_strides(dims, width)
+        return np.ascontiguousarray(storage).view(np.uint8).reshape(-1), dims, [int(x) for x in strides]
+    width = np.dtype(_NP[type_id]).itemsize
+    c, a, b = operand(condition, 1), operand(first, width), operand(second, width)
+    shape = broadcast_shape(c[1], broadcast_shape(a[1], b[1]))
+    out = np.empty(shape, _NP[type_id])
+    _select(width, _ptr(c[0]), _i64(c[1]), _i64(c[2]), len(c[1]), _ptr(a[0]), _i64(a[1]), _i64(a[2]), len(a[1]),
+            _ptr(b[0]), _i64(b[1]), _i64(b[2]), len(b[1]), _i64(shape), len(shape), _ptr(out))
     return out

@@ -296,6 +296,43 @@ def test_cast_and_copy_inference_and_admission():
     assert hc.prepare(CTX, hc.Copy(), D(DT.kFloat32, [0, 9])).dispatch_count() == 0
 
 
+def test_fill_and_select_inference_and_admission():
+    # src/compute_ops/operation.cc:1263-1275: Fill has no inputs; shape, type and scalar type must agree
+    one = hc.ScalarValue.of(DT.kFloat32, 1.0)
+    assert one.bits == 0x3F800000
+    assert hc.infer_output_descriptions(hc.Fill((3, 5), DT.kFloat32, one), []) == [D(DT.kFloat32, [3, 5])]
+    assert hc.infer_output_descriptions(hc.Fill((), DT.kBFloat16, hc.ScalarValue.from_bits(DT.kBFloat16, 0)), []) == [D(DT.kBFloat16, [])]
+    for bad in (hc.Fill((3,), DT.kBFloat16, one), hc.Fill((3,), DT.kUnknown, hc.ScalarValue()), hc.Fill((-1,), DT.kFloat32, one)):
+        with pytest.raises(hc.StatusError) as err:
+            hc.infer_output_descriptions(bad, [])
+        assert err.value.is_invalid_argument()
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Fill((3,), DT.kFloat32, one), [D(DT.kFloat32, [3])])
+    assert err.value.is_invalid_argument()
+    prepared = hc.prepare(CTX, hc.Fill((9496, 4096), DT.kBFloat16, hc.ScalarValue.of(DT.kBFloat16, -1.0)))
+    assert prepared.route_name() == "fill-pattern" and prepared.dispatch_count() == 1
+    assert prepared.workspace_requirement().size == 0
+    assert hc.prepare(CTX, hc.Fill((4, 0), DT.kInt32, hc.ScalarValue.of(DT.kInt32, 7))).dispatch_count() == 0
+    # src/compute_ops/operation.cc:1309-1330: Bool condition, equal branch types, three-way broadcast
+    assert hc.infer_output_descriptions(hc.Select(), [D(DT.kBool, [4, 1, 6]), D(DT.kInt8, [5, 6]), D(DT.kInt8, [4, 5, 1])]) \
+        == [D(DT.kInt8, [4, 5, 6])]
+    for bad in ([D(DT.kUInt8, [8]), D(DT.kFloat32, [8]), D(DT.kFloat32, [8])],
+                [D(DT.kBool, [8]), D(DT.kFloat32, [8]), D(DT.kFloat16, [8])],
+                [D(DT.kBool, [8]), D(DT.kFloat32, [3]), D(DT.kFloat32, [8])],
+                [D(DT.kBool, [8]), D(DT.kFloat32, [8])]):
+        with pytest.raises(hc.StatusError) as err:
+            hc.infer_output_descriptions(hc.Select(), bad)
+        assert err.value.is_invalid_argument()
+    # a branch whose descriptor is the output's may be overwritten (tensor_provider.cc:190-194)
+    prepared = hc.prepare(CTX, hc.Select(), D(DT.kBool, [8, 16]), D(DT.kFloat32, [8, 16]), D(DT.kFloat32, []))
+    assert prepared.route_name() == "select" and prepared.dispatch_count() == 1
+    assert [prepared.alias_support(0, i) for i in range(3)] == [False, True, False]
+    with pytest.raises(hc.StatusError) as err:  # blocked storage is not plain
+        hc.prepare(CTX, hc.Select(), D(DT.kBool, [64, 2]), hc.TensorDesc.gguf_q8_0_weight(DT.kBFloat16, 64, 2),
+                   hc.TensorDesc.gguf_q8_0_weight(DT.kBFloat16, 64, 2))
+    assert err.value.is_unimplemented()
+
+
 def test_stream_abi_is_exported_and_validates_without_a_device():
     from hyle_amd import capi
     from hyle_amd import file_stream as fs
