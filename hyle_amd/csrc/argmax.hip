@@ -177,17 +177,17 @@ hipError_t run(const ArgmaxParams &p, const void *x, void *values, int32_t *indi
 }  // namespace
 
 // Tiles are cut so that rows x tiles is about four blocks of 256 threads per compute unit:
-// measured on MI355X over logits[64, 151936] f32, scan and fold together take 11.4 us with 1024
+// measured on MI355X (256 units) over logits[64, 151936] f32, scan and fold together take 11.4 us with 1024
 // blocks, 11.8 with 768 or 1536, 12.3 with 2048, 13.3 with 512 and 12.9-14.0 with 3072-8192 (four
 // vectors in flight instead of two: 11.2-12.0 us over the same range).  64 rows of 151936 logits
 // become 64 x 16 blocks of 9496 elements; 1024 rows or more are one block each.  A tile is a
 // whole number of 16-byte vectors and never shorter than one pass of the block.
-void argmax_plan(uint64_t rows, uint32_t width, Elem type, ArgmaxParams *p) {
+void argmax_plan(uint64_t rows, uint32_t width, Elem type, uint32_t compute_units, ArgmaxParams *p) {
   p->shape.rows = rows;
   p->shape.width = width;
   const uint32_t vec = (uint32_t)elem_vec(type);
   const uint32_t pass = (uint32_t)(kVectorsInFlight * kBlockThreads) * vec;  // elements of one pass
-  const uint64_t blocks = 4u * 256u;
+  const uint64_t blocks = 4u * (uint64_t)compute_units;
   uint64_t wanted = rows == 0 ? 1 : (blocks + rows / 2) / rows;
   wanted = wanted < 1 ? 1 : wanted;
   const uint32_t row_vectors = (width + vec - 1) / vec;

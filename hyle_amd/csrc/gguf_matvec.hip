@@ -411,15 +411,16 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
   const dim3 grid(((uint32_t)p.rows + rows_per_block - 1) / rows_per_block), block(kBlockThreads);
   const size_t shared = (size_t)p.m * p.k * sizeof(float);
   const unsigned char *in = static_cast<const unsigned char *>(w);
+  const uint32_t units = p.compute_units;
   {
     // one activation row over rows of 2048 n values made of whole 16-byte vectors
     const bool lines = ((reinterpret_cast<uintptr_t>(w) | p.row_stride) & 15u) == 0;
     if (p.m == 1 && lines && p.k == 2048) {
       const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
       // three blocks per compute unit measured best (Q4_K [2048 -> 6144] 4.9 us and [2048 -> 151936]
-      // 45.9 us, against 6.4 and 47.7 us with five; counts that are not a multiple of the 256
+      // 45.9 us, against 6.4 and 47.7 us with five; counts that are not a multiple of the
       // compute units leave some of them a block short and are slower)
-      const dim3 machine(wanted < 256u * 3u ? wanted : 256u * 3u);
+      const dim3 machine(wanted < units * 3u ? wanted : units * 3u);
       hipLaunchKernelGGL((gguf_matvec_lines<kKind, TX, 1>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
                          p.row_stride);
       return hipGetLastError();
@@ -432,7 +433,7 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
     if (lines && p.k % 2048 == 0 && (p.k > 2048 || p.m > 1) && staged + parked <= 64 * 1024) {
       const uint32_t spans = p.k / 2048;
       const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
-      const dim3 machine(wanted < 256u * 3u ? wanted : 256u * 3u);
+      const dim3 machine(wanted < units * 3u ? wanted : units * 3u);
       if (p.m == 1)
         hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 1>), machine, block, staged, s, in, x, y,
                            (uint32_t)p.rows, p.row_stride, spans, p.m);

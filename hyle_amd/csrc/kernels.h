@@ -142,7 +142,7 @@ struct ArgmaxParams {
   uint32_t tiles = 0;        // tiles per row
   uint32_t tile_elems = 0;   // elements per tile
 };
-void argmax_plan(uint64_t rows, uint32_t width, Elem type, ArgmaxParams *p);
+void argmax_plan(uint64_t rows, uint32_t width, Elem type, uint32_t compute_units, ArgmaxParams *p);
 size_t argmax_workspace_bytes(const ArgmaxParams &p);
 hipError_t launch_argmax(Elem type, const ArgmaxParams &p, const void *x, void *values,
                          int32_t *indices, void *workspace, bool vectorised, hipStream_t stream);
@@ -188,6 +188,7 @@ struct MatVecParams {
   uint64_t row_stride = 0;  // bytes between physical weight rows
   uint8_t kind = 0;
   uint8_t codec = 0;        // HYLE_HIP_ACTIVATIONS_*: 0 exact f32 activations, 1 ggml's 8-bit activation blocks
+  uint32_t compute_units = 256;  // of the plan's device: the grids are three blocks per unit
 };
 size_t gguf_matvec_shared_bytes(uint32_t m, uint32_t k);
 // The 8-bit activation route: K = 2048 n, rows of whole 16-byte vectors, M <= 8.

@@ -695,6 +695,8 @@ hyle_hip_status admit(hyle_hip_plan *p) {
   const hyle_hip_op_desc &r = p->request;
   const Desc *in = r.inputs;
   const Desc &out = p->outputs[0];
+  // a plan made without a device is sized for the 256 units of an MI355X
+  const uint32_t units = p->context != nullptr && p->context->compute_units > 0 ? (uint32_t)p->context->compute_units : 256u;
   hyle_hip_status s;
   switch (r.op) {
     case HYLE_HIP_OP_UNARY:
@@ -903,7 +905,7 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       if (r.count == 1 && r.largest && innermost && !integer) {
         // the vocabulary argmax: a scan dispatch and a fold dispatch
         p->route = Route::kArgmax;
-        argmax_plan(p->output_elements[0], (uint32_t)in[0].dims[axis], p->elem, &p->argmax);
+        argmax_plan(p->output_elements[0], (uint32_t)in[0].dims[axis], p->elem, units, &p->argmax);
         p->workspace_size = argmax_workspace_bytes(p->argmax);
         p->workspace_alignment = 16;
         p->dispatches = 2;
@@ -984,6 +986,7 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       if (p->output_elements[0] == 0) return HYLE_HIP_OK;
       p->route = Route::kGgufMatVec;
       p->matvec.codec = (uint8_t)r.kind2;
+      p->matvec.compute_units = units;
       p->matvec.rows = (uint64_t)n;
       p->matvec.k = (uint32_t)k;
       p->matvec.m = (uint32_t)m;

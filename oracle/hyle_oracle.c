@@ -901,8 +901,9 @@ void hyle_oracle_q8_0_dequant_bf16(const void *blocks, size_t rows, size_t k,
  *         16; y = (d * scale) * (q - 32), q six bits from ql (low four) and qh
  *         (high two).
  * Products and the subtraction are separate f32 roundings, as the source
- * writes them.  PARITY UNPINNED against ggml itself: no vector of its output
- * exists in the reference tree. */
+ * writes them.  Pinned bit for bit against the two readings of these formats
+ * the reference tree holds (third_party/ggml_q4k_apple/ggml_q4k_apple.h:9-38;
+ * tests/compute_models/qwen27_original_nextn_reference.h:74-86,262-287). */
 static void q4_k_scale_min(int j, const unsigned char *q, unsigned *scale, unsigned *minimum) {
   if (j < 4) {
     *scale = q[j] & 63u;

@@ -18,10 +18,10 @@
  *     (oracle/_ref), plus the reference tests' known-answer vectors.
  *   - binary add/mul, broadcast offsets, reduce, index_of_max, topk1: pinned by
  *     IEEE closed forms, brute force and the reference tests' known answers.
- *   - q8_0 decode: the arithmetic lives in ggml (not in the reference tree);
- *     restated from the published block format, pinned by an exactness proof
- *     and exhaustive scale x quant enumeration against an independent
- *     integer/double evaluation.
+ *   - q8_0 decode: restated from the block format, pinned by an exactness
+ *     argument with exhaustive scale x quant enumeration against an independent
+ *     integer/double evaluation, and by the element values the reference's own
+ *     tests expect (see k_quant_dequant below).
  *   - rms_norm_bf16_native tile order: "parity unpinned" at the bit level (the
  *     reference sums each 128-wide tile with a Highway vector dot whose lane
  *     order is target-dependent); pinned only to tolerance.
@@ -37,6 +37,17 @@
  *     tests/compute_models/qwen27_original_nextn_reference.h:74-86,262-287):
  *     pinned bit for bit against both over random raw bytes, and against
  *     blocks packed field by field.
+ *   - gguf_matvec_q8 (MatMul as the reference's ggml route computes it): the
+ *     8-bit activation codecs, the centre and the bound are the ones the
+ *     reference's tests hold for that route; pinned against array-wise
+ *     restatements of those forms and a float64 product of independently
+ *     decoded weights.  No output vector of ggml itself exists in the tree, so
+ *     agreement is to the tests' bound, not bit for bit: PARITY UNPINNED at the
+ *     bit level.  gguf_matvec (exact weights, double accumulation) is the
+ *     mathematical product and is what the bound is centred on.
+ *   - fill, select: the reference route test's expectation
+ *     (tests/compute_route_vulkan/tensor_test.cc:255-283) and numpy's
+ *     broadcasting `where` over raw words.
  */
 #ifndef HYLE_ORACLE_H_
 #define HYLE_ORACLE_H_
@@ -284,8 +295,10 @@ void hyle_oracle_gguf_matvec_q8(int kind, const void *blocks, size_t rows, size_
 /* GGUF Q4_K (kind 0: 256 elements in 144 bytes) and Q6_K (kind 1: 256 in 210)
  * rows -> f32 and / or bf16 [rows, k] plus the f32 row sums of squares of the
  * exact f32 values.  Geometry from src/compute_ops/low_precision.cc:22-27; the
- * decode is ggml's, restated from the published block layouts (the source is
- * not in the reference tree: parity with it is unpinned). */
+ * decode is ggml's, restated from the published block layouts and pinned bit
+ * for bit against the two readings of them the reference tree holds
+ * (third_party/ggml_q4k_apple/ggml_q4k_apple.h:9-38;
+ * tests/compute_models/qwen27_original_nextn_reference.h:74-86,262-287). */
 void hyle_oracle_k_quant_dequant(int kind, const void *blocks, size_t rows, size_t k,
                                  size_t row_stride_bytes, float *out_f32, uint16_t *out_bf16,
                                  float *sumsq);

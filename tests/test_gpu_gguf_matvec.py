@@ -3,9 +3,9 @@ C ABI, against the oracle's float64 product of exactly decoded weights.
 
 Bar: |got - exact| <= 1e-5 * sum_k |w x| for f32 activations (the f32 sum of K products in the
 kernel's order); bf16 / f16 outputs within one unit in the last place of the rounded exact value
-unless inside that same bound.  This pins the product with exact weights; ggml's result for the
-same operation (8-bit activation blocks, integer dot products) is a different rounding of it and
-is not reproduced: parity with the reference's ggml route is unpinned.
+unless inside that same bound.  This is the product with exact weights (ActivationArithmetic.kExact);
+the product as the reference's ggml route computes it (8-bit activation blocks, integer dots) is
+the other arithmetic of the same operator and has its own test, test_gpu_gguf_matvec_q8.py.
 """
 from __future__ import annotations
 
