@@ -67,38 +67,37 @@ __device__ __forceinline__ int64_t mask_row_offset(const MaskRows &m, uint32_t r
 // at x, src/compute_provider_native/transformer.cc:44-57), so a causal mask saves half the reads.
 //
 // A mask broadcast over the leading axes (a [q, k] mask under [heads, q, k]) repeats every
-// `period` rows, `repeats` times.  With kRepeat > 1 a lane group takes row q of kRepeat
-// consecutive repeats: the mask row is read once and kept in registers, and the next row's loads
-// are issued before the current row is reduced.  The re-reads this saves never reached HBM (the
-// FETCH_SIZE counter shows the mask fetched once per launch either way) but they did cross the
-// cache fabric: measured on MI355X for S[32,4096,4096] f32 with an additive f32 mask, 804 us
-// with one head per lane group and 709 us with two.  A Boolean mask (a quarter of the bytes, and
-// half the rows' vectors never loaded) gains nothing from it.
-template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog, int kRepeat>
+// `period` rows, `repeats` times.  An additive mask is as large as one repeat of x (64 MiB for a
+// [4096, 4096] f32 mask), so in storage order every repeat streams it through the L2s again:
+// measured on MI355X for S[32,4096,4096] f32, the mask was fetched 16 times per launch (1.23 x the
+// algorithmic bytes) at 804 us with one head per lane group, or 709 us when a lane group kept its
+// mask row in registers across two heads.  With `steer` the blocks are re-ordered instead so that
+// the 32 heads of a mask row run next to each other on one XCD (693 us with one head per lane
+// group, 708 with two, 801 with four).  A Boolean mask (a quarter of the bytes, and half the
+// rows' vectors never loaded) fits the L2s and gains nothing from it.
+template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog>
 __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const void *mask, void *y,
                                                          uint32_t rows, uint32_t row_vectors,
                                                          float scale, MaskRows mrows, uint32_t period,
-                                                         uint32_t repeats) {
+                                                         uint32_t repeats, uint32_t steer) {
   constexpr int kVec = Traits<T>::kVec;
   constexpr int kWords = kVec / 4;  // mask bytes of one vector, as 32-bit words
   constexpr int kGroupsPerBlock = kThreads / kLanes;
   constexpr int kWaves = kThreads / kWaveLanes;
-  __shared__ float joint_max[2][kWaves], joint_sum[2][kWaves];
+  __shared__ float joint_max[kWaves], joint_sum[kWaves];
   const uint32_t lane = threadIdx.x % kLanes;
   const uint32_t group = blockIdx.x * kGroupsPerBlock + threadIdx.x / kLanes;
-  // row of repeat i: first_row + i * row_step, valid while i < valid_repeats
-  uint32_t first_row, row_step, valid_repeats;
-  if constexpr (kRepeat == 1) {
-    first_row = group;
-    row_step = 0;
-    valid_repeats = group < rows ? 1u : 0u;
-  } else {
-    const uint32_t chunk = group / period, first_repeat = chunk * kRepeat;
-    first_row = first_repeat * period + group % period;
-    row_step = period;
-    valid_repeats = first_repeat < repeats ? repeats - first_repeat : 0u;
+  uint32_t row = group;
+  if (steer != 0) {
+    // Blocks go to the eight XCDs round-robin and each XCD has an L2 of its own: every repeat of
+    // a mask row is given to one XCD, one after another in its queue, so the row is fetched into
+    // one L2 once and found there by the others (period is a multiple of 8 here, one group per
+    // block, so this is a permutation of the rows).
+    const uint32_t xcd = group % 8u, slot = group / 8u;
+    row = (slot % repeats) * period + (slot / repeats) * 8u + xcd;
   }
-  const uint32_t mask_row_index = first_row < rows ? first_row : rows - 1;
+  const bool row_ok = row < rows;
+  const uint32_t mask_row_index = row_ok ? row : rows - 1;
   const char *mask_row = nullptr;
   if (kMask != kMaskNone) mask_row = static_cast<const char *>(mask) + mask_row_offset(mrows, mask_row_index);
 
@@ -154,106 +153,94 @@ __global__ __launch_bounds__(kThreads) void softmax_rows(const void *x, const vo
     }
   }
 
-  u32x4 current[kVpl], next[kVpl];
-  auto issue = [&](int i, u32x4(&into)[kVpl]) {
-    const uint32_t row = first_row + (uint32_t)i * row_step;
-    const size_t row_base = (size_t)((uint32_t)i < valid_repeats ? row : mask_row_index) * row_vectors;
+  u32x4 current[kVpl];
+  {
+    const size_t row_base = (size_t)mask_row_index * row_vectors;
 #pragma unroll
     for (int k = 0; k < kVpl; ++k) {
-      into[k] = u32x4{0u, 0u, 0u, 0u};
+      current[k] = u32x4{0u, 0u, 0u, 0u};
       if constexpr (kMask == kMaskBoolean) {
-        if (wanted_vector[k]) into[k] = load16_stream(x, row_base + vec[k]);
+        if (wanted_vector[k]) current[k] = load16_stream(x, row_base + vec[k]);
       } else {
-        into[k] = load16_stream(x, row_base + vec[k]);
+        current[k] = load16_stream(x, row_base + vec[k]);
       }
     }
-  };
-  issue(0, current);
+  }
 #pragma unroll
-  for (int i = 0; i < kRepeat; ++i) {
-    if (i + 1 < kRepeat) issue(i + 1, next);
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) loads_issued(current[k]);
-    const bool row_ok = (uint32_t)i < valid_repeats;
-    const uint32_t row = first_row + (uint32_t)i * row_step;
+  for (int k = 0; k < kVpl; ++k) loads_issued(current[k]);
 
-    // ---- scale, mask --------------------------------------------------------------------
-    float v[kVpl][kVec];
+  // ---- scale, mask --------------------------------------------------------------------
+  float v[kVpl][kVec];
 #pragma unroll
-    for (int k = 0; k < kVpl; ++k) {
-      Traits<T>::unpack(current[k], v[k]);
+  for (int k = 0; k < kVpl; ++k) {
+    Traits<T>::unpack(current[k], v[k]);
 #pragma unroll
-      for (int j = 0; j < kVec; ++j) {
-        if constexpr (kMask == kMaskBoolean) {
-          const bool keep = ((bits[k][j / 4] >> (8 * (j % 4))) & 0xFFu) != 0;
-          v[k][j] = keep ? v[k][j] * scale : -INFINITY;
-        } else if constexpr (kMask == kMaskAdditive) {
-          v[k][j] = ok[k] ? v[k][j] * scale + addend[k][j] : -INFINITY;
-        } else {
-          v[k][j] = ok[k] ? v[k][j] * scale : -INFINITY;
-        }
+    for (int j = 0; j < kVec; ++j) {
+      if constexpr (kMask == kMaskBoolean) {
+        const bool keep = ((bits[k][j / 4] >> (8 * (j % 4))) & 0xFFu) != 0;
+        v[k][j] = keep ? v[k][j] * scale : -INFINITY;
+      } else if constexpr (kMask == kMaskAdditive) {
+        v[k][j] = ok[k] ? v[k][j] * scale + addend[k][j] : -INFINITY;
+      } else {
+        v[k][j] = ok[k] ? v[k][j] * scale : -INFINITY;
       }
     }
+  }
 
-    // ---- row maximum and validity -------------------------------------------------------
-    // A NaN or +inf anywhere makes the row undefined.  fmaxf never lets a NaN through, so a
-    // lane that met one reports +inf instead: after the reduction an infinite maximum of either
-    // sign (+inf: poisoned, -inf: nothing finite and unmasked) marks the row.
-    float peak = -INFINITY;
-    bool poisoned = false;
+  // ---- row maximum and validity -------------------------------------------------------
+  // A NaN or +inf anywhere makes the row undefined.  fmaxf never lets a NaN through, so a
+  // lane that met one reports +inf instead: after the reduction an infinite maximum of either
+  // sign (+inf: poisoned, -inf: nothing finite and unmasked) marks the row.
+  float peak = -INFINITY;
+  bool poisoned = false;
 #pragma unroll
-    for (int k = 0; k < kVpl; ++k)
+  for (int k = 0; k < kVpl; ++k)
 #pragma unroll
-      for (int j = 0; j < kVec; ++j) {
-        poisoned = poisoned || poisons_row(v[k][j]);
-        peak = fmaxf(peak, v[k][j]);
-      }
-    peak = row_max<kLanes>(poisoned ? INFINITY : peak, joint_max[i & 1]);
-    const bool invalid = __builtin_fabsf(peak) == INFINITY;
+    for (int j = 0; j < kVec; ++j) {
+      poisoned = poisoned || poisons_row(v[k][j]);
+      peak = fmaxf(peak, v[k][j]);
+    }
+  peak = row_max<kLanes>(poisoned ? INFINITY : peak, joint_max);
+  const bool invalid = __builtin_fabsf(peak) == INFINITY;
 
-    // ---- exponentials and their sum -----------------------------------------------------
-    // The logarithmic form keeps the maxima (exp = 1 each) out of the float sum and counts them
-    // instead: log(sum) = log1p((maxima - 1) + tail), which keeps a tail far below 1, as the
-    // reference does by leaving its one chosen maximum out
-    // (src/compute_provider_cuda/reduction_kernel.cu:178-196).
-    float total = 0.0f, maxima = 0.0f;
+  // ---- exponentials and their sum -----------------------------------------------------
+  // The logarithmic form keeps the maxima (exp = 1 each) out of the float sum and counts them
+  // instead: log(sum) = log1p((maxima - 1) + tail), which keeps a tail far below 1, as the
+  // reference does by leaving its one chosen maximum out
+  // (src/compute_provider_cuda/reduction_kernel.cu:178-196).
+  float total = 0.0f, maxima = 0.0f;
 #pragma unroll
-    for (int k = 0; k < kVpl; ++k)
+  for (int k = 0; k < kVpl; ++k)
 #pragma unroll
-      for (int j = 0; j < kVec; ++j) {
-        const float shifted = v[k][j] - peak;
-        if constexpr (kLog) {
-          const bool at_peak = shifted == 0.0f;
-          total += at_peak ? 0.0f : exp_scaled(shifted);
-          maxima += at_peak ? 1.0f : 0.0f;
-          v[k][j] = shifted;
-        } else {
-          v[k][j] = exp_scaled(shifted);
-          total += v[k][j];
-        }
-      }
-    total = row_sum<kLanes>(total, joint_sum[i & 1]);  // = 2^32 * sum(exp)
-    // joint_max[i & 1] is free again: every wave read it before the barrier of the sum above
-    if constexpr (kLog) maxima = row_sum<kLanes>(maxima, joint_max[i & 1]);
-
-    // ---- normalise and store ------------------------------------------------------------
-    // softmax: e * 2^32 * (1 / (sum * 2^32)).  log-softmax: (v - max) - log(sum).
-    // An undefined row gets a NaN normaliser: it turns every lane, masked zeros included,
-    // into NaN without a per-element select.
-    float normaliser = kLog ? log1pf((maxima - 1.0f) + total * 2.3283064365386963e-10f) : 1.0f / total;
-    if (invalid) normaliser = __builtin_nanf("");
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) {
-      if (row_ok && ok[k]) {
-        float r[kVec];
-#pragma unroll
-        for (int j = 0; j < kVec; ++j) r[j] = kLog ? v[k][j] - normaliser : v[k][j] * normaliser;
-        store16_stream(y, (size_t)row * row_vectors + vec[k], Traits<T>::pack(r));
+    for (int j = 0; j < kVec; ++j) {
+      const float shifted = v[k][j] - peak;
+      if constexpr (kLog) {
+        const bool at_peak = shifted == 0.0f;
+        total += at_peak ? 0.0f : exp_scaled(shifted);
+        maxima += at_peak ? 1.0f : 0.0f;
+        v[k][j] = shifted;
+      } else {
+        v[k][j] = exp_scaled(shifted);
+        total += v[k][j];
       }
     }
-    if (i + 1 < kRepeat) {
+  total = row_sum<kLanes>(total, joint_sum);  // = 2^32 * sum(exp)
+  // joint_max is free again: every wave read it before the barrier of the sum above
+  if constexpr (kLog) maxima = row_sum<kLanes>(maxima, joint_max);
+
+  // ---- normalise and store ------------------------------------------------------------
+  // softmax: e * 2^32 * (1 / (sum * 2^32)).  log-softmax: (v - max) - log(sum).
+  // An undefined row gets a NaN normaliser: it turns every lane, masked zeros included,
+  // into NaN without a per-element select.
+  float normaliser = kLog ? log1pf((maxima - 1.0f) + total * 2.3283064365386963e-10f) : 1.0f / total;
+  if (invalid) normaliser = __builtin_nanf("");
 #pragma unroll
-      for (int k = 0; k < kVpl; ++k) current[k] = next[k];
+  for (int k = 0; k < kVpl; ++k) {
+    if (row_ok && ok[k]) {
+      float r[kVec];
+#pragma unroll
+      for (int j = 0; j < kVec; ++j) r[j] = kLog ? v[k][j] - normaliser : v[k][j] * normaliser;
+      store16_stream(y, (size_t)row * row_vectors + vec[k], Traits<T>::pack(r));
     }
   }
 }
@@ -356,15 +343,13 @@ MaskRepeat mask_repeat(const SoftmaxParams &p) {
   return r;
 }
 
-template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog, int kRepeat>
+template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog>
 hipError_t run_rows_as(const SoftmaxParams &p, const void *x, const void *mask, void *y,
                        hipStream_t s) {
   constexpr int kGroupsPerBlock = kThreads / kLanes;
   const uint32_t rows = (uint32_t)p.shape.rows;
   const MaskRepeat repeat = mask_repeat(p);
-  const uint64_t groups =
-      kRepeat == 1 ? rows : (uint64_t)repeat.period * ((repeat.repeats + kRepeat - 1) / kRepeat);
-  const uint32_t blocks = (uint32_t)((groups + kGroupsPerBlock - 1) / kGroupsPerBlock);
+  const uint32_t blocks = (rows + kGroupsPerBlock - 1) / kGroupsPerBlock;
   MaskRows m{};
   m.outer_rank = p.outer_rank;
   for (int i = 0; i < kMaxRank; ++i) {
@@ -372,26 +357,29 @@ hipError_t run_rows_as(const SoftmaxParams &p, const void *x, const void *mask, 
     m.outer_strides[i] = p.mask_outer_strides[i];
   }
   m.inner_stride = p.mask_inner_stride;
-  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads, kMask, kLog, kRepeat>), dim3(blocks),
+  const uint32_t steer = kMask == kMaskAdditive && kGroupsPerBlock == 1 && repeat.repeats >= 2 &&
+                                 repeat.period % 8 == 0 && p.mask_inner_stride != 0
+                             ? 1u : 0u;
+  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads, kMask, kLog>), dim3(blocks),
                      dim3(kThreads), 0, s, x, mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, m,
-                     repeat.period, repeat.repeats);
+                     repeat.period, repeat.repeats, steer);
   return hipGetLastError();
 }
 
-template <class T, int kLanes, int kVpl, int kThreads = kBlockThreads, int kRepeat = 1>
+template <class T, int kLanes, int kVpl, int kThreads = kBlockThreads>
 hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, void *y,
                     hipStream_t s) {
   const bool log_form = p.log;
   switch ((int)p.mask_kind) {
     case kMaskBoolean:
-      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, true, kRepeat>(p, x, mask, y, s)
-                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, false, kRepeat>(p, x, mask, y, s);
+      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, true>(p, x, mask, y, s)
+                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, false>(p, x, mask, y, s);
     case kMaskAdditive:
-      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, true, kRepeat>(p, x, mask, y, s)
-                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, false, kRepeat>(p, x, mask, y, s);
+      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, true>(p, x, mask, y, s)
+                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, false>(p, x, mask, y, s);
     default:
-      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, true, 1>(p, x, mask, y, s)
-                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, false, 1>(p, x, mask, y, s);
+      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, true>(p, x, mask, y, s)
+                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, false>(p, x, mask, y, s);
   }
 }
 
@@ -411,12 +399,10 @@ hipError_t run_softmax(const SoftmaxParams &p, const void *x, const void *mask, 
   // one row per block 685; two waves x 8 vectors 706-737; four waves x 4 vectors 731; a plain
   // copy in the same shapes 688-737.  Boolean causal mask, masked vectors not loaded: four waves
   // x 4 vectors, one row per block 531; two rows per block 557; two or four heads per lane
-  // group 551-716.  Additive causal mask: eight waves x 2 vectors, one head per lane group 804,
-  // two heads 709, four heads 732; four waves x 4 vectors with two or four heads 730-815.
+  // group 551-716.  Additive causal mask, blocks steered so that a mask row stays on one XCD:
+  // eight waves x 2 vectors 693; four waves x 4 vectors 706.
   if (vectors <= 1024) {
     if ((int)p.mask_kind == kMaskBoolean) return run_rows<T, 256, 4, 256>(p, x, mask, y, s);
-    if ((int)p.mask_kind == kMaskAdditive && mask_repeat(p).repeats >= 2)
-      return run_rows<T, 512, 2, 512, 2>(p, x, mask, y, s);
     return run_rows<T, 512, 2, 512>(p, x, mask, y, s);
   }
   if (vectors <= 2048) return run_rows<T, 512, 4, 512>(p, x, mask, y, s);
