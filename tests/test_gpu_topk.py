@@ -124,6 +124,38 @@ def test_topk_when_the_first_bound_admits_every_key():
                 check(tag, data, [3, width], count, -1, largest, outputs)
 
 
+def test_topk_mostly_distinct_values_take_the_float_bound():
+    """Unordered, mostly distinct values: a tile's bound comes from the threads' float maxima and
+    only the few elements that reach it become keys; the lists of the tiles meet in the ranking
+    dispatch.  Winners that are zeros of either sign or infinities, NaNs among the losers, rows
+    whose last tile is short, more lists than one wave can sample, and two ranking stages."""
+    rng = np.random.default_rng(1158)
+    shapes = (([4, 151936], (64, 8, 256)),      # 19 tiles; count 256 merges in two stages
+              ([3, 20000], (100, 64)),           # 3 tiles, the last one short
+              ([2, 600000], (4, 33)),            # 74 tiles: more lists than one wave samples
+              ([5, 8192], (64,)),                # exactly one tile: the select dispatch writes the outputs
+              ([2, 8200], (17,)))                # a last tile of 8 elements, fewer than count
+    for tag in ("f32", "bf16", "f16"):
+        for dims, counts in shapes:
+            base = rng.normal(0, 2, dims).astype(np.float32)
+            for largest in (True, False):
+                sign = -1.0 if largest else 1.0
+                x = base.copy()
+                x[0] = sign * (np.abs(x[0]) + 1.0)                       # zeros are the best values of row 0
+                spots = rng.choice(dims[1], 24, replace=False)
+                x[0, spots[:12]] = 0.0
+                x[0, spots[12:]] = -0.0
+                x[1, rng.choice(dims[1], dims[1] // 50, replace=False)] = np.nan
+                x[1, rng.choice(dims[1], 5, replace=False)] = -sign * np.inf
+                x[-1, rng.choice(dims[1], 3, replace=False)] = sign * np.inf
+                stored = host_values(x, tag)
+                device = to_device(stored, tag)
+                for count in counts:
+                    note(f"topk float-bound path {tag} {dims} count {count} largest {largest}")
+                    outputs = run(hc.TopK(count=count, largest=largest), device)
+                    check(tag, stored, dims, count, -1, largest, outputs)
+
+
 def test_topk_vocabulary_shape_count_64():
     rng = np.random.default_rng(1160)
     x = rng.normal(0, 3, (64, 151936)).astype(np.float32)
