@@ -378,6 +378,180 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_lines(const unsi
   if (filled != 0) flush(row - (uint32_t)filled * stride, filled);
 }
 
+// ---- several activation rows: the integer dots on the matrix unit ------------------------------
+// v_mfma_i32_4x4x4i8 is sixteen independent 4 x 4 x 4 products, one per quad of lanes: lane q of a
+// quad gives row q of A (four int8 along k) and column q of B, and gets column q of D back, one
+// register per row.  With A = four weight rows at the same four positions and B = four activation
+// rows' codes at those positions, one instruction is the sixteen four-value dots that the vector
+// unit would take with sixteen v_dot4c.  So the four lanes of a quad decode four *different*
+// weight rows (the four a wave keeps in flight) at the *same* positions, each for one activation
+// row: lane (c, q) walks the 32-value shares of lanes 4 c .. 4 c + 3 of the one-row-per-wave
+// layout, on weight row q, against the codes of activation row q.  The decode of a weight row is
+// done once whatever the number of activation rows; what a group of 16 costs per lane beyond it is
+// two matrix instructions and four scale multiplies, for four rows by four activation rows.
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ i32x4 quad_dots(uint32_t weights, uint32_t codes, i32x4 sum) {
+  return __builtin_amdgcn_mfma_i32_4x4x4i8((int)weights, (int)codes, sum, 0, 0, 0);
+}
+// lane i of the caller's quad
+template <int kLane> __device__ __forceinline__ int quad_lane(int v) { return dpp_move<kLane * 0x55>(v); }
+template <int kLane> __device__ __forceinline__ float quad_lane(float v) { return dpp_move<kLane * 0x55>(v); }
+// sum over the sixteen quads of the wave, lane q of each: every lane ends with its column's total
+__device__ __forceinline__ float quads_sum(float v) {
+  v += dpp_move<0x1B>(dpp_move<kDppHalfMirror>(v));  // lane ^ 4: half-row mirror, then quad reversal
+  v += dpp_move<0x128>(v);                           // lane ^ 8: row_ror 8
+  v += __shfl_xor(v, 16, kWaveLanes);
+  v += __shfl_xor(v, 32, kWaveLanes);
+  return v;
+}
+
+// One decoded 32-value share of this lane's weight row against the codes `a` of the same
+// positions of this lane's activation row.  The codes go in as A and the weights as B, so the
+// lane gets its own weight row back against the quad's four activation rows: sums[i] gains
+// activation row i's part, and the weight row's scales are the lane's own.
+template <int kKind> struct QuadDot;
+template <> struct QuadDot<1> {  // Q6_K
+  static __device__ __forceinline__ void add(const SpanDot<1> &w, const LaneCodes &a, float (&sums)[4]) {
+    int total[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const i32x4 zero = {0, 0, 0, 0};
+      const i32x4 dots = quad_dots(a.codes[2 * g + 1], w.q[g][1], quad_dots(a.codes[2 * g], w.q[g][0], zero));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) total[i] = mad24(w.scale[g], dots[i], total[i]);
+    }
+    sums[0] += (w.step * quad_lane<0>(a.scale[0])) * (float)total[0];
+    sums[1] += (w.step * quad_lane<1>(a.scale[0])) * (float)total[1];
+    sums[2] += (w.step * quad_lane<2>(a.scale[0])) * (float)total[2];
+    sums[3] += (w.step * quad_lane<3>(a.scale[0])) * (float)total[3];
+  }
+};
+template <> struct QuadDot<2> {  // Q8_0
+  static __device__ __forceinline__ void add(const SpanDot<2> &w, const LaneCodes &a, float (&sums)[4]) {
+    i32x4 dots = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dots = quad_dots(a.codes[i], w.q[i], dots);
+    sums[0] += (w.d * quad_lane<0>(a.scale[0])) * (float)dots[0];
+    sums[1] += (w.d * quad_lane<1>(a.scale[0])) * (float)dots[1];
+    sums[2] += (w.d * quad_lane<2>(a.scale[0])) * (float)dots[2];
+    sums[3] += (w.d * quad_lane<3>(a.scale[0])) * (float)dots[3];
+  }
+};
+
+// kSets sets of four activation rows (rows past m repeat the last one and are not stored);
+// kRegisters: one span per row (K = 2048), the lane's codes live in registers for the whole kernel.
+// A wave takes weight rows first + n * stride four at a time, span by span.
+template <int kKind, class TX, int kSets, bool kRegisters>
+__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_quads(const unsigned char *weights, const void *x,
+                                                                      void *y, uint32_t rows, uint64_t row_stride,
+                                                                      uint32_t spans, uint32_t m) {
+  using Row = LinesRow<kKind, 1>;
+  using Kind = Lines<kKind>;
+  constexpr uint32_t kSpanBytes = Kind::kPassVectors * 16;
+  // the four lanes of a quad read the same offsets of four slots at once: 32 bytes between the
+  // slots' starts (mod 128) put them on different LDS banks
+  constexpr int kSlotStride = Row::kSlotBytes + 32;
+  __shared__ __align__(16) unsigned char slots[kWavesPerBlock][4][kSlotStride];
+  extern __shared__ __align__(16) uint32_t staged[];  // [m * spans][kCodeWords][64]
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  const uint32_t quad = lane / 4, own = lane % 4;  // positions of lanes 4 quad .. + 3; weight row and activation row `own`
+  const uint32_t k = spans * 2048;
+  for (uint32_t pair = wave; pair < m * spans; pair += kWavesPerBlock)
+    park(staged, pair, lane, quantise_span<kKind, TX>(x, (size_t)(pair / spans) * k, pair % spans, lane));
+  __syncthreads();
+  uint32_t token[kSets];
+#pragma unroll
+  for (int set = 0; set < kSets; ++set) token[set] = min(own + 4u * set, m - 1);
+  LaneCodes held[kRegisters ? kSets * 4 : 1];
+  if constexpr (kRegisters) {
+#pragma unroll
+    for (int set = 0; set < kSets; ++set)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) held[set * 4 + t] = fetch(staged, token[set], 4 * quad + t);
+  }
+  typename Kind::Lane at[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) at[t] = Kind::lane_of(0, 4 * quad + t);
+  const unsigned char *own_slot = slots[wave][own];
+  const uint32_t stride = gridDim.x * kWavesPerBlock;
+  const uint32_t first = blockIdx.x * kWavesPerBlock + wave;
+  if (first >= rows) return;  // no barrier follows
+  const uint32_t own_rows = (rows - first + stride - 1) / stride;
+  const uint32_t batches = (own_rows + 3) / 4;
+  // the loads of the next (batch, span) are in flight while this one is decoded
+  auto load_batch = [&](uint32_t batch, uint32_t span, Row (&into)[4]) {
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t n = 4 * batch + d;
+      // past the wave's last row: its first row again, a valid address whose bytes go unused
+      const unsigned char *source = weights + (size_t)(n < own_rows ? first + n * stride : first) * row_stride +
+                                    (size_t)(n < own_rows ? span : 0u) * kSpanBytes;
+      into[d] = Row::load(source, lane);
+    }
+  };
+  Row ring[4];
+  load_batch(0, 0, ring);
+  float sums[kSets][4] = {};
+  for (uint32_t batch = 0; batch < batches; ++batch) {
+    for (uint32_t span = 0; span < spans; ++span) {
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int i = 0; i < Row::kLoads; ++i)
+          *reinterpret_cast<u32x4 *>(slots[wave][d] + (size_t)(lane + i * kWaveLanes) * 16) = ring[d].v[i];
+      {
+        const bool last_span = span + 1 == spans;
+        const uint32_t next_batch = last_span ? batch + 1 : batch;
+        load_batch(next_batch < batches ? next_batch : 0u, last_span ? 0u : span + 1, ring);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        SpanDot<kKind> decoded;
+        decoded.decode(own_slot, at[t]);
+#pragma unroll
+        for (int set = 0; set < kSets; ++set) {
+          if constexpr (kRegisters) QuadDot<kKind>::add(decoded, held[set * 4 + t], sums[set]);
+          else QuadDot<kKind>::add(decoded, fetch(staged, token[set] * spans + span, 4 * quad + t), sums[set]);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    // the four rows are complete: lane (0, q) stores its weight row against every activation row
+#pragma unroll
+    for (int set = 0; set < kSets; ++set)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float total = quads_sum(sums[set][i]);
+        sums[set][i] = 0.0f;
+        const uint32_t n = 4 * batch + own, r = (uint32_t)i + 4u * set;
+        if (quad == 0 && n < own_rows && r < m) Traits<TX>::store(y, (size_t)r * rows + first + n * stride, total);
+      }
+  }
+}
+
+template <int kKind, class TX>
+hipError_t run_quads(const MatVecParams &p, const void *w, const void *x, void *y, uint32_t spans, dim3 grid,
+                     size_t shared, hipStream_t s) {
+  const unsigned char *in = static_cast<const unsigned char *>(w);
+#define HYLE_QUADS(SETS, REGISTERS)                                                                             \
+  hipLaunchKernelGGL((gguf_matvec_q8_quads<kKind, TX, SETS, REGISTERS>), grid, dim3(kBlockThreads), shared, s, in, x, \
+                     y, (uint32_t)p.rows, p.row_stride, spans, p.m)
+  if (p.m <= 4) {
+    if (spans == 1) HYLE_QUADS(1, true);
+    else HYLE_QUADS(1, false);
+  } else {
+    if (spans == 1) HYLE_QUADS(2, true);
+    else HYLE_QUADS(2, false);
+  }
+#undef HYLE_QUADS
+  return hipGetLastError();
+}
+
 template <int kKind, class TX, int kM>
 hipError_t run_registers(const MatVecParams &p, const void *w, const void *x, void *y, uint32_t spans, dim3 grid,
                          size_t shared, hipStream_t s) {
@@ -398,6 +572,12 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
   const uint32_t machine = (uint32_t)(compute_units > 0 ? compute_units : 256) * 3u;  // three blocks per compute unit
   const dim3 grid(wanted < machine ? wanted : machine);
   const size_t shared = gguf_matvec_q8_shared_bytes(p.m, p.k);
+  if constexpr (kKind != 0) {
+    // Q6_K and Q8_0 with several activation rows: the quad form, if its four row slots per wave
+    // fit beside the codes
+    const size_t slots = (size_t)kWavesPerBlock * 4 * (LinesRow<kKind, 1>::kSlotBytes + 32);
+    if (p.m >= 2 && slots + shared <= 64 * 1024) return run_quads<kKind, TX>(p, w, x, y, spans, grid, shared, s);
+  }
   if (p.m == 1) return run_registers<kKind, TX, 1>(p, w, x, y, spans, grid, shared, s);
   if (p.m == 2) return run_registers<kKind, TX, 2>(p, w, x, y, spans, grid, shared, s);
   if (p.m <= 4) return run_registers<kKind, TX, 4>(p, w, x, y, spans, grid, shared, s);
