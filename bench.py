@@ -602,14 +602,14 @@ def file_stream_rate(mib, ctx, torch, dev):
 # (profiles/hot_path_step_hbm_traffic_pmc.md: FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors
 # the same counters need to read a plain 1 GiB copy correctly).
 TRAFFIC = {
-    "cfg4_softmax_f32_causal": 3247181209,
-    "cfg4_softmax_f32_causal_additive": 5368804454,
-    "cfg3_swiglu_bf16": 302055219,
-    "cfg3_residual_add_bf16": 100736614,
-    "cfg1_broadcast_add_mul_f32": 67323085,
-    "cfg2_rmsnorm_bf16": 67236659,
-    "cfg4_argmax_f32": 39211827,
-    "cfg5_q8_0_dequant_sumsq": 38615859,
+    "cfg4_softmax_f32_causal": 3247166259,
+    "cfg4_softmax_f32_causal_additive": 4362172313,
+    "cfg3_swiglu_bf16": 302043955,
+    "cfg3_residual_add_bf16": 100731801,
+    "cfg1_broadcast_add_mul_f32": 67302297,
+    "cfg2_rmsnorm_bf16": 67215667,
+    "cfg4_argmax_f32": 39140659,
+    "cfg5_q8_0_dequant_sumsq": 38638592,
 }
 
 
