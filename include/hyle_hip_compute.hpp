@@ -229,6 +229,41 @@ enum class SoftmaxKind : std::uint8_t { kSoftmax = 0, kLogSoftmax };
 enum class MaskKind : std::uint8_t { kNone = 0, kAdditive, kBoolean };
 
 struct Copy final {};
+// Exact scalar payload of Fill (include/hyle/compute/operation.h:187-230): a type and the
+// element's bit pattern; low-precision floats come in through from_bits.
+class ScalarValue final {
+public:
+  constexpr ScalarValue() noexcept = default;
+  constexpr explicit ScalarValue(bool value) noexcept : type_(DataType::kBool), bits_(value ? 1u : 0u) {}
+  constexpr explicit ScalarValue(std::int8_t value) noexcept : type_(DataType::kInt8), bits_(static_cast<std::uint8_t>(value)) {}
+  constexpr explicit ScalarValue(std::uint8_t value) noexcept : type_(DataType::kUInt8), bits_(value) {}
+  constexpr explicit ScalarValue(std::int32_t value) noexcept : type_(DataType::kInt32), bits_(static_cast<std::uint32_t>(value)) {}
+  explicit ScalarValue(float value) noexcept : type_(DataType::kFloat32) {
+    std::uint32_t word;
+    std::memcpy(&word, &value, sizeof word);
+    bits_ = word;
+  }
+  static constexpr ScalarValue from_bits(DataType type, std::uint64_t bits) noexcept {
+    ScalarValue result;
+    result.type_ = type;
+    result.bits_ = bits;
+    return result;
+  }
+  constexpr bool valid() const noexcept { return type_ != DataType::kUnknown; }
+  constexpr DataType data_type() const noexcept { return type_; }
+  constexpr std::uint64_t bits() const noexcept { return bits_; }
+private:
+  DataType type_ = DataType::kUnknown;
+  std::uint64_t bits_ = 0;
+};
+// No inputs: a dense tensor of output_shape whose every element is `value`.
+struct Fill final {
+  std::vector<std::int64_t> output_shape;
+  DataType output_type = DataType::kUnknown;
+  ScalarValue value;
+};
+// Inputs (condition Bool, first, second), broadcast together: first where the condition holds.
+struct Select final {};
 struct Cast final { DataType output_type = DataType::kUnknown; };
 struct Unary final { UnaryKind kind = UnaryKind::kAbs; };
 struct Binary final { BinaryKind kind = BinaryKind::kAdd; };
@@ -286,9 +321,12 @@ struct Q8_0DequantSumSquares final {};
 // geometry of the descriptor), and MatMul(x, W) over such a weight for up to 8 activation rows
 // (inputs: weight, activations).
 using GgufDequantSumSquares = Q8_0DequantSumSquares;
-struct GgufMatVec final {};
+// kGgmlQ8: the activations are first quantised to ggml's 8-bit blocks and the block dots are
+// integers, as the reference's ggml route computes the product; kExact: exact weights times f32.
+enum class ActivationArithmetic : std::uint8_t { kExact = 0, kGgmlQ8 = 1 };
+struct GgufMatVec final { ActivationArithmetic activations = ActivationArithmetic::kExact; };
 
-using Operation = std::variant<Copy, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
+using Operation = std::variant<Copy, Fill, Select, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
                                Q8_0DequantSumSquares, GgufMatVec>;
 
 namespace detail {
@@ -300,6 +338,16 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
   struct Fill {
     hyle_hip_op_desc &r;
     void operator()(const Copy &) const { r.op = HYLE_HIP_OP_COPY; }
+    void operator()(const compute::Fill &o) const {
+      // the scalar's type travels as the output type; a scalar of another type is made invalid here
+      // so that the schema refuses it (src/compute_ops/operation.cc:1263-1275)
+      r.op = HYLE_HIP_OP_FILL;
+      r.kind = o.value.data_type() == o.output_type ? static_cast<std::uint32_t>(o.output_type) : 0u;
+      r.count = o.value.bits();
+      r.inputs[0].rank = static_cast<std::uint8_t>(o.output_shape.size() <= kMaxTensorRank ? o.output_shape.size() : 255);
+      for (std::size_t i = 0; i < o.output_shape.size() && i < kMaxTensorRank; ++i) r.inputs[0].dims[i] = o.output_shape[i];
+    }
+    void operator()(const Select &) const { r.op = HYLE_HIP_OP_SELECT; }
     void operator()(const Cast &o) const { r.op = HYLE_HIP_OP_CAST; r.kind = static_cast<std::uint32_t>(o.output_type); }
     void operator()(const Unary &o) const { r.op = HYLE_HIP_OP_UNARY; r.kind = static_cast<std::uint32_t>(o.kind); }
     void operator()(const Binary &o) const { r.op = HYLE_HIP_OP_BINARY; r.kind = static_cast<std::uint32_t>(o.kind); }
@@ -328,7 +376,7 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
       r.op = HYLE_HIP_OP_BINARY_CHAIN; r.kind = static_cast<std::uint32_t>(o.first); r.kind2 = static_cast<std::uint32_t>(o.second);
     }
     void operator()(const Q8_0DequantSumSquares &) const { r.op = HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ; }
-    void operator()(const GgufMatVec &) const { r.op = HYLE_HIP_OP_GGUF_MATVEC; }
+    void operator()(const GgufMatVec &o) const { r.op = HYLE_HIP_OP_GGUF_MATVEC; r.kind2 = static_cast<std::uint32_t>(o.activations); }
   };
   std::visit(Fill{r}, operation);
   r.input_count = static_cast<std::uint32_t>(count);
@@ -549,12 +597,19 @@ public:
     if (!s.ok()) { (void)hipEventDestroy(event); return s; }
     return Completion(event);
   }
+  Result<Completion> submit(Queue &queue, const TensorView &out) noexcept {
+    return submit(queue, std::initializer_list<ConstTensorView>{}, {out});
+  }
   Result<Completion> submit(Queue &queue, const ConstTensorView &a, const TensorView &out) noexcept {
     return submit(queue, {a}, {out});
   }
   Result<Completion> submit(Queue &queue, const ConstTensorView &a, const ConstTensorView &b,
                             const TensorView &out) noexcept {
     return submit(queue, {a, b}, {out});
+  }
+  Result<Completion> submit(Queue &queue, const ConstTensorView &a, const ConstTensorView &b, const ConstTensorView &c,
+                            const TensorView &out) noexcept {
+    return submit(queue, {a, b, c}, {out});
   }
 private:
   const hyle_hip_plan *plan_;
@@ -581,6 +636,9 @@ inline Result<PreparedOperation> prepare(const Context &context, const Operation
   Status s = detail::from_c(hyle_hip_plan_create(context.handle(), &request, nullptr, 0, &plan));
   if (!s.ok()) return s;
   return PreparedOperation(plan);
+}
+inline Result<PreparedOperation> prepare(const Context &c, const Operation &op) noexcept {
+  return prepare(c, op, std::initializer_list<TensorDesc>{});
 }
 inline Result<PreparedOperation> prepare(const Context &c, const Operation &op, const TensorDesc &a) noexcept {
   return prepare(c, op, {a});

@@ -152,6 +152,33 @@ HOST_TEST(CastAndCopyInferDenseOutputsAndDeclineUndefinedPairs) {
   EXPECT(prepare(context, Cast{DataType::kFloat32}, dense(DataType::kInt32, {2, 8})).has_value());
 }
 
+HOST_TEST(FillAndSelectFollowTheSchema) {
+  const Context context = Context::planning_only();
+  // src/compute_ops/operation.cc:1263-1275
+  auto out = infer_output_descriptions(Fill{{3, 5}, DataType::kFloat32, ScalarValue(1.0F)}, {});
+  REQUIRE(out.has_value());
+  EXPECT((*out)[0] == dense(DataType::kFloat32, {3, 5}));
+  EXPECT(infer_output_descriptions(Fill{{3}, DataType::kBFloat16, ScalarValue(1.0F)}, {}).error().IsInvalidArgument());
+  EXPECT(infer_output_descriptions(Fill{{3}, DataType::kUnknown, ScalarValue()}, {}).error().IsInvalidArgument());
+  auto filled = prepare(context, Fill{{8192, 2048}, DataType::kBFloat16, ScalarValue::from_bits(DataType::kBFloat16, 0x3F80)});
+  REQUIRE(filled.has_value());
+  EXPECT(filled->dispatch_count() == 1);
+  // src/compute_ops/operation.cc:1309-1330
+  out = infer_output_descriptions(Select{}, {dense(DataType::kBool, {4, 1, 6}), dense(DataType::kInt8, {5, 6}),
+                                             dense(DataType::kInt8, {4, 5, 1})});
+  REQUIRE(out.has_value());
+  EXPECT((*out)[0] == dense(DataType::kInt8, {4, 5, 6}));
+  EXPECT(infer_output_descriptions(Select{}, {dense(DataType::kUInt8, {8}), dense(DataType::kFloat32, {8}),
+                                              dense(DataType::kFloat32, {8})}).error().IsInvalidArgument());
+  EXPECT(infer_output_descriptions(Select{}, {dense(DataType::kBool, {8}), dense(DataType::kFloat32, {8}),
+                                              dense(DataType::kFloat16, {8})}).error().IsInvalidArgument());
+  auto selected = prepare(context, Select{}, dense(DataType::kBool, {8, 16}), dense(DataType::kFloat32, {8, 16}),
+                          dense(DataType::kFloat32, {}));
+  REQUIRE(selected.has_value());
+  EXPECT(!selected->alias_support(0, 0)->supported && selected->alias_support(0, 1)->supported &&
+         !selected->alias_support(0, 2)->supported);
+}
+
 HOST_TEST(SubmitWithoutDeviceIsFailedPrecondition) {
   Context context = Context::planning_only();
   EXPECT(context.create_queue().error().IsFailedPrecondition());
@@ -416,6 +443,44 @@ DEVICE_TEST(CastNarrowsWidensAndMaterialisesStridedInputBitExactly) {
   // Cast takes no alias: output over the input is refused
   EXPECT(prepared->create_invocation()->submit(fixture().queue, *ConstTensorView::create(wide, source),
                                                *TensorView::create(narrow, source)).error().IsInvalidArgument());
+}
+
+DEVICE_TEST(FillThenSelectKeepsBitsLikeTheReferenceRouteTest) {
+  // tests/compute_route_vulkan/tensor_test.cc:255-283: alternating flags, a NaN-payload scalar,
+  // Select(mask, input, filled) keeps the input's bits where the flag is set
+  constexpr std::int64_t count = 4099;
+  constexpr std::uint32_t scalar = 0xFFC00003U;
+  std::vector<std::uint32_t> raw(count);
+  std::mt19937 rng(7);
+  for (auto &word : raw) word = rng();
+  std::vector<std::uint8_t> flags(count);
+  for (std::int64_t i = 0; i < count; ++i) flags[i] = static_cast<std::uint8_t>(i % 2);
+  const TensorDesc values = dense(DataType::kFloat32, {count}), mask = dense(DataType::kBool, {count});
+  auto fill = prepare(fixture().context, Fill{{count}, DataType::kFloat32, ScalarValue::from_bits(DataType::kFloat32, scalar)});
+  REQUIRE(fill.has_value());
+  DeviceBuffer filled = DeviceBuffer::create(count * 4).value();
+  auto fill_invocation = fill->create_invocation();
+  REQUIRE(fill_invocation.has_value());
+  auto completion = fill_invocation->submit(fixture().queue, *TensorView::create(values, filled));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  EXPECT(download<std::uint32_t>(filled, count) == std::vector<std::uint32_t>(count, scalar));
+  auto select = prepare(fixture().context, Select{}, mask, values, values);
+  REQUIRE(select.has_value());
+  DeviceBuffer condition = upload(flags), input = upload(raw), out = DeviceBuffer::create(count * 4).value();
+  auto invocation = select->create_invocation();
+  REQUIRE(invocation.has_value());
+  completion = invocation->submit(fixture().queue, *ConstTensorView::create(mask, condition), *ConstTensorView::create(values, input),
+                                  *ConstTensorView::create(values, filled), *TensorView::create(values, out));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<std::uint32_t> want(count);
+  const std::int64_t dims[1] = {count}, byte_stride[1] = {1}, word_stride[1] = {4};
+  const std::vector<std::uint32_t> fill_words(count, scalar);
+  hyle_oracle_select(4, flags.data(), dims, byte_stride, 1, raw.data(), dims, word_stride, 1, fill_words.data(), dims,
+                     word_stride, 1, dims, 1, want.data());
+  for (std::int64_t i = 0; i < count; ++i) EXPECT(want[i] == (flags[i] ? raw[i] : scalar));
+  EXPECT(download<std::uint32_t>(out, count) == want);
 }
 
 DEVICE_TEST(RejectedSubmissionsEnqueueNothing) {
