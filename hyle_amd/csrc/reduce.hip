@@ -63,6 +63,18 @@ __global__ __launch_bounds__(kBlockThreads) void reduce_rows(const void *x, void
       const size_t base = (size_t)row * (width / kVec);
       const uint32_t last = end / kVec;
       uint32_t vec = begin / kVec + lane;
+      for (; vec + 3 * kLanes < last; vec += 4 * kLanes) {
+        u32x4 raw[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) raw[i] = load16_stream(x, base + vec + i * kLanes);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v[kVec];
+          Traits<TIn>::unpack(raw[i], v);
+#pragma unroll
+          for (int j = 0; j < kVec; ++j) acc = reduce_step<kKind>(acc, v[j]);
+        }
+      }
       for (; vec + kLanes < last; vec += 2 * kLanes) {
         u32x4 a = load16_stream(x, base + vec), b = load16_stream(x, base + vec + kLanes);
         float va[kVec], vb[kVec];
