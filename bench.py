@@ -218,7 +218,8 @@ def main() -> int:
             return [raw.to(dev)], [torch.empty((6144, 2048), dtype=torch.bfloat16, device=dev),
                                    torch.empty(6144, dtype=torch.float32, device=dev)]
         ops.append(Op(name, hc.GgufDequantSumSquares(), [hc.TensorDesc.gguf_weight(gguf, BF, 2048, 6144)], set_k, 16,
-                      6144 * (8 * block_bytes + 2048 * 2 + 4), 6144 * 2048, "u8/bf16", in_step=False))
+                      6144 * (8 * block_bytes + 2048 * 2 + 4), 6144 * 2048, "u8/bf16", in_step=False,
+                      ceiling="ceiling_copy_38mb"))
     # ---- decode-time MatMul over GGUF weights: one activation row against [K, N] ----------------
     EXACT, GGML_Q8 = hc.ActivationArithmetic.kExact, hc.ActivationArithmetic.kGgmlQ8
     for name, gguf, block_bytes, k, n_rows, sets, m, arithmetic in (
@@ -298,11 +299,11 @@ def main() -> int:
     # Reduce over the innermost axis, over the leading axis and over every axis (two dispatches
     # that meet in the workspace when there are too few results to fill the chip).
     reduce_lines = (
-        ("next_reduce_sum_rows_bf16", hc.ReductionKind.kSum, [-1], BF, torch.bfloat16, [8192, 2048], 16, 2 * 8192),
-        ("next_reduce_sum_columns_bf16", hc.ReductionKind.kSum, [0], BF, torch.bfloat16, [8192, 2048], 16, 2 * 2048),
-        ("next_reduce_max_all_f32", hc.ReductionKind.kMaximum, None, F32, torch.float32, [4096, 4096], 8, 4),
+        ("next_reduce_sum_rows_bf16", hc.ReductionKind.kSum, [-1], BF, torch.bfloat16, [8192, 2048], 16, 2 * 8192, "ceiling_scan_38mb"),
+        ("next_reduce_sum_columns_bf16", hc.ReductionKind.kSum, [0], BF, torch.bfloat16, [8192, 2048], 16, 2 * 2048, "ceiling_scan_38mb"),
+        ("next_reduce_max_all_f32", hc.ReductionKind.kMaximum, None, F32, torch.float32, [4096, 4096], 8, 4, "ceiling_scan_67mb"),
     )
-    for name, kind, axes, dtype, torch_dtype, dims, sets, out_bytes in reduce_lines:
+    for name, kind, axes, dtype, torch_dtype, dims, sets, out_bytes, ceiling in reduce_lines:
         if not want(name):
             continue
 
@@ -314,14 +315,14 @@ def main() -> int:
         ops.append(Op(name, hc.Reduce(kind, hc.Axes.all() if axes is None else hc.Axes.from_(axes),
                                       accumulation_type=F32),
                       [D(dtype, dims)], set_reduce, sets, dims[0] * dims[1] * size + out_bytes, dims[0] * dims[1],
-                      "f32" if dtype == F32 else "bf16", in_step=False))
+                      "f32" if dtype == F32 else "bf16", in_step=False, ceiling=ceiling))
     if want("next_topk64_f32"):
         def set_topk(i):
             logits = torch.empty((64, 151936), dtype=torch.float32, device=dev).normal_()
             return [logits], [torch.empty((64, 64), dtype=torch.float32, device=dev),
                               torch.empty((64, 64), dtype=torch.int32, device=dev)]
         ops.append(Op("next_topk64_f32", hc.TopK(count=64), [D(F32, [64, 151936])], set_topk, 14,
-                      64 * 151936 * 4 + 64 * 64 * 8, 64 * 151936, "f32", in_step=False))
+                      64 * 151936 * 4 + 64 * 64 * 8, 64 * 151936, "f32", in_step=False, ceiling="ceiling_scan_38mb"))
     if want("next_copy_bf16"):
         def set_copy(i):
             src = torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev).normal_()
