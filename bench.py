@@ -342,6 +342,14 @@ def main() -> int:
             return [mask, src, torch.zeros((), dtype=torch.bfloat16, device=dev)], [torch.empty_like(src)]
         ops.append(Op("next_select_bf16", hc.Select(), [D(hc.DataType.kBool, [8192, 6144]), D(BF, [8192, 6144]), D(BF, [])],
                       set_select, 3, 8192 * 6144 * 5, 8192 * 6144, "bf16", in_step=False))
+    if want("next_concat_bf16"):
+        # a join along the last axis: rows of 4 KiB and 8 KiB interleaved into rows of 12 KiB
+        def set_concat(i):
+            left = torch.empty((8192, 2048), dtype=torch.bfloat16, device=dev).normal_()
+            right = torch.empty((8192, 4096), dtype=torch.bfloat16, device=dev).normal_()
+            return [left, right], [torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev)]
+        ops.append(Op("next_concat_bf16", hc.Concat(-1), [D(BF, [8192, 2048]), D(BF, [8192, 4096])], set_concat, 3,
+                      8192 * 6144 * 4, 8192 * 6144, "bf16", in_step=False))
     # ---- practical ceilings for launches of 38 / 67 MB: a plain copy and a plain read-only scan (a
     # row maximum, one wave per row, one dispatch) of the traffic of the step's small shapes, through
     # the same C ABI and rotated the same way.  Kernels of this size run for 6 - 12 us, of which the

@@ -203,6 +203,7 @@ class OperationKind(enum.IntEnum):
     kRmsNorm = 9
     kLayerNorm = 10
     kGatedActivation = 12
+    kConcat = 15
     kSoftmax = 18
     kTopK = 19
     kBinaryChain = 0x100
@@ -313,6 +314,16 @@ class Fill:
 @dataclass(frozen=True)
 class Select:
     """Inputs (condition Bool, first, second) broadcast together; first where the condition holds."""
+
+
+@dataclass(frozen=True)
+class Concat:
+    """1..4 inputs of one type and rank joined along `axis`.  A wider Concat is issued in groups of
+    four into one output: `total` is then the output's extent on the axis and `start` the place
+    where this group begins."""
+    axis: int = 0
+    total: int = 0
+    start: int = 0
 
 
 @dataclass(frozen=True)
@@ -453,6 +464,8 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
             c.inputs[0].dims[i] = d
     elif isinstance(operation, Select):
         c.op = OperationKind.kSelect
+    elif isinstance(operation, Concat):
+        c.op, c.axis, c.kind, c.count = OperationKind.kConcat, operation.axis, operation.total, operation.start
     elif isinstance(operation, Unary):
         c.op, c.kind = OperationKind.kUnary, int(operation.kind)
     elif isinstance(operation, Binary):

@@ -245,4 +245,19 @@ struct SelectParams {
 hipError_t launch_select(const SelectParams &p, const void *condition, const void *first, const void *second, void *out,
                          bool vector_aligned, hipStream_t stream);
 
+// Concat of `inputs` (1..4) plain tensors along `axis` into a dense output seen as [outer, total,
+// inner]; input i covers [offset[i], offset[i] + extent[i]) of the axis.  dense: every input is
+// dense (runs of extent * inner elements are contiguous), otherwise byte strides per input.
+struct ConcatParams {
+  uint64_t elements = 0;   // of the output
+  uint32_t inputs = 0, outer = 1, inner = 1, total = 0;
+  uint32_t extent[4] = {}, offset[4] = {};
+  uint8_t size = 4;
+  bool dense = true;
+  int32_t rank = 0, axis = 0;
+  uint32_t dims[kMaxRank] = {};
+  int64_t strides[4][kMaxRank] = {};
+};
+hipError_t launch_concat(const ConcatParams &p, const void *const *inputs, void *out, hipStream_t stream);
+
 }  // namespace hyle_hip

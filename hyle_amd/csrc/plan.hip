@@ -295,6 +295,31 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
       if ((s = broadcast_shape(in[0].dims, in[0].rank, branches, branch_rank, dims, &rank)) != HYLE_HIP_OK) return s;
       return make_dense(in[1].dtype, dims, rank, &outs[0]);
     }
+    case HYLE_HIP_OP_CONCAT: {  // src/compute_ops/operation.cc:1516-1564
+      if ((s = expect_inputs(r, 1, HYLE_HIP_MAX_INPUTS)) != HYLE_HIP_OK) return s;
+      int axis;
+      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
+      int64_t dims[HYLE_HIP_MAX_RANK];
+      for (int a = 0; a < in[0].rank; ++a) dims[a] = in[0].dims[a];
+      for (uint32_t i = 1; i < r.input_count; ++i) {
+        if (in[i].dtype != in[0].dtype || in[i].rank != in[0].rank)
+          return fail(HYLE_HIP_INVALID_ARGUMENT, "Concat inputs must have equal data type and rank");
+        for (int a = 0; a < in[0].rank; ++a)
+          if (a != axis && in[i].dims[a] != dims[a])
+            return fail(HYLE_HIP_INVALID_ARGUMENT, "Concat non-axis dimensions must match");
+        if (in[i].dims[axis] > std::numeric_limits<int64_t>::max() - dims[axis])
+          return fail(HYLE_HIP_OUT_OF_RANGE, "Concat axis dimension overflows int64");
+        dims[axis] += in[i].dims[axis];
+      }
+      if (r.kind != 0) {  // one group of a wider Concat: the output's extent and this group's place in it
+        if (r.count > r.kind || (uint64_t)dims[axis] > r.kind - r.count)
+          return fail(HYLE_HIP_INVALID_ARGUMENT, "Concat group does not fit the output's extent on the axis");
+        dims[axis] = (int64_t)r.kind;
+      } else if (r.count != 0) {
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Concat group start needs the output's extent on the axis");
+      }
+      return make_dense(in[0].dtype, dims, in[0].rank, &outs[0]);
+    }
     case HYLE_HIP_OP_CAST: {  // src/compute_ops/operation.cc:1276-1285
       if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
       if (r.kind > 255 || dtype_size((uint8_t)r.kind) == 0 || !is_plain(in[0]))
@@ -509,6 +534,7 @@ enum class Route : uint8_t {
   kCast,
   kFill,
   kSelect,
+  kConcat,
 };
 
 const char *route_name(Route r) {
@@ -528,6 +554,7 @@ const char *route_name(Route r) {
     case Route::kCast: return "cast-copy";
     case Route::kFill: return "fill-pattern";
     case Route::kSelect: return "select";
+    case Route::kConcat: return "concat";
   }
   return "?";
 }
@@ -574,6 +601,9 @@ struct hyle_hip_plan {
   CastParams cast;
   FillParams fill;
   SelectParams select;
+  ConcatParams concat;
+  // Concat takes no alias and no overlap: bytes each input spans, for the launch's check
+  uint64_t concat_input_bytes[HYLE_HIP_MAX_INPUTS] = {0, 0, 0, 0};
   // Cast and Copy take no alias at all (AliasPolicy::kNone, src/compute_ops/operation.cc:935-957):
   // the bytes the input and the output occupy must not overlap.
   uint64_t no_overlap_input_bytes = 0, no_overlap_output_bytes = 0;
@@ -1047,6 +1077,52 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }
+    case HYLE_HIP_OP_CONCAT: {
+      // src/compute_provider_cuda/concat_provider.cc:40-90
+      for (uint32_t i = 0; i < r.input_count; ++i)
+        if (!is_plain(in[i])) return fail(HYLE_HIP_UNIMPLEMENTED, "Concat requires plain inputs and a dense output");
+      const uint64_t n = p->output_elements[0];
+      if (n > kMaxElements) return fail(HYLE_HIP_UNIMPLEMENTED, "Concat output exceeds INT32_MAX elements");
+      if (n == 0) return HYLE_HIP_OK;
+      int axis = 0;
+      normalize_axis(r.axis, out.rank, &axis);
+      ConcatParams &c = p->concat;
+      c.elements = n;
+      c.inputs = r.input_count;
+      c.size = (uint8_t)dtype_size(out.dtype);
+      c.rank = out.rank;
+      c.axis = axis;
+      c.total = (uint32_t)out.dims[axis];
+      c.outer = c.inner = 1;
+      for (int a = 0; a < out.rank; ++a) {
+        c.dims[a] = (uint32_t)out.dims[a];
+        if (a < axis) c.outer *= (uint32_t)out.dims[a];
+        if (a > axis) c.inner *= (uint32_t)out.dims[a];
+      }
+      uint32_t start = (uint32_t)r.count;
+      c.dense = true;
+      bool any = false;
+      for (uint32_t i = 0; i < r.input_count; ++i) {
+        c.extent[i] = (uint32_t)in[i].dims[axis];
+        c.offset[i] = start;
+        start += c.extent[i];
+        any = any || p->input_elements[i] != 0;
+        if (p->input_elements[i] == 0) continue;
+        c.dense = c.dense && is_dense(in[i]);
+        uint64_t last = 0;  // byte offset of the last element: TensorDesc::required_bytes
+        for (int a = 0; a < in[i].rank; ++a) {
+          c.strides[i][a] = in[i].byte_strides[a];
+          last += (uint64_t)(in[i].dims[a] - 1) * (uint64_t)in[i].byte_strides[a];
+        }
+        p->concat_input_bytes[i] = last + c.size;
+      }
+      if (!any) return HYLE_HIP_OK;  // an empty group: nothing to dispatch, no pointer is touched
+      if (!c.dense)
+        for (uint32_t i = 0; i < r.input_count; ++i) p->input_alignment[i] = 1;  // gathered bytewise
+      p->route = Route::kConcat;
+      p->dispatches = 1;
+      return HYLE_HIP_OK;
+    }
     case HYLE_HIP_OP_COPY:
     case HYLE_HIP_OP_CAST: {
       // src/compute_provider_native/cast.cc:127-176,256-279 (admitted pairs, plain input, dense
@@ -1412,6 +1488,18 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
     case Route::kSelect:
       err = launch_select(plan->select, inputs[0], inputs[1], inputs[2], outputs[0], vector, stream);
       break;
+    case Route::kConcat: {
+      const uintptr_t out_first = reinterpret_cast<uintptr_t>(outputs[0]);
+      const uint64_t out_bytes = plan->output_elements[0] * plan->concat.size;
+      for (uint32_t i = 0; i < input_count; ++i) {
+        if (plan->input_elements[i] == 0) continue;
+        const uintptr_t in_first = reinterpret_cast<uintptr_t>(inputs[i]);
+        if (in_first < out_first + out_bytes && out_first < in_first + plan->concat_input_bytes[i])
+          return fail(HYLE_HIP_INVALID_ARGUMENT, "input %u and output storage overlap; Concat takes no alias", i);
+      }
+      err = launch_concat(plan->concat, inputs, outputs[0], stream);
+      break;
+    }
   }
   if (err != hipSuccess) return hip_fail(err, "kernel launch");
   return HYLE_HIP_OK;

@@ -87,6 +87,11 @@ typedef enum hyle_hip_op_kind {
   /* in0 [.., n], optional scale [n], optional bias [n] (bias only with a scale) */
   HYLE_HIP_OP_LAYER_NORM = 10,
   HYLE_HIP_OP_GATED_ACTIVATION = 12,
+  /* Concat: 1..4 inputs of one type and rank joined along `axis` (negative counts from the end).
+   * A caller with more inputs issues one plan per group of four into the same output: `kind` is
+   * then the output's whole extent on the axis (0: the sum of this plan's inputs) and `count` the
+   * place on the axis where this group starts; the plan writes only its own inputs' part. */
+  HYLE_HIP_OP_CONCAT = 15,
   HYLE_HIP_OP_SOFTMAX = 18,
   HYLE_HIP_OP_TOP_K = 19,
   /* Fused forms with no single counterpart in the reference schema; a HYLE
@@ -188,7 +193,7 @@ typedef struct hyle_hip_op_desc {
   uint32_t keep_dimensions;  /* Reduce */
   float epsilon;             /* RmsNorm, LayerNorm */
   float scale;               /* Softmax */
-  uint64_t count;            /* TopK count; Fill: the scalar's bits */
+  uint64_t count;            /* TopK count; Fill: the scalar's bits; Concat: the group's start on the axis */
   uint32_t largest;          /* TopK: 1 = largest first, 0 = smallest first */
   uint32_t input_count;
   hyle_hip_tensor_desc inputs[HYLE_HIP_MAX_INPUTS];

@@ -1335,6 +1335,29 @@ void hyle_oracle_select(size_t width, const void *condition,
   }
 }
 
+/* src/compute_ops/operation.cc:1516-1564 (shape) and the storage rule of
+ * include/hyle/compute/providers/cuda.h:38-43: input `i` (dims equal to the
+ * output's except on `axis`, any byte strides) lands at `offset` on the axis of
+ * the dense output, its `width`-byte elements kept as they are.  One call per
+ * input. */
+void hyle_oracle_concat_part(size_t width, const void *src, const int64_t *dims,
+                             const int64_t *strides, int rank, int axis, int64_t offset,
+                             const int64_t *out_dims, void *dst) {
+  const size_t n = element_count(dims, rank);
+  unsigned char *d = (unsigned char *)dst;
+  for (size_t i = 0; i < n; ++i) {
+    size_t rest = i, to = 0, scale = 1;
+    for (int a = rank - 1; a >= 0; --a) {
+      const size_t c = rest % (size_t)dims[a];
+      rest /= (size_t)dims[a];
+      to += (a == axis ? c + (size_t)offset : c) * scale;
+      scale *= (size_t)out_dims[a];
+    }
+    memcpy(d + to * width,
+           (const unsigned char *)src + hyle_oracle_logical_byte_offset(dims, strides, rank, i), width);
+  }
+}
+
 /* ------------------------------------------------------------------------ */
 /* CPU baseline legs (row ranges, dense loops)                              */
 /* ------------------------------------------------------------------------ */

@@ -340,6 +340,15 @@ void hyle_oracle_select(size_t width, const void *condition,
                         const void *second, const int64_t *second_dims, const int64_t *second_strides, int second_rank,
                         const int64_t *out_dims, int out_rank, void *dst);
 
+/* ---- Concat ------------------------------------------------------------- */
+/* One input of a Concat along `axis` (src/compute_ops/operation.cc:1516-1564):
+ * `dims` / byte `strides` of the input, which equals the dense output's shape
+ * `out_dims` except on the axis, where it starts at `offset`; elements of
+ * `width` bytes are copied bit for bit. */
+void hyle_oracle_concat_part(size_t width, const void *src, const int64_t *dims,
+                             const int64_t *strides, int rank, int axis, int64_t offset,
+                             const int64_t *out_dims, void *dst);
+
 /* ---- CPU baseline legs ---------------------------------------------------
  * The same arithmetic as above in the loop shapes the reference's CPU provider
  * runs (dense rows, no per-element offset walk), over a contiguous row range

@@ -92,6 +92,7 @@ _matvec = _sig("hyle_oracle_gguf_matvec", None, C.c_int, _vp, _sz, _sz, _sz, _vp
 _fill = _sig("hyle_oracle_fill", None, C.c_size_t, C.c_uint64, C.c_size_t, _vp)
 _select = _sig("hyle_oracle_select", None, C.c_size_t, _vp, _i64p, _i64p, C.c_int, _vp, _i64p, _i64p, C.c_int,
                _vp, _i64p, _i64p, C.c_int, _i64p, C.c_int, _vp)
+_concat = _sig("hyle_oracle_concat_part", None, C.c_size_t, _vp, _i64p, _i64p, C.c_int, C.c_int, C.c_int64, _i64p, _vp)
 _cast = _sig("hyle_oracle_cast", C.c_int, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int, _vp)
 
 
@@ -542,4 +543,28 @@ def select(type_id: int, condition, first, second) -> np.ndarray:
     out = np.empty(shape, _NP[type_id])
     _select(width, _ptr(c[0]), _i64(c[1]), _i64(c[2]), len(c[1]), _ptr(a[0]), _i64(a[1]), _i64(a[2]), len(a[1]),
             _ptr(b[0]), _i64(b[1]), _i64(b[2]), len(b[1]), _i64(shape), len(shape), _ptr(out))
+    return out
+
+
+# ---- Concat ---------------------------------------------------------------
+def concat(type_id: int, parts, axis: int, total: int = 0, start: int = 0, into: np.ndarray | None = None) -> np.ndarray:
+    """Concat of `parts` = (storage, dims, byte_strides or None) along `axis`.  `total` / `start`
+    place the group inside a wider output (`into`, written in place) as the C ABI's grouped form
+    does; by default the output is exactly the parts joined."""
+    width = np.dtype(_NP[type_id]).itemsize
+    first = [int(d) for d in parts[0][1]]
+    axis = axis + len(first) if axis < 0 else axis
+    extent = sum(int(p[1][axis]) for p in parts)
+    shape = list(first)
+    shape[axis] = total if total else extent
+    out = into if into is not None else np.zeros(shape, _NP[type_id])
+    at = start
+    for storage, dims, strides in parts:
+        dims = [int(d) for d in dims]
+        if strides is None:
+            strides = _byte_strides(dims, width)
+        raw = np.ascontiguousarray(storage).view(np.uint8).reshape(-1)
+        if int(np.prod(dims)) != 0:
+            _concat(width, _ptr(raw), _i64(dims), _i64([int(x) for x in strides]), len(dims), axis, at, _i64(shape), _ptr(out))
+        at += dims[axis]
     return out

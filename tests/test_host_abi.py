@@ -333,6 +333,25 @@ def test_fill_and_select_inference_and_admission():
     assert err.value.is_unimplemented()
 
 
+def test_concat_inference_and_admission():
+    # src/compute_ops/operation.cc:1516-1564
+    assert hc.infer_output_descriptions(hc.Concat(1), [D(DT.kInt8, [2, 3, 5]), D(DT.kInt8, [2, 0, 5]), D(DT.kInt8, [2, 4, 5])]) \
+        == [D(DT.kInt8, [2, 7, 5])]
+    assert hc.infer_output_descriptions(hc.Concat(-1, total=40, start=8), [D(DT.kFloat32, [3, 8])]) == [D(DT.kFloat32, [3, 40])]
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Concat(2), [D(DT.kFloat32, [3, 8])])
+    assert err.value.is_out_of_range()
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Concat(0), [D(DT.kFloat32, [3, 8]), D(DT.kFloat32, [3, 9])])
+    assert err.value.is_invalid_argument()
+    prepared = hc.prepare(CTX, hc.Concat(0), D(DT.kBFloat16, [8192, 2048]), D(DT.kBFloat16, [64, 2048]))
+    assert prepared.route_name() == "concat" and prepared.dispatch_count() == 1 and prepared.workspace_requirement().size == 0
+    assert hc.prepare(CTX, hc.Concat(0), D(DT.kBFloat16, [0, 2048]), D(DT.kBFloat16, [0, 2048])).dispatch_count() == 0
+    with pytest.raises(hc.StatusError) as err:  # blocked storage is not plain
+        hc.prepare(CTX, hc.Concat(0), hc.TensorDesc.gguf_q8_0_weight(DT.kBFloat16, 64, 2))
+    assert err.value.is_unimplemented()
+
+
 def test_stream_abi_is_exported_and_validates_without_a_device():
     from hyle_amd import capi
     from hyle_amd import file_stream as fs
