@@ -100,6 +100,8 @@ EXPORTS = {
     "hyle_hip_plan_route_name": (C.c_char_p, [C.c_void_p]),
     "hyle_hip_plan_launch": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_uint32, C.POINTER(C.c_void_p),
                                        C.c_uint32, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "hyle_hip_plan_device_status": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
+    "hyle_hip_plan_device_status_offset": (C.c_int, [C.c_void_p, C.POINTER(C.c_size_t)]),
     "hyle_hip_plan_launch_static": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_uint32, C.POINTER(C.c_void_p),
                                               C.c_uint32, C.c_void_p]),
     "hyle_hip_static_scratch_bytes": (C.c_size_t, []),

@@ -74,16 +74,26 @@ GGUF_BLOCKS = {GgufQuantizedType.kQ4K: (256, 144), GgufQuantizedType.kQ6K: (256,
 class DataType(enum.IntEnum):  # include/hyle/compute/tensor_desc.h:17-34
     kUnknown = 0
     kBool = 1
+    kFloat8E4M3FN = 2
+    kFloat8E5M2 = 3
     kFloat16 = 4
     kBFloat16 = 5
     kFloat32 = 6
+    kFloat64 = 7
     kInt8 = 8
     kUInt8 = 9
+    kInt16 = 10
+    kUInt16 = 11
     kInt32 = 12
+    kUInt32 = 13
+    kInt64 = 14
+    kUInt64 = 15
 
 
-_SIZES = {DataType.kBool: 1, DataType.kInt8: 1, DataType.kUInt8: 1, DataType.kFloat16: 2,
-          DataType.kBFloat16: 2, DataType.kFloat32: 4, DataType.kInt32: 4}
+_SIZES = {DataType.kBool: 1, DataType.kFloat8E4M3FN: 1, DataType.kFloat8E5M2: 1, DataType.kInt8: 1, DataType.kUInt8: 1,
+          DataType.kFloat16: 2, DataType.kBFloat16: 2, DataType.kInt16: 2, DataType.kUInt16: 2,
+          DataType.kFloat32: 4, DataType.kInt32: 4, DataType.kUInt32: 4,
+          DataType.kFloat64: 8, DataType.kInt64: 8, DataType.kUInt64: 8}
 
 
 def data_type_size(dtype: DataType) -> int:
@@ -203,6 +213,7 @@ class OperationKind(enum.IntEnum):
     kRmsNorm = 9
     kLayerNorm = 10
     kGatedActivation = 12
+    kGather = 13
     kConcat = 15
     kSoftmax = 18
     kTopK = 19
@@ -288,6 +299,10 @@ class ScalarValue:
             return ScalarValue(data_type, int(np.array(value, np.float32).view(np.uint32)))
         if data_type == DataType.kFloat16:
             return ScalarValue(data_type, int(np.array(value, np.float16).view(np.uint16)))
+        if data_type == DataType.kFloat64:
+            return ScalarValue(data_type, int(np.array(value, np.float64).view(np.uint64)))
+        if data_type in (DataType.kFloat8E4M3FN, DataType.kFloat8E5M2):
+            raise StatusError(capi.INVALID_ARGUMENT, "8-bit float scalars are given by their bits (from_bits)")
         if data_type == DataType.kBFloat16:
             word = int(np.array(value, np.float32).view(np.uint32))
             if (word & 0x7FFFFFFF) > 0x7F800000:
@@ -324,6 +339,20 @@ class Concat:
     axis: int = 0
     total: int = 0
     start: int = 0
+
+
+class IndexBoundsPolicy(enum.IntEnum):  # include/hyle/compute/operation.h:102-105
+    kChecked = 0
+    kUnchecked = 1
+
+
+@dataclass(frozen=True)
+class Gather:
+    """Inputs (source, Int32 / Int64 indices): the source with `axis` replaced by the shape of the
+    indices (include/hyle/compute/operation.h:367-370).  With checked bounds an index outside the
+    axis leaves the output untouched and `OperationInvocation.wait` raises OutOfRange."""
+    axis: int = 0
+    bounds: IndexBoundsPolicy = IndexBoundsPolicy.kChecked
 
 
 @dataclass(frozen=True)
@@ -466,6 +495,8 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
         c.op = OperationKind.kSelect
     elif isinstance(operation, Concat):
         c.op, c.axis, c.kind, c.count = OperationKind.kConcat, operation.axis, operation.total, operation.start
+    elif isinstance(operation, Gather):
+        c.op, c.axis, c.kind2 = OperationKind.kGather, operation.axis, int(operation.bounds)
     elif isinstance(operation, Unary):
         c.op, c.kind = OperationKind.kUnary, int(operation.kind)
     elif isinstance(operation, Binary):
@@ -621,6 +652,13 @@ class OperationInvocation:
         _check(capi.load().hyle_hip_plan_launch(
             self._prepared._handle, self._in, len(inputs), self._out, len(outputs),
             self._workspace, self._workspace_size, stream))
+
+    def wait(self, stream: int, static_scratch: bool = False) -> None:
+        """Completion::wait for launches whose kernels can refuse their input (checked Gather):
+        waits for `stream` and raises StatusError(OutOfRange) when the device said so.  Plans
+        without a device verdict return at once."""
+        _check(capi.load().hyle_hip_plan_device_status(
+            self._prepared._handle, None if static_scratch else self._workspace, stream))
 
     def submit_without_workspace(self, stream: int, inputs: Sequence[int], outputs: Sequence[int]) -> None:
         """The same launch through hyle_hip_plan_launch_static: the route's workspace is the

@@ -38,6 +38,7 @@ __global__ __launch_bounds__(kBlockThreads) void concat_runs(ConcatOperands p, u
     const uint32_t u = (piece * kRunSteps + j) * kBlockThreads + threadIdx.x;
     if (u >= units_per_run) break;
     if constexpr (kUnit == 16) store16_stream(to, u, load16_stream(from, u));
+    else if constexpr (kUnit == 8) reinterpret_cast<uint64_t *>(to)[u] = reinterpret_cast<const uint64_t *>(from)[u];
     else if constexpr (kUnit == 4) reinterpret_cast<uint32_t *>(to)[u] = reinterpret_cast<const uint32_t *>(from)[u];
     else if constexpr (kUnit == 2) reinterpret_cast<uint16_t *>(to)[u] = reinterpret_cast<const uint16_t *>(from)[u];
     else to[u] = from[u];
@@ -111,6 +112,7 @@ hipError_t launch_concat(const ConcatParams &p, const void *const *inputs, void 
     const dim3 grid((uint32_t)blocks, p.inputs), block(kBlockThreads);
     switch (unit) {
       case 16: hipLaunchKernelGGL((concat_runs<16>), grid, block, 0, stream, c, o); break;
+      case 8: hipLaunchKernelGGL((concat_runs<8>), grid, block, 0, stream, c, o); break;
       case 4: hipLaunchKernelGGL((concat_runs<4>), grid, block, 0, stream, c, o); break;
       case 2: hipLaunchKernelGGL((concat_runs<2>), grid, block, 0, stream, c, o); break;
       default: hipLaunchKernelGGL((concat_runs<1>), grid, block, 0, stream, c, o); break;
@@ -130,6 +132,7 @@ hipError_t launch_concat(const ConcatParams &p, const void *const *inputs, void 
   }
   const dim3 grid(blocks_for(most), p.inputs), block(kBlockThreads);
   switch (p.size) {
+    case 8: hipLaunchKernelGGL((concat_general<8>), grid, block, 0, stream, l, o); break;
     case 4: hipLaunchKernelGGL((concat_general<4>), grid, block, 0, stream, l, o); break;
     case 2: hipLaunchKernelGGL((concat_general<2>), grid, block, 0, stream, l, o); break;
     default: hipLaunchKernelGGL((concat_general<1>), grid, block, 0, stream, l, o); break;

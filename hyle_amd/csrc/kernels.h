@@ -222,10 +222,10 @@ struct CastParams {
 hipError_t launch_cast(const CastParams &p, const void *in, void *out, bool vectorised,
                        hipStream_t stream);
 
-// Fill: `elements` elements of `size` bytes (1, 2 or 4) set to the low bytes of `bits`.
+// Fill: `elements` elements of `size` bytes (1, 2, 4 or 8) set to the low bytes of `bits`.
 struct FillParams {
   uint64_t elements = 0;
-  uint32_t bits = 0;
+  uint64_t bits = 0;
   uint8_t size = 4;
 };
 hipError_t launch_fill(const FillParams &p, void *out, hipStream_t stream);
@@ -259,5 +259,31 @@ struct ConcatParams {
   int64_t strides[4][kMaxRank] = {};
 };
 hipError_t launch_concat(const ConcatParams &p, const void *const *inputs, void *out, hipStream_t stream);
+
+// Gather along one axis of a plain source by Int32 / Int64 indices into a dense output seen as
+// [outer, index_count, inner].  rows: the elements after the axis are contiguous and the axes
+// before it fold into outer_pitch, so whole rows move; otherwise the output is walked by
+// coordinate with source_strides / index_out_strides per output axis.  checked: a first dispatch
+// leaves one flag per block in the workspace (32-bit words from its start) and the moving dispatch
+// writes nothing when any is set; word kGatherStatusWord then reads 1, else 0.
+constexpr uint32_t kGatherStatusWord = 256;
+constexpr size_t kGatherWorkspaceBytes = (kGatherStatusWord + 1) * 4;
+struct GatherParams {
+  uint64_t elements = 0;  // of the output
+  uint64_t extent = 0;    // of the source on the axis
+  uint64_t inner = 1;     // elements after the axis
+  uint64_t outer_pitch = 0, axis_pitch = 0;  // bytes
+  uint32_t outer = 1, index_count = 0;
+  uint8_t size = 4;
+  bool wide_indices = false, dense_indices = true, checked = true, rows = false;
+  int32_t index_rank = 0;
+  uint32_t index_dims[kMaxRank] = {};
+  int64_t index_strides[kMaxRank] = {};
+  int32_t rank = 0;  // of the output
+  uint32_t dims[kMaxRank] = {};
+  int64_t source_strides[kMaxRank] = {}, index_out_strides[kMaxRank] = {};
+};
+hipError_t launch_gather(const GatherParams &p, const void *source, const void *indices, void *out, void *workspace,
+                         hipStream_t stream);
 
 }  // namespace hyle_hip

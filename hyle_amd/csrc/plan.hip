@@ -44,21 +44,32 @@ typedef hyle_hip_tensor_desc Desc;
 size_t dtype_size(uint8_t dtype) {
   switch (dtype) {
     case HYLE_HIP_DTYPE_BOOL:
+    case HYLE_HIP_DTYPE_F8_E4M3FN:
+    case HYLE_HIP_DTYPE_F8_E5M2:
     case HYLE_HIP_DTYPE_I8:
     case HYLE_HIP_DTYPE_U8: return 1;
     case HYLE_HIP_DTYPE_F16:
-    case HYLE_HIP_DTYPE_BF16: return 2;
+    case HYLE_HIP_DTYPE_BF16:
+    case HYLE_HIP_DTYPE_I16:
+    case HYLE_HIP_DTYPE_U16: return 2;
     case HYLE_HIP_DTYPE_F32:
-    case HYLE_HIP_DTYPE_I32: return 4;
+    case HYLE_HIP_DTYPE_I32:
+    case HYLE_HIP_DTYPE_U32: return 4;
+    case HYLE_HIP_DTYPE_F64:
+    case HYLE_HIP_DTYPE_I64:
+    case HYLE_HIP_DTYPE_U64: return 8;
     default: return 0;
   }
 }
+bool is_index(uint8_t dtype) { return dtype == HYLE_HIP_DTYPE_I32 || dtype == HYLE_HIP_DTYPE_I64; }
+// The schema's type classes (src/compute_ops/operation.cc:20-56); what the kernels compute in is
+// narrower and decided at admission (to_elem).
 bool is_floating(uint8_t dtype) {
-  return dtype == HYLE_HIP_DTYPE_F16 || dtype == HYLE_HIP_DTYPE_BF16 || dtype == HYLE_HIP_DTYPE_F32;
+  return dtype == HYLE_HIP_DTYPE_F8_E4M3FN || dtype == HYLE_HIP_DTYPE_F8_E5M2 || dtype == HYLE_HIP_DTYPE_F16 ||
+         dtype == HYLE_HIP_DTYPE_BF16 || dtype == HYLE_HIP_DTYPE_F32 || dtype == HYLE_HIP_DTYPE_F64;
 }
 bool is_numeric(uint8_t dtype) {
-  return is_floating(dtype) || dtype == HYLE_HIP_DTYPE_I8 || dtype == HYLE_HIP_DTYPE_U8 ||
-         dtype == HYLE_HIP_DTYPE_I32;
+  return is_floating(dtype) || (dtype >= HYLE_HIP_DTYPE_I8 && dtype <= HYLE_HIP_DTYPE_U64);
 }
 bool to_elem(uint8_t dtype, Elem *out) {
   switch (dtype) {
@@ -465,6 +476,22 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
       }
       return make_dense(in[0].dtype, in[0].dims, in[0].rank, &outs[0]);
     }
+    case HYLE_HIP_OP_GATHER: {  // src/compute_ops/operation.cc:112-118,616-637,1470-1489
+      if ((s = expect_inputs(r, 2, 2)) != HYLE_HIP_OK) return s;
+      if (r.kind2 > HYLE_HIP_BOUNDS_UNCHECKED)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Gather bounds policy is invalid");
+      if (!is_index(in[1].dtype)) return fail(HYLE_HIP_INVALID_ARGUMENT, "Gather indices must use Int32 or Int64");
+      int axis;
+      if ((s = normalize_axis(r.axis, in[0].rank, &axis)) != HYLE_HIP_OK) return s;
+      if (in[0].rank - 1 + in[1].rank > HYLE_HIP_MAX_RANK)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Gather output rank exceeds limit");
+      int64_t dims[HYLE_HIP_MAX_RANK];
+      int rank = 0;
+      for (int a = 0; a < axis; ++a) dims[rank++] = in[0].dims[a];
+      for (int a = 0; a < in[1].rank; ++a) dims[rank++] = in[1].dims[a];
+      for (int a = axis + 1; a < in[0].rank; ++a) dims[rank++] = in[0].dims[a];
+      return make_dense(in[0].dtype, dims, rank, &outs[0]);
+    }
     case HYLE_HIP_OP_TOP_K: {
       if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
       if (!is_numeric(in[0].dtype) || in[0].rank == 0)
@@ -535,6 +562,7 @@ enum class Route : uint8_t {
   kFill,
   kSelect,
   kConcat,
+  kGather,
 };
 
 const char *route_name(Route r) {
@@ -555,6 +583,7 @@ const char *route_name(Route r) {
     case Route::kFill: return "fill-pattern";
     case Route::kSelect: return "select";
     case Route::kConcat: return "concat";
+    case Route::kGather: return "gather";
   }
   return "?";
 }
@@ -602,7 +631,8 @@ struct hyle_hip_plan {
   FillParams fill;
   SelectParams select;
   ConcatParams concat;
-  // Concat takes no alias and no overlap: bytes each input spans, for the launch's check
+  GatherParams gather;
+  // Concat and Gather take no alias and no overlap: bytes each input spans, for the launch's check
   uint64_t concat_input_bytes[HYLE_HIP_MAX_INPUTS] = {0, 0, 0, 0};
   // Cast and Copy take no alias at all (AliasPolicy::kNone, src/compute_ops/operation.cc:935-957):
   // the bytes the input and the output occupy must not overlap.
@@ -1038,7 +1068,7 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->route = Route::kFill;
       p->dispatches = 1;
       p->fill.elements = n;
-      p->fill.bits = (uint32_t)r.count;
+      p->fill.bits = r.count;
       p->fill.size = (uint8_t)size;
       return HYLE_HIP_OK;
     }
@@ -1123,6 +1153,77 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }
+    case HYLE_HIP_OP_GATHER: {
+      // src/compute_provider_cuda/collectives_provider.cc:92-125: plain source and indices, at
+      // most INT32_MAX output elements and indices
+      if (!is_plain(in[0]) || !is_plain(in[1]) || in[0].rank == 0)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Gather requires a plain source of rank >= 1 and plain indices");
+      const uint64_t n = p->output_elements[0];
+      if (n > kMaxElements || p->input_elements[1] > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Gather output or index count exceeds INT32_MAX");
+      if (n == 0) return HYLE_HIP_OK;
+      int axis = 0;
+      normalize_axis(r.axis, in[0].rank, &axis);
+      GatherParams &g = p->gather;
+      const int64_t size = (int64_t)dtype_size(out.dtype);
+      g.elements = n;
+      g.size = (uint8_t)size;
+      g.extent = (uint64_t)in[0].dims[axis];
+      g.wide_indices = in[1].dtype == HYLE_HIP_DTYPE_I64;
+      g.dense_indices = is_dense(in[1]);
+      g.checked = r.kind2 == HYLE_HIP_BOUNDS_CHECKED;
+      g.index_count = (uint32_t)p->input_elements[1];
+      g.index_rank = in[1].rank;
+      for (int a = 0; a < in[1].rank; ++a) {
+        g.index_dims[a] = (uint32_t)in[1].dims[a];
+        g.index_strides[a] = in[1].dims[a] == 1 ? 0 : in[1].byte_strides[a];
+      }
+      g.axis_pitch = (uint64_t)in[0].byte_strides[axis];
+      g.outer = 1;
+      g.inner = 1;
+      for (int a = 0; a < axis; ++a) g.outer *= (uint32_t)in[0].dims[a];
+      for (int a = axis + 1; a < in[0].rank; ++a) g.inner *= (uint64_t)in[0].dims[a];
+      // whole rows move when the elements after the axis are contiguous and the axes before it
+      // fold into one pitch (axes of extent 1 have no say)
+      g.rows = true;
+      int64_t expected = size;
+      for (int a = in[0].rank - 1; a > axis; --a) {
+        if (in[0].dims[a] != 1 && in[0].byte_strides[a] != expected) g.rows = false;
+        expected *= in[0].dims[a];
+      }
+      bool first = true;
+      expected = 0;
+      for (int a = axis - 1; a >= 0; --a) {
+        if (in[0].dims[a] == 1) continue;
+        if (first) g.outer_pitch = (uint64_t)in[0].byte_strides[a];
+        else if (in[0].byte_strides[a] != expected) g.rows = false;
+        first = false;
+        expected = in[0].byte_strides[a] * in[0].dims[a];
+      }
+      // the coordinate walk: per output axis, the source's stride or the indices'
+      g.rank = out.rank;
+      for (int a = 0; a < out.rank; ++a) {
+        g.dims[a] = (uint32_t)out.dims[a];
+        if (a < axis) g.source_strides[a] = in[0].byte_strides[a];
+        else if (a < axis + in[1].rank) g.index_out_strides[a] = g.index_strides[a - axis];
+        else g.source_strides[a] = in[0].byte_strides[a - in[1].rank + 1];
+      }
+      // strided operands may sit at any byte: they are read bytewise
+      if (!is_dense(in[0])) p->input_alignment[0] = 1;
+      if (!g.dense_indices) p->input_alignment[1] = 1;
+      for (int i = 0; i < 2; ++i) {
+        uint64_t last = 0;  // byte offset of the last element: TensorDesc::required_bytes
+        for (int a = 0; a < in[i].rank; ++a) last += (uint64_t)(in[i].dims[a] - 1) * (uint64_t)in[i].byte_strides[a];
+        p->concat_input_bytes[i] = p->input_elements[i] == 0 ? 0 : last + dtype_size(in[i].dtype);
+      }
+      p->route = Route::kGather;
+      p->dispatches = g.checked ? 2 : 1;
+      if (g.checked) {
+        p->workspace_size = kGatherWorkspaceBytes;
+        p->workspace_alignment = 256;
+      }
+      return HYLE_HIP_OK;
+    }
     case HYLE_HIP_OP_COPY:
     case HYLE_HIP_OP_CAST: {
       // src/compute_provider_native/cast.cc:127-176,256-279 (admitted pairs, plain input, dense
@@ -1153,8 +1254,6 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       if (n > kMaxElements)
         return fail(HYLE_HIP_UNIMPLEMENTED, "Cast / Copy output exceeds INT32_MAX elements");
       if (n == 0) return HYLE_HIP_OK;
-      p->route = Route::kCast;
-      p->dispatches = 1;
       c.elements = n;
       c.dense_input = is_dense(in[0]);
       c.rank = in[0].rank;
@@ -1164,6 +1263,18 @@ hyle_hip_status admit(hyle_hip_plan *p) {
         c.strides[a] = in[0].byte_strides[a];
         last += (uint64_t)(in[0].dims[a] - 1) * (uint64_t)in[0].byte_strides[a];
       }
+      if (c.copy_size == 8) {
+        // an 8-byte element moves as two 4-byte halves: one more innermost axis of extent 2
+        if (2 * n > kMaxElements || (!c.dense_input && c.rank == kMaxRank))
+          return fail(HYLE_HIP_UNIMPLEMENTED, "Copy of 8-byte elements exceeds INT32_MAX halves or rank 7 with strides");
+        c.copy_size = 4;
+        c.elements = 2 * n;
+        c.dims[c.rank] = 2;
+        c.strides[c.rank] = 4;
+        c.rank += 1;
+      }
+      p->route = Route::kCast;
+      p->dispatches = 1;
       // byte strides need not keep elements aligned (cast.cc:113-116): such inputs are read bytewise
       if (!c.dense_input) p->input_alignment[0] = 1;
       p->no_overlap_input_bytes = last + dtype_size(in[0].dtype);
@@ -1500,8 +1611,43 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
       err = launch_concat(plan->concat, inputs, outputs[0], stream);
       break;
     }
+    case Route::kGather: {
+      // src/compute_provider_native/indexing.cc:189-195
+      if (plan->gather.extent == 0) return fail(HYLE_HIP_OUT_OF_RANGE, "Gather cannot index an empty axis");
+      const uintptr_t out_first = reinterpret_cast<uintptr_t>(outputs[0]);
+      const uint64_t out_bytes = plan->output_elements[0] * plan->gather.size;
+      for (uint32_t i = 0; i < 2; ++i) {
+        const uintptr_t in_first = reinterpret_cast<uintptr_t>(inputs[i]);
+        if (in_first < out_first + out_bytes && out_first < in_first + plan->concat_input_bytes[i])
+          return fail(HYLE_HIP_INVALID_ARGUMENT, "input %u and output storage overlap; Gather takes no alias", i);
+      }
+      err = launch_gather(plan->gather, inputs[0], inputs[1], outputs[0], workspace, stream);
+      break;
+    }
   }
   if (err != hipSuccess) return hip_fail(err, "kernel launch");
+  return HYLE_HIP_OK;
+}
+
+int hyle_hip_plan_device_status_offset(const hyle_hip_plan *plan, size_t *offset) {
+  if (plan == nullptr || plan->route != Route::kGather || !plan->gather.checked) return 0;
+  if (offset != nullptr) *offset = (size_t)kGatherStatusWord * 4;
+  return 1;
+}
+
+hyle_hip_status hyle_hip_plan_device_status(const hyle_hip_plan *plan, const void *workspace, void *stream_handle) {
+  if (plan == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "plan is null");
+  size_t offset = 0;
+  if (!hyle_hip_plan_device_status_offset(plan, &offset)) return HYLE_HIP_OK;
+  if (workspace == nullptr) workspace = plan->context != nullptr ? plan->context->static_scratch : nullptr;
+  if (workspace == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "workspace is null");
+  hipStream_t stream = static_cast<hipStream_t>(stream_handle);
+  uint32_t word = 0;
+  hipError_t err = hipMemcpyAsync(&word, static_cast<const unsigned char *>(workspace) + offset, sizeof(word),
+                                  hipMemcpyDeviceToHost, stream);
+  if (err == hipSuccess) err = hipStreamSynchronize(stream);
+  if (err != hipSuccess) return hip_fail(err, "reading the device status word");
+  if (word != 0) return fail(HYLE_HIP_OUT_OF_RANGE, "Gather index is outside the selected axis");
   return HYLE_HIP_OK;
 }
 

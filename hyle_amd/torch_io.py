@@ -14,7 +14,11 @@ from . import compute as hc
 _TO_HYLE = {torch.float32: hc.DataType.kFloat32, torch.float16: hc.DataType.kFloat16,
             torch.bfloat16: hc.DataType.kBFloat16, torch.bool: hc.DataType.kBool,
             torch.uint8: hc.DataType.kUInt8, torch.int8: hc.DataType.kInt8,
-            torch.int32: hc.DataType.kInt32}
+            torch.int32: hc.DataType.kInt32, torch.float64: hc.DataType.kFloat64,
+            torch.int16: hc.DataType.kInt16, torch.int64: hc.DataType.kInt64,
+            torch.uint16: hc.DataType.kUInt16, torch.uint32: hc.DataType.kUInt32,
+            torch.uint64: hc.DataType.kUInt64, torch.float8_e4m3fn: hc.DataType.kFloat8E4M3FN,
+            torch.float8_e5m2: hc.DataType.kFloat8E5M2}
 _TO_TORCH = {v: k for k, v in _TO_HYLE.items()}
 
 
@@ -69,4 +73,5 @@ def run(context: hc.Context, operation, *inputs: torch.Tensor, outputs: Optional
     bound.submit(inputs, outs)
     # the workspace must outlive the enqueued kernels
     torch.cuda.current_stream().synchronize()
+    bound.invocation.wait(current_stream_handle())  # the device's verdict, where the route has one
     return outs

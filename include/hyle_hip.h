@@ -54,16 +54,33 @@ typedef enum hyle_hip_status {
   HYLE_HIP_UNAVAILABLE = 14
 } hyle_hip_status;
 
+/* hyle::compute::DataType (include/hyle/compute/tensor_desc.h:17-34).  Arithmetic serves F32 / F16 /
+ * BF16 (TopK also I32, Cast also Bool and I32 sources); every type is storage for the operations
+ * that only move bits (Copy, Fill, Select, Concat, Gather), and I32 / I64 index Gather. */
 typedef enum hyle_hip_dtype {
   HYLE_HIP_DTYPE_UNKNOWN = 0,
   HYLE_HIP_DTYPE_BOOL = 1,
+  HYLE_HIP_DTYPE_F8_E4M3FN = 2,
+  HYLE_HIP_DTYPE_F8_E5M2 = 3,
   HYLE_HIP_DTYPE_F16 = 4,
   HYLE_HIP_DTYPE_BF16 = 5,
   HYLE_HIP_DTYPE_F32 = 6,
+  HYLE_HIP_DTYPE_F64 = 7,
   HYLE_HIP_DTYPE_I8 = 8,
   HYLE_HIP_DTYPE_U8 = 9,
-  HYLE_HIP_DTYPE_I32 = 12
+  HYLE_HIP_DTYPE_I16 = 10,
+  HYLE_HIP_DTYPE_U16 = 11,
+  HYLE_HIP_DTYPE_I32 = 12,
+  HYLE_HIP_DTYPE_U32 = 13,
+  HYLE_HIP_DTYPE_I64 = 14,
+  HYLE_HIP_DTYPE_U64 = 15
 } hyle_hip_dtype;
+
+/* hyle::compute::IndexBoundsPolicy (include/hyle/compute/operation.h:102-105) */
+typedef enum hyle_hip_index_bounds {
+  HYLE_HIP_BOUNDS_CHECKED = 0,
+  HYLE_HIP_BOUNDS_UNCHECKED = 1
+} hyle_hip_index_bounds;
 
 typedef enum hyle_hip_op_kind {
   /* Copy: any plain input (dense or strided) materialised as a dense tensor of the same type.
@@ -87,6 +104,14 @@ typedef enum hyle_hip_op_kind {
   /* in0 [.., n], optional scale [n], optional bias [n] (bias only with a scale) */
   HYLE_HIP_OP_LAYER_NORM = 10,
   HYLE_HIP_OP_GATED_ACTIVATION = 12,
+  /* Gather (include/hyle/compute/operation.h:367-370): in0 a plain source of any storage type,
+   * in1 plain I32 / I64 indices of any rank; out0 is the source with `axis` replaced by the shape
+   * of the indices, bits kept.  `kind2` = hyle_hip_index_bounds.  Checked bounds take two
+   * dispatches and a small workspace: an index below 0 or at / past the axis extent leaves every
+   * byte of the output as it was and shows as OUT_OF_RANGE in hyle_hip_plan_device_status once
+   * the launch has completed.  Unchecked bounds take one dispatch and trust the caller.  No alias:
+   * the output overlaps neither input. */
+  HYLE_HIP_OP_GATHER = 13,
   /* Concat: 1..4 inputs of one type and rank joined along `axis` (negative counts from the end).
    * A caller with more inputs issues one plan per group of four into the same output: `kind` is
    * then the output's whole extent on the axis (0: the sum of this plan's inputs) and `count` the
@@ -186,8 +211,9 @@ typedef struct hyle_hip_op_desc {
   uint32_t op;               /* hyle_hip_op_kind */
   uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind; Cast, Fill: output hyle_hip_dtype */
   uint32_t kind2;            /* BINARY_CHAIN: second BinaryKind; GATED: GatedInputKind;
-                                SOFTMAX: SoftmaxKind; GGUF_MATVEC: HYLE_HIP_ACTIVATIONS_* */
-  int32_t axis;              /* Softmax / TopK axis (negative counts from the end) */
+                                SOFTMAX: SoftmaxKind; GGUF_MATVEC: HYLE_HIP_ACTIVATIONS_*;
+                                GATHER: hyle_hip_index_bounds */
+  int32_t axis;              /* Softmax / TopK / Concat / Gather axis (negative counts from the end) */
   uint32_t mask;             /* Softmax MaskKind */
   uint32_t accumulation;     /* hyle_hip_dtype; UNKNOWN or F32 */
   uint32_t keep_dimensions;  /* Reduce */
@@ -266,6 +292,19 @@ HYLE_HIP_API hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan,
                                                   void *const *outputs, uint32_t output_count,
                                                   void *workspace, size_t workspace_size,
                                                   void *stream);
+
+/* The device-side verdict of a launch whose kernels can refuse their input: checked Gather, whose
+ * reference counterpart fails the Completion with OutOfRange when an index lies outside the axis
+ * (src/compute_provider_cuda/collectives.cu:123-145; tests/compute_provider_cuda/
+ * gather_collectives_test.cc:176-212).  Waits for `stream`, reads the plan's status word from
+ * `workspace` (the one the launch was given; NULL after hyle_hip_plan_launch_static) and returns
+ * OK or OUT_OF_RANGE.  Plans without such a word return OK at once, without waiting.  An adapter
+ * calls this from Completion::wait; hyle_hip_plan_device_status_offset gives the word's place in
+ * the workspace (a uint32, non-zero = refused) for one that prefers its own asynchronous copy,
+ * and returns 0 when the plan has no such word. */
+HYLE_HIP_API hyle_hip_status hyle_hip_plan_device_status(const hyle_hip_plan *plan, const void *workspace,
+                                                         void *stream);
+HYLE_HIP_API int hyle_hip_plan_device_status_offset(const hyle_hip_plan *plan, size_t *offset);
 
 /* hyle_hip_plan_launch for callers that cannot allocate device memory and have no workspace to
  * pass: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It

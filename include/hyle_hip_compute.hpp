@@ -264,6 +264,14 @@ struct Fill final {
 };
 // Inputs (condition Bool, first, second), broadcast together: first where the condition holds.
 struct Select final {};
+// Up to four inputs joined along `axis` (include/hyle/compute/operation.h:384-386).  A wider Concat is
+// prepared as groups of consecutive inputs: `total` is then the output's whole extent along the axis
+// and `start` the extent that precedes the group; both stay 0 when one group is the whole Concat.
+struct Concat final {
+  std::int32_t axis = 0;
+  std::uint64_t total = 0;
+  std::uint64_t start = 0;
+};
 struct Cast final { DataType output_type = DataType::kUnknown; };
 struct Unary final { UnaryKind kind = UnaryKind::kAbs; };
 struct Binary final { BinaryKind kind = BinaryKind::kAdd; };
@@ -326,7 +334,7 @@ using GgufDequantSumSquares = Q8_0DequantSumSquares;
 enum class ActivationArithmetic : std::uint8_t { kExact = 0, kGgmlQ8 = 1 };
 struct GgufMatVec final { ActivationArithmetic activations = ActivationArithmetic::kExact; };
 
-using Operation = std::variant<Copy, Fill, Select, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
+using Operation = std::variant<Copy, Fill, Select, Concat, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
                                Q8_0DequantSumSquares, GgufMatVec>;
 
 namespace detail {
@@ -348,6 +356,9 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
       for (std::size_t i = 0; i < o.output_shape.size() && i < kMaxTensorRank; ++i) r.inputs[0].dims[i] = o.output_shape[i];
     }
     void operator()(const Select &) const { r.op = HYLE_HIP_OP_SELECT; }
+    void operator()(const Concat &o) const {
+      r.op = HYLE_HIP_OP_CONCAT; r.axis = o.axis; r.kind = static_cast<std::uint32_t>(o.total); r.count = o.start;
+    }
     void operator()(const Cast &o) const { r.op = HYLE_HIP_OP_CAST; r.kind = static_cast<std::uint32_t>(o.output_type); }
     void operator()(const Unary &o) const { r.op = HYLE_HIP_OP_UNARY; r.kind = static_cast<std::uint32_t>(o.kind); }
     void operator()(const Binary &o) const { r.op = HYLE_HIP_OP_BINARY; r.kind = static_cast<std::uint32_t>(o.kind); }

@@ -1358,6 +1358,66 @@ void hyle_oracle_concat_part(size_t width, const void *src, const int64_t *dims,
   }
 }
 
+/* ---- Gather -------------------------------------------------------------- */
+/* src/compute_provider_native/indexing.cc:57-91,143-276: the output is the
+ * source with `axis` replaced by the shape of the indices; output element at
+ * coordinates (before, item.., after) is the source element at (before,
+ * indices[item..], after), `width` bytes kept as they are.  Checked bounds look
+ * at every index first: one below 0 or at / past the axis extent returns 1 and
+ * writes nothing (indexing.cc:75-91), as does an axis of extent 0 under either
+ * policy (indexing.cc:189-195). */
+static int64_t read_gather_index(const unsigned char *indices, int wide, size_t offset) {
+  if (wide) {
+    int64_t value;
+    memcpy(&value, indices + offset, sizeof value);
+    return value;
+  }
+  int32_t value;
+  memcpy(&value, indices + offset, sizeof value);
+  return value;
+}
+
+int hyle_oracle_gather(size_t width, const void *src, const int64_t *dims, const int64_t *strides, int rank,
+                       int axis, const void *indices, int wide, const int64_t *index_dims,
+                       const int64_t *index_strides, int index_rank, int checked, void *dst) {
+  int64_t out_dims[16];
+  int out_rank = 0;
+  for (int a = 0; a < axis; ++a) out_dims[out_rank++] = dims[a];
+  for (int a = 0; a < index_rank; ++a) out_dims[out_rank++] = index_dims[a];
+  for (int a = axis + 1; a < rank; ++a) out_dims[out_rank++] = dims[a];
+  const size_t n = element_count(out_dims, out_rank);
+  if (n == 0) return 0;
+  if (dims[axis] == 0) return 1;
+  const size_t index_count = element_count(index_dims, index_rank);
+  const unsigned char *ids = (const unsigned char *)indices;
+  if (checked) {
+    for (size_t i = 0; i < index_count; ++i) {
+      const int64_t value =
+          read_gather_index(ids, wide, hyle_oracle_logical_byte_offset(index_dims, index_strides, index_rank, i));
+      if (value < 0 || (uint64_t)value >= (uint64_t)dims[axis]) return 1;
+    }
+  }
+  unsigned char *d = (unsigned char *)dst;
+  for (size_t i = 0; i < n; ++i) {
+    size_t coordinate[16];
+    size_t rest = i;
+    for (int a = out_rank - 1; a >= 0; --a) {
+      coordinate[a] = rest % (size_t)out_dims[a];
+      rest /= (size_t)out_dims[a];
+    }
+    size_t index_offset = 0;
+    for (int a = 0; a < index_rank; ++a) index_offset += coordinate[axis + a] * (size_t)index_strides[a];
+    const int64_t selected = read_gather_index(ids, wide, index_offset);
+    size_t from = 0;
+    for (int a = 0; a < rank; ++a) {
+      const size_t c = a < axis ? coordinate[a] : a == axis ? (size_t)selected : coordinate[a - 1 + index_rank];
+      from += c * (size_t)strides[a];
+    }
+    memcpy(d + i * width, (const unsigned char *)src + from, width);
+  }
+  return 0;
+}
+
 /* ------------------------------------------------------------------------ */
 /* CPU baseline legs (row ranges, dense loops)                              */
 /* ------------------------------------------------------------------------ */

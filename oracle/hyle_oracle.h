@@ -48,6 +48,11 @@
  *   - fill, select: the reference route test's expectation
  *     (tests/compute_route_vulkan/tensor_test.cc:255-283) and numpy's
  *     broadcasting `where` over raw words.
+ *   - concat_part: numpy.concatenate over raw words in the shape of the
+ *     reference route test (tests/compute_route_vulkan/concat_test.cc:9-88).
+ *   - gather: numpy.take over raw words in the shape of the reference tests
+ *     (tests/compute_provider_cuda/gather_collectives_test.cc,
+ *     collectives_test_support.h:257-314) and their checked-failure cases.
  */
 #ifndef HYLE_ORACLE_H_
 #define HYLE_ORACLE_H_
@@ -348,6 +353,16 @@ void hyle_oracle_select(size_t width, const void *condition,
 void hyle_oracle_concat_part(size_t width, const void *src, const int64_t *dims,
                              const int64_t *strides, int rank, int axis, int64_t offset,
                              const int64_t *out_dims, void *dst);
+
+/* ---- Gather -------------------------------------------------------------- */
+/* Gather along `axis` (src/compute_provider_native/indexing.cc:57-91,143-276):
+ * source `dims` / byte `strides`, Int32 (`wide` = 0) or Int64 indices with their
+ * own dims / byte strides; the dense output has the axis replaced by the shape
+ * of the indices.  Returns 0, or 1 without writing when the bounds are checked
+ * and an index lies outside the axis, or when the axis is empty. */
+int hyle_oracle_gather(size_t width, const void *src, const int64_t *dims, const int64_t *strides, int rank,
+                       int axis, const void *indices, int wide, const int64_t *index_dims,
+                       const int64_t *index_strides, int index_rank, int checked, void *dst);
 
 /* ---- CPU baseline legs ---------------------------------------------------
  * The same arithmetic as above in the loop shapes the reference's CPU provider

@@ -19,7 +19,10 @@ ADD, SUBTRACT, MULTIPLY, DIVIDE, MINIMUM, MAXIMUM = range(6)
 SUM, MEAN, MIN, MAX = range(4)
 MASK_NONE, MASK_ADDITIVE, MASK_BOOLEAN = range(3)
 
-_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16, BOOL: np.uint8, I32: np.int32}
+RAW1, RAW2, RAW4, RAW8 = 10, 11, 12, 13  # storage words for the operations that only move bits
+
+_NP = {F32: np.float32, F16: np.uint16, BF16: np.uint16, BOOL: np.uint8, I32: np.int32,
+       RAW1: np.uint8, RAW2: np.uint16, RAW4: np.uint32, RAW8: np.uint64}
 
 
 def build() -> None:
@@ -92,6 +95,8 @@ _matvec = _sig("hyle_oracle_gguf_matvec", None, C.c_int, _vp, _sz, _sz, _sz, _vp
 _fill = _sig("hyle_oracle_fill", None, C.c_size_t, C.c_uint64, C.c_size_t, _vp)
 _select = _sig("hyle_oracle_select", None, C.c_size_t, _vp, _i64p, _i64p, C.c_int, _vp, _i64p, _i64p, C.c_int,
                _vp, _i64p, _i64p, C.c_int, _i64p, C.c_int, _vp)
+_gather = _sig("hyle_oracle_gather", C.c_int, C.c_size_t, _vp, _i64p, _i64p, C.c_int, C.c_int, _vp, C.c_int, _i64p, _i64p,
+               C.c_int, C.c_int, _vp)
 _concat = _sig("hyle_oracle_concat_part", None, C.c_size_t, _vp, _i64p, _i64p, C.c_int, C.c_int, C.c_int64, _i64p, _vp)
 _cast = _sig("hyle_oracle_cast", C.c_int, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int, _vp)
 
@@ -568,3 +573,26 @@ def concat(type_id: int, parts, axis: int, total: int = 0, start: int = 0, into:
             _concat(width, _ptr(raw), _i64(dims), _i64([int(x) for x in strides]), len(dims), axis, at, _i64(shape), _ptr(out))
         at += dims[axis]
     return out
+
+
+# ---- Gather ---------------------------------------------------------------
+def gather(source: np.ndarray, dims, strides, axis: int, indices: np.ndarray, index_dims, index_strides,
+           checked: bool = True, into: np.ndarray | None = None, width: int | None = None, wide: bool | None = None):
+    """Gather along `axis`.  `source` / `indices` are the storage, described by dims and byte
+    strides (None = dense).  The element width and the index width (`wide` = Int64) come from the
+    arrays' dtypes unless given, as they must be for raw byte storage.  Returns (status, output):
+    status 1 means an index was refused and the output (`into`, or zeros) was left as it was."""
+    width = source.dtype.itemsize if width is None else width
+    wide = indices.dtype.itemsize == 8 if wide is None else wide
+    dims = [int(d) for d in dims]
+    index_dims = [int(d) for d in index_dims]
+    axis = axis + len(dims) if axis < 0 else axis
+    strides = _byte_strides(dims, width) if strides is None else [int(x) for x in strides]
+    index_strides = _byte_strides(index_dims, 8 if wide else 4) if index_strides is None else [int(x) for x in index_strides]
+    shape = dims[:axis] + index_dims + dims[axis + 1:]
+    out = into if into is not None else np.zeros(shape, source.dtype)
+    raw = np.ascontiguousarray(source).view(np.uint8).reshape(-1)
+    ids = np.ascontiguousarray(indices).view(np.uint8).reshape(-1)
+    status = _gather(width, _ptr(raw), _i64(dims), _i64(strides), len(dims), axis, _ptr(ids), 1 if wide else 0,
+                     _i64(index_dims), _i64(index_strides), len(index_dims), 1 if checked else 0, _ptr(out))
+    return status, out

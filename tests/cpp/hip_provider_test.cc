@@ -179,6 +179,27 @@ HOST_TEST(FillAndSelectFollowTheSchema) {
          !selected->alias_support(0, 2)->supported);
 }
 
+HOST_TEST(ConcatFollowsTheSchema) {
+  const Context context = Context::planning_only();
+  // src/compute_ops/operation.cc:1516-1564: equal types and extents off the axis, negative axes count from the end
+  auto out = infer_output_descriptions(Concat{-1}, {dense(DataType::kFloat16, {2, 3, 5}), dense(DataType::kFloat16, {2, 3, 0}),
+                                                    dense(DataType::kFloat16, {2, 3, 7})});
+  REQUIRE(out.has_value());
+  EXPECT((*out)[0] == dense(DataType::kFloat16, {2, 3, 12}));
+  EXPECT(infer_output_descriptions(Concat{0}, {dense(DataType::kFloat16, {2, 3}), dense(DataType::kFloat32, {2, 3})}).error().IsInvalidArgument());
+  EXPECT(infer_output_descriptions(Concat{0}, {dense(DataType::kFloat16, {2, 3}), dense(DataType::kFloat16, {2, 4})}).error().IsInvalidArgument());
+  EXPECT(infer_output_descriptions(Concat{2}, {dense(DataType::kFloat16, {2, 3})}).error().IsOutOfRange());  // operation.cc:228-242
+  // a group of a wider Concat: the output keeps its whole extent, the group says where it starts
+  out = infer_output_descriptions(Concat{1, 20, 9}, {dense(DataType::kInt32, {4, 3}), dense(DataType::kInt32, {4, 5})});
+  REQUIRE(out.has_value());
+  EXPECT((*out)[0] == dense(DataType::kInt32, {4, 20}));
+  EXPECT(infer_output_descriptions(Concat{1, 20, 15}, {dense(DataType::kInt32, {4, 3}), dense(DataType::kInt32, {4, 5})}).error().IsInvalidArgument());
+  auto prepared = prepare(context, Concat{1}, dense(DataType::kBFloat16, {8192, 2048}), dense(DataType::kBFloat16, {8192, 4096}));
+  REQUIRE(prepared.has_value());
+  EXPECT(prepared->dispatch_count() == 1);
+  EXPECT(!prepared->alias_support(0, 0)->supported && !prepared->alias_support(0, 1)->supported);
+}
+
 HOST_TEST(SubmitWithoutDeviceIsFailedPrecondition) {
   Context context = Context::planning_only();
   EXPECT(context.create_queue().error().IsFailedPrecondition());
@@ -481,6 +502,43 @@ DEVICE_TEST(FillThenSelectKeepsBitsLikeTheReferenceRouteTest) {
                      word_stride, 1, dims, 1, want.data());
   for (std::int64_t i = 0; i < count; ++i) EXPECT(want[i] == (flags[i] ? raw[i] : scalar));
   EXPECT(download<std::uint32_t>(out, count) == want);
+}
+
+DEVICE_TEST(ConcatJoinsRawWordsAlongTheMiddleAxis) {
+  // tests/compute_route_vulkan/concat_test.cc:9-70: base [2, 3, 5], parts of 3, 0 and 4 along axis 1
+  const std::int64_t extents[3] = {3, 0, 4}, out_dims[3] = {2, 7, 5};
+  const TensorDesc joined = dense(DataType::kFloat32, {2, 7, 5});
+  std::mt19937 rng(11);
+  std::vector<std::vector<std::uint32_t>> parts;
+  std::vector<DeviceBuffer> buffers;
+  std::vector<TensorDesc> descs;
+  std::vector<std::uint32_t> want(2 * 7 * 5, 0);
+  std::int64_t offset = 0;
+  for (std::int64_t extent : extents) {
+    std::vector<std::uint32_t> words(2 * extent * 5);
+    for (auto &word : words) word = rng();
+    const std::int64_t dims[3] = {2, extent, 5}, strides[3] = {extent * 20, 20, 4};
+    hyle_oracle_concat_part(4, words.data(), dims, strides, 3, 1, offset, out_dims, want.data());
+    offset += extent;
+    descs.push_back(dense(DataType::kFloat32, {2, extent, 5}));
+    buffers.push_back(words.empty() ? DeviceBuffer::create(4).value() : upload(words));
+    parts.push_back(std::move(words));
+  }
+  auto concat = prepare(fixture().context, Concat{1}, descs[0], descs[1], descs[2]);
+  REQUIRE(concat.has_value());
+  DeviceBuffer out = DeviceBuffer::create(want.size() * 4).value();
+  auto invocation = concat->create_invocation();
+  REQUIRE(invocation.has_value());
+  auto completion = invocation->submit(fixture().queue, *ConstTensorView::create(descs[0], buffers[0]),
+                                       *ConstTensorView::create(descs[1], buffers[1]), *ConstTensorView::create(descs[2], buffers[2]),
+                                       *TensorView::create(joined, out));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  for (std::int64_t i = 0; i < 2; ++i)
+    for (std::int64_t j = 0; j < 7; ++j)
+      for (std::int64_t k = 0; k < 5; ++k)
+        EXPECT(want[(i * 7 + j) * 5 + k] == (j < 3 ? parts[0][(i * 3 + j) * 5 + k] : parts[2][(i * 4 + j - 3) * 5 + k]));
+  EXPECT(download<std::uint32_t>(out, want.size()) == want);
 }
 
 DEVICE_TEST(RejectedSubmissionsEnqueueNothing) {

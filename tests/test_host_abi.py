@@ -352,6 +352,61 @@ def test_concat_inference_and_admission():
     assert err.value.is_unimplemented()
 
 
+def test_gather_inference_and_admission():
+    # src/compute_ops/operation.cc:616-637,1470-1489
+    assert hc.infer_output_descriptions(hc.Gather(1), [D(DT.kFloat64, [2, 7, 3]), D(DT.kInt64, [2, 3])]) \
+        == [D(DT.kFloat64, [2, 2, 3, 3])]
+    assert hc.infer_output_descriptions(hc.Gather(-1), [D(DT.kBFloat16, [5, 9]), D(DT.kInt32, [])]) == [D(DT.kBFloat16, [5])]
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Gather(0), [D(DT.kFloat32, [4, 3]), D(DT.kFloat32, [2])])
+    assert err.value.is_invalid_argument()   # indices must be Int32 or Int64
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.Gather(2), [D(DT.kFloat32, [4, 3]), D(DT.kInt32, [2])])
+    assert err.value.is_out_of_range()
+    with pytest.raises(hc.StatusError) as err:  # rank 5 - 1 + 5 > 8
+        hc.infer_output_descriptions(hc.Gather(0), [D(DT.kFloat32, [2] * 5), D(DT.kInt32, [1] * 5)])
+    assert err.value.is_invalid_argument()
+    checked = hc.prepare(CTX, hc.Gather(0), D(DT.kBFloat16, [151936, 2048]), D(DT.kInt32, [8192]))
+    assert checked.route_name() == "gather" and checked.dispatch_count() == 2
+    assert 0 < checked.workspace_requirement().size <= 4096
+    assert not checked.alias_support(0, 0) and not checked.alias_support(0, 1)
+    trusted = hc.prepare(CTX, hc.Gather(0, hc.IndexBoundsPolicy.kUnchecked), D(DT.kBFloat16, [151936, 2048]), D(DT.kInt32, [8192]))
+    assert trusted.dispatch_count() == 1 and trusted.workspace_requirement().size == 0
+    assert hc.prepare(CTX, hc.Gather(0), D(DT.kInt32, [4, 0]), D(DT.kInt32, [4])).dispatch_count() == 0
+    with pytest.raises(hc.StatusError) as err:  # blocked storage is not plain
+        hc.prepare(CTX, hc.Gather(0), hc.TensorDesc.gguf_q8_0_weight(DT.kBFloat16, 64, 2), D(DT.kInt32, [4]))
+    assert err.value.is_unimplemented()
+
+
+def test_every_scalar_type_is_storage_and_only_floats_are_arithmetic():
+    # include/hyle/compute/providers/cuda.h:19-24: Copy / Fill / Select keep 1/2/4/8-byte storage,
+    # arithmetic is FP32 / FP16 / BF16
+    sizes = {DT.kBool: 1, DT.kFloat8E4M3FN: 1, DT.kFloat8E5M2: 1, DT.kInt8: 1, DT.kUInt8: 1, DT.kFloat16: 2, DT.kBFloat16: 2,
+             DT.kInt16: 2, DT.kUInt16: 2, DT.kFloat32: 4, DT.kInt32: 4, DT.kUInt32: 4, DT.kFloat64: 8, DT.kInt64: 8, DT.kUInt64: 8}
+    for kind, size in sizes.items():
+        assert hc.data_type_size(kind) == size
+        d = D(kind, [6, 10])
+        assert d.byte_strides == (10 * size, size)
+        assert hc.prepare(CTX, hc.Copy(), d).dispatch_count() == 1
+        assert hc.prepare(CTX, hc.Copy(), hc.TensorDesc.strided_bytes(kind, [6, 10], [size, 6 * size + 1])).dispatch_count() == 1
+        assert hc.prepare(CTX, hc.Fill((6, 10), kind, hc.ScalarValue.from_bits(kind, 1))).dispatch_count() == 1
+        assert hc.prepare(CTX, hc.Select(), D(DT.kBool, [6, 10]), d, D(kind, [])).dispatch_count() == 1
+        assert hc.prepare(CTX, hc.Concat(0), d, d).dispatch_count() == 1
+        if kind not in (DT.kFloat16, DT.kBFloat16, DT.kFloat32):
+            for operation in (hc.Binary(hc.BinaryKind.kAdd),):
+                with pytest.raises(hc.StatusError) as err:
+                    hc.prepare(CTX, operation, d, d)
+                assert err.value.is_unimplemented()
+            with pytest.raises(hc.StatusError) as err:   # the schema takes every float, the kernels three of them
+                hc.prepare(CTX, hc.Softmax(), d)
+            floating = kind in (DT.kFloat8E4M3FN, DT.kFloat8E5M2, DT.kFloat64)
+            assert err.value.is_unimplemented() if floating else err.value.is_invalid_argument()
+    with pytest.raises(hc.StatusError) as err:   # bits wider than the element
+        hc.prepare(CTX, hc.Fill((4,), DT.kUInt32, hc.ScalarValue.from_bits(DT.kUInt32, 1 << 32)))
+    assert err.value.is_invalid_argument()
+    assert hc.prepare(CTX, hc.Fill((4,), DT.kUInt64, hc.ScalarValue.from_bits(DT.kUInt64, (1 << 64) - 1))).dispatch_count() == 1
+
+
 def test_stream_abi_is_exported_and_validates_without_a_device():
     from hyle_amd import capi
     from hyle_amd import file_stream as fs
