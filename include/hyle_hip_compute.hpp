@@ -100,13 +100,16 @@ inline constexpr std::size_t kMaxTensorRank = HYLE_HIP_MAX_RANK;
 
 // include/hyle/compute/tensor_desc.h:17-34
 enum class DataType : std::uint8_t {
-  kUnknown = 0, kBool = 1, kFloat16 = 4, kBFloat16 = 5, kFloat32 = 6, kInt8 = 8, kUInt8 = 9, kInt32 = 12,
+  kUnknown = 0, kBool = 1, kFloat8E4M3FN = 2, kFloat8E5M2 = 3, kFloat16 = 4, kBFloat16 = 5, kFloat32 = 6, kFloat64 = 7,
+  kInt8 = 8, kUInt8 = 9, kInt16 = 10, kUInt16 = 11, kInt32 = 12, kUInt32 = 13, kInt64 = 14, kUInt64 = 15,
 };
 inline std::size_t data_type_size(DataType type) noexcept {
   switch (type) {
-    case DataType::kBool: case DataType::kInt8: case DataType::kUInt8: return 1;
-    case DataType::kFloat16: case DataType::kBFloat16: return 2;
-    case DataType::kFloat32: case DataType::kInt32: return 4;
+    case DataType::kBool: case DataType::kFloat8E4M3FN: case DataType::kFloat8E5M2: case DataType::kInt8:
+    case DataType::kUInt8: return 1;
+    case DataType::kFloat16: case DataType::kBFloat16: case DataType::kInt16: case DataType::kUInt16: return 2;
+    case DataType::kFloat32: case DataType::kInt32: case DataType::kUInt32: return 4;
+    case DataType::kFloat64: case DataType::kInt64: case DataType::kUInt64: return 8;
     default: return 0;
   }
 }
@@ -272,6 +275,14 @@ struct Concat final {
   std::uint64_t total = 0;
   std::uint64_t start = 0;
 };
+// include/hyle/compute/operation.h:102-105,367-370.  Inputs (source, Int32 / Int64 indices): the
+// source with `axis` replaced by the shape of the indices.  With checked bounds an index outside
+// the axis leaves the output untouched and fails the Completion with OutOfRange.
+enum class IndexBoundsPolicy : std::uint8_t { kChecked = 0, kUnchecked = 1 };
+struct Gather final {
+  std::int32_t axis = 0;
+  IndexBoundsPolicy bounds = IndexBoundsPolicy::kChecked;
+};
 struct Cast final { DataType output_type = DataType::kUnknown; };
 struct Unary final { UnaryKind kind = UnaryKind::kAbs; };
 struct Binary final { BinaryKind kind = BinaryKind::kAdd; };
@@ -334,7 +345,7 @@ using GgufDequantSumSquares = Q8_0DequantSumSquares;
 enum class ActivationArithmetic : std::uint8_t { kExact = 0, kGgmlQ8 = 1 };
 struct GgufMatVec final { ActivationArithmetic activations = ActivationArithmetic::kExact; };
 
-using Operation = std::variant<Copy, Fill, Select, Concat, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
+using Operation = std::variant<Copy, Fill, Select, Concat, Gather, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
                                Q8_0DequantSumSquares, GgufMatVec>;
 
 namespace detail {
@@ -358,6 +369,9 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
     void operator()(const Select &) const { r.op = HYLE_HIP_OP_SELECT; }
     void operator()(const Concat &o) const {
       r.op = HYLE_HIP_OP_CONCAT; r.axis = o.axis; r.kind = static_cast<std::uint32_t>(o.total); r.count = o.start;
+    }
+    void operator()(const Gather &o) const {
+      r.op = HYLE_HIP_OP_GATHER; r.axis = o.axis; r.kind2 = static_cast<std::uint32_t>(o.bounds);
     }
     void operator()(const Cast &o) const { r.op = HYLE_HIP_OP_CAST; r.kind = static_cast<std::uint32_t>(o.output_type); }
     void operator()(const Unary &o) const { r.op = HYLE_HIP_OP_UNARY; r.kind = static_cast<std::uint32_t>(o.kind); }
@@ -490,15 +504,30 @@ private:
 class Completion final {
 public:
   explicit Completion(hipEvent_t event) noexcept : event_(event) {}
-  Completion(Completion &&o) noexcept : event_(o.event_) { o.event_ = nullptr; }
-  Completion &operator=(Completion &&o) noexcept { std::swap(event_, o.event_); return *this; }
+  // A launch whose kernels can refuse their input (checked Gather): the plan's status word in
+  // `workspace` is read once the event has passed.
+  Completion(hipEvent_t event, const hyle_hip_plan *plan, const void *workspace, hipStream_t stream) noexcept
+      : event_(event), plan_(plan), workspace_(workspace), stream_(stream) {}
+  Completion(Completion &&o) noexcept : event_(o.event_), plan_(o.plan_), workspace_(o.workspace_), stream_(o.stream_) {
+    o.event_ = nullptr;
+  }
+  Completion &operator=(Completion &&o) noexcept {
+    std::swap(event_, o.event_); plan_ = o.plan_; workspace_ = o.workspace_; stream_ = o.stream_;
+    return *this;
+  }
   Completion(const Completion &) = delete;
   ~Completion() { if (event_ != nullptr) (void)hipEventDestroy(event_); }
   Status wait() noexcept {
-    return event_ == nullptr ? Status::Ok() : detail::from_hip(hipEventSynchronize(event_), "hipEventSynchronize");
+    if (event_ == nullptr) return Status::Ok();
+    Status s = detail::from_hip(hipEventSynchronize(event_), "hipEventSynchronize");
+    if (!s.ok() || plan_ == nullptr) return s;
+    return detail::from_c(hyle_hip_plan_device_status(plan_, workspace_, stream_));
   }
 private:
   hipEvent_t event_ = nullptr;
+  const hyle_hip_plan *plan_ = nullptr;
+  const void *workspace_ = nullptr;
+  hipStream_t stream_ = nullptr;
 };
 
 class Queue final {  // one HIP stream (src/compute_backend_cuda: stream-per-Queue)
@@ -606,6 +635,7 @@ public:
     if (!s.ok()) return s;
     s = detail::from_hip(hipEventRecord(event, queue.stream()), "hipEventRecord");
     if (!s.ok()) { (void)hipEventDestroy(event); return s; }
+    if (hyle_hip_plan_device_status_offset(plan_, nullptr)) return Completion(event, plan_, workspace_, queue.stream());
     return Completion(event);
   }
   Result<Completion> submit(Queue &queue, const TensorView &out) noexcept {

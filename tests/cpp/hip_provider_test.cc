@@ -200,6 +200,23 @@ HOST_TEST(ConcatFollowsTheSchema) {
   EXPECT(!prepared->alias_support(0, 0)->supported && !prepared->alias_support(0, 1)->supported);
 }
 
+HOST_TEST(GatherFollowsTheSchema) {
+  const Context context = Context::planning_only();
+  // src/compute_ops/operation.cc:616-637,1470-1489
+  auto out = infer_output_descriptions(Gather{1}, {dense(DataType::kFloat64, {2, 7, 3}), dense(DataType::kInt64, {2, 3})});
+  REQUIRE(out.has_value());
+  EXPECT((*out)[0] == dense(DataType::kFloat64, {2, 2, 3, 3}));
+  EXPECT(infer_output_descriptions(Gather{0}, {dense(DataType::kFloat32, {4, 3}), dense(DataType::kFloat32, {2})}).error().IsInvalidArgument());
+  EXPECT(infer_output_descriptions(Gather{2}, {dense(DataType::kFloat32, {4, 3}), dense(DataType::kInt32, {2})}).error().IsOutOfRange());
+  auto checked = prepare(context, Gather{0}, dense(DataType::kBFloat16, {151936, 2048}), dense(DataType::kInt32, {8192}));
+  REQUIRE(checked.has_value());
+  EXPECT(checked->dispatch_count() == 2 && checked->workspace_requirement().size != 0);
+  auto trusted = prepare(context, Gather{0, IndexBoundsPolicy::kUnchecked}, dense(DataType::kBFloat16, {151936, 2048}),
+                         dense(DataType::kInt32, {8192}));
+  REQUIRE(trusted.has_value());
+  EXPECT(trusted->dispatch_count() == 1 && trusted->workspace_requirement().size == 0);
+}
+
 HOST_TEST(SubmitWithoutDeviceIsFailedPrecondition) {
   Context context = Context::planning_only();
   EXPECT(context.create_queue().error().IsFailedPrecondition());
@@ -539,6 +556,48 @@ DEVICE_TEST(ConcatJoinsRawWordsAlongTheMiddleAxis) {
       for (std::int64_t k = 0; k < 5; ++k)
         EXPECT(want[(i * 7 + j) * 5 + k] == (j < 3 ? parts[0][(i * 3 + j) * 5 + k] : parts[2][(i * 4 + j - 3) * 5 + k]));
   EXPECT(download<std::uint32_t>(out, want.size()) == want);
+}
+
+DEVICE_TEST(CheckedGatherFailsTheCompletionAndKeepsTheOutput) {
+  // tests/compute_provider_cuda/gather_collectives_test.cc:172-212: [4, 3] source, two Int64 indices;
+  // -1, the extent, the largest and the smallest index fail with OutOfRange and write nothing
+  const TensorDesc source = dense(DataType::kFloat64, {4, 3}), indices = dense(DataType::kInt64, {2});
+  const std::vector<std::uint64_t> data{1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12}, poison{8, 7, 6, 5, 4, 3};
+  auto gather = prepare(fixture().context, Gather{}, source, indices);
+  REQUIRE(gather.has_value());
+  const TensorDesc result = gather->output_description().value();
+  EXPECT(result == dense(DataType::kFloat64, {2, 3}));
+  DeviceBuffer input = upload(data);
+  DeviceBuffer scratch = DeviceBuffer::create(gather->workspace_requirement().size).value();
+  const std::int64_t dims[2] = {4, 3}, strides[2] = {24, 8}, index_dims[1] = {2}, index_strides[1] = {8};
+  for (std::int64_t invalid : {std::int64_t{-1}, std::int64_t{4}, std::numeric_limits<std::int64_t>::max(),
+                               std::numeric_limits<std::int64_t>::min()}) {
+    const std::vector<std::int64_t> ids{0, invalid};
+    DeviceBuffer picked = upload(ids), out = upload(poison);
+    auto invocation = gather->create_invocation(scratch.data(), scratch.size());
+    REQUIRE(invocation.has_value());
+    auto completion = invocation->submit(fixture().queue, *ConstTensorView::create(source, input),
+                                         *ConstTensorView::create(indices, picked), *TensorView::create(result, out));
+    REQUIRE(completion.has_value());
+    EXPECT(completion->wait().IsOutOfRange());
+    EXPECT(download<std::uint64_t>(out, 6) == poison);
+    std::vector<std::uint64_t> untouched = poison;
+    EXPECT(hyle_oracle_gather(8, data.data(), dims, strides, 2, 0, ids.data(), 1, index_dims, index_strides, 1, 1,
+                              untouched.data()) == 1);
+    EXPECT(untouched == poison);
+  }
+  const std::vector<std::int64_t> ids{3, 1};
+  DeviceBuffer picked = upload(ids), out = upload(poison);
+  auto invocation = gather->create_invocation(scratch.data(), scratch.size());
+  REQUIRE(invocation.has_value());
+  auto completion = invocation->submit(fixture().queue, *ConstTensorView::create(source, input),
+                                       *ConstTensorView::create(indices, picked), *TensorView::create(result, out));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  std::vector<std::uint64_t> want(6);
+  EXPECT(hyle_oracle_gather(8, data.data(), dims, strides, 2, 0, ids.data(), 1, index_dims, index_strides, 1, 1, want.data()) == 0);
+  EXPECT(want == (std::vector<std::uint64_t>{10, 11, 12, 4, 5, 6}));
+  EXPECT(download<std::uint64_t>(out, 6) == want);
 }
 
 DEVICE_TEST(RejectedSubmissionsEnqueueNothing) {

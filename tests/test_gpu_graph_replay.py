@@ -73,8 +73,9 @@ def test_captured_step_replays_bit_identically():
 
 def test_captured_two_dispatch_routes_replay_bit_identically():
     """The routes that pass partial results through the caller's workspace (Reduce over few long
-    rows or over columns, TopK by selection and by sorted tiles), plus Cast, LayerNorm, LogSoftmax
-    and the K-quant decoder: captured once, replayed three times, same bits as eager."""
+    rows or over columns, TopK by selection and by sorted tiles, Gather with checked indices), plus
+    Cast, LayerNorm, LogSoftmax, the K-quant decoder, Concat and Select: captured once, replayed
+    three times, same bits as eager."""
     ctx = context()
     rng = np.random.default_rng(1600)
     f32 = hc.DataType.kFloat32
@@ -86,6 +87,9 @@ def test_captured_two_dispatch_routes_replay_bit_identically():
     raw.view(32, 8, 144)[:, :, 1] &= 0x3B
     raw.view(32, 8, 144)[:, :, 3] &= 0x3B
     weights = raw.to(DEVICE)
+    table = to_device(rng.normal(0, 1, (5000, 256)).astype(np.float32), "f32")
+    ids = torch.from_numpy(rng.integers(0, 5000, 3000).astype(np.int32)).to(DEVICE)
+    flags = torch.from_numpy(rng.integers(0, 2, (64, 2048)).astype(np.uint8)).to(DEVICE).view(torch.bool)
     ops = [
         (hc.Reduce(hc.ReductionKind.kSum, hc.Axes.from_([-1])), [long_rows], None),
         (hc.Reduce(hc.ReductionKind.kMaximum, hc.Axes.from_([0])), [columns], None),
@@ -96,6 +100,9 @@ def test_captured_two_dispatch_routes_replay_bit_identically():
         (hc.Softmax(kind=hc.SoftmaxKind.kLogSoftmax), [hidden], None),
         (hc.GgufDequantSumSquares(), [weights],
          [hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ4K, hc.DataType.kBFloat16, 2048, 32)]),
+        (hc.Gather(0), [table, ids], None),   # checked: the flags of the first dispatch live in the workspace
+        (hc.Concat(-1), [hidden, hidden], None),
+        (hc.Select(), [flags, hidden, torch.zeros((), device=DEVICE)], None),
     ]
     bounds = [(tio.Bound(ctx, op, descs or [tio.desc_of(t) for t in inputs]), inputs) for op, inputs, descs in ops]
     routes = [b.prepared.route_name() for b, _ in bounds]
@@ -128,6 +135,8 @@ def test_captured_two_dispatch_routes_replay_bit_identically():
         assert np.isfinite(scratch)
         graph.replay()
         torch.cuda.synchronize()
+        for bound, _ in bounds:                      # the device's verdict (checked Gather): accepted
+            bound.invocation.wait(tio.current_stream_handle())
         for outs, expected in zip(graph_outs, want):
             for t, e in zip(outs, expected):
                 got = to_host(t)
