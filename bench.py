@@ -365,6 +365,22 @@ def main() -> int:
             ops.append(Op("next_gather_unchecked_bf16", hc.Gather(0, hc.IndexBoundsPolicy.kUnchecked),
                           [D(BF, [151936, 2048]), D(hc.DataType.kInt32, [8192])], set_gather, 8, gather_bytes, 8192 * 2048,
                           "bf16", in_step=False, ceiling="ceiling_copy_67mb"))
+    if want("next_categorical_f32"):
+        # one draw per row of the argmax shape, with the selected log probability: the row is read once
+        def set_categorical(i):
+            logits = torch.empty((64, 151936), dtype=torch.float32, device=dev).normal_(0, 3)
+            ids = torch.randint(0, 1 << 31, (64, 4), dtype=torch.int64, device=dev).to(torch.int32)
+            return [logits, ids], [torch.empty(64, dtype=torch.int32, device=dev), torch.empty(64, dtype=torch.float32, device=dev)]
+        ops.append(Op("next_categorical_f32", hc.Categorical(True), [D(F32, [64, 151936]), D(hc.DataType.kUInt32, [64, 4])],
+                      set_categorical, 16, 64 * 151936 * 4 + 64 * 24, 64 * 151936, "f32", in_step=False,
+                      ceiling="ceiling_scan_38mb"))
+    if want("next_random_bits_u32"):
+        # Philox4x32-10 words: ten rounds of two 32 x 32 -> 64 products per 16 bytes written (integer work, not bytes, bounds it)
+        def set_bits(i):
+            ids = torch.randint(0, 1 << 31, (4096, 4), dtype=torch.int64, device=dev).to(torch.int32)
+            return [ids], [torch.empty((4096, 4096), dtype=torch.int32, device=dev)]
+        ops.append(Op("next_random_bits_u32", hc.RandomBits(4096), [D(hc.DataType.kUInt32, [4096, 4])], set_bits, 4,
+                      4096 * 4096 * 4 + 4096 * 16, 4096 * 4096, "u32", in_step=False))
     # ---- practical ceilings for launches of 38 / 67 MB: a plain copy and a plain read-only scan (a
     # row maximum, one wave per row, one dispatch) of the traffic of the step's small shapes, through
     # the same C ABI and rotated the same way.  Kernels of this size run for 6 - 12 us, of which the

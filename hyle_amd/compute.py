@@ -220,6 +220,8 @@ class OperationKind(enum.IntEnum):
     kBinaryChain = 0x100
     kQ8_0DequantSumSquares = 0x101
     kGgufMatVec = 0x102
+    kRandomBits = 0x103
+    kCategorical = 0x104
 
 
 class UnaryKind(enum.IntEnum):
@@ -473,6 +475,21 @@ class GgufMatVec:
     activations: ActivationArithmetic = ActivationArithmetic.kExact
 
 
+@dataclass(frozen=True)
+class RandomBits:
+    """sampling_ops::RandomBits (include/hyle/compute/sampling_ops.h:12-35): input U32 [R, 4]
+    identities (key low / high, draw low / high); output U32 [R, word_count] Philox4x32-10 words."""
+    word_count: int = 4
+
+
+@dataclass(frozen=True)
+class Categorical:
+    """sampling_ops::Categorical (include/hyle/compute/sampling_ops.h:37-66): inputs (log-weights
+    [R, V], U32 [R, 4] identities); outputs I32 [R] indices and, when asked, F32 [R] normalised log
+    probabilities.  A row without valid mass fails `OperationInvocation.wait` with InvalidArgument."""
+    return_log_probability: bool = False
+
+
 def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
     c = capi.OpDescC()
     c.abi_version = capi.ABI_VERSION
@@ -524,6 +541,12 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
         c.op = OperationKind.kQ8_0DequantSumSquares
     elif isinstance(operation, GgufMatVec):
         c.op, c.kind2 = OperationKind.kGgufMatVec, int(operation.activations)
+    elif isinstance(operation, RandomBits):
+        if operation.word_count < 0:
+            raise StatusError(capi.INVALID_ARGUMENT, "RandomBits word count is negative")
+        c.op, c.count = OperationKind.kRandomBits, operation.word_count
+    elif isinstance(operation, Categorical):
+        c.op, c.kind2 = OperationKind.kCategorical, 1 if operation.return_log_probability else 0
     else:
         raise StatusError(capi.UNIMPLEMENTED, f"operation {type(operation).__name__} is not served by this provider")
     if len(inputs) > capi.MAX_INPUTS:

@@ -66,7 +66,7 @@ struct GatherVerdict {
 __device__ __forceinline__ bool indices_refused(const GatherVerdict &verdict) {
   if (verdict.flags == nullptr) return false;
   const int bad = __syncthreads_or(threadIdx.x < verdict.flag_count ? (int)verdict.flags[threadIdx.x] : 0);
-  if (blockIdx.x == 0 && threadIdx.x == 0) *verdict.status = bad ? 1u : 0u;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *verdict.status = bad ? kStatusIndexOutOfRange : 0u;
   return bad != 0;
 }
 

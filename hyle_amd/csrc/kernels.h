@@ -286,4 +286,30 @@ struct GatherParams {
 hipError_t launch_gather(const GatherParams &p, const void *source, const void *indices, void *out, void *workspace,
                          hipStream_t stream);
 
+// What a status word in the workspace says after a launch whose kernels can refuse their input
+// (the reference's DeviceStatusCode): 0 accepted.
+constexpr uint32_t kStatusIndexOutOfRange = 1, kStatusInvalidNumericInput = 2;
+
+// RandomBits: U32[rows, 4] identities -> U32[rows, word_count] Philox4x32-10 words.
+struct RandomBitsParams {
+  uint32_t rows = 0, word_count = 0;
+};
+hipError_t launch_random_bits(const RandomBitsParams &p, const void *identities, void *out, hipStream_t stream);
+
+// Categorical over dense [rows, width] log-weights: `tiles` tiles of kCategoricalTile elements per
+// row, one CategoricalTile each at the start of the workspace, the status word at status_offset.
+constexpr int kCategoricalTile = 4096;
+struct CategoricalTile {
+  float maximum;     // of the tile (-inf: no finite element)
+  uint32_t invalid;  // the tile holds NaN or +inf
+  double mass;       // sum of exp(x - maximum)
+};
+struct CategoricalParams {
+  uint32_t rows = 0, width = 0, tiles = 0;
+  bool scored = false;  // also the selected element's normalised log probability
+  size_t status_offset = 0;
+};
+hipError_t launch_categorical(Elem type, const CategoricalParams &p, const void *logits, const void *identities, void *indices,
+                              void *scores, void *workspace, bool vector_aligned, hipStream_t stream);
+
 }  // namespace hyle_hip

@@ -492,6 +492,38 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
       for (int a = axis + 1; a < in[0].rank; ++a) dims[rank++] = in[0].dims[a];
       return make_dense(in[0].dtype, dims, rank, &outs[0]);
     }
+    case HYLE_HIP_OP_RANDOM_BITS:
+    case HYLE_HIP_OP_CATEGORICAL: {  // src/compute_ops/sampling_ops.cc:8-63
+      const bool bits = r.op == HYLE_HIP_OP_RANDOM_BITS;
+      if ((s = expect_inputs(r, bits ? 1 : 2, bits ? 1 : 2)) != HYLE_HIP_OK) return s;
+      const Desc &counters = in[bits ? 0 : 1];
+      if (!is_plain(counters) || !is_dense(counters) || counters.dtype != HYLE_HIP_DTYPE_U32 || counters.rank != 2 ||
+          counters.dims[1] != 4)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "sampling counters require dense U32[R,4] key/draw words");
+      if (bits) {
+        if (r.count > (uint64_t)std::numeric_limits<int32_t>::max())
+          return fail(HYLE_HIP_OUT_OF_RANGE, "RandomBits word count exceeds I32");
+        const int64_t dims[2] = {counters.dims[0], (int64_t)r.count};
+        return make_dense(HYLE_HIP_DTYPE_U32, dims, 2, &outs[0]);
+      }
+      if (r.kind2 > 1) return fail(HYLE_HIP_INVALID_ARGUMENT, "Categorical input/output arity differs");
+      const Desc &logits = in[0];
+      if (!is_plain(logits) || !is_dense(logits) || logits.rank != 2 ||
+          (logits.dtype != HYLE_HIP_DTYPE_F16 && logits.dtype != HYLE_HIP_DTYPE_BF16 && logits.dtype != HYLE_HIP_DTYPE_F32))
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Categorical requires dense F16/BF16/F32[R,V] log-weights");
+      if (logits.dims[0] != counters.dims[0])
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "Categorical counter row count differs");
+      if (logits.dims[1] == 0) return fail(HYLE_HIP_INVALID_ARGUMENT, "Categorical requires positive vocabulary");
+      if (logits.dims[1] > (int64_t)std::numeric_limits<int32_t>::max())
+        return fail(HYLE_HIP_OUT_OF_RANGE, "Categorical vocabulary exceeds I32 indices");
+      const int64_t dims[1] = {logits.dims[0]};
+      if ((s = make_dense(HYLE_HIP_DTYPE_I32, dims, 1, &outs[0])) != HYLE_HIP_OK) return s;
+      if (r.kind2 == 1) {
+        *out_count = 2;
+        return make_dense(HYLE_HIP_DTYPE_F32, dims, 1, &outs[1]);
+      }
+      return HYLE_HIP_OK;
+    }
     case HYLE_HIP_OP_TOP_K: {
       if ((s = expect_inputs(r, 1, 1)) != HYLE_HIP_OK) return s;
       if (!is_numeric(in[0].dtype) || in[0].rank == 0)
@@ -563,6 +595,8 @@ enum class Route : uint8_t {
   kSelect,
   kConcat,
   kGather,
+  kRandomBits,
+  kCategorical,
 };
 
 const char *route_name(Route r) {
@@ -584,6 +618,8 @@ const char *route_name(Route r) {
     case Route::kSelect: return "select";
     case Route::kConcat: return "concat";
     case Route::kGather: return "gather";
+    case Route::kRandomBits: return "philox-words";
+    case Route::kCategorical: return "categorical-tiles";
   }
   return "?";
 }
@@ -632,6 +668,8 @@ struct hyle_hip_plan {
   SelectParams select;
   ConcatParams concat;
   GatherParams gather;
+  RandomBitsParams random_bits;
+  CategoricalParams categorical;
   // Concat and Gather take no alias and no overlap: bytes each input spans, for the launch's check
   uint64_t concat_input_bytes[HYLE_HIP_MAX_INPUTS] = {0, 0, 0, 0};
   // Cast and Copy take no alias at all (AliasPolicy::kNone, src/compute_ops/operation.cc:935-957):
@@ -1153,6 +1191,39 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }
+    case HYLE_HIP_OP_RANDOM_BITS: {
+      // src/compute_provider_cuda/sampling_provider.cc:26-71
+      if (p->input_elements[0] / 4 > kMaxElements || p->output_elements[0] > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "RandomBits requires at most INT32_MAX rows and output words");
+      p->input_alignment[0] = 16;  // a row's four identity words are read as one vector
+      if (p->output_elements[0] == 0) return HYLE_HIP_OK;
+      p->route = Route::kRandomBits;
+      p->dispatches = 1;
+      p->random_bits.rows = (uint32_t)in[0].dims[0];
+      p->random_bits.word_count = (uint32_t)r.count;
+      return HYLE_HIP_OK;
+    }
+    case HYLE_HIP_OP_CATEGORICAL: {
+      // src/compute_provider_cuda/sampling_provider.cc:26-71: fixed shapes, row and tile grids within I32
+      if (!to_elem(in[0].dtype, &p->elem)) return fail(HYLE_HIP_UNIMPLEMENTED, "Categorical requires float32/float16/bfloat16");
+      const uint64_t rows = (uint64_t)in[0].dims[0], width = (uint64_t)in[0].dims[1];
+      const uint64_t tiles = (width + kCategoricalTile - 1) / kCategoricalTile;
+      if (rows > kMaxElements || rows * tiles > kMaxElements)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "Categorical row or tile grid capacity exceeded");
+      p->input_alignment[1] = 16;
+      if (rows == 0) return HYLE_HIP_OK;
+      CategoricalParams &c = p->categorical;
+      c.rows = (uint32_t)rows;
+      c.width = (uint32_t)width;
+      c.tiles = (uint32_t)tiles;
+      c.scored = r.kind2 == 1;
+      c.status_offset = (rows * tiles * sizeof(CategoricalTile) + 255) / 256 * 256;
+      p->workspace_size = c.status_offset + 256;
+      p->workspace_alignment = 256;
+      p->route = Route::kCategorical;
+      p->dispatches = 2;
+      return HYLE_HIP_OK;
+    }
     case HYLE_HIP_OP_GATHER: {
       // src/compute_provider_cuda/collectives_provider.cc:92-125: plain source and indices, at
       // most INT32_MAX output elements and indices
@@ -1624,15 +1695,29 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
       err = launch_gather(plan->gather, inputs[0], inputs[1], outputs[0], workspace, stream);
       break;
     }
+    case Route::kRandomBits:
+      err = launch_random_bits(plan->random_bits, inputs[0], outputs[0], stream);
+      break;
+    case Route::kCategorical:
+      err = launch_categorical(plan->elem, plan->categorical, inputs[0], inputs[1], outputs[0],
+                               output_count > 1 ? outputs[1] : nullptr, workspace, aligned(inputs[0], 16), stream);
+      break;
   }
   if (err != hipSuccess) return hip_fail(err, "kernel launch");
   return HYLE_HIP_OK;
 }
 
 int hyle_hip_plan_device_status_offset(const hyle_hip_plan *plan, size_t *offset) {
-  if (plan == nullptr || plan->route != Route::kGather || !plan->gather.checked) return 0;
-  if (offset != nullptr) *offset = (size_t)kGatherStatusWord * 4;
-  return 1;
+  if (plan == nullptr) return 0;
+  if (plan->route == Route::kGather && plan->gather.checked) {
+    if (offset != nullptr) *offset = (size_t)kGatherStatusWord * 4;
+    return 1;
+  }
+  if (plan->route == Route::kCategorical) {
+    if (offset != nullptr) *offset = plan->categorical.status_offset;
+    return 1;
+  }
+  return 0;
 }
 
 hyle_hip_status hyle_hip_plan_device_status(const hyle_hip_plan *plan, const void *workspace, void *stream_handle) {
@@ -1647,7 +1732,10 @@ hyle_hip_status hyle_hip_plan_device_status(const hyle_hip_plan *plan, const voi
                                   hipMemcpyDeviceToHost, stream);
   if (err == hipSuccess) err = hipStreamSynchronize(stream);
   if (err != hipSuccess) return hip_fail(err, "reading the device status word");
-  if (word != 0) return fail(HYLE_HIP_OUT_OF_RANGE, "Gather index is outside the selected axis");
+  if (word == kStatusIndexOutOfRange) return fail(HYLE_HIP_OUT_OF_RANGE, "Gather index is outside the selected axis");
+  if (word == kStatusInvalidNumericInput)
+    return fail(HYLE_HIP_INVALID_ARGUMENT, "Categorical requires valid nonzero row mass");
+  if (word != 0) return fail(HYLE_HIP_INTERNAL, "device status word holds %u", word);
   return HYLE_HIP_OK;
 }
 

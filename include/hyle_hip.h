@@ -140,7 +140,20 @@ typedef enum hyle_hip_op_kind {
    * weight, Q8_K blocks for Q4_K / Q6_K) and the block dot products are integers
    * (tests/compute_models/qwen27_original_nextn_reference.h:94-167,193-257 holds that
    * arithmetic and the bound the reference accepts of it). */
-  HYLE_HIP_OP_GGUF_MATVEC = 0x102
+  HYLE_HIP_OP_GGUF_MATVEC = 0x102,
+  /* sampling_ops::RandomBits (include/hyle/compute/sampling_ops.h:12-35): in0 dense U32 [R, 4]
+   * identities (key low / high, draw low / high), `count` = word_count; out0 dense U32
+   * [R, word_count] of Philox4x32-10 words, word j = lane j % 4 of the block with counter
+   * {j / 4, draw}.  Bit for bit the words of every backend of the reference. */
+  HYLE_HIP_OP_RANDOM_BITS = 0x103,
+  /* sampling_ops::Categorical (include/hyle/compute/sampling_ops.h:37-66): in0 dense F32 / F16 /
+   * BF16 [R, V] log-weights, in1 dense U32 [R, 4] identities; out0 I32 [R] indices and, with
+   * `kind2` = 1, out1 F32 [R] normalised log probabilities of the selected elements.  -Inf is
+   * zero mass.  Two dispatches and a workspace; a row with NaN, +Inf or no finite element writes
+   * nothing and shows as INVALID_ARGUMENT in hyle_hip_plan_device_status.  The draw is the CPU
+   * provider's inverse CDF on the 52-bit uniform of the row's first Philox block; like the
+   * reference's own backends it promises the distribution, not equal indices across backends. */
+  HYLE_HIP_OP_CATEGORICAL = 0x104
 } hyle_hip_op_kind;
 
 /* UnaryKind (include/hyle/compute/operation.h:57-73) */
@@ -212,14 +225,15 @@ typedef struct hyle_hip_op_desc {
   uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind; Cast, Fill: output hyle_hip_dtype */
   uint32_t kind2;            /* BINARY_CHAIN: second BinaryKind; GATED: GatedInputKind;
                                 SOFTMAX: SoftmaxKind; GGUF_MATVEC: HYLE_HIP_ACTIVATIONS_*;
-                                GATHER: hyle_hip_index_bounds */
+                                GATHER: hyle_hip_index_bounds; CATEGORICAL: 1 = also log probabilities */
   int32_t axis;              /* Softmax / TopK / Concat / Gather axis (negative counts from the end) */
   uint32_t mask;             /* Softmax MaskKind */
   uint32_t accumulation;     /* hyle_hip_dtype; UNKNOWN or F32 */
   uint32_t keep_dimensions;  /* Reduce */
   float epsilon;             /* RmsNorm, LayerNorm */
   float scale;               /* Softmax */
-  uint64_t count;            /* TopK count; Fill: the scalar's bits; Concat: the group's start on the axis */
+  uint64_t count;            /* TopK count; Fill: the scalar's bits; Concat: the group's start on the axis;
+                                RandomBits: word_count */
   uint32_t largest;          /* TopK: 1 = largest first, 0 = smallest first */
   uint32_t input_count;
   hyle_hip_tensor_desc inputs[HYLE_HIP_MAX_INPUTS];
@@ -296,9 +310,10 @@ HYLE_HIP_API hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan,
 /* The device-side verdict of a launch whose kernels can refuse their input: checked Gather, whose
  * reference counterpart fails the Completion with OutOfRange when an index lies outside the axis
  * (src/compute_provider_cuda/collectives.cu:123-145; tests/compute_provider_cuda/
- * gather_collectives_test.cc:176-212).  Waits for `stream`, reads the plan's status word from
+ * gather_collectives_test.cc:176-212), and Categorical, which fails it with InvalidArgument for a
+ * row without valid mass (src/compute_provider_cuda/sampling_kernel.cu:47-79).  Waits for `stream`, reads the plan's status word from
  * `workspace` (the one the launch was given; NULL after hyle_hip_plan_launch_static) and returns
- * OK or OUT_OF_RANGE.  Plans without such a word return OK at once, without waiting.  An adapter
+ * OK, OUT_OF_RANGE or INVALID_ARGUMENT.  Plans without such a word return OK at once, without waiting.  An adapter
  * calls this from Completion::wait; hyle_hip_plan_device_status_offset gives the word's place in
  * the workspace (a uint32, non-zero = refused) for one that prefers its own asynchronous copy,
  * and returns 0 when the plan has no such word. */

@@ -1418,6 +1418,104 @@ int hyle_oracle_gather(size_t width, const void *src, const int64_t *dims, const
   return 0;
 }
 
+/* ---- Sampling ------------------------------------------------------------ */
+/* Philox4x32-10 as the reference addresses it (third_party/random123_counter/
+ * philox.h:20-44; include/hyle/compute/sampling_ops.h:12-16): identity = key
+ * low / high, draw low / high; block `index` is the counter {index low, index
+ * high, draw low, draw high} under that key. */
+void hyle_oracle_philox_block(const uint32_t identity[4], uint64_t index, uint32_t out[4]) {
+  uint32_t x0 = (uint32_t)index, x1 = (uint32_t)(index >> 32), x2 = identity[2], x3 = identity[3];
+  uint32_t key0 = identity[0], key1 = identity[1];
+  for (int round = 0; round < 10; ++round) {
+    const uint64_t first = (uint64_t)0xD2511F53u * x0;
+    const uint64_t second = (uint64_t)0xCD9E8D57u * x2;
+    const uint32_t y0 = (uint32_t)(second >> 32) ^ x1 ^ key0;
+    const uint32_t y2 = (uint32_t)(first >> 32) ^ x3 ^ key1;
+    x1 = (uint32_t)second;
+    x3 = (uint32_t)first;
+    x0 = y0;
+    x2 = y2;
+    key0 += 0x9E3779B9u;
+    key1 += 0xBB67AE85u;
+  }
+  out[0] = x0, out[1] = x1, out[2] = x2, out[3] = x3;
+}
+
+/* RandomBits (src/compute_provider_native/sampling.cc:77-88): word j of row r
+ * is lane j % 4 of block j / 4 under the row's identity. */
+void hyle_oracle_random_bits(const uint32_t *identities, size_t rows, size_t word_count, uint32_t *out) {
+  for (size_t r = 0; r < rows; ++r)
+    for (size_t column = 0; column < word_count; column += 4) {
+      uint32_t words[4];
+      hyle_oracle_philox_block(identities + 4 * r, column / 4, words);
+      for (size_t lane = 0; lane < 4 && column + lane < word_count; ++lane) out[r * word_count + column + lane] = words[lane];
+    }
+}
+
+/* The uniform of a row's draw (sampling.cc:155-158): the 52-bit midpoint of the
+ * first two words of block 0, in (0, 1). */
+double hyle_oracle_categorical_uniform(const uint32_t identity[4]) {
+  uint32_t words[4];
+  hyle_oracle_philox_block(identity, 0, words);
+  return ((double)words[0] * 0x1p20 + (double)(words[1] >> 12) + 0.5) * 0x1p-52;
+}
+
+/* Categorical (sampling.cc:119-182,184-215): per row the maximum, the mass
+ * total = sum of expf(x - max) in double, and the first index whose running
+ * mass exceeds total * uniform; a threshold that rounding leaves past the last
+ * boundary selects the last element equal to the maximum.  The optional score
+ * is (x[selected] - max) - log(total) in double, narrowed.  NaN, +Inf or a row
+ * without finite elements returns 1 and writes nothing. */
+static void load_row_f32(int type, const void *base, size_t first, size_t count, float *dst) {
+  const unsigned char *bytes = (const unsigned char *)base + first * type_size(type);
+  for (size_t i = 0; i < count; ++i) dst[i] = load_as_f32(type, bytes + i * type_size(type));
+}
+
+int hyle_oracle_categorical(int type, const void *logits, const uint32_t *identities, size_t rows, size_t width,
+                            int32_t *indices, float *log_probabilities) {
+  float *row = (float *)malloc((width ? width : 1) * sizeof(float));
+  float *maxima = (float *)malloc((rows ? rows : 1) * sizeof(float));
+  int invalid = 0;
+  for (size_t r = 0; r < rows; ++r) {
+    load_row_f32(type, logits, r * width, width, row);
+    float maximum = -INFINITY;
+    for (size_t c = 0; c < width; ++c) {
+      if (isnan(row[c]) || row[c] == INFINITY) invalid = 1;
+      maximum = row[c] > maximum ? row[c] : maximum;
+    }
+    if (!isfinite(maximum)) invalid = 1;
+    maxima[r] = maximum;
+  }
+  for (size_t r = 0; r < rows && !invalid; ++r) {
+    load_row_f32(type, logits, r * width, width, row);
+    const float maximum = maxima[r];
+    double total = 0;
+    for (size_t c = 0; c < width; ++c) total += (double)expf(row[c] - maximum);
+    const double threshold = total * hyle_oracle_categorical_uniform(identities + 4 * r);
+    double cumulative = 0;
+    size_t selected = width;
+    for (size_t c = 0; c < width; ++c) {
+      cumulative += (double)expf(row[c] - maximum);
+      if (cumulative > threshold) {
+        selected = c;
+        break;
+      }
+    }
+    if (selected == width)
+      for (selected = width; selected > 0; --selected)
+        if (row[selected - 1] == maximum) {
+          --selected;
+          break;
+        }
+    indices[r] = (int32_t)selected;
+    if (log_probabilities != NULL)
+      log_probabilities[r] = (float)((double)row[selected] - (double)maximum - log(total));
+  }
+  free(row);
+  free(maxima);
+  return invalid;
+}
+
 /* ------------------------------------------------------------------------ */
 /* CPU baseline legs (row ranges, dense loops)                              */
 /* ------------------------------------------------------------------------ */

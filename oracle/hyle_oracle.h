@@ -50,6 +50,15 @@
  *     broadcasting `where` over raw words.
  *   - concat_part: numpy.concatenate over raw words in the shape of the
  *     reference route test (tests/compute_route_vulkan/concat_test.cc:9-88).
+ *   - philox_block, random_bits: the published Random123 known-answer vectors
+ *     for philox4x32_10 and the independent array form in the reference's
+ *     tests (tests/compute_models/sampling_fixture.h:70-91).
+ *   - categorical: restated from the CPU recipe; checked against a float64
+ *     inverse-CDF in numpy, the reference test's properties (one positive
+ *     mass, row permutation, score within 2e-5 of the float64 normaliser,
+ *     tests/compute_models/sampling_fixture.h:153-283) and its seven-sigma
+ *     quality gate.  Selected indices need not match across the reference's
+ *     own backends (include/hyle/compute/sampling_ops.h:50-55).
  *   - gather: numpy.take over raw words in the shape of the reference tests
  *     (tests/compute_provider_cuda/gather_collectives_test.cc,
  *     collectives_test_support.h:257-314) and their checked-failure cases.
@@ -363,6 +372,22 @@ void hyle_oracle_concat_part(size_t width, const void *src, const int64_t *dims,
 int hyle_oracle_gather(size_t width, const void *src, const int64_t *dims, const int64_t *strides, int rank,
                        int axis, const void *indices, int wide, const int64_t *index_dims,
                        const int64_t *index_strides, int index_rank, int checked, void *dst);
+
+/* ---- Sampling ------------------------------------------------------------ */
+/* Philox4x32-10 under the reference's addressing (third_party/random123_counter/
+ * philox.h:20-44): identity = key low / high, draw low / high; block `index`
+ * holds words 4 * index .. 4 * index + 3 of the row's stream. */
+void hyle_oracle_philox_block(const uint32_t identity[4], uint64_t index, uint32_t out[4]);
+/* RandomBits (src/compute_provider_native/sampling.cc:77-88): identities U32[rows, 4]
+ * -> U32[rows, word_count]. */
+void hyle_oracle_random_bits(const uint32_t *identities, size_t rows, size_t word_count, uint32_t *out);
+/* The uniform in (0, 1) of a row's categorical draw (sampling.cc:155-158). */
+double hyle_oracle_categorical_uniform(const uint32_t identity[4]);
+/* Categorical over dense [rows, width] log-weights of `type` (sampling.cc:119-215):
+ * I32 indices and, when log_probabilities is not NULL, F32 scores.  Returns 0, or 1
+ * without writing when a row holds NaN or +Inf or no finite element. */
+int hyle_oracle_categorical(int type, const void *logits, const uint32_t *identities, size_t rows, size_t width,
+                            int32_t *indices, float *log_probabilities);
 
 /* ---- CPU baseline legs ---------------------------------------------------
  * The same arithmetic as above in the loop shapes the reference's CPU provider

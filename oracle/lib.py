@@ -97,6 +97,11 @@ _select = _sig("hyle_oracle_select", None, C.c_size_t, _vp, _i64p, _i64p, C.c_in
                _vp, _i64p, _i64p, C.c_int, _i64p, C.c_int, _vp)
 _gather = _sig("hyle_oracle_gather", C.c_int, C.c_size_t, _vp, _i64p, _i64p, C.c_int, C.c_int, _vp, C.c_int, _i64p, _i64p,
                C.c_int, C.c_int, _vp)
+_u32p = C.POINTER(C.c_uint32)
+_philox = _sig("hyle_oracle_philox_block", None, _vp, C.c_uint64, _vp)
+_random_bits = _sig("hyle_oracle_random_bits", None, _vp, C.c_size_t, C.c_size_t, _vp)
+_uniform = _sig("hyle_oracle_categorical_uniform", C.c_double, _vp)
+_categorical = _sig("hyle_oracle_categorical", C.c_int, C.c_int, _vp, _vp, C.c_size_t, C.c_size_t, _vp, _vp)
 _concat = _sig("hyle_oracle_concat_part", None, C.c_size_t, _vp, _i64p, _i64p, C.c_int, C.c_int, C.c_int64, _i64p, _vp)
 _cast = _sig("hyle_oracle_cast", C.c_int, C.c_int, C.c_int, _vp, _i64p, _i64p, C.c_int, _vp)
 
@@ -596,3 +601,34 @@ def gather(source: np.ndarray, dims, strides, axis: int, indices: np.ndarray, in
     status = _gather(width, _ptr(raw), _i64(dims), _i64(strides), len(dims), axis, _ptr(ids), 1 if wide else 0,
                      _i64(index_dims), _i64(index_strides), len(index_dims), 1 if checked else 0, _ptr(out))
     return status, out
+
+
+# ---- Sampling -------------------------------------------------------------
+def philox_block(identity, index: int) -> np.ndarray:
+    """Words 4 * index .. 4 * index + 3 of the stream of `identity` = (key low, key high, draw low, draw high)."""
+    ident = np.ascontiguousarray(identity, np.uint32)
+    out = np.empty(4, np.uint32)
+    _philox(_ptr(ident), int(index), _ptr(out))
+    return out
+
+
+def random_bits(identities: np.ndarray, word_count: int) -> np.ndarray:
+    ident = np.ascontiguousarray(identities, np.uint32).reshape(-1, 4)
+    out = np.empty((ident.shape[0], word_count), np.uint32)
+    _random_bits(_ptr(ident), ident.shape[0], word_count, _ptr(out))
+    return out
+
+
+def categorical_uniform(identity) -> float:
+    return float(_uniform(_ptr(np.ascontiguousarray(identity, np.uint32))))
+
+
+def categorical(type_id: int, logits: np.ndarray, identities: np.ndarray, scored: bool = False):
+    """(status, indices, scores or None); status 1: a row without valid mass, nothing written."""
+    logits = _c(logits, _NP[type_id])
+    rows, width = logits.shape
+    ident = np.ascontiguousarray(identities, np.uint32).reshape(rows, 4)
+    indices = np.full(rows, -1, np.int32)
+    scores = np.full(rows, np.nan, np.float32) if scored else None
+    status = _categorical(type_id, _ptr(logits), _ptr(ident), rows, width, _ptr(indices), _ptr(scores))
+    return status, indices, scores
