@@ -345,8 +345,12 @@ using GgufDequantSumSquares = Q8_0DequantSumSquares;
 enum class ActivationArithmetic : std::uint8_t { kExact = 0, kGgmlQ8 = 1 };
 struct GgufMatVec final { ActivationArithmetic activations = ActivationArithmetic::kExact; };
 
+// sampling_ops::RandomBits / Categorical (include/hyle/compute/sampling_ops.h:12-75)
+struct RandomBits final { std::uint32_t word_count = 4; };
+struct Categorical final { bool return_log_probability = false; };
+
 using Operation = std::variant<Copy, Fill, Select, Concat, Gather, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
-                               Q8_0DequantSumSquares, GgufMatVec>;
+                               Q8_0DequantSumSquares, GgufMatVec, RandomBits, Categorical>;
 
 namespace detail {
 inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *inputs, std::size_t count) noexcept {
@@ -402,6 +406,8 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
     }
     void operator()(const Q8_0DequantSumSquares &) const { r.op = HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ; }
     void operator()(const GgufMatVec &o) const { r.op = HYLE_HIP_OP_GGUF_MATVEC; r.kind2 = static_cast<std::uint32_t>(o.activations); }
+    void operator()(const RandomBits &o) const { r.op = HYLE_HIP_OP_RANDOM_BITS; r.count = o.word_count; }
+    void operator()(const Categorical &o) const { r.op = HYLE_HIP_OP_CATEGORICAL; r.kind2 = o.return_log_probability ? 1u : 0u; }
   };
   std::visit(Fill{r}, operation);
   r.input_count = static_cast<std::uint32_t>(count);

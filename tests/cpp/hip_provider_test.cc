@@ -600,6 +600,51 @@ DEVICE_TEST(CheckedGatherFailsTheCompletionAndKeepsTheOutput) {
   EXPECT(download<std::uint64_t>(out, 6) == want);
 }
 
+DEVICE_TEST(CategoricalDrawsTheOraclesIndexAndFailsOnInvalidRows) {
+  // tests/compute_models/sampling_fixture.h:262-283: three rows of seven equal weights, then +Inf, NaN
+  // and an all -Inf row fail with InvalidArgument, and the same key / draw succeeds again unchanged
+  const TensorDesc logits = dense(DataType::kFloat32, {3, 7}), counters = dense(DataType::kUInt32, {3, 4});
+  std::vector<std::uint32_t> identities;
+  for (std::uint32_t row = 0; row < 3; ++row) {
+    const std::uint32_t words[4] = {row * 0x9E3779B9U, 0xFEDCBA98U ^ (row * 17), 73 + row, 0};
+    identities.insert(identities.end(), words, words + 4);
+  }
+  auto draw = prepare(fixture().context, Categorical{true}, logits, counters);
+  REQUIRE(draw.has_value());
+  EXPECT(draw->output_description(1).value() == dense(DataType::kFloat32, {3}));
+  DeviceBuffer scratch = DeviceBuffer::create(draw->workspace_requirement().size).value();
+  DeviceBuffer keys = upload(identities);
+  auto run = [&](const std::vector<float> &values, std::vector<std::int32_t> *picked, std::vector<float> *scores) {
+    DeviceBuffer input = upload(values), ids = upload(std::vector<std::int32_t>(3, -7)), logp = upload(std::vector<float>(3, 0.0F));
+    auto invocation = draw->create_invocation(scratch.data(), scratch.size());
+    auto completion = invocation->submit(fixture().queue, {*ConstTensorView::create(logits, input), *ConstTensorView::create(counters, keys)},
+                                         {*TensorView::create(dense(DataType::kInt32, {3}), ids),
+                                          *TensorView::create(dense(DataType::kFloat32, {3}), logp)});
+    if (!completion.has_value()) return completion.error();
+    Status status = completion->wait();
+    *picked = download<std::int32_t>(ids, 3);
+    *scores = download<float>(logp, 3);
+    return status;
+  };
+  const std::vector<float> valid(21, 0.25F);
+  std::vector<std::int32_t> before, after, want(3);
+  std::vector<float> before_scores, after_scores, want_scores(3);
+  EXPECT(run(valid, &before, &before_scores).ok());
+  EXPECT(hyle_oracle_categorical(HYLE_ORACLE_F32, valid.data(), identities.data(), 3, 7, want.data(), want_scores.data()) == 0);
+  EXPECT(before == want);
+  for (int row = 0; row < 3; ++row) EXPECT(std::fabs(before_scores[row] - want_scores[row]) <= 2e-5F);
+  for (int kind = 0; kind < 3; ++kind) {
+    std::vector<float> bad = valid;
+    if (kind == 0) bad[9] = std::numeric_limits<float>::infinity();
+    if (kind == 1) bad[9] = std::numeric_limits<float>::quiet_NaN();
+    if (kind == 2) std::fill(bad.begin() + 7, bad.begin() + 14, -std::numeric_limits<float>::infinity());
+    EXPECT(run(bad, &after, &after_scores).IsInvalidArgument());
+    EXPECT(hyle_oracle_categorical(HYLE_ORACLE_F32, bad.data(), identities.data(), 3, 7, want.data(), want_scores.data()) == 1);
+    EXPECT(run(valid, &after, &after_scores).ok());
+    EXPECT(after == before && after_scores == before_scores);
+  }
+}
+
 DEVICE_TEST(RejectedSubmissionsEnqueueNothing) {
   const TensorDesc d = dense(DataType::kFloat32, {8, 64}), row = dense(DataType::kFloat32, {64});
   auto prepared = prepare(fixture().context, Binary{BinaryKind::kMultiply}, d, row);

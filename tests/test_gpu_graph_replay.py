@@ -74,8 +74,8 @@ def test_captured_step_replays_bit_identically():
 def test_captured_two_dispatch_routes_replay_bit_identically():
     """The routes that pass partial results through the caller's workspace (Reduce over few long
     rows or over columns, TopK by selection and by sorted tiles, Gather with checked indices), plus
-    Cast, LayerNorm, LogSoftmax, the K-quant decoder, Concat and Select: captured once, replayed
-    three times, same bits as eager."""
+    Cast, LayerNorm, LogSoftmax, the K-quant decoder, Concat, Select, Categorical and RandomBits:
+    captured once, replayed three times, same bits as eager."""
     ctx = context()
     rng = np.random.default_rng(1600)
     f32 = hc.DataType.kFloat32
@@ -90,6 +90,8 @@ def test_captured_two_dispatch_routes_replay_bit_identically():
     table = to_device(rng.normal(0, 1, (5000, 256)).astype(np.float32), "f32")
     ids = torch.from_numpy(rng.integers(0, 5000, 3000).astype(np.int32)).to(DEVICE)
     flags = torch.from_numpy(rng.integers(0, 2, (64, 2048)).astype(np.uint8)).to(DEVICE).view(torch.bool)
+    keys = torch.from_numpy(rng.integers(0, 1 << 31, (4, 4)).astype(np.int32)).to(DEVICE)
+    key_desc = hc.TensorDesc.dense(hc.DataType.kUInt32, [4, 4])
     ops = [
         (hc.Reduce(hc.ReductionKind.kSum, hc.Axes.from_([-1])), [long_rows], None),
         (hc.Reduce(hc.ReductionKind.kMaximum, hc.Axes.from_([0])), [columns], None),
@@ -103,6 +105,8 @@ def test_captured_two_dispatch_routes_replay_bit_identically():
         (hc.Gather(0), [table, ids], None),   # checked: the flags of the first dispatch live in the workspace
         (hc.Concat(-1), [hidden, hidden], None),
         (hc.Select(), [flags, hidden, torch.zeros((), device=DEVICE)], None),
+        (hc.Categorical(True), [logits, keys], [tio.desc_of(logits), key_desc]),   # tile records and the status word
+        (hc.RandomBits(33), [keys], [key_desc]),
     ]
     bounds = [(tio.Bound(ctx, op, descs or [tio.desc_of(t) for t in inputs]), inputs) for op, inputs, descs in ops]
     routes = [b.prepared.route_name() for b, _ in bounds]

@@ -407,6 +407,37 @@ def test_every_scalar_type_is_storage_and_only_floats_are_arithmetic():
     assert hc.prepare(CTX, hc.Fill((4,), DT.kUInt64, hc.ScalarValue.from_bits(DT.kUInt64, (1 << 64) - 1))).dispatch_count() == 1
 
 
+def test_sampling_inference_and_admission():
+    # src/compute_ops/sampling_ops.cc:8-63
+    U32 = DT.kUInt32
+    assert hc.infer_output_descriptions(hc.RandomBits(17), [D(U32, [5, 4])]) == [D(U32, [5, 17])]
+    assert hc.infer_output_descriptions(hc.RandomBits(0), [D(U32, [0, 4])]) == [D(U32, [0, 0])]
+    for bad in (D(U32, [5, 3]), D(DT.kInt32, [5, 4]), D(U32, [20]), hc.TensorDesc.strided_bytes(U32, [5, 4], [32, 4])):
+        with pytest.raises(hc.StatusError) as err:
+            hc.infer_output_descriptions(hc.RandomBits(4), [bad])
+        assert err.value.is_invalid_argument()
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.RandomBits(1 << 31), [D(U32, [5, 4])])
+    assert err.value.is_out_of_range()
+    assert hc.infer_output_descriptions(hc.Categorical(), [D(DT.kBFloat16, [13, 17]), D(U32, [13, 4])]) == [D(DT.kInt32, [13])]
+    assert hc.infer_output_descriptions(hc.Categorical(True), [D(DT.kFloat32, [13, 17]), D(U32, [13, 4])]) \
+        == [D(DT.kInt32, [13]), D(DT.kFloat32, [13])]
+    for logits, counters in ((D(DT.kFloat64, [13, 17]), D(U32, [13, 4])), (D(DT.kFloat32, [13, 17]), D(U32, [12, 4])),
+                             (D(DT.kFloat32, [13, 0]), D(U32, [13, 4])), (D(DT.kFloat32, [13 * 17]), D(U32, [13, 4])),
+                             (hc.TensorDesc.strided_bytes(DT.kFloat32, [13, 17], [128, 4]), D(U32, [13, 4]))):
+        with pytest.raises(hc.StatusError) as err:
+            hc.infer_output_descriptions(hc.Categorical(), [logits, counters])
+        assert err.value.is_invalid_argument()
+    bits = hc.prepare(CTX, hc.RandomBits(4096), D(U32, [4096, 4]))
+    assert bits.route_name() == "philox-words" and bits.dispatch_count() == 1 and bits.workspace_requirement().size == 0
+    assert hc.prepare(CTX, hc.RandomBits(0), D(U32, [7, 4])).dispatch_count() == 0
+    draw = hc.prepare(CTX, hc.Categorical(True), D(DT.kFloat32, [64, 151936]), D(U32, [64, 4]))
+    assert draw.route_name() == "categorical-tiles" and draw.dispatch_count() == 2
+    assert draw.workspace_requirement().size == 64 * 38 * 16 + 256    # a 16-byte record per tile of 4096, then the status word
+    assert not draw.alias_support(0, 0) and not draw.alias_support(1, 0)
+    assert hc.prepare(CTX, hc.Categorical(), D(DT.kFloat32, [0, 7]), D(U32, [0, 4])).dispatch_count() == 0
+
+
 def test_stream_abi_is_exported_and_validates_without_a_device():
     from hyle_amd import capi
     from hyle_amd import file_stream as fs
