@@ -365,6 +365,16 @@ def main() -> int:
             ops.append(Op("next_gather_unchecked_bf16", hc.Gather(0, hc.IndexBoundsPolicy.kUnchecked),
                           [D(BF, [151936, 2048]), D(hc.DataType.kInt32, [8192])], set_gather, 8, gather_bytes, 8192 * 2048,
                           "bf16", in_step=False, ceiling="ceiling_copy_67mb"))
+    if want("next_rope_bf16"):
+        # the queries of a prefill: [1, 8192, 16, 128] bf16 rotated in the half-split layout, one position per step
+        def set_rope(i):
+            x = torch.empty((1, 8192, 16, 128), dtype=torch.bfloat16, device=dev).normal_()
+            positions = torch.arange(8192, dtype=torch.int32, device=dev)
+            frequencies = (1000000.0 ** (-torch.arange(64, dtype=torch.float32, device=dev) / 64.0)).contiguous()
+            return [x, positions, frequencies], [torch.empty_like(x)]
+        ops.append(Op("next_rope_bf16", hc.RoPE(128, 1, hc.RopeLayout.kHalfSplit),
+                      [D(BF, [1, 8192, 16, 128]), D(hc.DataType.kInt32, [8192]), D(F32, [64])], set_rope, 10,
+                      8192 * 16 * 128 * 4 + 8192 * 4 + 256, 8192 * 16 * 128, "bf16", in_step=False, ceiling="ceiling_copy_67mb"))
     if want("next_categorical_f32"):
         # one draw per row of the argmax shape, with the selected log probability: the row is read once
         def set_categorical(i):

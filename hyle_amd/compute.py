@@ -215,6 +215,7 @@ class OperationKind(enum.IntEnum):
     kGatedActivation = 12
     kGather = 13
     kConcat = 15
+    kRoPE = 16
     kSoftmax = 18
     kTopK = 19
     kBinaryChain = 0x100
@@ -475,6 +476,21 @@ class GgufMatVec:
     activations: ActivationArithmetic = ActivationArithmetic.kExact
 
 
+class RopeLayout(enum.IntEnum):  # include/hyle/compute/operation.h:112-115
+    kInterleaved = 0
+    kHalfSplit = 1
+
+
+@dataclass(frozen=True)
+class RoPE:
+    """Inputs (data, Int32 / Int64 positions, F32 frequencies): the first `rotary_dimensions`
+    elements of every row rotated pair by pair through frequency * position
+    (include/hyle/compute/operation.h:388-392)."""
+    rotary_dimensions: int = 0
+    sequence_axis: int = -2
+    layout: RopeLayout = RopeLayout.kInterleaved
+
+
 @dataclass(frozen=True)
 class RandomBits:
     """sampling_ops::RandomBits (include/hyle/compute/sampling_ops.h:12-35): input U32 [R, 4]
@@ -541,6 +557,10 @@ def _op_desc(operation, inputs: Sequence[TensorDesc]) -> capi.OpDescC:
         c.op = OperationKind.kQ8_0DequantSumSquares
     elif isinstance(operation, GgufMatVec):
         c.op, c.kind2 = OperationKind.kGgufMatVec, int(operation.activations)
+    elif isinstance(operation, RoPE):
+        if operation.rotary_dimensions < 0:
+            raise StatusError(capi.INVALID_ARGUMENT, "RoPE rotary dimension must be positive, even and fit the last axis")
+        c.op, c.count, c.axis, c.kind2 = OperationKind.kRoPE, operation.rotary_dimensions, operation.sequence_axis, int(operation.layout)
     elif isinstance(operation, RandomBits):
         if operation.word_count < 0:
             raise StatusError(capi.INVALID_ARGUMENT, "RandomBits word count is negative")

@@ -286,6 +286,17 @@ struct GatherParams {
 hipError_t launch_gather(const GatherParams &p, const void *source, const void *indices, void *out, void *workspace,
                          hipStream_t stream);
 
+// RoPE over a dense tensor seen as `rows` rows of `depth` elements; row r belongs to sequence step
+// (r / inner) % sequence.  Positions are [sequence] or, batched, one per (r / inner); frequencies
+// are f32 [rotary / 2] or, stepped, [sequence, rotary / 2].
+struct RopeParams {
+  uint64_t rows = 0;
+  uint32_t depth = 0, rotary = 0, sequence = 1, inner = 1;
+  bool half_split = false, wide_positions = false, batched_positions = false, stepped_frequencies = false;
+};
+hipError_t launch_rope(Elem type, const RopeParams &p, const void *in, const void *positions, const void *frequencies, void *out,
+                       bool vector_aligned, hipStream_t stream);
+
 // What a status word in the workspace says after a launch whose kernels can refuse their input
 // (the reference's DeviceStatusCode): 0 accepted.
 constexpr uint32_t kStatusIndexOutOfRange = 1, kStatusInvalidNumericInput = 2;

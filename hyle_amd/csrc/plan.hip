@@ -492,6 +492,34 @@ hyle_hip_status infer(const hyle_hip_op_desc &r, Desc *outs, uint32_t *out_count
       for (int a = axis + 1; a < in[0].rank; ++a) dims[rank++] = in[0].dims[a];
       return make_dense(in[0].dtype, dims, rank, &outs[0]);
     }
+    case HYLE_HIP_OP_ROPE: {  // src/compute_ops/operation.cc:127-132,639-696,1566-1574
+      if ((s = expect_inputs(r, 3, 3)) != HYLE_HIP_OK) return s;
+      if (r.kind2 > HYLE_HIP_ROPE_HALF_SPLIT) return fail(HYLE_HIP_INVALID_ARGUMENT, "RoPE layout is invalid");
+      const Desc &data = in[0], &positions = in[1], &frequencies = in[2];
+      if (!is_floating(data.dtype) || !is_floating(frequencies.dtype) || !is_index(positions.dtype))
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "RoPE requires floating data/frequencies and i32/i64 positions");
+      if (data.rank < 2 || r.count == 0 || (r.count & 1u) != 0 || r.count > (uint64_t)data.dims[data.rank - 1])
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "RoPE rotary dimension must be positive, even and fit the last axis");
+      int sequence_axis;
+      if ((s = normalize_axis(r.axis, data.rank, &sequence_axis)) != HYLE_HIP_OK) return s;
+      if (sequence_axis == data.rank - 1)
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "RoPE sequence axis cannot be the rotary depth axis");
+      const int64_t extent = data.dims[sequence_axis];
+      if (positions.rank == 0 || (positions.rank == 1 && positions.dims[0] != extent))
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "RoPE positions must include the complete sequence axis");
+      if (positions.rank > 1) {
+        if (positions.rank != sequence_axis + 1)
+          return fail(HYLE_HIP_INVALID_ARGUMENT, "RoPE batched positions must match the data prefix through sequence");
+        for (int a = 0; a < positions.rank; ++a)
+          if (positions.dims[a] != data.dims[a])
+            return fail(HYLE_HIP_INVALID_ARGUMENT, "RoPE batched position shape does not match data prefix");
+      }
+      if (frequencies.rank == 0 || frequencies.dims[frequencies.rank - 1] != (int64_t)(r.count / 2))
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "RoPE frequency last dimension must equal rotary_dimensions / 2");
+      if (frequencies.rank > 2 || (frequencies.rank == 2 && frequencies.dims[0] != extent))
+        return fail(HYLE_HIP_INVALID_ARGUMENT, "RoPE frequencies must be [pairs] or [sequence,pairs]");
+      return make_dense(data.dtype, data.dims, data.rank, &outs[0]);
+    }
     case HYLE_HIP_OP_RANDOM_BITS:
     case HYLE_HIP_OP_CATEGORICAL: {  // src/compute_ops/sampling_ops.cc:8-63
       const bool bits = r.op == HYLE_HIP_OP_RANDOM_BITS;
@@ -597,6 +625,7 @@ enum class Route : uint8_t {
   kGather,
   kRandomBits,
   kCategorical,
+  kRope,
 };
 
 const char *route_name(Route r) {
@@ -620,6 +649,7 @@ const char *route_name(Route r) {
     case Route::kGather: return "gather";
     case Route::kRandomBits: return "philox-words";
     case Route::kCategorical: return "categorical-tiles";
+    case Route::kRope: return "rope-rows";
   }
   return "?";
 }
@@ -670,6 +700,7 @@ struct hyle_hip_plan {
   GatherParams gather;
   RandomBitsParams random_bits;
   CategoricalParams categorical;
+  RopeParams rope;
   // Concat and Gather take no alias and no overlap: bytes each input spans, for the launch's check
   uint64_t concat_input_bytes[HYLE_HIP_MAX_INPUTS] = {0, 0, 0, 0};
   // Cast and Copy take no alias at all (AliasPolicy::kNone, src/compute_ops/operation.cc:935-957):
@@ -1191,6 +1222,34 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->dispatches = 1;
       return HYLE_HIP_OK;
     }
+    case HYLE_HIP_OP_ROPE: {
+      // the reference's explicit-frequency route takes dense operands and f32 frequencies
+      // (src/compute_ggml_runtime/explicit_rope.h:11-40)
+      if (!to_elem(in[0].dtype, &p->elem) || !is_dense(in[0]) || !is_plain(in[0]))
+        return fail(HYLE_HIP_UNIMPLEMENTED, "RoPE requires dense float32/float16/bfloat16 data");
+      if (!is_plain(in[1]) || !is_dense(in[1]) || !is_plain(in[2]) || !is_dense(in[2]) || in[2].dtype != HYLE_HIP_DTYPE_F32)
+        return fail(HYLE_HIP_UNIMPLEMENTED, "RoPE requires dense positions and dense float32 frequencies");
+      const uint64_t n = p->output_elements[0];
+      if (n > kMaxElements) return fail(HYLE_HIP_UNIMPLEMENTED, "RoPE requires at most INT32_MAX elements");
+      p->alias_inputs[0] = 1;  // a thread reads both elements of its pairs before it writes them
+      if (n == 0) return HYLE_HIP_OK;
+      int sequence_axis = 0;
+      normalize_axis(r.axis, in[0].rank, &sequence_axis);
+      RopeParams &rope = p->rope;
+      rope.depth = (uint32_t)in[0].dims[in[0].rank - 1];
+      rope.rows = n / rope.depth;
+      rope.rotary = (uint32_t)r.count;
+      rope.sequence = (uint32_t)in[0].dims[sequence_axis];
+      rope.inner = 1;
+      for (int a = sequence_axis + 1; a < in[0].rank - 1; ++a) rope.inner *= (uint32_t)in[0].dims[a];
+      rope.half_split = r.kind2 == HYLE_HIP_ROPE_HALF_SPLIT;
+      rope.wide_positions = in[1].dtype == HYLE_HIP_DTYPE_I64;
+      rope.batched_positions = in[1].rank > 1;
+      rope.stepped_frequencies = in[2].rank == 2;
+      p->route = Route::kRope;
+      p->dispatches = 1;
+      return HYLE_HIP_OK;
+    }
     case HYLE_HIP_OP_RANDOM_BITS: {
       // src/compute_provider_cuda/sampling_provider.cc:26-71
       if (p->input_elements[0] / 4 > kMaxElements || p->output_elements[0] > kMaxElements)
@@ -1695,6 +1754,10 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
       err = launch_gather(plan->gather, inputs[0], inputs[1], outputs[0], workspace, stream);
       break;
     }
+    case Route::kRope:
+      err = launch_rope(plan->elem, plan->rope, inputs[0], inputs[1], inputs[2], outputs[0],
+                        aligned(inputs[0], 16) && aligned(outputs[0], 16), stream);
+      break;
     case Route::kRandomBits:
       err = launch_random_bits(plan->random_bits, inputs[0], outputs[0], stream);
       break;

@@ -76,6 +76,13 @@ typedef enum hyle_hip_dtype {
   HYLE_HIP_DTYPE_U64 = 15
 } hyle_hip_dtype;
 
+/* hyle::compute::RopeLayout (include/hyle/compute/operation.h:112-115): pairs are (2i, 2i + 1) or
+ * (i, i + rotary / 2). */
+typedef enum hyle_hip_rope_layout {
+  HYLE_HIP_ROPE_INTERLEAVED = 0,
+  HYLE_HIP_ROPE_HALF_SPLIT = 1
+} hyle_hip_rope_layout;
+
 /* hyle::compute::IndexBoundsPolicy (include/hyle/compute/operation.h:102-105) */
 typedef enum hyle_hip_index_bounds {
   HYLE_HIP_BOUNDS_CHECKED = 0,
@@ -117,6 +124,13 @@ typedef enum hyle_hip_op_kind {
    * then the output's whole extent on the axis (0: the sum of this plan's inputs) and `count` the
    * place on the axis where this group starts; the plan writes only its own inputs' part. */
   HYLE_HIP_OP_CONCAT = 15,
+  /* RoPE (include/hyle/compute/operation.h:388-392): in0 dense F32 / F16 / BF16 data of rank >= 2,
+   * in1 dense I32 / I64 positions ([S] or the data's leading dimensions through the sequence
+   * axis), in2 dense F32 frequencies ([rotary / 2] or [S, rotary / 2]); out0 like in0.  `count` =
+   * rotary_dimensions (positive, even, at most the last extent), `axis` = sequence_axis (not the
+   * last), `kind2` = hyle_hip_rope_layout.  Arithmetic in f32 with phase = frequency * f32(position);
+   * elements past rotary_dimensions pass through.  out0 may alias in0. */
+  HYLE_HIP_OP_ROPE = 16,
   HYLE_HIP_OP_SOFTMAX = 18,
   HYLE_HIP_OP_TOP_K = 19,
   /* Fused forms with no single counterpart in the reference schema; a HYLE
@@ -225,15 +239,16 @@ typedef struct hyle_hip_op_desc {
   uint32_t kind;             /* Unary/Binary/Reduction/GatedActivation kind; Cast, Fill: output hyle_hip_dtype */
   uint32_t kind2;            /* BINARY_CHAIN: second BinaryKind; GATED: GatedInputKind;
                                 SOFTMAX: SoftmaxKind; GGUF_MATVEC: HYLE_HIP_ACTIVATIONS_*;
-                                GATHER: hyle_hip_index_bounds; CATEGORICAL: 1 = also log probabilities */
-  int32_t axis;              /* Softmax / TopK / Concat / Gather axis (negative counts from the end) */
+                                GATHER: hyle_hip_index_bounds; CATEGORICAL: 1 = also log probabilities;
+                                ROPE: hyle_hip_rope_layout */
+  int32_t axis;              /* Softmax / TopK / Concat / Gather axis, RoPE sequence axis (negative counts from the end) */
   uint32_t mask;             /* Softmax MaskKind */
   uint32_t accumulation;     /* hyle_hip_dtype; UNKNOWN or F32 */
   uint32_t keep_dimensions;  /* Reduce */
   float epsilon;             /* RmsNorm, LayerNorm */
   float scale;               /* Softmax */
   uint64_t count;            /* TopK count; Fill: the scalar's bits; Concat: the group's start on the axis;
-                                RandomBits: word_count */
+                                RandomBits: word_count; RoPE: rotary_dimensions */
   uint32_t largest;          /* TopK: 1 = largest first, 0 = smallest first */
   uint32_t input_count;
   hyle_hip_tensor_desc inputs[HYLE_HIP_MAX_INPUTS];

@@ -345,12 +345,19 @@ using GgufDequantSumSquares = Q8_0DequantSumSquares;
 enum class ActivationArithmetic : std::uint8_t { kExact = 0, kGgmlQ8 = 1 };
 struct GgufMatVec final { ActivationArithmetic activations = ActivationArithmetic::kExact; };
 
+// include/hyle/compute/operation.h:112-115,388-392.  Inputs (data, Int32 / Int64 positions, F32 frequencies).
+enum class RopeLayout : std::uint8_t { kInterleaved = 0, kHalfSplit = 1 };
+struct RoPE final {
+  std::size_t rotary_dimensions = 0;
+  std::int32_t sequence_axis = -2;
+  RopeLayout layout = RopeLayout::kInterleaved;
+};
 // sampling_ops::RandomBits / Categorical (include/hyle/compute/sampling_ops.h:12-75)
 struct RandomBits final { std::uint32_t word_count = 4; };
 struct Categorical final { bool return_log_probability = false; };
 
 using Operation = std::variant<Copy, Fill, Select, Concat, Gather, Cast, Unary, Binary, Reduce, RmsNorm, LayerNorm, GatedActivation, Softmax, TopK, BinaryChain,
-                               Q8_0DequantSumSquares, GgufMatVec, RandomBits, Categorical>;
+                               Q8_0DequantSumSquares, GgufMatVec, RandomBits, Categorical, RoPE>;
 
 namespace detail {
 inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *inputs, std::size_t count) noexcept {
@@ -406,6 +413,9 @@ inline hyle_hip_op_desc to_c(const Operation &operation, const TensorDesc *input
     }
     void operator()(const Q8_0DequantSumSquares &) const { r.op = HYLE_HIP_OP_Q8_0_DEQUANT_SUMSQ; }
     void operator()(const GgufMatVec &o) const { r.op = HYLE_HIP_OP_GGUF_MATVEC; r.kind2 = static_cast<std::uint32_t>(o.activations); }
+    void operator()(const RoPE &o) const {
+      r.op = HYLE_HIP_OP_ROPE; r.count = o.rotary_dimensions; r.axis = o.sequence_axis; r.kind2 = static_cast<std::uint32_t>(o.layout);
+    }
     void operator()(const RandomBits &o) const { r.op = HYLE_HIP_OP_RANDOM_BITS; r.count = o.word_count; }
     void operator()(const Categorical &o) const { r.op = HYLE_HIP_OP_CATEGORICAL; r.kind2 = o.return_log_probability ? 1u : 0u; }
   };

@@ -1418,6 +1418,45 @@ int hyle_oracle_gather(size_t width, const void *src, const int64_t *dims, const
   return 0;
 }
 
+/* ---- RoPE ---------------------------------------------------------------- */
+/* src/compute_ggml_runtime/explicit_rope.h:11-74: data widened to f32, positions
+ * converted to f32, phase = frequency * position in f32, cosf / sinf of the
+ * phase, a' = a * cos - b * sin and b' = a * sin + b * cos with every product
+ * and sum a separate f32 operation, one rounding to the storage type; elements
+ * past `rotary` are copied.  Pairs: (2i, 2i + 1) interleaved, (i, i + rotary / 2)
+ * half-split.  Positions are [S] or (batched) the data's leading dimensions
+ * through the sequence axis; frequencies [rotary / 2] or (stepped) [S, rotary / 2]. */
+void hyle_oracle_rope(int type, const void *data, const int64_t *dims, int rank, int sequence_axis,
+                      const void *positions, int wide, int batched, const float *frequencies, int stepped,
+                      int64_t rotary, int half_split, void *dst) {
+  const size_t depth = (size_t)dims[rank - 1], pairs = (size_t)rotary / 2;
+  const size_t n = element_count(dims, rank);
+  if (n == 0) return;
+  const size_t rows = n / depth, sequence = (size_t)dims[sequence_axis];
+  size_t inner = 1;
+  for (int a = sequence_axis + 1; a < rank - 1; ++a) inner *= (size_t)dims[a];
+  const size_t size = type_size(type);
+  const unsigned char *src = (const unsigned char *)data;
+  unsigned char *out = (unsigned char *)dst;
+  for (size_t r = 0; r < rows; ++r) {
+    const size_t step_index = r / inner, step = step_index % sequence;
+    const size_t at = batched ? step_index : step;
+    const float position = wide ? (float)((const int64_t *)positions)[at] : (float)((const int32_t *)positions)[at];
+    const float *row_frequencies = frequencies + (stepped ? step * pairs : 0);
+    const size_t base = r * depth;
+    for (size_t i = 0; i < pairs; ++i) {
+      const size_t first = base + (half_split ? i : 2 * i), second = half_split ? first + pairs : first + 1;
+      const volatile float phase = row_frequencies[i] * position;
+      const float c = cosf(phase), sn = sinf(phase);
+      const float a = load_as_f32(type, src + first * size), b = load_as_f32(type, src + second * size);
+      const volatile float ac = a * c, bs = b * sn, as = a * sn, bc = b * c;
+      store_from_f32(type, out + first * size, ac - bs);
+      store_from_f32(type, out + second * size, as + bc);
+    }
+    for (size_t i = (size_t)rotary; i < depth; ++i) memcpy(out + (base + i) * size, src + (base + i) * size, size);
+  }
+}
+
 /* ---- Sampling ------------------------------------------------------------ */
 /* Philox4x32-10 as the reference addresses it (third_party/random123_counter/
  * philox.h:20-44; include/hyle/compute/sampling_ops.h:12-16): identity = key

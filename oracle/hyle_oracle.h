@@ -50,6 +50,12 @@
  *     broadcasting `where` over raw words.
  *   - concat_part: numpy.concatenate over raw words in the shape of the
  *     reference route test (tests/compute_route_vulkan/concat_test.cc:9-88).
+ *   - rope: the reference tests' known answers (tests/compute_provider_ggml/
+ *     cpu_provider_test.cc:1571-1760, incl. the long-position phases), a
+ *     float64 rotation, and what rotations obey (zero position or frequency is
+ *     the identity, norms of pairs are kept, the tail passes through).  libm's
+ *     cosf / sinf stand for ggml's: agreement is to tolerance, PARITY UNPINNED
+ *     at the bit level.
  *   - philox_block, random_bits: the published Random123 known-answer vectors
  *     for philox4x32_10 and the independent array form in the reference's
  *     tests (tests/compute_models/sampling_fixture.h:70-91).
@@ -372,6 +378,15 @@ void hyle_oracle_concat_part(size_t width, const void *src, const int64_t *dims,
 int hyle_oracle_gather(size_t width, const void *src, const int64_t *dims, const int64_t *strides, int rank,
                        int axis, const void *indices, int wide, const int64_t *index_dims,
                        const int64_t *index_strides, int index_rank, int checked, void *dst);
+
+/* ---- RoPE ---------------------------------------------------------------- */
+/* RoPE with explicit frequencies over dense data of `type` (src/compute_ggml_runtime/
+ * explicit_rope.h:11-74): all arithmetic in f32, phase = frequency * f32(position).
+ * positions: int32 or (`wide`) int64, [S] or (`batched`) the data's leading dimensions
+ * through the sequence axis; frequencies: f32 [rotary / 2] or (`stepped`) [S, rotary / 2]. */
+void hyle_oracle_rope(int type, const void *data, const int64_t *dims, int rank, int sequence_axis,
+                      const void *positions, int wide, int batched, const float *frequencies, int stepped,
+                      int64_t rotary, int half_split, void *dst);
 
 /* ---- Sampling ------------------------------------------------------------ */
 /* Philox4x32-10 under the reference's addressing (third_party/random123_counter/

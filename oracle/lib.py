@@ -97,6 +97,8 @@ _select = _sig("hyle_oracle_select", None, C.c_size_t, _vp, _i64p, _i64p, C.c_in
                _vp, _i64p, _i64p, C.c_int, _i64p, C.c_int, _vp)
 _gather = _sig("hyle_oracle_gather", C.c_int, C.c_size_t, _vp, _i64p, _i64p, C.c_int, C.c_int, _vp, C.c_int, _i64p, _i64p,
                C.c_int, C.c_int, _vp)
+_rope = _sig("hyle_oracle_rope", None, C.c_int, _vp, _i64p, C.c_int, C.c_int, _vp, C.c_int, C.c_int, _vp, C.c_int, C.c_int64,
+             C.c_int, _vp)
 _u32p = C.POINTER(C.c_uint32)
 _philox = _sig("hyle_oracle_philox_block", None, _vp, C.c_uint64, _vp)
 _random_bits = _sig("hyle_oracle_random_bits", None, _vp, C.c_size_t, C.c_size_t, _vp)
@@ -632,3 +634,19 @@ def categorical(type_id: int, logits: np.ndarray, identities: np.ndarray, scored
     scores = np.full(rows, np.nan, np.float32) if scored else None
     status = _categorical(type_id, _ptr(logits), _ptr(ident), rows, width, _ptr(indices), _ptr(scores))
     return status, indices, scores
+
+
+# ---- RoPE -----------------------------------------------------------------
+def rope(type_id: int, data: np.ndarray, positions: np.ndarray, frequencies: np.ndarray, rotary: int,
+         sequence_axis: int = -2, half_split: bool = False) -> np.ndarray:
+    """RoPE over dense `data` (storage dtype of type_id); positions int32 / int64 of rank 1 or the
+    data's leading dimensions through the sequence axis; frequencies float32 [rotary / 2] or [S, rotary / 2]."""
+    data = _c(data, _NP[type_id])
+    positions = np.ascontiguousarray(positions)
+    frequencies = np.ascontiguousarray(frequencies, np.float32)
+    axis = sequence_axis + data.ndim if sequence_axis < 0 else sequence_axis
+    out = np.empty_like(data)
+    _rope(type_id, _ptr(data), _i64(data.shape), data.ndim, axis, _ptr(positions), 1 if positions.dtype.itemsize == 8 else 0,
+          1 if positions.ndim > 1 else 0, _ptr(frequencies), 1 if frequencies.ndim == 2 else 0, int(rotary),
+          1 if half_split else 0, _ptr(out))
+    return out

@@ -645,6 +645,40 @@ DEVICE_TEST(CategoricalDrawsTheOraclesIndexAndFailsOnInvalidRows) {
   }
 }
 
+DEVICE_TEST(RopeMatchesTheReferenceTestsKnownAnswers) {
+  // tests/compute_provider_ggml/cpu_provider_test.cc:1609-1648: f32 [1, 2, 1, 8], positions {0, 2},
+  // frequencies {0.5, 0.25}, rotary 4, half-split; in place
+  const TensorDesc data = dense(DataType::kFloat32, {1, 2, 1, 8});
+  std::vector<float> values(16);
+  for (int i = 0; i < 16; ++i) values[i] = static_cast<float>(i + 1);
+  auto rope = prepare(fixture().context, RoPE{4, 1, RopeLayout::kHalfSplit}, data, dense(DataType::kInt32, {2}),
+                      dense(DataType::kFloat32, {2}));
+  REQUIRE(rope.has_value());
+  EXPECT(rope->alias_support(0, 0)->supported);
+  DeviceBuffer x = upload(values), positions = upload(std::vector<std::int32_t>{0, 2}), frequencies = upload(std::vector<float>{0.5F, 0.25F});
+  auto invocation = rope->create_invocation();
+  REQUIRE(invocation.has_value());
+  auto completion = invocation->submit(fixture().queue, *ConstTensorView::create(data, x),
+                                       *ConstTensorView::create(dense(DataType::kInt32, {2}), positions),
+                                       *ConstTensorView::create(dense(DataType::kFloat32, {2}), frequencies), *TensorView::create(data, x));
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  const std::vector<float> got = download<float>(x, 16);
+  std::vector<double> want(16);
+  for (int i = 0; i < 16; ++i) want[i] = i + 1;
+  want[8] = 9.0 * std::cos(1.0) - 11.0 * std::sin(1.0);
+  want[9] = 10.0 * std::cos(0.5) - 12.0 * std::sin(0.5);
+  want[10] = 9.0 * std::sin(1.0) + 11.0 * std::cos(1.0);
+  want[11] = 10.0 * std::sin(0.5) + 12.0 * std::cos(0.5);
+  for (int i = 0; i < 16; ++i) EXPECT(std::fabs(got[i] - want[i]) <= 1e-5);
+  std::vector<float> oracle(16);
+  const std::int64_t dims[4] = {1, 2, 1, 8};
+  const std::int32_t steps[2] = {0, 2};
+  const float rates[2] = {0.5F, 0.25F};
+  hyle_oracle_rope(HYLE_ORACLE_F32, values.data(), dims, 4, 1, steps, 0, 0, rates, 0, 4, 1, oracle.data());
+  for (int i = 0; i < 16; ++i) EXPECT(std::fabs(got[i] - oracle[i]) <= 4e-6F * 24.0F);
+}
+
 DEVICE_TEST(RejectedSubmissionsEnqueueNothing) {
   const TensorDesc d = dense(DataType::kFloat32, {8, 64}), row = dense(DataType::kFloat32, {64});
   auto prepared = prepare(fixture().context, Binary{BinaryKind::kMultiply}, d, row);

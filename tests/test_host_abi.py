@@ -438,6 +438,38 @@ def test_sampling_inference_and_admission():
     assert hc.prepare(CTX, hc.Categorical(), D(DT.kFloat32, [0, 7]), D(U32, [0, 4])).dispatch_count() == 0
 
 
+def test_rope_inference_and_admission():
+    # src/compute_ops/operation.cc:639-696,1566-1574
+    data, positions, frequencies = D(DT.kBFloat16, [1, 8192, 16, 128]), D(DT.kInt32, [8192]), D(DT.kFloat32, [64])
+    rope = hc.RoPE(128, 1, hc.RopeLayout.kHalfSplit)
+    assert hc.infer_output_descriptions(rope, [data, positions, frequencies]) == [data]
+    assert hc.infer_output_descriptions(hc.RoPE(64, 1), [data, D(DT.kInt64, [1, 8192]), D(DT.kFloat32, [8192, 32])]) == [data]
+    bad = [
+        (hc.RoPE(0, 1), [data, positions, frequencies]), (hc.RoPE(3, 1), [data, positions, frequencies]),
+        (hc.RoPE(130, 1), [data, positions, frequencies]), (hc.RoPE(128, 3), [data, positions, frequencies]),
+        (rope, [data, D(DT.kInt32, [8191]), frequencies]), (rope, [data, D(DT.kInt32, [2, 8192]), frequencies]),
+        (rope, [data, D(DT.kFloat32, [8192]), frequencies]), (rope, [data, positions, D(DT.kFloat32, [63])]),
+        (rope, [data, positions, D(DT.kFloat32, [16, 64])]), (rope, [data, positions, D(DT.kInt32, [64])]),
+        (rope, [D(DT.kBFloat16, [128]), positions, frequencies]),
+    ]
+    for operation, inputs in bad:
+        with pytest.raises(hc.StatusError) as err:
+            hc.infer_output_descriptions(operation, inputs)
+        assert err.value.is_invalid_argument()
+    with pytest.raises(hc.StatusError) as err:
+        hc.infer_output_descriptions(hc.RoPE(128, 7), [data, positions, frequencies])
+    assert err.value.is_out_of_range()
+    prepared = hc.prepare(CTX, rope, data, positions, frequencies)
+    assert prepared.route_name() == "rope-rows" and prepared.dispatch_count() == 1 and prepared.workspace_requirement().size == 0
+    assert prepared.alias_support(0, 0) and not prepared.alias_support(0, 1)
+    for inputs in ([D(DT.kFloat64, [2, 3, 8]), D(DT.kInt32, [3]), D(DT.kFloat32, [2])],       # the schema's floats the kernels do not serve
+                   [D(DT.kFloat32, [2, 3, 8]), D(DT.kInt32, [3]), D(DT.kBFloat16, [2])],
+                   [hc.TensorDesc.strided_bytes(DT.kFloat32, [2, 3, 8], [128, 40, 4]), D(DT.kInt32, [3]), D(DT.kFloat32, [2])]):
+        with pytest.raises(hc.StatusError) as err:
+            hc.prepare(CTX, hc.RoPE(4, 1), *inputs)
+        assert err.value.is_unimplemented()
+
+
 def test_stream_abi_is_exported_and_validates_without_a_device():
     from hyle_amd import capi
     from hyle_amd import file_stream as fs
