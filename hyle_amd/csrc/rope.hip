@@ -132,40 +132,67 @@ __global__ __launch_bounds__(kBlockThreads) void rope_steps(RopeOperands p, cons
   }
   __syncthreads();
   const uint32_t rotating = (kHalfSplit ? p.pairs : p.rotary) / kVec, partner = p.pairs / kVec;
-  const uint32_t per_step = p.inner * places;
-  for (uint32_t u = threadIdx.x; u < own * per_step; u += kBlockThreads) {
+  const uint32_t per_step = p.inner * places, total = own * per_step;
+  // a unit is one place of one row; its loads are issued one unit ahead of its arithmetic
+  struct Unit {
+    size_t at;        // the vector in the tensor
+    uint32_t table;   // where the unit's cos values start; 0xFFFFFFFF: a tail vector that is copied
+    u32x4 lower, upper;
+  };
+  auto fetch = [&](uint32_t u) {
+    Unit unit;
     const uint32_t local = u / per_step, within = u - local * per_step;
     const uint32_t h = within / places, place = within - h * places;
     const size_t row = ((size_t)(first_step + local) * p.inner + h) * vectors_per_row;
     if (place >= rotating) {
-      const size_t at = row + p.rotary / kVec + (place - rotating);
-      store16_stream(out, at, load16_stream(in, at));
-      continue;
-    }
-    const size_t at = row + place;
-    const float *c = table + 2 * local * p.pairs + place * kPairs, *s = c + p.pairs;
-    if constexpr (kHalfSplit) {
-      float a[kVec], b[kVec], ra[kVec], rb[kVec];
-      const u32x4 lower = load16_stream(in, at), upper = load16_stream(in, at + partner);
-      Traits<T>::unpack(lower, a);
-      Traits<T>::unpack(upper, b);
-#pragma unroll
-      for (int j = 0; j < kVec; ++j) {
-        ra[j] = a[j] * c[j] - b[j] * s[j];
-        rb[j] = a[j] * s[j] + b[j] * c[j];
-      }
-      store16_stream(out, at, Traits<T>::pack(ra));
-      store16_stream(out, at + partner, Traits<T>::pack(rb));
+      unit.at = row + p.rotary / kVec + (place - rotating);
+      unit.table = 0xFFFFFFFFu;
+      unit.lower = load16_stream(in, unit.at);
+      unit.upper = unit.lower;
     } else {
-      float x[kVec], r[kVec];
-      Traits<T>::unpack(load16_stream(in, at), x);
-#pragma unroll
-      for (int j = 0; j < kVec / 2; ++j) {
-        r[2 * j] = x[2 * j] * c[j] - x[2 * j + 1] * s[j];
-        r[2 * j + 1] = x[2 * j] * s[j] + x[2 * j + 1] * c[j];
-      }
-      store16_stream(out, at, Traits<T>::pack(r));
+      unit.at = row + place;
+      unit.table = 2 * local * p.pairs + place * kPairs;
+      unit.lower = load16_stream(in, unit.at);
+      unit.upper = kHalfSplit ? load16_stream(in, unit.at + partner) : unit.lower;
     }
+    return unit;
+  };
+  uint32_t u = threadIdx.x;
+  if (u >= total) return;
+  Unit current = fetch(u);
+  while (true) {
+    const uint32_t following = u + kBlockThreads;
+    Unit next = current;
+    if (following < total) next = fetch(following);
+    if (current.table == 0xFFFFFFFFu) {
+      store16_stream(out, current.at, current.lower);
+    } else {
+      const float *c = table + current.table, *s = c + p.pairs;
+      if constexpr (kHalfSplit) {
+        float a[kVec], b[kVec], ra[kVec], rb[kVec];
+        Traits<T>::unpack(current.lower, a);
+        Traits<T>::unpack(current.upper, b);
+#pragma unroll
+        for (int j = 0; j < kVec; ++j) {
+          ra[j] = a[j] * c[j] - b[j] * s[j];
+          rb[j] = a[j] * s[j] + b[j] * c[j];
+        }
+        store16_stream(out, current.at, Traits<T>::pack(ra));
+        store16_stream(out, current.at + partner, Traits<T>::pack(rb));
+      } else {
+        float x[kVec], r[kVec];
+        Traits<T>::unpack(current.lower, x);
+#pragma unroll
+        for (int j = 0; j < kVec / 2; ++j) {
+          r[2 * j] = x[2 * j] * c[j] - x[2 * j + 1] * s[j];
+          r[2 * j + 1] = x[2 * j] * s[j] + x[2 * j + 1] * c[j];
+        }
+        store16_stream(out, current.at, Traits<T>::pack(r));
+      }
+    }
+    if (following >= total) break;
+    current = next;
+    u = following;
   }
 }
 
@@ -207,11 +234,12 @@ hipError_t run_rope(const RopeParams &p, const void *in, const void *positions, 
     const uint64_t units = p.rows / p.inner * groups * places;  // at most INT32_MAX elements / kVec
     const uint64_t steps = p.rows / p.inner;
     if (p.rotary / 2 <= 2048) {
-      // Thin blocks: the steps that give a block about 128 places.  Measured on MI355X for
-      // [1, 8192, 16, 128] bf16, half-split: 13.3 us with one step (128 places) per block, 13.6 /
-      // 13.9 / 14.8 / 17.7 us with 2 / 4 / 8 / 16; 14.9 us when every thread takes cos and sin
-      // itself for eight rows, 31.2 us when it does so for each row.
-      uint32_t per_block = 128 / (p.inner * places);
+      // The steps that give a block about 512 places, two per thread with the second one's loads
+      // issued before the first one's arithmetic.  Measured on MI355X for [1, 8192, 16, 128] bf16,
+      // half-split: 13.5 us so (14.2 / 13.6 / 13.8 / 15.3 us with 128 / 256 / 1024 / 2048 places);
+      // 14.9 us when every thread takes cos and sin itself for eight rows, 31.2 us when it does
+      // so for each row; the plain copy of the same bytes 11.1 us.
+      uint32_t per_block = 512 / (p.inner * places);
       per_block = per_block < 1 ? 1 : per_block;
       while (per_block > 1 && (size_t)per_block * p.rotary * sizeof(float) > 32768) --per_block;
       const size_t lds = (size_t)per_block * p.rotary * sizeof(float);
