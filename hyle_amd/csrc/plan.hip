@@ -1254,7 +1254,6 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       // src/compute_provider_cuda/sampling_provider.cc:26-71
       if (p->input_elements[0] / 4 > kMaxElements || p->output_elements[0] > kMaxElements)
         return fail(HYLE_HIP_UNIMPLEMENTED, "RandomBits requires at most INT32_MAX rows and output words");
-      p->input_alignment[0] = 16;  // a row's four identity words are read as one vector
       if (p->output_elements[0] == 0) return HYLE_HIP_OK;
       p->route = Route::kRandomBits;
       p->dispatches = 1;
@@ -1269,7 +1268,6 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       const uint64_t tiles = (width + kCategoricalTile - 1) / kCategoricalTile;
       if (rows > kMaxElements || rows * tiles > kMaxElements)
         return fail(HYLE_HIP_UNIMPLEMENTED, "Categorical row or tile grid capacity exceeded");
-      p->input_alignment[1] = 16;
       if (rows == 0) return HYLE_HIP_OK;
       CategoricalParams &c = p->categorical;
       c.rows = (uint32_t)rows;

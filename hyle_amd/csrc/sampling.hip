@@ -45,8 +45,8 @@ __global__ __launch_bounds__(kBlockThreads) void random_bits(const uint32_t *ide
   const uint64_t total = (uint64_t)rows * blocks_per_row;
   for (uint64_t i = (uint64_t)blockIdx.x * kBlockThreads + threadIdx.x; i < total; i += (uint64_t)gridDim.x * kBlockThreads) {
     const uint32_t row = (uint32_t)(i / blocks_per_row), column = (uint32_t)(i - (uint64_t)row * blocks_per_row);
-    const u32x4 identity = load16(identities, row);
-    const PhiloxWords w = philox_block(identity.x, identity.y, identity.z, identity.w, column);
+    const uint32_t *identity = identities + (size_t)row * 4;  // element-aligned, as the reference asks
+    const PhiloxWords w = philox_block(identity[0], identity[1], identity[2], identity[3], column);
     uint32_t *to = out + (uint64_t)row * word_count + (uint64_t)column * 4;
     if (vector) {
       store16_stream(to, 0, u32x4{w.x0, w.x1, w.x2, w.x3});
@@ -223,7 +223,8 @@ __global__ __launch_bounds__(kBlockThreads) void categorical_rows(const void *lo
   const uint32_t row = blockIdx.x;
   const CategoricalTile *mine = parts + (size_t)row * tiles;
   const void *base = static_cast<const unsigned char *>(logits) + (size_t)row * width * Traits<T>::kSize;
-  const u32x4 identity = load16(identities, row);
+  const uint32_t *identity = identities + (size_t)row * 4;
+  const uint32_t key0 = identity[0], key1 = identity[1], draw0 = identity[2], draw1 = identity[3];
   // the row's maximum; a tile with NaN or +inf counts as +inf, which no valid tile reaches
   float maximum = -kInfinity;
   for (uint32_t t = threadIdx.x; t < tiles; t += kBlockThreads) maximum = fmaxf(maximum, mine[t].invalid ? kInfinity : mine[t].maximum);
@@ -241,7 +242,7 @@ __global__ __launch_bounds__(kBlockThreads) void categorical_rows(const void *lo
   for (uint32_t t = begin; t < end; ++t) own += mine[t].mass * (double)scale_of(t);
   double total = 0, through = 0;
   const double before = block_scan(own, wave_totals, &through, &total);
-  const PhiloxWords draw = philox_block(identity.x, identity.y, identity.z, identity.w, 0);
+  const PhiloxWords draw = philox_block(key0, key1, draw0, draw1, 0);
   // the 52-bit midpoint is exact in double at both ends (sampling.cc:155-158)
   const double uniform = ((double)draw.x0 * 0x1p20 + (double)(draw.x1 >> 12) + 0.5) * 0x1p-52;
   const double threshold = total * uniform;

@@ -31,15 +31,16 @@ def on_device(raw: np.ndarray) -> torch.Tensor:
     return torch.from_numpy(flat.copy()).to(DEVICE) if flat.size else torch.empty(16, dtype=torch.uint8, device=DEVICE)
 
 
-def random_bits_on_device(ids: np.ndarray, count: int) -> np.ndarray:
+def random_bits_on_device(ids: np.ndarray, count: int, lead: int = 0) -> np.ndarray:
+    """`lead`: bytes the identities sit past a 256-byte boundary (the reference asks element alignment only)."""
     rows = ids.shape[0]
     prepared = hc.prepare(context(), hc.RandomBits(count), hc.TensorDesc.dense(DT.kUInt32, [rows, 4]))
     assert prepared.output_description() == hc.TensorDesc.dense(DT.kUInt32, [rows, count])
     assert prepared.workspace_requirement().size == 0
     assert prepared.dispatch_count() == (1 if rows * count else 0)
-    source = on_device(ids)
+    source = on_device(np.concatenate([np.zeros(lead, np.uint8), np.ascontiguousarray(ids).view(np.uint8).reshape(-1)]))
     out = torch.full((rows * count * 4 + 16,), 0x5A, dtype=torch.uint8, device=DEVICE)
-    prepared.create_invocation().submit(torch.cuda.current_stream().cuda_stream, [source.data_ptr()], [out.data_ptr()])
+    prepared.create_invocation().submit(torch.cuda.current_stream().cuda_stream, [source.data_ptr() + lead], [out.data_ptr()])
     torch.cuda.synchronize()
     host = out.cpu().numpy()
     assert (host[rows * count * 4:] == 0x5A).all()
@@ -57,6 +58,7 @@ def test_random_bits_match_philox_word_for_word():
     ids = np.random.default_rng(9).integers(0, 1 << 32, (4096, 4), dtype=np.uint64).astype(np.uint32)
     assert np.array_equal(random_bits_on_device(ids, 1024), orc.random_bits(ids, 1024))
     assert np.array_equal(random_bits_on_device(ids[:333], 1001), orc.random_bits(ids[:333], 1001))
+    assert np.array_equal(random_bits_on_device(ids[:333], 64, lead=4), orc.random_bits(ids[:333], 64))
 
 
 def categorical_on_device(type_id, stored: np.ndarray, ids: np.ndarray, scored: bool, static: bool = False):
