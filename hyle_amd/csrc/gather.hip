@@ -97,8 +97,8 @@ template <int kUnit> __device__ __forceinline__ void store_unit(unsigned char *t
   else reinterpret_cast<typename UnitWord<kUnit>::type *>(to)[u] = word;
 }
 
-// Rows of at least 256 units: a row is cut into chunks of 256 units and a block of 512 threads
-// takes two consecutive chunks -- of one long row or of two short ones --, one unit per thread, so
+// Rows of at least 256 units, fewer than 4096 chunks in all: a row is cut into chunks of 256 units
+// and a block of 512 threads takes two consecutive chunks -- of one long row or of two short ones --, one unit per thread, so
 // a chunk's row, its index and both addresses are the same for 256 threads.  Measured on MI355X
 // for 8192 rows of 4 KiB picked at random from 622 MB: 12.5 us in this form (11.4 us when the
 // picked rows are consecutive, 11.1 us for a plain copy of the same bytes); blocks that take 4 to
@@ -118,6 +118,54 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows(GatherRows p, GatherI
   const int64_t selected = index_at<kWide, kDense>(v, item);
   const unsigned char *from = p.source + (uint64_t)outer * p.outer_pitch + (uint64_t)selected * p.axis_pitch;
   store_unit<kUnit>(out + (uint64_t)row * p.row_units * kUnit, unit, load_unit<kUnit>(from, unit));
+}
+
+// The same chunks, sixteen per block of 512 threads: sixteen threads resolve the chunks' rows and
+// indices into LDS first, then every lane streams eight units one after another, its stores
+// after its last load, as the plain copy kernel does.
+constexpr int kFatChunks = 16;
+template <int kUnit, bool kWide, bool kDense>
+__global__ __launch_bounds__(kRowThreads) void gather_rows_fat(GatherRows p, GatherIndexView v, GatherVerdict verdict,
+                                                               unsigned char *out, uint32_t chunks_per_row, uint32_t chunks) {
+  __shared__ const unsigned char *from_of[kFatChunks];
+  __shared__ unsigned char *to_of[kFatChunks];
+  __shared__ uint32_t units_of[kFatChunks];
+  if (indices_refused(verdict)) return;
+  if (threadIdx.x < kFatChunks) {
+    const uint32_t chunk = blockIdx.x * kFatChunks + threadIdx.x;
+    uint32_t units = 0;
+    if (chunk < chunks) {
+      const uint32_t row = chunk / chunks_per_row, piece = chunk - row * chunks_per_row;
+      const uint32_t outer = row / p.index_count, item = row - outer * p.index_count;
+      const int64_t selected = index_at<kWide, kDense>(v, item);
+      const uint32_t first = piece * kBlockThreads;
+      units = p.row_units - first < (uint32_t)kBlockThreads ? p.row_units - first : (uint32_t)kBlockThreads;
+      from_of[threadIdx.x] = p.source + (uint64_t)outer * p.outer_pitch + (uint64_t)selected * p.axis_pitch + (size_t)first * kUnit;
+      to_of[threadIdx.x] = out + ((uint64_t)row * p.row_units + first) * kUnit;
+    }
+    units_of[threadIdx.x] = units;
+  }
+  __syncthreads();
+  constexpr int kSteps = kFatChunks * kBlockThreads / kRowThreads;  // 8
+  const uint32_t lane = threadIdx.x % kBlockThreads, half = threadIdx.x / kBlockThreads;
+  typename UnitWord<kUnit>::type held[kSteps];
+  bool live[kSteps];
+  auto load = [&](int j) {
+    const int c = j * (kRowThreads / kBlockThreads) + half;
+    live[j] = lane < units_of[c];
+    held[j] = load_unit<kUnit>(from_of[c], live[j] ? lane : 0u);  // a lane past the chunk reads its first unit and drops it
+  };
+  load(0);
+#pragma unroll
+  for (int j = 0; j < kSteps; ++j) {
+    if constexpr (kUnit == 16) loads_issued(held[j]);
+    if (j + 1 < kSteps) load(j + 1);
+  }
+#pragma unroll
+  for (int j = 0; j < kSteps; ++j) {
+    const int c = j * (kRowThreads / kBlockThreads) + half;
+    if (live[j]) store_unit<kUnit>(to_of[c], lane, held[j]);
+  }
 }
 
 // Short rows: one unit per thread, rows packed into blocks.
@@ -177,8 +225,14 @@ void run_rows(const GatherRows &rows, const GatherIndexView &view, const GatherV
     const uint32_t per_row = (rows.row_units + kBlockThreads - 1) / kBlockThreads;
     const uint64_t chunks = (uint64_t)per_row * rows.rows;  // at most INT32_MAX bytes / 256
     const uint32_t per_block = kRowThreads / kBlockThreads;
-    hipLaunchKernelGGL((gather_rows<kUnit, kWide, kDense>), dim3((uint32_t)((chunks + per_block - 1) / per_block)),
-                       dim3(kRowThreads), 0, stream, rows, view, verdict, out, per_row, (uint32_t)chunks);
+    // Enough chunks to give every compute unit a fat block: sixteen chunks per block, resolved
+    // first and then streamed (11.8 us against 12.6 us for 8192 rows of 4 KiB picked at random).
+    if (chunks >= 4096)
+      hipLaunchKernelGGL((gather_rows_fat<kUnit, kWide, kDense>), dim3((uint32_t)((chunks + kFatChunks - 1) / kFatChunks)),
+                         dim3(kRowThreads), 0, stream, rows, view, verdict, out, per_row, (uint32_t)chunks);
+    else
+      hipLaunchKernelGGL((gather_rows<kUnit, kWide, kDense>), dim3((uint32_t)((chunks + per_block - 1) / per_block)),
+                         dim3(kRowThreads), 0, stream, rows, view, verdict, out, per_row, (uint32_t)chunks);
   } else {
     const uint64_t units = (uint64_t)rows.rows * rows.row_units;
     hipLaunchKernelGGL((gather_units<kUnit, kWide, kDense>), dim3((uint32_t)((units + kBlockThreads - 1) / kBlockThreads)),
