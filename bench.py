@@ -234,6 +234,7 @@ def main() -> int:
             ("next_matvec_ggml_q8_q4_k_ffn", hc.GgufQuantizedType.kQ4K, 144, 2048, 6144, 80, 1, GGML_Q8),
             ("next_matvec_ggml_q8_q4_k_ffn_down", hc.GgufQuantizedType.kQ4K, 144, 6144, 2048, 80, 1, GGML_Q8),
             ("next_matvec_ggml_q8_q4_k_vocab", hc.GgufQuantizedType.kQ4K, 144, 2048, 151936, 4, 1, GGML_Q8),
+            ("next_matvec_ggml_q8_q4_k_vocab_4_tokens", hc.GgufQuantizedType.kQ4K, 144, 2048, 151936, 4, 4, GGML_Q8),
             ("next_matvec_ggml_q8_q6_k_vocab", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 1, GGML_Q8),
             ("next_matvec_ggml_q8_q6_k_vocab_4_tokens", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 4, GGML_Q8),
             ("next_matvec_ggml_q8_q6_k_vocab_8_tokens", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 8, GGML_Q8),

@@ -188,10 +188,45 @@ template <int kCount> __device__ __forceinline__ float joint_sum(float (&v)[kCou
   return mine;
 }
 
+// Six-bit sc (or m) of sub-block j from the twelve scale bytes of a Q4_K block, s0 = bytes 0..3,
+// s1 = 4..7, s2 = 8..11: sub-blocks 0..3 keep them whole in bytes j and j + 4, sub-blocks 4..7 keep
+// four bits in a nibble of byte j + 4 and two more in the top of byte j - 4 (sc) or j (m).
+__device__ __forceinline__ int q4k_six_bits(uint32_t s0, uint32_t s1, uint32_t s2, uint32_t j, bool minimum) {
+  const uint32_t shift = 8 * (j % 4), own = minimum ? s1 : s0;
+  if (j < 4) return (int)((own >> shift) & 63u);
+  return (int)(((s2 >> (shift + (minimum ? 4u : 0u))) & 15u) | (((own >> (shift + 6)) & 3u) << 4));
+}
+
 template <> struct SpanDot<0> {  // Q4_K
   uint32_t low[2][2], high[2][2];
   int sc_low[2], sc_high[2], m_low[2], m_high[2];
   float d[2], dmin[2];
+  // The same without the block's other lanes (in the quad layout they hold other weight rows):
+  // the lane works out the four factors of its two sub-blocks, 2 chunk and 2 chunk + 1, itself.
+  // They are the same for the four shares a quad lane walks, so they are taken once per span.
+  __device__ __forceinline__ void scales_alone(const unsigned char *slot, const Lines<0>::Lane &at, uint32_t chunk) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const u32x4 head = *reinterpret_cast<const u32x4 *>(slot + at.header[i]);
+      d[i] = f16_to_f32((uint16_t)head.x);
+      dmin[i] = f16_to_f32((uint16_t)(head.x >> 16));
+      sc_low[i] = q4k_six_bits(head.y, head.z, head.w, 2 * chunk, false);
+      sc_high[i] = q4k_six_bits(head.y, head.z, head.w, 2 * chunk + 1, false);
+      m_low[i] = q4k_six_bits(head.y, head.z, head.w, 2 * chunk, true);
+      m_high[i] = q4k_six_bits(head.y, head.z, head.w, 2 * chunk + 1, true);
+    }
+  }
+  __device__ __forceinline__ void quants_alone(const unsigned char *slot, const Lines<0>::Lane &at) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t *words = reinterpret_cast<const uint32_t *>(slot + at.quants[i]);
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        low[i][w] = words[w] & 0x0F0F0F0Fu;
+        high[i][w] = (words[w] >> 4) & 0x0F0F0F0Fu;
+      }
+    }
+  }
   __device__ __forceinline__ void decode(const unsigned char *slot, const Lines<0>::Lane &at) {
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -426,6 +461,46 @@ template <> struct QuadDot<1> {  // Q6_K
     sums[3] += (w.step * quad_lane<3>(a.scale[0])) * (float)total[3];
   }
 };
+// Q4_K.  The four shares a quad lane walks in a span lie in the same two weight blocks and the
+// same two activation blocks, so their integer dots are accumulated in the matrix unit across the
+// shares -- codes . low nibbles, codes . high nibbles and, for the minima, codes . m with m as four
+// equal bytes -- and the scales are applied once per span.
+template <> struct QuadDot<0> {
+  struct Sums {
+    i32x4 lows[2], highs[2], minima[2];
+  };
+  static __device__ __forceinline__ void clear(Sums &acc) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) acc.lows[i] = acc.highs[i] = acc.minima[i] = i32x4{0, 0, 0, 0};
+  }
+  static __device__ __forceinline__ void add(const SpanDot<0> &w, const LaneCodes &a, Sums &acc) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const uint32_t m_low = (uint32_t)w.m_low[i] * 0x01010101u, m_high = (uint32_t)w.m_high[i] * 0x01010101u;
+      acc.lows[i] = quad_dots(a.codes[4 * i + 1], w.low[i][1], quad_dots(a.codes[4 * i], w.low[i][0], acc.lows[i]));
+      acc.highs[i] = quad_dots(a.codes[4 * i + 3], w.high[i][1], quad_dots(a.codes[4 * i + 2], w.high[i][0], acc.highs[i]));
+      acc.minima[i] = quad_dots(a.codes[4 * i + 1], m_low, quad_dots(a.codes[4 * i], m_low, acc.minima[i]));
+      acc.minima[i] = quad_dots(a.codes[4 * i + 3], m_high, quad_dots(a.codes[4 * i + 2], m_high, acc.minima[i]));
+    }
+  }
+  template <int kRow>
+  static __device__ __forceinline__ float row(const SpanDot<0> &w, const float (&scale)[2], const Sums &acc) {
+    float total = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int scaled = mad24(w.sc_low[i], acc.lows[i][kRow], __mul24(w.sc_high[i], acc.highs[i][kRow]));
+      total += quad_lane<kRow>(scale[i]) * (w.d[i] * (float)scaled - w.dmin[i] * (float)acc.minima[i][kRow]);
+    }
+    return total;
+  }
+  // scale: the activation blocks' scales of this lane's activation row (the same for the four shares)
+  static __device__ __forceinline__ void close(const SpanDot<0> &w, const float (&scale)[2], const Sums &acc, float (&sums)[4]) {
+    sums[0] += row<0>(w, scale, acc);
+    sums[1] += row<1>(w, scale, acc);
+    sums[2] += row<2>(w, scale, acc);
+    sums[3] += row<3>(w, scale, acc);
+  }
+};
 template <> struct QuadDot<2> {  // Q8_0
   static __device__ __forceinline__ void add(const SpanDot<2> &w, const LaneCodes &a, float (&sums)[4]) {
     i32x4 dots = {0, 0, 0, 0};
@@ -508,14 +583,39 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_quads(const unsi
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      if constexpr (kKind == 0) {
+        // Q4_K: the four shares one after another in a loop that is not unrolled (unrolled, their
+        // decodes are all hoisted to the front and the kernel needs every register there is: 256
+        // + 67 against 90), the codes fetched from LDS share by share
+        SpanDot<0> decoded;
+        decoded.scales_alone(own_slot, Kind::lane_of(0, 4 * quad), quad % 4);  // chunk = (4 quad + t) % 16 / 4
+        typename QuadDot<0>::Sums acc[kSets];
+        float scale[kSets][2];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        SpanDot<kKind> decoded;
-        decoded.decode(own_slot, at[t]);
+        for (int set = 0; set < kSets; ++set) QuadDot<0>::clear(acc[set]);
+#pragma unroll 1
+        for (int t = 0; t < 4; ++t) {
+          decoded.quants_alone(own_slot, Kind::lane_of(0, 4 * quad + t));
 #pragma unroll
-        for (int set = 0; set < kSets; ++set) {
-          if constexpr (kRegisters) QuadDot<kKind>::add(decoded, held[set * 4 + t], sums[set]);
-          else QuadDot<kKind>::add(decoded, fetch(staged, token[set] * spans + span, 4 * quad + t), sums[set]);
+          for (int set = 0; set < kSets; ++set) {
+            const LaneCodes a = fetch(staged, token[set] * spans + span, 4 * quad + t);
+            scale[set][0] = a.scale[0];
+            scale[set][1] = a.scale[1];
+            QuadDot<0>::add(decoded, a, acc[set]);
+          }
+        }
+#pragma unroll
+        for (int set = 0; set < kSets; ++set) QuadDot<0>::close(decoded, scale[set], acc[set], sums[set]);
+      } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          SpanDot<kKind> decoded;
+          decoded.decode(own_slot, at[t]);
+#pragma unroll
+          for (int set = 0; set < kSets; ++set) {
+            if constexpr (kRegisters) QuadDot<kKind>::add(decoded, held[set * 4 + t], sums[set]);
+            else QuadDot<kKind>::add(decoded, fetch(staged, token[set] * spans + span, 4 * quad + t), sums[set]);
+          }
         }
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -541,11 +641,12 @@ hipError_t run_quads(const MatVecParams &p, const void *w, const void *x, void *
 #define HYLE_QUADS(SETS, REGISTERS)                                                                             \
   hipLaunchKernelGGL((gguf_matvec_q8_quads<kKind, TX, SETS, REGISTERS>), grid, dim3(kBlockThreads), shared, s, in, x, \
                      y, (uint32_t)p.rows, p.row_stride, spans, p.m)
+  const bool registers = spans == 1 && kKind != 0;  // Q4_K fetches its codes from LDS share by share
   if (p.m <= 4) {
-    if (spans == 1) HYLE_QUADS(1, true);
+    if (registers) HYLE_QUADS(1, true);
     else HYLE_QUADS(1, false);
   } else {
-    if (spans == 1) HYLE_QUADS(2, true);
+    if (registers) HYLE_QUADS(2, true);
     else HYLE_QUADS(2, false);
   }
 #undef HYLE_QUADS
@@ -572,9 +673,8 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
   const uint32_t machine = (uint32_t)(compute_units > 0 ? compute_units : 256) * 3u;  // three blocks per compute unit
   const dim3 grid(wanted < machine ? wanted : machine);
   const size_t shared = gguf_matvec_q8_shared_bytes(p.m, p.k);
-  if constexpr (kKind != 0) {
-    // Q6_K and Q8_0 with several activation rows: the quad form, if its four row slots per wave
-    // fit beside the codes
+  {
+    // several activation rows: the quad form, if its four row slots per wave fit beside the codes
     const size_t slots = (size_t)kWavesPerBlock * 4 * (LinesRow<kKind, 1>::kSlotBytes + 32);
     if (p.m >= 2 && slots + shared <= 64 * 1024) return run_quads<kKind, TX>(p, w, x, y, spans, grid, shared, s);
   }

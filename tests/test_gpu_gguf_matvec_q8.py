@@ -98,7 +98,7 @@ def test_q8_route_raw_bytes_zero_blocks_ties_and_padded_rows(tag):
     check(tag, "f32", padded, rows, k, x, row_stride=row_bytes + 48)
 
 
-@pytest.mark.parametrize("tag,m", [("q6_k", 4), ("q4_k", 1), ("q8_0", 2)])
+@pytest.mark.parametrize("tag,m", [("q6_k", 4), ("q4_k", 1), ("q4_k", 3), ("q4_k", 8), ("q8_0", 2)])
 def test_q8_route_vocabulary_sized_weight(tag, m):
     rng = np.random.default_rng(1802)
     rows, k = 151936, 2048
