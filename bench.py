@@ -351,7 +351,7 @@ def main() -> int:
             return [left, right], [torch.empty((8192, 6144), dtype=torch.bfloat16, device=dev)]
         ops.append(Op("next_concat_bf16", hc.Concat(-1), [D(BF, [8192, 2048]), D(BF, [8192, 4096])], set_concat, 3,
                       8192 * 6144 * 4, 8192 * 6144, "bf16", in_step=False))
-    if want("next_gather_bf16") or want("next_gather_unchecked_bf16"):
+    if want("next_gather_bf16") or want("next_gather_unchecked_bf16") or want("next_gather_last_rows_bf16"):
         # the embedding lookup: 8192 rows of 4 KiB picked from a [151936, 2048] table by Int32 ids; one
         # table for both lines (622 MB).  Checked bounds add the dispatch that looks at every id.
         table = torch.empty((151936, 2048), dtype=torch.bfloat16, device=dev).normal_()
@@ -362,6 +362,14 @@ def main() -> int:
         if want("next_gather_bf16"):
             ops.append(Op("next_gather_bf16", hc.Gather(0), [D(BF, [151936, 2048]), D(hc.DataType.kInt32, [8192])], set_gather,
                           8, gather_bytes + 8192 * 4, 8192 * 2048, "bf16", in_step=False, ceiling="ceiling_copy_67mb"))
+        if want("next_gather_last_rows_bf16"):
+            # what a step does for its last tokens: 64 checked row picks out of [8192, 2048] hidden states
+            hidden = torch.empty((8192, 2048), dtype=torch.bfloat16, device=dev).normal_()
+            def set_last(i):
+                ids = torch.randint(0, 8192, (64,), dtype=torch.int32, device=dev)
+                return [hidden, ids], [torch.empty((64, 2048), dtype=torch.bfloat16, device=dev)]
+            ops.append(Op("next_gather_last_rows_bf16", hc.Gather(0), [D(BF, [8192, 2048]), D(hc.DataType.kInt32, [64])], set_last,
+                          8, 64 * 2048 * 4 + 64 * 4, 64 * 2048, "bf16", in_step=False))
         if want("next_gather_unchecked_bf16"):
             ops.append(Op("next_gather_unchecked_bf16", hc.Gather(0, hc.IndexBoundsPolicy.kUnchecked),
                           [D(BF, [151936, 2048]), D(hc.DataType.kInt32, [8192])], set_gather, 8, gather_bytes, 8192 * 2048,

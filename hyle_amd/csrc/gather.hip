@@ -55,16 +55,37 @@ __global__ __launch_bounds__(kBlockThreads) void gather_check(GatherIndexView v,
   if (threadIdx.x == 0) flags[blockIdx.x] = bad ? 1u : 0u;
 }
 
-// What the moving kernels know of the check: flags == nullptr for unchecked bounds.
+// What the moving kernels know of the check.  flags != nullptr: a dispatch of gather_check went
+// first.  flags == nullptr and status != nullptr: there are few indices and every block looks at
+// all of them itself before it moves anything (one dispatch instead of two; the blocks agree
+// because they read the same indices).  Both nullptr: unchecked bounds.
 struct GatherVerdict {
   const uint32_t *flags;
   uint32_t flag_count;  // <= kBlockThreads
-  uint32_t *status;     // 0 or 1 after the launch, for the host
+  uint32_t *status;     // 0 or kStatusIndexOutOfRange after the launch, for the host
+  uint64_t extent;
 };
 
-// Every block folds the flags; none writes a byte of the output when an index was refused.
+// Every block reaches the same verdict; none writes a byte of the output when an index was refused.
+template <bool kWide, bool kDense>
+__device__ __forceinline__ bool indices_refused(const GatherVerdict &verdict, const GatherIndexView &v) {
+  if (verdict.status == nullptr) return false;
+  int bad = 0;
+  if (verdict.flags != nullptr) {
+    bad = threadIdx.x < verdict.flag_count ? (int)verdict.flags[threadIdx.x] : 0;
+  } else {
+    for (uint32_t i = threadIdx.x; i < v.count; i += blockDim.x) {
+      const int64_t value = index_at<kWide, kDense>(v, i);
+      bad |= (value < 0 || (uint64_t)value >= verdict.extent) ? 1 : 0;
+    }
+  }
+  bad = __syncthreads_or(bad);
+  if (blockIdx.x == 0 && threadIdx.x == 0) *verdict.status = bad ? kStatusIndexOutOfRange : 0u;
+  return bad != 0;
+}
+// The coordinate walk has no index view of its own: it always follows a dispatch of gather_check.
 __device__ __forceinline__ bool indices_refused(const GatherVerdict &verdict) {
-  if (verdict.flags == nullptr) return false;
+  if (verdict.status == nullptr) return false;
   const int bad = __syncthreads_or(threadIdx.x < verdict.flag_count ? (int)verdict.flags[threadIdx.x] : 0);
   if (blockIdx.x == 0 && threadIdx.x == 0) *verdict.status = bad ? kStatusIndexOutOfRange : 0u;
   return bad != 0;
@@ -108,7 +129,7 @@ constexpr int kRowThreads = 2 * kBlockThreads;
 template <int kUnit, bool kWide, bool kDense>
 __global__ __launch_bounds__(kRowThreads) void gather_rows(GatherRows p, GatherIndexView v, GatherVerdict verdict,
                                                            unsigned char *out, uint32_t chunks_per_row, uint32_t chunks) {
-  if (indices_refused(verdict)) return;
+  if (indices_refused<kWide, kDense>(verdict, v)) return;
   const uint32_t chunk = blockIdx.x * (kRowThreads / kBlockThreads) + threadIdx.x / kBlockThreads;
   if (chunk >= chunks) return;
   const uint32_t row = chunk / chunks_per_row, piece = chunk - row * chunks_per_row;
@@ -130,7 +151,7 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_fat(GatherRows p, Gat
   __shared__ const unsigned char *from_of[kFatChunks];
   __shared__ unsigned char *to_of[kFatChunks];
   __shared__ uint32_t units_of[kFatChunks];
-  if (indices_refused(verdict)) return;
+  if (indices_refused<kWide, kDense>(verdict, v)) return;
   if (threadIdx.x < kFatChunks) {
     const uint32_t chunk = blockIdx.x * kFatChunks + threadIdx.x;
     uint32_t units = 0;
@@ -172,7 +193,7 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_fat(GatherRows p, Gat
 template <int kUnit, bool kWide, bool kDense>
 __global__ __launch_bounds__(kBlockThreads) void gather_units(GatherRows p, GatherIndexView v, GatherVerdict verdict,
                                                               unsigned char *out, uint32_t units) {
-  if (indices_refused(verdict)) return;
+  if (indices_refused<kWide, kDense>(verdict, v)) return;
   const uint32_t g = blockIdx.x * kBlockThreads + threadIdx.x;
   if (g >= units) return;
   const uint32_t row = g / p.row_units, u = g - row * p.row_units;
@@ -275,11 +296,13 @@ hipError_t launch_gather(const GatherParams &p, const void *source, const void *
   }
   // strided indices are read bytewise; dense ones at their natural alignment
   const bool dense_indices = p.dense_indices && reinterpret_cast<uintptr_t>(indices) % (p.wide_indices ? 8 : 4) == 0;
-  GatherVerdict verdict{nullptr, 0, nullptr};
-  if (p.checked) {
+  GatherVerdict verdict{nullptr, 0, nullptr, p.extent};
+  if (p.checked && p.fused_check) {
+    verdict.status = static_cast<uint32_t *>(workspace) + kGatherStatusWord;
+  } else if (p.checked) {
     uint32_t *words = static_cast<uint32_t *>(workspace);
     const uint32_t blocks = std::min<uint32_t>(kBlockThreads, (p.index_count + kBlockThreads - 1) / kBlockThreads);
-    verdict = GatherVerdict{words, blocks, words + kGatherStatusWord};
+    verdict = GatherVerdict{words, blocks, words + kGatherStatusWord, p.extent};
     const dim3 grid(blocks), block(kBlockThreads);
     if (p.wide_indices) {
       if (dense_indices) hipLaunchKernelGGL((gather_check<true, true>), grid, block, 0, stream, view, p.extent, words);

@@ -265,7 +265,8 @@ hipError_t launch_concat(const ConcatParams &p, const void *const *inputs, void 
 // before it fold into outer_pitch, so whole rows move; otherwise the output is walked by
 // coordinate with source_strides / index_out_strides per output axis.  checked: a first dispatch
 // leaves one flag per block in the workspace (32-bit words from its start) and the moving dispatch
-// writes nothing when any is set; word kGatherStatusWord then reads 1, else 0.
+// writes nothing when any is set -- or, with few indices, every moving block checks them all
+// itself; word kGatherStatusWord then reads 1, else 0.
 constexpr uint32_t kGatherStatusWord = 256;
 constexpr size_t kGatherWorkspaceBytes = (kGatherStatusWord + 1) * 4;
 struct GatherParams {
@@ -276,6 +277,7 @@ struct GatherParams {
   uint32_t outer = 1, index_count = 0;
   uint8_t size = 4;
   bool wide_indices = false, dense_indices = true, checked = true, rows = false;
+  bool fused_check = false;  // checked, few indices, whole rows: every moving block looks at all indices itself
   int32_t index_rank = 0;
   uint32_t index_dims[kMaxRank] = {};
   int64_t index_strides[kMaxRank] = {};

@@ -1344,8 +1344,13 @@ hyle_hip_status admit(hyle_hip_plan *p) {
         for (int a = 0; a < in[i].rank; ++a) last += (uint64_t)(in[i].dims[a] - 1) * (uint64_t)in[i].byte_strides[a];
         p->concat_input_bytes[i] = p->input_elements[i] == 0 ? 0 : last + dtype_size(in[i].dtype);
       }
+      // Few indices (the rows a step picks for its last tokens, a decode batch's embeddings): every
+      // moving block looks at all of them itself, which saves the checking dispatch.  At most 1024
+      // indices, and at most 8 MiB of index reads over all blocks, counted for the narrowest units.
+      const uint64_t index_bytes = (uint64_t)g.index_count * (g.wide_indices ? 8 : 4);
+      g.fused_check = g.checked && g.rows && g.index_count <= 1024 && (n + 255) / 256 * index_bytes <= (8u << 20);
       p->route = Route::kGather;
-      p->dispatches = g.checked ? 2 : 1;
+      p->dispatches = g.checked && !g.fused_check ? 2 : 1;
       if (g.checked) {
         p->workspace_size = kGatherWorkspaceBytes;
         p->workspace_alignment = 256;

@@ -47,7 +47,9 @@ def gather_on_device(kind, size, storage, lead, shape, strides, dense, axis, ind
     out_shape = list(shape[:normal]) + list(index_shape) + list(shape[normal + 1:])
     assert prepared.output_description() == hc.TensorDesc.dense(kind, out_shape)
     count = int(np.prod(out_shape)) if out_shape else 1
-    assert prepared.dispatch_count() == (0 if count == 0 else (2 if checked else 1))
+    # checked bounds: a dispatch that looks at the indices first, unless they are few and whole rows
+    # move, when every moving block looks at them itself
+    assert prepared.dispatch_count() == (0 if count == 0 else 1) or (checked and prepared.dispatch_count() == 2)
     source, ids = on_device(storage), on_device(index_storage)
     out = torch.full((out_lead + max(count, 1) * size + 16,), poison, dtype=torch.uint8, device=DEVICE)
     need = prepared.workspace_requirement()
@@ -217,6 +219,24 @@ def test_empty_operands_and_rejected_bindings():
     with pytest.raises(hc.StatusError) as refused:
         hollow.create_invocation(0, 0).submit(stream, [source.data_ptr(), ids.data_ptr()], [out.data_ptr()])
     assert refused.value.code == capi.OUT_OF_RANGE
+
+
+def test_few_checked_indices_take_one_dispatch():
+    wide = hc.prepare(context(), hc.Gather(0), hc.TensorDesc.dense(DT.kBFloat16, [4096, 2048]), hc.TensorDesc.dense(DT.kInt32, [8]))
+    many = hc.prepare(context(), hc.Gather(0), hc.TensorDesc.dense(DT.kBFloat16, [4096, 2048]), hc.TensorDesc.dense(DT.kInt32, [2000]))
+    assert wide.dispatch_count() == 1 and many.dispatch_count() == 2
+    assert wide.workspace_requirement().size == many.workspace_requirement().size > 0   # the status word lives there either way
+    rows, width = 4096, 2048
+    values = np.random.default_rng(8).integers(0, 1 << 16, (rows, width), dtype=np.uint64).astype(np.uint16)
+    for count in (1, 8, 1000):
+        ids = np.random.default_rng(count).integers(0, rows, count).astype(np.int64)
+        note(f"gather {count} checked indices in one dispatch")
+        status, got = gather_on_device(DT.kBFloat16, 2, values, 0, [rows, width], None, True, 0, ids, 0, [count], None, True, True)
+        assert status == 0 and np.array_equal(got, values[ids])
+        ids[count // 2] = rows
+        status, got = gather_on_device(DT.kBFloat16, 2, values, 0, [rows, width], None, True, 0, ids, 0, [count], None, True, True,
+                                       poison=0x33)
+        assert status == capi.OUT_OF_RANGE and (got.view(np.uint8) == 0x33).all()
 
 
 def test_embedding_sized_lookup():

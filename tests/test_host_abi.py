@@ -370,6 +370,8 @@ def test_gather_inference_and_admission():
     assert checked.route_name() == "gather" and checked.dispatch_count() == 2
     assert 0 < checked.workspace_requirement().size <= 4096
     assert not checked.alias_support(0, 0) and not checked.alias_support(0, 1)
+    few = hc.prepare(CTX, hc.Gather(0), D(DT.kBFloat16, [4096, 2048]), D(DT.kInt32, [8]))
+    assert few.dispatch_count() == 1 and few.workspace_requirement().size == checked.workspace_requirement().size
     trusted = hc.prepare(CTX, hc.Gather(0, hc.IndexBoundsPolicy.kUnchecked), D(DT.kBFloat16, [151936, 2048]), D(DT.kInt32, [8192]))
     assert trusted.dispatch_count() == 1 and trusted.workspace_requirement().size == 0
     assert hc.prepare(CTX, hc.Gather(0), D(DT.kInt32, [4, 0]), D(DT.kInt32, [4])).dispatch_count() == 0
