@@ -66,22 +66,38 @@ struct GatherVerdict {
   uint64_t extent;
 };
 
-// Every block reaches the same verdict; none writes a byte of the output when an index was refused.
+// This thread's share of the verdict: its flag word, or its share of all indices.
 template <bool kWide, bool kDense>
-__device__ __forceinline__ bool indices_refused(const GatherVerdict &verdict, const GatherIndexView &v) {
-  if (verdict.status == nullptr) return false;
+__device__ __forceinline__ int refusals_seen(const GatherVerdict &verdict, const GatherIndexView &v) {
   int bad = 0;
   if (verdict.flags != nullptr) {
     bad = threadIdx.x < verdict.flag_count ? (int)verdict.flags[threadIdx.x] : 0;
   } else {
-    for (uint32_t i = threadIdx.x; i < v.count; i += blockDim.x) {
-      const int64_t value = index_at<kWide, kDense>(v, i);
-      bad |= (value < 0 || (uint64_t)value >= verdict.extent) ? 1 : 0;
+    // eight indices per thread at a time, their loads in flight together
+    constexpr int kBatch = 8;
+    for (uint32_t first = threadIdx.x; first < v.count; first += kBatch * blockDim.x) {
+      int64_t value[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const uint32_t i = first + j * blockDim.x;
+        value[j] = index_at<kWide, kDense>(v, i < v.count ? i : first);
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) bad |= (value[j] < 0 || (uint64_t)value[j] >= verdict.extent) ? 1 : 0;
     }
   }
+  return bad;
+}
+// Every block reaches the same verdict; none writes a byte of the output when an index was refused.
+__device__ __forceinline__ bool block_refuses(const GatherVerdict &verdict, int bad) {
   bad = __syncthreads_or(bad);
   if (blockIdx.x == 0 && threadIdx.x == 0) *verdict.status = bad ? kStatusIndexOutOfRange : 0u;
   return bad != 0;
+}
+template <bool kWide, bool kDense>
+__device__ __forceinline__ bool indices_refused(const GatherVerdict &verdict, const GatherIndexView &v) {
+  if (verdict.status == nullptr) return false;
+  return block_refuses(verdict, refusals_seen<kWide, kDense>(verdict, v));
 }
 // The coordinate walk has no index view of its own: it always follows a dispatch of gather_check.
 __device__ __forceinline__ bool indices_refused(const GatherVerdict &verdict) {
@@ -151,14 +167,18 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_fat(GatherRows p, Gat
   __shared__ const unsigned char *from_of[kFatChunks];
   __shared__ unsigned char *to_of[kFatChunks];
   __shared__ uint32_t units_of[kFatChunks];
-  if (indices_refused<kWide, kDense>(verdict, v)) return;
+  // A block that checks the indices itself does so while its rows are on their way: it reads from
+  // where its own indices point, held inside the axis, and stores only after the verdict.
+  const bool checks_itself = verdict.status != nullptr && verdict.flags == nullptr;
+  if (!checks_itself && indices_refused<kWide, kDense>(verdict, v)) return;
   if (threadIdx.x < kFatChunks) {
     const uint32_t chunk = blockIdx.x * kFatChunks + threadIdx.x;
     uint32_t units = 0;
     if (chunk < chunks) {
       const uint32_t row = chunk / chunks_per_row, piece = chunk - row * chunks_per_row;
       const uint32_t outer = row / p.index_count, item = row - outer * p.index_count;
-      const int64_t selected = index_at<kWide, kDense>(v, item);
+      int64_t selected = index_at<kWide, kDense>(v, item);
+      if (checks_itself) selected = selected < 0 ? 0 : ((uint64_t)selected >= verdict.extent ? (int64_t)verdict.extent - 1 : selected);
       const uint32_t first = piece * kBlockThreads;
       units = p.row_units - first < (uint32_t)kBlockThreads ? p.row_units - first : (uint32_t)kBlockThreads;
       from_of[threadIdx.x] = p.source + (uint64_t)outer * p.outer_pitch + (uint64_t)selected * p.axis_pitch + (size_t)first * kUnit;
@@ -182,6 +202,7 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_fat(GatherRows p, Gat
     if constexpr (kUnit == 16) loads_issued(held[j]);
     if (j + 1 < kSteps) load(j + 1);
   }
+  if (checks_itself && block_refuses(verdict, refusals_seen<kWide, kDense>(verdict, v))) return;
 #pragma unroll
   for (int j = 0; j < kSteps; ++j) {
     const int c = j * (kRowThreads / kBlockThreads) + half;

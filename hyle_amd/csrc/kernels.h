@@ -277,7 +277,7 @@ struct GatherParams {
   uint32_t outer = 1, index_count = 0;
   uint8_t size = 4;
   bool wide_indices = false, dense_indices = true, checked = true, rows = false;
-  bool fused_check = false;  // checked, few indices, whole rows: every moving block looks at all indices itself
+  bool fused_check = false;  // checked, whole rows, few indices or a large launch: every moving block looks at all indices itself
   int32_t index_rank = 0;
   uint32_t index_dims[kMaxRank] = {};
   int64_t index_strides[kMaxRank] = {};

@@ -1347,8 +1347,17 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       // Few indices (the rows a step picks for its last tokens, a decode batch's embeddings): every
       // moving block looks at all of them itself, which saves the checking dispatch.  At most 1024
       // indices, and at most 8 MiB of index reads over all blocks, counted for the narrowest units.
+      // Long rows in a launch large enough for the blocks of sixteen chunks (4096 chunks of 4 KiB,
+      // whatever unit the addresses allow) check while their rows are on the way, which hides the
+      // index reads: up to 16384 indices and 32 MiB of index reads, counted for 16-byte units
+      // (8192 checked rows of 4 KiB: 12.4 us in one dispatch against 14.5 us in two).
       const uint64_t index_bytes = (uint64_t)g.index_count * (g.wide_indices ? 8 : 4);
-      g.fused_check = g.checked && g.rows && g.index_count <= 1024 && (n + 255) / 256 * index_bytes <= (8u << 20);
+      const uint64_t row_bytes = g.inner * (uint64_t)size, row_count = (uint64_t)g.outer * g.index_count;
+      const uint64_t chunks = (row_bytes + 4095) / 4096 * row_count;
+      const bool few = g.index_count <= 1024 && (n + 255) / 256 * index_bytes <= (8u << 20);
+      const bool overlapped = row_bytes >= 4096 && chunks >= 4096 && g.index_count <= 16384 &&
+                              (chunks + 15) / 16 * index_bytes <= (32u << 20);
+      g.fused_check = g.checked && g.rows && (few || overlapped);
       p->route = Route::kGather;
       p->dispatches = g.checked && !g.fused_check ? 2 : 1;
       if (g.checked) {

@@ -239,6 +239,39 @@ def test_few_checked_indices_take_one_dispatch():
         assert status == capi.OUT_OF_RANGE and (got.view(np.uint8) == 0x33).all()
 
 
+def test_many_long_checked_rows_check_themselves_while_they_load():
+    """A launch large enough for the blocks of sixteen chunks takes one dispatch up to 16384 indices: valid
+    indices move every row, one bad index (negative, past the axis, first or last) moves none; both index
+    widths, rows of 4 KiB and of 4 KiB + 16 bytes (a short last chunk), and an outer group."""
+    D = hc.TensorDesc.dense
+    one = hc.prepare(context(), hc.Gather(0), D(DT.kBFloat16, [5000, 2048]), D(DT.kInt32, [8192]))
+    two = hc.prepare(context(), hc.Gather(0), D(DT.kBFloat16, [5000, 2048]), D(DT.kInt32, [20000]))
+    short = hc.prepare(context(), hc.Gather(0), D(DT.kBFloat16, [5000, 1024]), D(DT.kInt32, [8192]))
+    assert one.dispatch_count() == 1 and two.dispatch_count() == 2 and short.dispatch_count() == 2
+    for rows, width, shape, wide in ((5000, 2048, [4096], False), (3000, 2056, [64, 80], True), (2, 2048, [4100], False)):
+        count = int(np.prod(shape))
+        values = np.random.default_rng(rows).integers(0, 1 << 16, (rows, width), dtype=np.uint64).astype(np.uint16)
+        ids = np.random.default_rng(width).integers(0, rows, shape).astype(np.int64 if wide else np.int32)
+        note(f"gather {shape} checked rows of {2 * width} bytes out of {rows}, one dispatch")
+        status, got = gather_on_device(DT.kBFloat16, 2, values, 0, [rows, width], None, True, 0, ids, 0, shape, None, True, wide)
+        assert status == 0 and np.array_equal(got, values[ids])
+        for place, value in ((0, -1), (count - 1, rows), (count // 3, 1 << 30)):
+            bad = ids.copy().reshape(-1)
+            bad[place] = value
+            status, got = gather_on_device(DT.kBFloat16, 2, values, 0, [rows, width], None, True, 0, bad.reshape(shape), 0, shape,
+                                           None, True, wide, poison=0x77)
+            assert status == capi.OUT_OF_RANGE and (got.view(np.uint8) == 0x77).all()
+    note("gather [3, 1500, 2048] along axis 1 by 1400 checked indices, one dispatch")
+    values = np.random.default_rng(5).integers(0, 1 << 16, (3, 1500, 2048), dtype=np.uint64).astype(np.uint16)
+    ids = np.random.default_rng(6).integers(0, 1500, 1400).astype(np.int32)
+    status, got = gather_on_device(DT.kBFloat16, 2, values, 0, [3, 1500, 2048], None, True, 1, ids, 0, [1400], None, True, False)
+    assert status == 0 and np.array_equal(got, values[:, ids])
+    ids[700] = 1500
+    status, got = gather_on_device(DT.kBFloat16, 2, values, 0, [3, 1500, 2048], None, True, 1, ids, 0, [1400], None, True, False,
+                                   poison=0x42)
+    assert status == capi.OUT_OF_RANGE and (got.view(np.uint8) == 0x42).all()
+
+
 def test_embedding_sized_lookup():
     note("gather embedding [151936, 2048] bf16 by 8192 int32 indices")
     rows, width, count = 151936, 2048, 8192
