@@ -210,7 +210,11 @@ HOST_TEST(GatherFollowsTheSchema) {
   EXPECT(infer_output_descriptions(Gather{2}, {dense(DataType::kFloat32, {4, 3}), dense(DataType::kInt32, {2})}).error().IsOutOfRange());
   auto checked = prepare(context, Gather{0}, dense(DataType::kBFloat16, {151936, 2048}), dense(DataType::kInt32, {8192}));
   REQUIRE(checked.has_value());
-  EXPECT(checked->dispatch_count() == 2 && checked->workspace_requirement().size != 0);
+  // large enough to check inside the moving blocks: one dispatch; 20000 indices take the checking dispatch first
+  EXPECT(checked->dispatch_count() == 1 && checked->workspace_requirement().size != 0);
+  auto many = prepare(context, Gather{0}, dense(DataType::kBFloat16, {151936, 2048}), dense(DataType::kInt32, {20000}));
+  REQUIRE(many.has_value());
+  EXPECT(many->dispatch_count() == 2 && many->workspace_requirement().size == checked->workspace_requirement().size);
   auto trusted = prepare(context, Gather{0, IndexBoundsPolicy::kUnchecked}, dense(DataType::kBFloat16, {151936, 2048}),
                          dense(DataType::kInt32, {8192}));
   REQUIRE(trusted.has_value());

@@ -366,8 +366,10 @@ def test_gather_inference_and_admission():
     with pytest.raises(hc.StatusError) as err:  # rank 5 - 1 + 5 > 8
         hc.infer_output_descriptions(hc.Gather(0), [D(DT.kFloat32, [2] * 5), D(DT.kInt32, [1] * 5)])
     assert err.value.is_invalid_argument()
-    checked = hc.prepare(CTX, hc.Gather(0), D(DT.kBFloat16, [151936, 2048]), D(DT.kInt32, [8192]))
+    checked = hc.prepare(CTX, hc.Gather(0), D(DT.kBFloat16, [151936, 2048]), D(DT.kInt32, [20000]))
     assert checked.route_name() == "gather" and checked.dispatch_count() == 2
+    large = hc.prepare(CTX, hc.Gather(0), D(DT.kBFloat16, [151936, 2048]), D(DT.kInt32, [8192]))   # checks inside the moving blocks
+    assert large.dispatch_count() == 1 and large.workspace_requirement().size == checked.workspace_requirement().size
     assert 0 < checked.workspace_requirement().size <= 4096
     assert not checked.alias_support(0, 0) and not checked.alias_support(0, 1)
     few = hc.prepare(CTX, hc.Gather(0), D(DT.kBFloat16, [4096, 2048]), D(DT.kInt32, [8]))
