@@ -394,7 +394,7 @@ def main() -> int:
                       set_categorical, 16, 64 * 151936 * 4 + 64 * 24, 64 * 151936, "f32", in_step=False,
                       ceiling="ceiling_scan_38mb"))
     if want("next_random_bits_u32"):
-        # Philox4x32-10 words: ten rounds of two 32 x 32 -> 64 products per 16 bytes written (integer work, not bytes, bounds it)
+        # Philox4x32-10 words: ten rounds of two 32 x 32 -> 64 products per 16 bytes written
         def set_bits(i):
             ids = torch.randint(0, 1 << 31, (4096, 4), dtype=torch.int64, device=dev).to(torch.int32)
             return [ids], [torch.empty((4096, 4096), dtype=torch.int32, device=dev)]

@@ -39,7 +39,7 @@ __device__ __forceinline__ PhiloxWords philox_block(uint32_t key0, uint32_t key1
   return v;
 }
 
-// One Philox block (four words) per thread.
+// One Philox block (four words) per thread over the flat block index: short or unaligned rows.
 __global__ __launch_bounds__(kBlockThreads) void random_bits(const uint32_t *identities, uint32_t *out, uint32_t rows,
                                                              uint32_t word_count, uint32_t blocks_per_row, bool vector) {
   const uint64_t total = (uint64_t)rows * blocks_per_row;
@@ -56,6 +56,27 @@ __global__ __launch_bounds__(kBlockThreads) void random_bits(const uint32_t *ide
 #pragma unroll
       for (uint32_t lane = 0; lane < 4; ++lane)
         if (lane < left) to[lane] = words[lane];
+    }
+  }
+}
+
+// Long rows: the row is the block's (its identity sits in scalar registers and nothing is
+// divided), a thread makes four blocks 256 apart, so every store of a wave is 1 KiB in one piece
+// and a thread's earlier stores drain while it works on the next block.
+constexpr int kBitsPerThread = 4;
+__global__ __launch_bounds__(kBlockThreads) void random_bits_rows(const uint32_t *identities, uint32_t *out, uint32_t rows,
+                                                                  uint32_t word_count, uint32_t blocks_per_row) {
+  for (uint32_t row = blockIdx.y; row < rows; row += gridDim.y) {
+    const uint32_t *identity = identities + (size_t)row * 4;
+    const uint32_t key0 = identity[0], key1 = identity[1], draw0 = identity[2], draw1 = identity[3];
+    uint32_t *to = out + (uint64_t)row * word_count;
+#pragma unroll
+    for (int j = 0; j < kBitsPerThread; ++j) {
+      const uint32_t column = (blockIdx.x * kBitsPerThread + j) * kBlockThreads + threadIdx.x;
+      if (column < blocks_per_row) {
+        const PhiloxWords w = philox_block(key0, key1, draw0, draw1, column);
+        store16_stream(to, column, u32x4{w.x0, w.x1, w.x2, w.x3});
+      }
     }
   }
 }
@@ -360,6 +381,13 @@ hipError_t launch_random_bits(const RandomBitsParams &p, const void *identities,
   uint64_t blocks = (total + kBlockThreads - 1) / kBlockThreads;
   blocks = blocks > 65535 ? 65535 : blocks;
   const bool vector = p.word_count % 4 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  if (vector && blocks_per_row >= kBlockThreads) {
+    const uint32_t per_block = kBlockThreads * kBitsPerThread;
+    const dim3 grid((blocks_per_row + per_block - 1) / per_block, p.rows < 65535u ? p.rows : 65535u);
+    hipLaunchKernelGGL(random_bits_rows, grid, dim3(kBlockThreads), 0, stream, static_cast<const uint32_t *>(identities),
+                       static_cast<uint32_t *>(out), p.rows, p.word_count, blocks_per_row);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL(random_bits, dim3((uint32_t)blocks), dim3(kBlockThreads), 0, stream, static_cast<const uint32_t *>(identities),
                      static_cast<uint32_t *>(out), p.rows, p.word_count, blocks_per_row, vector);
   return hipGetLastError();

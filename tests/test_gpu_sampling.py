@@ -59,6 +59,12 @@ def test_random_bits_match_philox_word_for_word():
     assert np.array_equal(random_bits_on_device(ids, 1024), orc.random_bits(ids, 1024))
     assert np.array_equal(random_bits_on_device(ids[:333], 1001), orc.random_bits(ids[:333], 1001))
     assert np.array_equal(random_bits_on_device(ids[:333], 64, lead=4), orc.random_bits(ids[:333], 64))
+    note("random bits, long rows (a block per row piece): 3 x 4100, 2 x 16388, 5 x 1024 past an odd lead, 66000 x 1024")
+    assert np.array_equal(random_bits_on_device(ids[:3], 4100), orc.random_bits(ids[:3], 4100))
+    assert np.array_equal(random_bits_on_device(ids[:2], 16388), orc.random_bits(ids[:2], 16388))
+    assert np.array_equal(random_bits_on_device(ids[:5], 1024, lead=12), orc.random_bits(ids[:5], 1024))
+    many = np.random.default_rng(10).integers(0, 1 << 32, (66000, 4), dtype=np.uint64).astype(np.uint32)   # more rows than grid.y holds
+    assert np.array_equal(random_bits_on_device(many, 1024), orc.random_bits(many, 1024))
 
 
 def categorical_on_device(type_id, stored: np.ndarray, ids: np.ndarray, scored: bool, static: bool = False):
