@@ -257,8 +257,82 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_lines(const unsigne
   }
 }
 
-// Longer rows (K = 2048 n from 4096 up to 10240 or 12288) and two to eight activation rows (any
-// K = 2048 n whose activations fit): the same walk over spans of 2048 values, with the
+// One activation row against rows of kSpans spans of 2048 values, a wave of the block per span:
+// the wave keeps its span of x in registers as the kernel above does (no staging of x through
+// LDS, so a block starts on its rows at once, which is most of the time when a wave has only a
+// row or two to walk: Q4_K [6144 -> 2048] has 2048 rows for 1024 compute-unit SIMDs), walks the
+// block's rows span by span and leaves its share of each row in LDS, where the first wave adds
+// the spans' shares in span order.
+template <int kKind, class TX, int kSpans>
+__global__ __launch_bounds__(kSpans * kWaveLanes) void gguf_matvec_spans(const unsigned char *weights, const void *x, void *y,
+                                                                       uint32_t rows, uint64_t row_stride) {
+  using Row = LinesRow<kKind, 1>;
+  using Kind = Lines<kKind>;
+  constexpr uint32_t kSpanBytes = Kind::kPassVectors * 16;
+  __shared__ __align__(16) unsigned char slots[kSpans][Row::kSlotBytes];
+  __shared__ float shares[kSpans][kLinesDepth];
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t span = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  unsigned char *slot = slots[span];
+  float xs[32], xsum[4];
+  const typename Kind::Lane at = Kind::lane_of(0, lane);
+#pragma unroll
+  for (int e = 0; e < 32; ++e) xs[e] = Traits<TX>::load(x, Kind::position(span, lane, e));
+#pragma unroll
+  for (int part = 0; part < 4; ++part) {
+    xsum[part] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) xsum[part] += xs[8 * part + t];
+  }
+  const uint32_t stride = gridDim.x, first = blockIdx.x;  // first < rows: the grid has at most `rows` blocks
+  const unsigned char *mine = weights + (size_t)span * kSpanBytes;
+  Row ring[kLinesDepth];
+#pragma unroll
+  for (int d = 0; d < kLinesDepth; ++d) {
+    const uint64_t wanted = (uint64_t)first + (uint64_t)d * stride;
+    ring[d] = Row::load(mine + (size_t)(wanted < rows ? (uint32_t)wanted : first) * row_stride, lane);
+  }
+  for (uint64_t base = first; base < rows; base += (uint64_t)kLinesDepth * stride) {
+    float totals[kLinesDepth] = {};
+#pragma unroll
+    for (int d = 0; d < kLinesDepth; ++d) {
+      const uint64_t row = base + (uint64_t)d * stride;
+      if (row >= rows) break;
+#pragma unroll
+      for (int i = 0; i < Row::kLoads; ++i)
+        *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = ring[d].v[i];
+      const uint64_t wanted = row + (uint64_t)kLinesDepth * stride;
+      ring[d] = Row::load(mine + (size_t)(wanted < rows ? (uint32_t)wanted : first) * row_stride, lane);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      totals[d] = Kind::dot(slot, at, xs, xsum);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    // as above: lane l < 4 ends with row l's sum over the wave
+    static_assert(kLinesDepth == 4, "the joint reduction is written for four rows");
+    const bool odd = (lane & 1u) != 0, upper = (lane & 2u) != 0;
+    const float pair01 = (odd ? totals[1] : totals[0]) + __shfl_xor(odd ? totals[0] : totals[1], 1);
+    const float pair23 = (odd ? totals[3] : totals[2]) + __shfl_xor(odd ? totals[2] : totals[3], 1);
+    float share = (upper ? pair23 : pair01) + __shfl_xor(upper ? pair01 : pair23, 2);
+#pragma unroll
+    for (int step = 4; step < kWaveLanes; step *= 2) share += __shfl_xor(share, step);
+    if (lane < (uint32_t)kLinesDepth) shares[span][lane] = share;
+    __syncthreads();
+    const uint64_t row = base + (uint64_t)lane * stride;
+    if (span == 0 && lane < (uint32_t)kLinesDepth && row < rows) {
+      float whole = shares[0][lane];
+#pragma unroll
+      for (int other = 1; other < kSpans; ++other) whole += shares[other][lane];
+      Traits<TX>::store(y, (size_t)row, whole);
+    }
+    __syncthreads();
+  }
+}
+
+// Two to eight activation rows (any K = 2048 n whose activations fit) and one row longer than six
+// spans: the same walk over spans of 2048 values, with the
 // activations as f32 in LDS instead of registers.  They are laid out [span][e / 4][lane][e % 4], so
 // that a lane fetches its 32 values of a span with eight 16-byte reads that are contiguous across
 // the wave; Q4_K's per-lane sums of x sit beside them.  A wave walks the spans of its rows one
@@ -425,11 +499,29 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
                          p.row_stride);
       return hipGetLastError();
     }
-    // longer rows: x in LDS, as long as it fits in a block's 64 KiB beside the waves' row buffers
-    // (for K = 4096 this measured slightly faster than 64 activations in registers: 13.8 against
-    // 14.4 us for Q4_K [4096 -> 14336])
+    // several activation rows, or more spans: x in LDS, as long as it fits in a block's 64 KiB
+    // beside the waves' row buffers
     const size_t staged = (size_t)p.m * (p.k / 2048) * (2048 + (kKind == 0 ? 256 : 0)) * sizeof(float);
     const size_t parked = (size_t)kWavesPerBlock * LinesRow<kKind, 1>::kSlotBytes;
+    // one activation row, two to six spans: a wave per span, twelve waves per compute unit
+    // (Q4_K [6144 -> 2048]: 4.8 us with 4 blocks of three waves per unit, 4.9 / 5.4 / 6.6 / 7.3 us
+    // with 3 / 2 / 6 / 8; [4096 -> 14336]: 11.7 us with 6 blocks of two waves, 13.4 / 13.7 us with
+    // 4 / 8; with the activations staged in LDS as below: 8.1 and 14.3 us, and 24 against 15 us
+    // for [12288 -> 4096])
+    if (p.m == 1 && lines && p.k % 2048 == 0 && p.k >= 4096 && p.k <= 12288) {
+      const uint32_t spans = p.k / 2048;
+      const uint32_t most = units * (12u / spans);
+      const dim3 machine((uint32_t)p.rows < most ? (uint32_t)p.rows : most);
+      const uint32_t rows = (uint32_t)p.rows;
+      switch (spans) {
+        case 2: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 2>), machine, dim3(2 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+        case 3: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 3>), machine, dim3(3 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+        case 4: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 4>), machine, dim3(4 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+        case 5: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 5>), machine, dim3(5 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+        default: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 6>), machine, dim3(6 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      }
+      return hipGetLastError();
+    }
     if (lines && p.k % 2048 == 0 && (p.k > 2048 || p.m > 1) && staged + parked <= 64 * 1024) {
       const uint32_t spans = p.k / 2048;
       const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);

@@ -110,11 +110,13 @@ def test_matvec_single_token_forms(tag, x_tag):
 @pytest.mark.parametrize("x_tag", ["f32", "bf16"])
 @pytest.mark.parametrize("tag", ["q4_k", "q6_k", "q8_0"])
 def test_matvec_single_token_long_rows(tag, x_tag):
-    """One activation row over 6144 to 12288 values (whole 2048-value spans): activations in LDS,
-    a wave walks the spans of its rows.  Row counts around the number of waves of the grid, and
-    one past the LDS limit that falls back to the general kernel."""
+    """One activation row over two to six whole 2048-value spans: a wave of the block per span, its
+    activations in registers, the spans' shares added in LDS.  Row counts below, at and around the
+    number of blocks of the grid (twelve waves per compute unit), blocks that take more than the
+    four rows they keep in flight; seven spans take the kernel that stages the activations in LDS."""
     rng = np.random.default_rng(1704)
-    for rows, k in ((2048, 6144), (3, 8192), (3100, 10240), (37, 12288)):
+    for rows, k in ((2048, 6144), (3, 8192), (3100, 10240), (37, 12288), (7000, 4096), (1025, 6144), (4100, 8192),
+                    (40, 14336)):
         raw = weights_for(tag, rng, rows, k)
         note(f"matvec {tag} long rows {rows} k {k} x {x_tag}")
         check(tag, x_tag, raw, rows, k, rng.normal(0, 1, k).astype(np.float32))
