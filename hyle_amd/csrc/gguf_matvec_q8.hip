@@ -413,6 +413,71 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_lines(const unsi
   if (filled != 0) flush(row - (uint32_t)filled * stride, filled);
 }
 
+// One activation row, one to six spans: a wave of the block per span.  The wave quantises its own
+// span of x straight into registers (nothing is parked in LDS and no barrier precedes the first
+// row), walks the block's rows at its span and leaves its share of each row in LDS, where the
+// first wave adds the spans' shares in span order.
+template <int kKind, class TX, int kSpans>
+__global__ __launch_bounds__(kSpans * kWaveLanes) void gguf_matvec_q8_spans(const unsigned char *weights, const void *x, void *y,
+                                                                          uint32_t rows, uint64_t row_stride) {
+  using Row = LinesRow<kKind, 1>;
+  using Kind = Lines<kKind>;
+  constexpr uint32_t kSpanBytes = Kind::kPassVectors * 16;
+  __shared__ __align__(16) unsigned char slots[kSpans][Row::kSlotBytes];
+  __shared__ float shares[kSpans][kLinesDepth];
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t span = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  unsigned char *slot = slots[span];
+  const typename Kind::Lane at = Kind::lane_of(0, lane);
+  const uint32_t stride = gridDim.x, first = blockIdx.x;  // first < rows: the grid has at most `rows` blocks
+  const unsigned char *mine = weights + (size_t)span * kSpanBytes;
+  Row ring[kLinesDepth];
+#pragma unroll
+  for (int d = 0; d < kLinesDepth; ++d) {
+    const uint64_t wanted = (uint64_t)first + (uint64_t)d * stride;
+    ring[d] = Row::load(mine + (size_t)(wanted < rows ? (uint32_t)wanted : first) * row_stride, lane);
+  }
+  const LaneCodes held = quantise_span<kKind, TX>(x, 0, span, lane);  // while the first rows are on their way
+  for (uint64_t base = first; base < rows; base += (uint64_t)kLinesDepth * stride) {
+    float totals[kLinesDepth] = {};
+#pragma unroll
+    for (int d = 0; d < kLinesDepth; ++d) {
+      const uint64_t row = base + (uint64_t)d * stride;
+      if (row >= rows) break;
+#pragma unroll
+      for (int i = 0; i < Row::kLoads; ++i)
+        *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = ring[d].v[i];
+      const uint64_t wanted = row + (uint64_t)kLinesDepth * stride;
+      ring[d] = Row::load(mine + (size_t)(wanted < rows ? (uint32_t)wanted : first) * row_stride, lane);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      SpanDot<kKind> decoded;
+      decoded.decode(slot, at);
+      totals[d] = decoded.against(held);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+    static_assert(kLinesDepth == 4, "the joint sum is taken over four rows");
+    const float share = joint_sum<kLinesDepth>(totals, lane);  // lane l < 4: row l over the wave
+    if constexpr (kSpans == 1) {
+      const uint64_t row = base + (uint64_t)lane * stride;
+      if (lane < (uint32_t)kLinesDepth && row < rows) Traits<TX>::store(y, (size_t)row, share);
+    } else {
+      if (lane < (uint32_t)kLinesDepth) shares[span][lane] = share;
+      __syncthreads();
+      const uint64_t row = base + (uint64_t)lane * stride;
+      if (span == 0 && lane < (uint32_t)kLinesDepth && row < rows) {
+        float whole = shares[0][lane];
+#pragma unroll
+        for (int other = 1; other < kSpans; ++other) whole += shares[other][lane];
+        Traits<TX>::store(y, (size_t)row, whole);
+      }
+      __syncthreads();
+    }
+  }
+}
+
 // ---- several activation rows: the integer dots on the matrix unit ------------------------------
 // v_mfma_i32_4x4x4i8 is sixteen independent 4 x 4 x 4 products, one per quad of lanes: lane q of a
 // quad gives row q of A (four int8 along k) and column q of B, and gets column q of D back, one
@@ -677,6 +742,27 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
     // several activation rows: the quad form, if its four row slots per wave fit beside the codes
     const size_t slots = (size_t)kWavesPerBlock * 4 * (LinesRow<kKind, 1>::kSlotBytes + 32);
     if (p.m >= 2 && slots + shared <= 64 * 1024) return run_quads<kKind, TX>(p, w, x, y, spans, grid, shared, s);
+  }
+  if (p.m == 1 && spans <= 6) {
+    // One activation row: a wave per span.  Eight waves per compute unit measured best or equal in
+    // 25 of 27 shapes (three formats, K = 2048 ... 12288, 1024 ... 151936 rows: 0-30 % below the
+    // kernel that parks the codes in LDS first); Q4_K over many rows wants twelve
+    // ([4096 -> 151936]: 79 us with 12, 90 us with 8, 93 us parked).
+    const uint32_t units = (uint32_t)(compute_units > 0 ? compute_units : 256);
+    const uint32_t waves = kKind == 0 && p.rows * spans >= 65536 ? 12u : 8u;
+    const uint32_t most = units * (waves / spans);
+    const dim3 blocks((uint32_t)p.rows < most ? (uint32_t)p.rows : most);
+    const unsigned char *in = static_cast<const unsigned char *>(w);
+    const uint32_t rows = (uint32_t)p.rows;
+    switch (spans) {
+      case 1: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 1>), blocks, dim3(1 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      case 2: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 2>), blocks, dim3(2 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      case 3: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 3>), blocks, dim3(3 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      case 4: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 4>), blocks, dim3(4 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      case 5: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 5>), blocks, dim3(5 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      default: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 6>), blocks, dim3(6 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+    }
+    return hipGetLastError();
   }
   if (p.m == 1) return run_registers<kKind, TX, 1>(p, w, x, y, spans, grid, shared, s);
   if (p.m == 2) return run_registers<kKind, TX, 2>(p, w, x, y, spans, grid, shared, s);

@@ -72,7 +72,10 @@ def test_q8_route_shapes_and_batches(tag, x_tag):
     rng = np.random.default_rng(1800)
     for rows, k, m in ((1, 2048, 1), (67, 2048, 1), (130, 2048, 2), (9, 2048, 3), (33, 2048, 4), (21, 2048, 5),
                        (40, 2048, 8), (6, 4096, 1), (19, 4096, 2), (13, 4096, 4), (9000, 2048, 3), (5, 6144, 1),
-                       (3, 12288, 1), (7, 8192, 1)):
+                       (3, 12288, 1), (7, 8192, 1),
+                       # one row, a wave per span: blocks with one row, with more than the four in flight, five and
+                       # seven spans (the last parks its codes in LDS)
+                       (9000, 2048, 1), (5000, 4096, 1), (1030, 6144, 1), (600, 10240, 1), (5, 14336, 1)):
         raw = weights_for(tag, rng, rows, k)
         x = rng.normal(0, 1.5, (m, k) if m > 1 else (k,)).astype(np.float32)
         note(f"q8 matvec {tag} x {x_tag} rows {rows} k {k} m {m}")
