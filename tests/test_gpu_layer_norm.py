@@ -22,7 +22,7 @@ from gpu_support import (DEVICE, TYPES, assert_close_f32, assert_narrow_ulp, con
 pytestmark = pytest.mark.gpu
 
 
-def layer_bar(got, want, tag):
+def layer_bar(got, want, tag, bias=None):
     if tag == "f32":
         # the reference's mean is a running f32 sum, whose error bound grows with the row
         # length; beyond 4096 columns the floor grows with it (width / 4096)
@@ -35,7 +35,13 @@ def layer_bar(got, want, tag):
         oid = TYPES[tag][1]
         width = want.shape[-1]
         g, w = orc.to_f32(oid, got).astype(np.float64), orc.to_f32(oid, want).astype(np.float64)
-        near_mean = np.abs(g - w) <= 2e-6 * max(1.0, width / 4096.0)
+        floor = 2e-6 * max(1.0, width / 4096.0)
+        if bias is not None:
+            # fma(normalised * scale, bias): where the two nearly cancel, the result carries the product's
+            # error (the inverse deviation's: running against tree sums of `width` squares), not its own
+            shift = bias if bias.dtype == np.float32 else orc.to_f32(oid, bias)   # f32 parameters, or the input's own type
+            floor = floor + 1e-5 * max(1.0, width / 4096.0) * np.abs(shift.astype(np.float64))
+        near_mean = np.abs(g - w) <= floor
         assert np.array_equal(np.isnan(g), np.isnan(w))
         assert_narrow_ulp(np.where(near_mean, want, got), want, tag)
 
@@ -113,6 +119,30 @@ def test_layer_norm_schema_errors_and_declines():
     with pytest.raises(hc.StatusError) as err:  # strided input: left to another provider
         hc.prepare(ctx, hc.LayerNorm(), hc.TensorDesc.strided_bytes(DT.kFloat32, [4, 64], [512, 4]))
     assert err.value.is_unimplemented()
+
+
+@pytest.mark.parametrize("tag,param_tag", [("f32", "f32"), ("bf16", "bf16"), ("bf16", "f32"), ("f16", "f16")])
+def test_layer_norm_launches_that_cover_the_tensor_exactly(tag, param_tag):
+    """64 rows of every width that fills a launch shape's lanes with whole vectors: the kernels that mask
+    nothing (the other test's row counts and widths leave lanes or rows over), in all three parameter forms."""
+    oid, pid = TYPES[tag][1], TYPES[param_tag][1]
+    rng = np.random.default_rng(502)
+    per_vector = 4 if tag == "f32" else 8
+    for vectors in (8, 16, 32, 64, 128, 256, 512, 1024, 2048, 4096, 8192):
+        rows, width = 64, vectors * per_vector
+        x = host_values((rng.normal(-0.3, 1, (rows, width)) * rng.uniform(0.1, 10, (rows, 1))).astype(np.float32), tag)
+        scale = host_values(rng.normal(1, 0.1, width).astype(np.float32), param_tag)
+        bias = host_values(rng.normal(0, 0.5, width).astype(np.float32), param_tag)
+        dx, ds, db = to_device(x, tag), to_device(scale, param_tag), to_device(bias, param_tag)
+        op = hc.LayerNorm(epsilon=1e-6)
+        note(f"LayerNorm {tag} (params {param_tag}) [{rows}, {width}] exact cover: plain, scale, affine")
+        if tag == param_tag:
+            (out,) = run(op, dx)
+            layer_bar(to_host(out), orc.layer_norm(oid, x, None, None, 1e-6), tag)
+        (out,) = run(op, dx, ds)
+        layer_bar(to_host(out), orc.layer_norm(oid, x, scale, None, 1e-6, param_type=pid), tag)
+        (out,) = run(op, dx, ds, db)
+        layer_bar(to_host(out), orc.layer_norm(oid, x, scale, bias, 1e-6, param_type=pid), tag, bias=bias)
 
 
 def test_layer_norm_bench_shape_and_shift_invariance():
