@@ -14,133 +14,10 @@
 //   LayerNorm  mean = sum(x) / n, inv = 1 / sqrt(sum((x - mean)^2) / n + eps),
 //              then fma((x - mean) * inv, scale, bias); scale alone multiplies
 // with a true divide and square root and one RN-even store.
-#include <type_traits>
-
-#include "device_common.h"
-#include "kernels.h"
+#include "norm_rows.h"
 
 namespace hyle_hip {
 namespace {
-
-template <class W, int kVec>
-__device__ __forceinline__ void load_weight(const void *w, uint32_t vec, float (&out)[kVec]) {
-  if constexpr (Traits<W>::kVec == kVec) {
-    Traits<W>::unpack(load16(w, vec), out);
-  } else {  // f32 parameters under a narrow input: two vectors per input vector
-    float lo[4], hi[4];
-    Traits<F32>::unpack(load16(w, 2 * (size_t)vec), lo);
-    Traits<F32>::unpack(load16(w, 2 * (size_t)vec + 1), hi);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      out[j] = lo[j];
-      out[4 + j] = hi[j];
-    }
-  }
-}
-
-enum : int { kPlain = 0, kScale = 1, kScaleBias = 2 };  // learned parameters of a launch
-
-// `kRows` consecutive rows share one group of lanes.  Loads carry no branches (a lane outside
-// the row, or a row outside the tensor, reads a clamped, valid address and zeroes the value).
-// The rows are loaded one after another (the kVpl loads of a row together, the next row once
-// they have arrived), the parameter vectors are fetched once for all rows, and every store
-// follows the last load: a block reads in one phase and writes in another, which for tensors of
-// a few tens of MB measured 10-15 % faster on MI355X than issuing all loads of a lane at once.
-// `kExact` launches cover the tensor exactly (every lane a vector of every row of its group), so
-// nothing is masked, and `kParameters` is fixed per instantiation: per element the bf16 LayerNorm
-// is ten vector instructions instead of sixteen.  One such instruction per element is 0.44 us of
-// every SIMD's time for 16.7 M elements, which the loads do not hide once all waves of a launch
-// are resident together and move through their phases side by side.
-template <class T, class W, int kLanes, int kVpl, int kThreads, int kRows, bool kLayer, int kParameters, bool kExact>
-__global__ __launch_bounds__(kThreads) void norm_rows(const void *x, const void *w, const void *b,
-                                                      void *y, uint32_t rows, uint32_t row_vectors,
-                                                      float width, float epsilon) {
-  constexpr int parameters = kParameters;
-  constexpr int kVec = Traits<T>::kVec;
-  constexpr int kGroupsPerBlock = kThreads / kLanes;
-  __shared__ float joint[kLayer ? 2 : 1][kRows][kThreads / kWaveLanes];
-  const uint32_t lane = threadIdx.x % kLanes;
-  const uint32_t first_row = (blockIdx.x * kGroupsPerBlock + threadIdx.x / kLanes) * kRows;
-
-  u32x4 raw[kRows][kVpl];
-  uint32_t vec[kVpl];
-#pragma unroll
-  for (int k = 0; k < kVpl; ++k) {
-    const uint32_t wanted = lane + k * kLanes;
-    vec[k] = kExact || wanted < row_vectors ? wanted : row_vectors - 1;
-  }
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const uint32_t row = kExact || first_row + r < rows ? first_row + r : rows - 1;
-    const size_t row_base = (size_t)row * row_vectors;
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) raw[r][k] = load16_stream(x, row_base + vec[k]);
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) loads_issued(raw[r][k]);
-  }
-  float scale[kVpl][kVec], bias[kVpl][kVec];
-  if constexpr (parameters != kPlain) {
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) load_weight<W, kVec>(w, vec[k], scale[k]);
-  }
-  if constexpr (kLayer && parameters == kScaleBias) {
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) load_weight<W, kVec>(b, vec[k], bias[k]);
-  }
-  // Row by row: measured on MI355X, reducing the statistics of both rows behind one barrier
-  // is slower (RMSNorm over [8192, 2048] bf16: 13.5 us against 11.4 us).
-  float v[kRows][kVpl][kVec];
-  float inverse[kRows];
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    bool ok[kVpl];
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) {
-      ok[k] = kExact || (first_row + r < rows && lane + k * kLanes < row_vectors);
-      Traits<T>::unpack(raw[r][k], v[r][k]);
-    }
-    if constexpr (kLayer) {
-      float sum = 0.0f;
-#pragma unroll
-      for (int k = 0; k < kVpl; ++k)
-#pragma unroll
-        for (int j = 0; j < kVec; ++j) sum += ok[k] ? v[r][k][j] : 0.0f;
-      const float mean = row_sum<kLanes>(sum, joint[1][r]) / width;
-#pragma unroll
-      for (int k = 0; k < kVpl; ++k)
-#pragma unroll
-        for (int j = 0; j < kVec; ++j) v[r][k][j] -= mean;
-    }
-    float squares = 0.0f;
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k)
-#pragma unroll
-      for (int j = 0; j < kVec; ++j) {
-        v[r][k][j] = ok[k] ? v[r][k][j] : 0.0f;
-        squares = __builtin_fmaf(v[r][k][j], v[r][k][j], squares);
-      }
-    squares = row_sum<kLanes>(squares, joint[0][r]);
-    inverse[r] = 1.0f / sqrtf(squares / width + epsilon);
-  }
-#pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const uint32_t row = first_row + r;
-    const size_t row_base = (size_t)row * row_vectors;
-#pragma unroll
-    for (int k = 0; k < kVpl; ++k) {
-      if (kExact || (row < rows && lane + k * kLanes < row_vectors)) {
-        float out[kVec];
-#pragma unroll
-        for (int j = 0; j < kVec; ++j) {
-          out[j] = v[r][k][j] * inverse[r];
-          if constexpr (kLayer && parameters == kScaleBias) out[j] = __builtin_fmaf(out[j], scale[k][j], bias[k][j]);
-          else if constexpr (parameters != kPlain) out[j] = out[j] * scale[k][j];
-        }
-        store16_stream(y, row_base + vec[k], Traits<T>::pack(out));
-      }
-    }
-  }
-}
 
 // Any width, any element alignment: one block per row, the row is re-read for each pass
 // (the re-reads come from cache).
@@ -172,11 +49,6 @@ __global__ __launch_bounds__(kBlockThreads) void norm_generic(const void *x, con
     Traits<T>::store(y, base + i, r);
   }
 }
-
-struct Bound {
-  const void *x, *w, *b;
-  void *y;
-};
 
 template <class T, class W, bool kLayer, int kLanes, int kVpl, int kThreads = kBlockThreads, int kRows = 1>
 hipError_t run_rows(const NormParams &p, const Bound &io, int parameters, hipStream_t s) {
@@ -258,6 +130,11 @@ hipError_t run_typed(Elem type, const NormParams &p, const Bound &io, bool vecto
 hipError_t launch_norm(Elem type, const NormParams &p, const void *x, const void *w, const void *b,
                        void *y, bool vectorised, hipStream_t stream) {
   if (p.shape.rows == 0 || p.shape.width == 0) return hipSuccess;
+  if (vectorised) {  // a shape that covers the tensor exactly, when there is one
+    const bool launched = p.layer ? launch_norm_exact_layer(type, p, x, w, b, y, stream)
+                                  : launch_norm_exact_rms(type, p, x, w, y, stream);
+    if (launched) return hipGetLastError();
+  }
   const Bound io{x, w, b, y};
   return p.layer ? run_typed<true>(type, p, io, vectorised, stream)
                  : run_typed<false>(type, p, io, vectorised, stream);

@@ -261,6 +261,35 @@ def test_rms_norm_domain_values_every_route(tag, weight_tag):
             assert_narrow_ulp(to_host(out), want, tag)
 
 
+@pytest.mark.parametrize("tag,weight_tag", [("bf16", "bf16"), ("bf16", "f32"), ("f16", "f16"), ("f32", "f32")])
+def test_rms_norm_launches_that_cover_the_tensor_exactly(tag, weight_tag):
+    """An even number of rows of 64 n, 128 n or 256 n whole vectors (n <= 8): the launch shapes that mask
+    nothing, with and without the weight; one width past them and an odd row count take the masked shapes."""
+    oid, wid = TYPES[tag][1], TYPES[weight_tag][1]
+    rng = np.random.default_rng(77)
+    per_vector = 4 if tag == "f32" else 8
+    for rows, vectors in ((6, 320), (6, 384), (6, 448), (6, 512), (6, 640), (6, 768), (6, 896), (6, 1024), (6, 1280),
+                          (6, 1536), (6, 1792), (6, 2048), (64, 512), (6, 2304), (7, 512)):
+        hidden = vectors * per_vector
+        vals = (rng.normal(0, 1, (rows, hidden)) * rng.uniform(0.1, 10, (rows, 1))).astype(np.float32)
+        scale = rng.normal(1, 0.1, hidden).astype(np.float32)
+        xs, ws = host_values(vals, tag), host_values(scale, weight_tag)
+        note(f"rmsnorm {tag}/{weight_tag} [{rows}, {hidden}]: with and without weight")
+        (out,) = run(hc.RmsNorm(epsilon=1e-6), to_device(xs, tag), to_device(ws, weight_tag))
+        want = orc.rms_norm(oid, xs, ws, 1e-6, weight_type=wid)
+        if tag == "f32":
+            assert_close_f32(to_host(out), want, rel=1e-5)
+        else:
+            assert_narrow_ulp(to_host(out), want, tag)
+        if tag == weight_tag:
+            (out,) = run(hc.RmsNorm(epsilon=1e-6), to_device(xs, tag))
+            want = orc.rms_norm(oid, xs, None, 1e-6)
+            if tag == "f32":
+                assert_close_f32(to_host(out), want, rel=1e-5)
+            else:
+                assert_narrow_ulp(to_host(out), want, tag)
+
+
 def test_rms_norm_zero_rows_and_zero_hidden():
     for shape in ((0, 128), (4, 0)):
         note(f"rmsnorm empty {shape}")
