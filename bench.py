@@ -279,6 +279,20 @@ def main() -> int:
         ops.append(Op("next_layer_norm_bf16", hc.LayerNorm(epsilon=1e-6),
                       [D(BF, [8192, 2048]), D(BF, [2048]), D(BF, [2048])], set_ln, 10,
                       2 * 8192 * 2048 * 2 + 2 * 4096, 8192 * 2048, "bf16", in_step=False))
+    # the norms at other hidden sizes (the same 67 MB): launch shapes that cover the tensor exactly
+    for name, layer, rows_n, hidden_n in (("next_rms_norm_bf16_hidden_4096", False, 4096, 4096),
+                                         ("next_layer_norm_bf16_hidden_8192", True, 2048, 8192)):
+        if not want(name):
+            continue
+
+        def set_wide(i, layer=layer, rows_n=rows_n, hidden_n=hidden_n):
+            dx = torch.empty((rows_n, hidden_n), dtype=torch.bfloat16, device=dev).normal_()
+            scale = torch.empty(hidden_n, dtype=torch.bfloat16, device=dev).normal_(1.0, 0.1)
+            return ([dx, scale, scale.clone()] if layer else [dx, scale]), [torch.empty_like(dx)]
+        descs = [D(BF, [rows_n, hidden_n]), D(BF, [hidden_n])] + ([D(BF, [hidden_n])] if layer else [])
+        ops.append(Op(name, hc.LayerNorm(epsilon=1e-6) if layer else hc.RmsNorm(epsilon=1e-6), descs, set_wide, 10,
+                      2 * rows_n * hidden_n * 2 + (2 if layer else 1) * hidden_n * 2, rows_n * hidden_n, "bf16",
+                      in_step=False, ceiling="ceiling_copy_67mb"))
     if want("next_geglu_tanh_bf16") or want("next_gelu_bf16"):
         gate_g, up_g = wl.config3_swiglu()
 
