@@ -134,7 +134,7 @@ def test_layer_norm_launches_that_cover_the_tensor_exactly(tag, param_tag):
     oid, pid = TYPES[tag][1], TYPES[param_tag][1]
     rng = np.random.default_rng(502)
     per_vector = 4 if tag == "f32" else 8
-    for vectors in (8, 16, 32, 64, 128, 192, 256, 320, 384, 448, 512, 640, 768, 896, 1024, 1280, 1536, 1792, 2048, 4096, 8192):
+    for vectors in (8, 16, 32, 64, 128, 192, 256, 320, 384, 448, 512, 576, 640, 768, 896, 1024, 1280, 1536, 1792, 2048, 4096, 8192):
         rows, width = 64, vectors * per_vector
         x = host_values((rng.normal(-0.3, 1, (rows, width)) * rng.uniform(0.1, 10, (rows, 1))).astype(np.float32), tag)
         scale = host_values(rng.normal(1, 0.1, width).astype(np.float32), param_tag)

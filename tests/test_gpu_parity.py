@@ -268,7 +268,7 @@ def test_rms_norm_launches_that_cover_the_tensor_exactly(tag, weight_tag):
     oid, wid = TYPES[tag][1], TYPES[weight_tag][1]
     rng = np.random.default_rng(77)
     per_vector = 4 if tag == "f32" else 8
-    for rows, vectors in ((6, 320), (6, 384), (6, 448), (6, 512), (6, 640), (6, 768), (6, 896), (6, 1024), (6, 1280),
+    for rows, vectors in ((6, 320), (6, 384), (6, 448), (6, 512), (6, 576), (6, 640), (6, 768), (6, 896), (6, 1024), (6, 1280),
                           (6, 1536), (6, 1792), (6, 2048), (64, 512), (6, 2304), (7, 512)):
         hidden = vectors * per_vector
         vals = (rng.normal(0, 1, (rows, hidden)) * rng.uniform(0.1, 10, (rows, 1))).astype(np.float32)
