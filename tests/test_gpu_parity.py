@@ -263,12 +263,13 @@ def test_rms_norm_domain_values_every_route(tag, weight_tag):
 
 @pytest.mark.parametrize("tag,weight_tag", [("bf16", "bf16"), ("bf16", "f32"), ("f16", "f16"), ("f32", "f32")])
 def test_rms_norm_launches_that_cover_the_tensor_exactly(tag, weight_tag):
-    """An even number of rows of 64 n, 128 n or 256 n whole vectors (n <= 8): the launch shapes that mask
-    nothing, with and without the weight; one width past them and an odd row count take the masked shapes."""
+    """Rows of 16 to 128 whole vectors in multiples of a block's rows, and an even number of rows of 64 n,
+    128 n or 256 n vectors: the launch shapes that mask nothing, with and without the weight; one width past
+    them and an odd row count take the masked shapes."""
     oid, wid = TYPES[tag][1], TYPES[weight_tag][1]
     rng = np.random.default_rng(77)
     per_vector = 4 if tag == "f32" else 8
-    for rows, vectors in ((6, 320), (6, 384), (6, 448), (6, 512), (6, 576), (6, 640), (6, 768), (6, 896), (6, 1024), (6, 1280),
+    for rows, vectors in ((64, 16), (64, 32), (64, 64), (64, 128), (96, 64), (6, 192), (6, 320), (6, 384), (6, 448), (6, 512), (6, 576), (6, 640), (6, 768), (6, 896), (6, 1024), (6, 1280),
                           (6, 1536), (6, 1792), (6, 2048), (64, 512), (6, 2304), (7, 512)):
         hidden = vectors * per_vector
         vals = (rng.normal(0, 1, (rows, hidden)) * rng.uniform(0.1, 10, (rows, 1))).astype(np.float32)
