@@ -161,8 +161,9 @@ bool run_exact(const NormParams &p, const Bound &io, int parameters, hipStream_t
 
 }  // namespace
 
-// Launches the shape that covers [rows, width] exactly, if there is one: an even number of rows
-// of 64 n, 128 n or 256 n whole vectors, n <= 8.  False: nothing was launched, take the masked shapes.
+// Launches the shape that covers [rows, width] exactly, if there is one (norm_exact.h lists them:
+// rows of 16 to 128 vectors in multiples of a block's rows, an even number of rows of 64 n, 128 n
+// or 256 n vectors).  False: nothing was launched, take the masked shapes.
 bool launch_norm_exact_rms(Elem type, const NormParams &p, const void *x, const void *w, void *y, hipStream_t stream);
 bool launch_norm_exact_layer(Elem type, const NormParams &p, const void *x, const void *w, const void *b, void *y,
                              hipStream_t stream);
