@@ -279,6 +279,13 @@ def main() -> int:
         ops.append(Op("next_layer_norm_bf16", hc.LayerNorm(epsilon=1e-6),
                       [D(BF, [8192, 2048]), D(BF, [2048]), D(BF, [2048])], set_ln, 10,
                       2 * 8192 * 2048 * 2 + 2 * 4096, 8192 * 2048, "bf16", in_step=False))
+    if want("next_softmax_bf16_unmasked"):
+        # attention rows without a mask (a decode step over its cache, an encoder): [4096, 4096] bf16
+        def set_rows(i):
+            dx = torch.empty((4096, 4096), dtype=torch.bfloat16, device=dev).normal_(0.0, 3.0)
+            return [dx], [torch.empty_like(dx)]
+        ops.append(Op("next_softmax_bf16_unmasked", hc.Softmax(), [D(BF, [4096, 4096])], set_rows, 10,
+                      2 * 4096 * 4096 * 2, 4096 * 4096, "bf16", in_step=False, ceiling="ceiling_copy_67mb"))
     # the norms at other hidden sizes (the same 67 MB): launch shapes that cover the tensor exactly
     for name, layer, rows_n, hidden_n in (("next_rms_norm_bf16_hidden_4096", False, 4096, 4096),
                                          ("next_layer_norm_bf16_hidden_8192", True, 2048, 8192)):

@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libhyle_hip.so")
 
-SOURCES = ["plan.hip", "elementwise.hip", "norm.hip", "norm_exact_rms.hip", "norm_exact_layer.hip", "softmax.hip", "reduce.hip", "argmax.hip", "topk.hip", "q8_0.hip", "gguf_k.hip", "gguf_matvec.hip", "gguf_matvec_q8.hip", "cast.hip", "select_fill.hip", "concat.hip", "gather.hip", "sampling.hip", "rope.hip", "file_stream.hip", "backend.hip"]
+SOURCES = ["plan.hip", "elementwise.hip", "norm.hip", "norm_exact_rms.hip", "norm_exact_layer.hip", "softmax.hip", "softmax_exact.hip", "reduce.hip", "argmax.hip", "topk.hip", "q8_0.hip", "gguf_k.hip", "gguf_matvec.hip", "gguf_matvec_q8.hip", "cast.hip", "select_fill.hip", "concat.hip", "gather.hip", "sampling.hip", "rope.hip", "file_stream.hip", "backend.hip"]
 
 # -ffp-contract=off: (a + b) * s and x * scale + mask keep two roundings, as the reference does.
 # packed-fp32 instructions are switched off for every device function.

@@ -13,32 +13,12 @@
 // double); the exponentials are carried scaled by 2^32 and the scale is folded
 // into the normaliser, so results down to the smallest subnormal are produced by
 // an ordinary multiply instead of being flushed by the hardware exp2.
-#include "device_common.h"
-#include "kernels.h"
+#include "softmax_math.h"
 
 namespace hyle_hip {
 namespace {
 
 enum : int { kMaskNone = 0, kMaskAdditive = 1, kMaskBoolean = 2 };
-
-// exp(t) * 2^32 for t <= 0.  t * log2(e) is taken as a rounded product plus its exact
-// residual (one fma), so the hardware exp2 sees an argument good to about 2e-8 * |t|
-// and the result stays within 2e-6 relative down to the subnormal range.
-__device__ __forceinline__ float exp_scaled(float t) {
-  constexpr float kLog2e = 1.44269504088896340736f;
-  constexpr float kLn2 = 0.69314718055994530942f;
-  t = fmaxf(t, -200.0f);  // exp(-200) * 2^32 is below every subnormal; also tames -inf
-  const float hi = t * kLog2e;
-  const float lo = __builtin_fmaf(t, kLog2e, -hi);
-  const float p = __builtin_amdgcn_exp2f(hi + 32.0f);
-  return __builtin_fmaf(p, lo * kLn2, p);
-}
-
-// NaN or +inf: the values that make a softmax row undefined
-// (src/simd/math/activations.cc:181-186).
-__device__ __forceinline__ bool poisons_row(float v) {
-  return __builtin_amdgcn_class(v, 0x001 | 0x002 | 0x200);  // sNaN | qNaN | +inf
-}
 
 struct MaskRows {
   int32_t outer_rank;
@@ -434,6 +414,7 @@ hipError_t launch_softmax(Elem type, const SoftmaxParams &p, const void *x, cons
                           void *y, bool vectorised, int /*compute_units*/, hipStream_t stream) {
   if (p.shape.rows == 0 || p.shape.width == 0) return hipSuccess;
   if (!vectorised) return hipErrorInvalidValue;  // the caller routes those to the general kernel
+  if ((int)p.mask_kind == kMaskNone && launch_softmax_exact(type, p, x, y, stream)) return hipGetLastError();
   switch (type) {
     case Elem::kF32: return run_softmax<F32>(p, x, mask, y, stream);
     case Elem::kF16: return run_softmax<F16>(p, x, mask, y, stream);

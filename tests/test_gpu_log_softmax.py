@@ -94,6 +94,27 @@ def test_log_softmax_widths_masks_every_route(tag):
         log_bar(to_host(out), orc.softmax(oid, x, mask_kind=orc.MASK_ADDITIVE, mask=add, log=True), tag)
 
 
+@pytest.mark.parametrize("tag", ["f32", "bf16", "f16"])
+def test_log_softmax_unmasked_launches_that_cover_the_tensor_exactly(tag):
+    """The logarithmic form over the same exact launch shapes as the softmax test: 32 unmasked rows of
+    every width with a shape of its own, undefined rows (NaN, +inf, only -inf) and -inf elements (-inf out)."""
+    oid = TYPES[tag][1]
+    rng = np.random.default_rng(1207)
+    per_vector = 4 if tag == "f32" else 8
+    for vectors in (16, 32, 64, 128, 192, 256, 320, 384, 448, 512, 640, 768, 896, 1024, 1280, 1536, 1792, 2048):
+        rows, width = 32, vectors * per_vector
+        values = rng.normal(0, 3, (rows, width)).astype(np.float32)
+        values[3, 5] = np.nan
+        values[4, width - 1] = np.inf
+        values[5, :] = -np.inf
+        values[6, ::3] = -np.inf
+        values[7, 1::2] = values[7, 0]            # many equal maxima or equal values
+        x = host_values(values, tag)
+        note(f"log-softmax {tag} [{rows}, {width}] unmasked")
+        (out,) = run(hc.Softmax(kind=LOG), to_device(x, tag))
+        log_bar(to_host(out), orc.softmax(oid, x, log=True), tag)
+
+
 def test_log_softmax_other_axes_views_and_undefined_rows():
     rng = np.random.default_rng(1207)
     for tag in ("f32", "bf16"):

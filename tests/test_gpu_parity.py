@@ -396,6 +396,33 @@ def test_softmax_widths_masks_every_route(tag):
         softmax_bar(to_host(out), want) if tag == "f32" else assert_narrow_ulp(to_host(out), want, tag)
 
 
+@pytest.mark.parametrize("tag", ["f32", "bf16", "f16"])
+def test_softmax_unmasked_launches_that_cover_the_tensor_exactly(tag):
+    """Unmasked rows of every width that has a launch shape of its own (sub-wave groups with two vectors
+    per lane and four rows, then 64, 128 or 256 lanes with three to eight vectors and two rows), 32 rows
+    each; with a scale; a row with a NaN, one with +inf, one of -inf only (all three undefined: NaN) and
+    one with -inf elements (zeros).  33 rows of one width take the masked shapes."""
+    oid = TYPES[tag][1]
+    rng = np.random.default_rng(107)
+    per_vector = 4 if tag == "f32" else 8
+    for rows, vectors in [(32, v) for v in (16, 32, 64, 128, 192, 256, 320, 384, 448, 512, 640, 768, 896, 1024, 1280,
+                                            1536, 1792, 2048)] + [(33, 512)]:
+        width = vectors * per_vector
+        values = rng.normal(0, 3, (rows, width)).astype(np.float32)
+        values[3, 5] = np.nan
+        values[4, width - 1] = np.inf
+        values[5, :] = -np.inf
+        values[6, ::3] = -np.inf
+        x = host_values(values, tag)
+        for scale in (1.0, 0.125):
+            note(f"softmax {tag} [{rows}, {width}] unmasked, scale {scale}")
+            (out,) = run(hc.Softmax(scale=scale), to_device(x, tag))
+            want = orc.softmax(oid, x, scale=scale)
+            decoded = want if tag == "f32" else orc.to_f32(oid, want)
+            assert np.isnan(decoded[3:6]).all() and (decoded[6, ::3] == 0).all()
+            softmax_bar(to_host(out), want) if tag == "f32" else assert_narrow_ulp(to_host(out), want, tag)
+
+
 @pytest.mark.parametrize("tag", ["f32", "bf16"])
 def test_softmax_boolean_mask_hides_specials_additive_mask_does_not(tag):
     # A masked element is replaced by -inf before anything looks at it
