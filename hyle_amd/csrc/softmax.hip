@@ -18,26 +18,6 @@
 namespace hyle_hip {
 namespace {
 
-enum : int { kMaskNone = 0, kMaskAdditive = 1, kMaskBoolean = 2 };
-
-struct MaskRows {
-  int32_t outer_rank;
-  uint32_t outer_dims[kMaxRank];
-  int64_t outer_strides[kMaxRank];
-  int64_t inner_stride;
-};
-
-__device__ __forceinline__ int64_t mask_row_offset(const MaskRows &m, uint32_t row) {
-  int64_t offset = 0;
-  uint32_t rest = row;
-  for (int axis = m.outer_rank - 1; axis >= 0; --axis) {
-    const uint32_t extent = m.outer_dims[axis];
-    offset += (int64_t)(rest % extent) * m.outer_strides[axis];
-    rest /= extent;
-  }
-  return offset;
-}
-
 // A lane group (kLanes lanes, each with kVpl 16-byte vectors) owns one row at a time.
 //
 // Loads carry no branches: a lane outside the row (or a row outside the tensor) reads a clamped,
@@ -414,7 +394,7 @@ hipError_t launch_softmax(Elem type, const SoftmaxParams &p, const void *x, cons
                           void *y, bool vectorised, int /*compute_units*/, hipStream_t stream) {
   if (p.shape.rows == 0 || p.shape.width == 0) return hipSuccess;
   if (!vectorised) return hipErrorInvalidValue;  // the caller routes those to the general kernel
-  if ((int)p.mask_kind == kMaskNone && launch_softmax_exact(type, p, x, y, stream)) return hipGetLastError();
+  if (launch_softmax_exact(type, p, x, mask, y, stream)) return hipGetLastError();
   switch (type) {
     case Elem::kF32: return run_softmax<F32>(p, x, mask, y, stream);
     case Elem::kF16: return run_softmax<F16>(p, x, mask, y, stream);

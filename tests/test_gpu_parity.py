@@ -423,6 +423,57 @@ def test_softmax_unmasked_launches_that_cover_the_tensor_exactly(tag):
             softmax_bar(to_host(out), want) if tag == "f32" else assert_narrow_ulp(to_host(out), want, tag)
 
 
+@pytest.mark.parametrize("log_form", [False, True])
+@pytest.mark.parametrize("tag", ["f32", "bf16", "f16"])
+def test_softmax_masked_launches_that_cover_the_tensor_exactly(tag, log_form):
+    """[heads, 16, width] under a [16, width] mask, widths with a launch shape of their own: a staircase
+    Boolean mask (whole vectors left out, one row left out entirely -> NaN) from 512 vectors per row on,
+    an additive mask with -inf columns for every width; specials under and beside the mask."""
+    oid = TYPES[tag][1]
+    rng = np.random.default_rng(108)
+    per_vector = 4 if tag == "f32" else 8
+    kind = hc.SoftmaxKind.kLogSoftmax if log_form else hc.SoftmaxKind.kSoftmax
+    for vectors in (16, 64, 128, 192, 256, 320, 512, 640, 768, 1024, 1536, 2048):
+        heads, q, width = 2, 16, vectors * per_vector
+        values = rng.normal(0, 3, (heads, q, width)).astype(np.float32)
+        keep = (np.arange(width)[None, :] <= (np.arange(q)[:, None] + 1) * (width // q) - 3).astype(np.uint8)
+        keep[5, :] = 0                                  # nothing kept: NaN for every head
+        values[0, 7, width - 1] = np.nan               # under the mask: hidden
+        values[1, 9, 0] = np.inf                       # kept: the row is undefined
+        x = host_values(values, tag)
+        note(f"softmax {tag} log={log_form} [{heads}, {q}, {width}] staircase Bool mask, scale 0.25")
+        dmask = torch.from_numpy(keep).to(DEVICE).view(torch.bool)
+        (out,) = run(hc.Softmax(scale=0.25, kind=kind, mask=hc.MaskKind.kBoolean), to_device(x, tag), dmask)
+        want = orc.softmax(oid, x, scale=0.25, mask_kind=orc.MASK_BOOLEAN, mask=keep, log=log_form)
+        got = to_host(out)
+        if tag != "f32":
+            assert_narrow_ulp(got, want, tag)
+        elif log_form:
+            assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
+            ok = np.isfinite(want)
+            assert np.all(np.abs(got[ok].astype(np.float64) - want[ok]) <= np.abs(want[ok]) * 4e-6 + 2e-7)
+        else:
+            softmax_bar(got, want)
+        note(f"softmax {tag} log={log_form} [{heads}, {q}, {width}] additive mask [{q}, {width}] with -inf columns")
+        add = np.where(rng.random((q, width)) < 0.3, -np.inf, rng.normal(0, 1, (q, width))).astype(np.float32)
+        add[:, 1] = 0
+        values[0, 7, width - 1] = 1.0
+        values[1, 9, 0] = -2.0
+        x = host_values(values, tag)
+        addend = host_values(add, tag)
+        (out,) = run(hc.Softmax(kind=kind, mask=hc.MaskKind.kAdditive), to_device(x, tag), to_device(addend, tag))
+        want = orc.softmax(oid, x, mask_kind=orc.MASK_ADDITIVE, mask=addend, log=log_form)
+        got = to_host(out)
+        if tag != "f32":
+            assert_narrow_ulp(got, want, tag)
+        elif log_form:
+            assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
+            ok = np.isfinite(want)
+            assert np.all(np.abs(got[ok].astype(np.float64) - want[ok]) <= np.abs(want[ok]) * 4e-6 + 2e-7)
+        else:
+            softmax_bar(got, want)
+
+
 @pytest.mark.parametrize("tag", ["f32", "bf16"])
 def test_softmax_boolean_mask_hides_specials_additive_mask_does_not(tag):
     # A masked element is replaced by -inf before anything looks at it
