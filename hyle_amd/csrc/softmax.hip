@@ -377,7 +377,14 @@ hipError_t run_softmax(const SoftmaxParams &p, const void *x, const void *mask, 
   // group 551-716.  Additive causal mask, blocks steered so that a mask row stays on one XCD:
   // eight waves x 2 vectors 693; four waves x 4 vectors 706.
   if (vectors <= 1024) {
-    if ((int)p.mask_kind == kMaskBoolean) return run_rows<T, 256, 4, 256>(p, x, mask, y, s);
+    if ((int)p.mask_kind == kMaskBoolean) {
+      // exactly 1024 vectors: one wave per row, sixteen vectors per lane, no block barrier.  With
+      // the launch covering the tensor exactly (see run_rows_as) this measured 549-552 us for
+      // S[32, 4096, 4096] f32 against 554-560 us for four waves per row on the same machine
+      // (two waves 560-566, eight 573-600, two rows per block 566-592).
+      if (vectors == 1024) return run_rows<T, 64, 16, 64>(p, x, mask, y, s);
+      return run_rows<T, 256, 4, 256>(p, x, mask, y, s);
+    }
     return run_rows<T, 512, 2, 512>(p, x, mask, y, s);
   }
   if (vectors <= 2048) return run_rows<T, 512, 4, 512>(p, x, mask, y, s);
