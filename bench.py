@@ -682,7 +682,7 @@ def file_stream_rate(mib, ctx, torch, dev):
 # (profiles/hot_path_step_hbm_traffic_pmc.md: FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors
 # the same counters need to read a plain 1 GiB copy correctly).
 TRAFFIC = {
-    "cfg4_softmax_f32_causal": 3250951987,
+    "cfg4_softmax_f32_causal": 3256479642,
     "cfg4_softmax_f32_causal_additive": 4362172313,
     "cfg3_swiglu_bf16": 302043955,
     "cfg3_residual_add_bf16": 100731801,
