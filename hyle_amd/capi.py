@@ -98,6 +98,9 @@ EXPORTS = {
     "hyle_hip_plan_alias_support": (C.c_int, [C.c_void_p, C.c_uint32, C.c_uint32]),
     "hyle_hip_plan_dispatch_count": (C.c_uint32, [C.c_void_p]),
     "hyle_hip_plan_route_name": (C.c_char_p, [C.c_void_p]),
+    "hyle_hip_variant_count": (C.c_uint32, []),
+    "hyle_hip_variant_label": (C.c_char_p, [C.c_uint32]),
+    "hyle_hip_last_launch_variant": (C.c_char_p, []),
     "hyle_hip_plan_launch": (C.c_int, [C.c_void_p, C.POINTER(C.c_void_p), C.c_uint32, C.POINTER(C.c_void_p),
                                        C.c_uint32, C.c_void_p, C.c_size_t, C.c_void_p]),
     "hyle_hip_plan_device_status": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),

@@ -715,6 +715,17 @@ class OperationInvocation:
             self._prepared._handle, self._in, len(inputs), self._out, len(outputs), stream))
 
 
+def launch_variants() -> list:
+    """Labels of every kernel launch shape compiled into the library (diagnostics)."""
+    lib = capi.load()
+    return [lib.hyle_hip_variant_label(i).decode() for i in range(lib.hyle_hip_variant_count())]
+
+
+def last_launch_variant() -> str:
+    """Label(s) of the dispatches this thread's last submit enqueued, joined by ' + '."""
+    return capi.load().hyle_hip_last_launch_variant().decode()
+
+
 def prepare(context: Context, operation, *inputs: TensorDesc,
             outputs: Optional[Sequence[TensorDesc]] = None) -> PreparedOperation:
     """hyle::compute::prepare(context, operation, input descriptors...)."""

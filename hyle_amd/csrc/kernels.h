@@ -7,7 +7,29 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <string>
+
 namespace hyle_hip {
+
+// ---- launch-shape labels ------------------------------------------------------
+// Which kernel shape a launcher picks depends on sizes, strides and alignment seen at launch.
+// Every launcher notes a label for the shape it chose on the calling thread, and every label
+// registers itself when the library loads, so the list (hyle_hip_variant_label) holds exactly
+// the launch shapes compiled in.  A label names the shape (lanes x vectors x rows, mask form,
+// exact or masked), not the storage type: tests use it to prove that a case reached the kernel
+// it was written for.
+namespace variants {
+const char *add(const std::string &label);  // registers a label, returns its stable text
+void note(const char *label);               // the calling thread is about to launch this shape
+}  // namespace variants
+
+// Tag::text() is the label; the first use of Variant<Tag>::label anywhere in the library makes
+// the label part of the list.
+template <class Tag> struct Variant {
+  static const char *const label;
+};
+template <class Tag> const char *const Variant<Tag>::label = variants::add(Tag::text());
+template <class Tag> inline void note_variant() { variants::note(Variant<Tag>::label); }
 
 enum class Elem : uint8_t { kF32 = 0, kF16 = 1, kBF16 = 2 };
 

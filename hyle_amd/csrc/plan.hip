@@ -11,6 +11,8 @@
 #include <limits>
 #include <mutex>
 #include <new>
+#include <string>
+#include <vector>
 
 #include "../../include/hyle_hip.h"
 #include "kernels.h"
@@ -35,6 +37,22 @@ hyle_hip_status fail(hyle_hip_status status, const char *format, ...) {
 hyle_hip_status hip_fail(hipError_t error, const char *what) {
   return fail(HYLE_HIP_INTERNAL, "%s: %s", what, hipGetErrorString(error));
 }
+
+// ---------------------------------------------------------------------------------
+// launch-shape labels (kernels.h)
+// ---------------------------------------------------------------------------------
+struct VariantList {
+  std::mutex mutex;
+  std::vector<std::string *> labels;  // never freed: the texts are handed out as C strings
+};
+VariantList &variant_list() {
+  static VariantList *list = new VariantList;  // outlives every static of the library
+  return *list;
+}
+constexpr int kNotedVariants = 4;  // dispatches of one launch
+thread_local const char *g_noted[kNotedVariants];
+thread_local int g_noted_count = 0;
+thread_local char g_noted_text[512];
 
 // ---------------------------------------------------------------------------------
 // descriptors
@@ -1432,6 +1450,22 @@ bool aligned(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) &
 
 }  // namespace
 
+namespace hyle_hip {
+namespace variants {
+const char *add(const std::string &label) {
+  VariantList &list = variant_list();
+  std::lock_guard<std::mutex> lock(list.mutex);
+  for (const std::string *known : list.labels)
+    if (*known == label) return known->c_str();
+  list.labels.push_back(new std::string(label));
+  return list.labels.back()->c_str();
+}
+void note(const char *label) {
+  if (g_noted_count < kNotedVariants) g_noted[g_noted_count++] = label;
+}
+}  // namespace variants
+}  // namespace hyle_hip
+
 // ---------------------------------------------------------------------------------
 // Device scratch of hyle_hip_plan_launch_static: the workspace of the two-dispatch routes for
 // callers that cannot allocate.  Every device the library runs on holds its own copy of the
@@ -1628,9 +1662,33 @@ const char *hyle_hip_plan_route_name(const hyle_hip_plan *plan) {
   return route_name(plan->route);
 }
 
+uint32_t hyle_hip_variant_count(void) {
+  VariantList &list = variant_list();
+  std::lock_guard<std::mutex> lock(list.mutex);
+  return (uint32_t)list.labels.size();
+}
+
+const char *hyle_hip_variant_label(uint32_t index) {
+  VariantList &list = variant_list();
+  std::lock_guard<std::mutex> lock(list.mutex);
+  return index < list.labels.size() ? list.labels[index]->c_str() : "";
+}
+
+const char *hyle_hip_last_launch_variant(void) {
+  size_t used = 0;
+  g_noted_text[0] = 0;
+  for (int i = 0; i < g_noted_count; ++i) {
+    const int wrote = snprintf(g_noted_text + used, sizeof g_noted_text - used, "%s%s", i ? " + " : "", g_noted[i]);
+    if (wrote < 0 || (size_t)wrote >= sizeof g_noted_text - used) break;
+    used += (size_t)wrote;
+  }
+  return g_noted_text;
+}
+
 hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *const *inputs,
                                      uint32_t input_count, void *const *outputs, uint32_t output_count,
                                      void *workspace, size_t workspace_size, void *stream_handle) {
+  g_noted_count = 0;
   if (plan == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "plan is null");
   if (input_count != plan->request.input_count || output_count != plan->output_count)
     return fail(HYLE_HIP_INVALID_ARGUMENT, "launch binding counts differ from the plan");
@@ -1697,7 +1755,7 @@ hyle_hip_status hyle_hip_plan_launch(const hyle_hip_plan *plan, const void *cons
                         aligned(inputs[0], 16) && aligned(outputs[0], 16) &&
                         (mask == nullptr || aligned(mask, 16)) &&
                         plan->softmax.shape.width % kvec == 0 &&
-                        plan->softmax.shape.width / kvec <= 16u * 256u;
+                        plan->softmax.shape.width / kvec <= 8u * 1024u;  // the widest row shape: 1024 lanes x 8 vectors
       if (rows)
         err = launch_softmax(plan->elem, plan->softmax, inputs[0], mask, outputs[0], true,
                              plan->context->compute_units, stream);
@@ -1819,6 +1877,7 @@ size_t hyle_hip_static_scratch_bytes(void) { return kStaticScratchBytes; }
 hyle_hip_status hyle_hip_plan_launch_static(const hyle_hip_plan *plan, const void *const *inputs,
                                             uint32_t input_count, void *const *outputs, uint32_t output_count,
                                             void *stream_handle) {
+  g_noted_count = 0;
   if (plan == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "plan is null");
   if (plan->workspace_size > kStaticScratchBytes)
     return fail(HYLE_HIP_RESOURCE_EXHAUSTED,

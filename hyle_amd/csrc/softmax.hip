@@ -310,7 +310,25 @@ MaskRepeat mask_repeat(const SoftmaxParams &p) {
   return r;
 }
 
-template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog>
+inline const char *mask_word(int mask) {
+  return mask == kMaskBoolean ? "boolean" : (mask == kMaskAdditive ? "additive" : "unmasked");
+}
+
+// softmax_rows/<lanes>x<vectors per lane>/<threads per block>/<mask>/<exact|ragged>[/steered]
+template <int kLanes, int kVpl, int kThreads, int kMask, bool kExact, bool kSteered> struct RowsTag {
+  static std::string text() {
+    return "softmax_rows/" + std::to_string(kLanes) + "x" + std::to_string(kVpl) + "/" + std::to_string(kThreads) + "/" +
+           mask_word(kMask) + (kExact ? "/exact" : "/ragged") + (kSteered ? "/steered" : "");
+  }
+};
+struct GeneralTag {
+  static std::string text() { return "softmax_general"; }
+};
+
+// kForms: bit 0 the ragged kernel (lanes and rows test whether they are inside), bit 1 the exact one.
+constexpr int kRagged = 1, kExactForm = 2, kBothForms = 3;
+
+template <class T, int kLanes, int kVpl, int kThreads, int kMask, bool kLog, int kForms>
 hipError_t run_rows_as(const SoftmaxParams &p, const void *x, const void *mask, void *y,
                        hipStream_t s) {
   constexpr int kGroupsPerBlock = kThreads / kLanes;
@@ -329,33 +347,59 @@ hipError_t run_rows_as(const SoftmaxParams &p, const void *x, const void *mask, 
                              ? 1u : 0u;
   // A launch that covers the tensor exactly takes the instantiation without the in-the-row and
   // in-the-tensor tests (S[32, 4096, 4096] f32 under the Boolean mask: 531 us against 544 us).
-  if (rows % kGroupsPerBlock == 0 && p.shape.width / Traits<T>::kVec == (uint32_t)(kLanes * kVpl)) {
-    hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads, kMask, kLog, true>), dim3(blocks),
+  constexpr bool kMaySteer = kMask == kMaskAdditive && kGroupsPerBlock == 1;
+  const bool exact = rows % kGroupsPerBlock == 0 && p.shape.width / Traits<T>::kVec == (uint32_t)(kLanes * kVpl);
+  if constexpr ((kForms & kExactForm) != 0) {
+    if (exact) {
+      if constexpr (kMaySteer) {
+        if (steer != 0) note_variant<RowsTag<kLanes, kVpl, kThreads, kMask, true, true>>();
+      }
+      if (steer == 0) note_variant<RowsTag<kLanes, kVpl, kThreads, kMask, true, false>>();
+      hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads, kMask, kLog, true>), dim3(blocks),
+                         dim3(kThreads), 0, s, x, mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, m,
+                         repeat.period, repeat.repeats, steer);
+      return hipGetLastError();
+    }
+  }
+  if constexpr ((kForms & kRagged) != 0) {
+    if constexpr (kMaySteer) {
+      if (steer != 0) note_variant<RowsTag<kLanes, kVpl, kThreads, kMask, false, true>>();
+    }
+    if (steer == 0) note_variant<RowsTag<kLanes, kVpl, kThreads, kMask, false, false>>();
+    hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads, kMask, kLog>), dim3(blocks),
                        dim3(kThreads), 0, s, x, mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, m,
                        repeat.period, repeat.repeats, steer);
     return hipGetLastError();
   }
-  hipLaunchKernelGGL((softmax_rows<T, kLanes, kVpl, kThreads, kMask, kLog>), dim3(blocks),
-                     dim3(kThreads), 0, s, x, mask, y, rows, p.shape.width / Traits<T>::kVec, p.scale, m,
-                     repeat.period, repeat.repeats, steer);
-  return hipGetLastError();
+  return hipErrorInvalidValue;
 }
 
-template <class T, int kLanes, int kVpl, int kThreads = kBlockThreads>
+// kMasks: the mask forms this launch shape is ever chosen for (bit kMask...), so that only those
+// are compiled.
+constexpr int kAnyMask = 7, kBooleanOnly = 1 << kMaskBoolean, kNotBoolean = kAnyMask & ~kBooleanOnly;
+
+template <class T, int kLanes, int kVpl, int kThreads = kBlockThreads, int kMasks = kAnyMask, int kForms = kBothForms>
 hipError_t run_rows(const SoftmaxParams &p, const void *x, const void *mask, void *y,
                     hipStream_t s) {
   const bool log_form = p.log;
   switch ((int)p.mask_kind) {
     case kMaskBoolean:
-      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, true>(p, x, mask, y, s)
-                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, false>(p, x, mask, y, s);
+      if constexpr ((kMasks >> kMaskBoolean) & 1)
+        return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, true, kForms>(p, x, mask, y, s)
+                        : run_rows_as<T, kLanes, kVpl, kThreads, kMaskBoolean, false, kForms>(p, x, mask, y, s);
+      break;
     case kMaskAdditive:
-      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, true>(p, x, mask, y, s)
-                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, false>(p, x, mask, y, s);
+      if constexpr ((kMasks >> kMaskAdditive) & 1)
+        return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, true, kForms>(p, x, mask, y, s)
+                        : run_rows_as<T, kLanes, kVpl, kThreads, kMaskAdditive, false, kForms>(p, x, mask, y, s);
+      break;
     default:
-      return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, true>(p, x, mask, y, s)
-                      : run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, false>(p, x, mask, y, s);
+      if constexpr ((kMasks >> kMaskNone) & 1)
+        return log_form ? run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, true, kForms>(p, x, mask, y, s)
+                        : run_rows_as<T, kLanes, kVpl, kThreads, kMaskNone, false, kForms>(p, x, mask, y, s);
+      break;
   }
+  return hipErrorInvalidValue;
 }
 
 template <class T>
@@ -382,10 +426,11 @@ hipError_t run_softmax(const SoftmaxParams &p, const void *x, const void *mask, 
       // the launch covering the tensor exactly (see run_rows_as) this measured 549-552 us for
       // S[32, 4096, 4096] f32 against 554-560 us for four waves per row on the same machine
       // (two waves 560-566, eight 573-600, two rows per block 566-592).
-      if (vectors == 1024) return run_rows<T, 64, 16, 64>(p, x, mask, y, s);
-      return run_rows<T, 256, 4, 256>(p, x, mask, y, s);
+      // (1024 vectors in one-wave blocks always cover the tensor exactly; 513-1023 never fill 256 x 4)
+      if (vectors == 1024) return run_rows<T, 64, 16, 64, kBooleanOnly, kExactForm>(p, x, mask, y, s);
+      return run_rows<T, 256, 4, 256, kBooleanOnly, kRagged>(p, x, mask, y, s);
     }
-    return run_rows<T, 512, 2, 512>(p, x, mask, y, s);
+    return run_rows<T, 512, 2, 512, kNotBoolean>(p, x, mask, y, s);
   }
   if (vectors <= 2048) return run_rows<T, 512, 4, 512>(p, x, mask, y, s);
   if (vectors <= 4096) return run_rows<T, 1024, 4, 1024>(p, x, mask, y, s);
@@ -404,6 +449,7 @@ hipError_t run_general(const SoftmaxGeneralParams &p, const void *x, const void 
     g.in_strides[i] = p.in_strides[i];
     g.mask_strides[i] = p.mask_strides[i];
   }
+  note_variant<GeneralTag>();
   hipLaunchKernelGGL((softmax_general<T>), dim3((uint32_t)(p.outer * p.inner)), dim3(kBlockThreads),
                      0, s, static_cast<const char *>(x), static_cast<const char *>(mask), y, p.width,
                      p.scale, (int)p.mask_kind, p.log ? 1 : 0, g);

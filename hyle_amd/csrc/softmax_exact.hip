@@ -154,6 +154,14 @@ void launch_form(bool log_form, dim3 grid, hipStream_t s, const void *x, const v
                        row_vectors, scale, m);
 }
 
+// softmax_rows_exact/<lanes>x<vectors per lane>/<threads per block>/<rows per lane group>/<mask>
+template <int kLanes, int kVpl, int kThreads, int kRows, int kMask> struct ExactTag {
+  static std::string text() {
+    return "softmax_rows_exact/" + std::to_string(kLanes) + "x" + std::to_string(kVpl) + "/" + std::to_string(kThreads) + "/" +
+           std::to_string(kRows) + "/" + (kMask == kMaskBoolean ? "boolean" : (kMask == kMaskAdditive ? "additive" : "unmasked"));
+  }
+};
+
 template <class T, int kLanes, int kVpl, int kThreads, int kRows>
 bool run_exact(const SoftmaxParams &p, const void *x, const void *mask, void *y, hipStream_t s) {
   constexpr int kRowsPerBlock = kThreads / kLanes * kRows;
@@ -168,9 +176,23 @@ bool run_exact(const SoftmaxParams &p, const void *x, const void *mask, void *y,
   m.inner_stride = p.mask_inner_stride;
   const dim3 grid(rows / kRowsPerBlock);
   switch ((int)p.mask_kind) {
-    case kMaskBoolean: launch_form<T, kLanes, kVpl, kThreads, kRows, kMaskBoolean>(p.log, grid, s, x, mask, y, row_vectors, p.scale, m); break;
-    case kMaskAdditive: launch_form<T, kLanes, kVpl, kThreads, kRows, kMaskAdditive>(p.log, grid, s, x, mask, y, row_vectors, p.scale, m); break;
-    default: launch_form<T, kLanes, kVpl, kThreads, kRows, kMaskNone>(p.log, grid, s, x, mask, y, row_vectors, p.scale, m); break;
+    case kMaskBoolean:
+      // a Boolean mask takes these shapes from 512 vectors per row on (run_exact_shape)
+      if constexpr (kLanes * kVpl >= 512) {
+        note_variant<ExactTag<kLanes, kVpl, kThreads, kRows, kMaskBoolean>>();
+        launch_form<T, kLanes, kVpl, kThreads, kRows, kMaskBoolean>(p.log, grid, s, x, mask, y, row_vectors, p.scale, m);
+        break;
+      } else {
+        return false;
+      }
+    case kMaskAdditive:
+      note_variant<ExactTag<kLanes, kVpl, kThreads, kRows, kMaskAdditive>>();
+      launch_form<T, kLanes, kVpl, kThreads, kRows, kMaskAdditive>(p.log, grid, s, x, mask, y, row_vectors, p.scale, m);
+      break;
+    default:
+      note_variant<ExactTag<kLanes, kVpl, kThreads, kRows, kMaskNone>>();
+      launch_form<T, kLanes, kVpl, kThreads, kRows, kMaskNone>(p.log, grid, s, x, mask, y, row_vectors, p.scale, m);
+      break;
   }
   return true;
 }

@@ -309,6 +309,17 @@ HYLE_HIP_API uint32_t hyle_hip_plan_dispatch_count(const hyle_hip_plan *plan);
 /* Name of the kernel route the plan selected (diagnostics, profiling). */
 HYLE_HIP_API const char *hyle_hip_plan_route_name(const hyle_hip_plan *plan);
 
+/* Diagnostics for tests and profiling; no counterpart in the reference.  Inside a route the
+ * launcher picks a kernel shape from the sizes, strides and alignments it sees at launch.  Every
+ * shape compiled into the library has a label ("softmax_rows/512x2/additive/exact/steered");
+ * hyle_hip_variant_count / hyle_hip_variant_label list them, and hyle_hip_last_launch_variant
+ * returns the label(s) of the dispatches the calling thread's last hyle_hip_plan_launch or
+ * hyle_hip_plan_launch_static enqueued, joined by " + " (empty when it enqueued nothing).  The
+ * text stays valid until the thread's next call of the same function. */
+HYLE_HIP_API uint32_t hyle_hip_variant_count(void);
+HYLE_HIP_API const char *hyle_hip_variant_label(uint32_t index);
+HYLE_HIP_API const char *hyle_hip_last_launch_variant(void);
+
 /* ProviderPreparedVTable::shared_submit
  * (include/hyle/compute/detail/prepared_callbacks.h:26-30): enqueue on `stream`
  * (a hipStream_t; NULL is the default stream) and return without waiting.
