@@ -96,7 +96,11 @@ def main() -> int:
             # does not need and does not issue (no bandwidth is claimed for bytes never moved).
             self.credited = algorithmic_bytes if credited_bytes is None else credited_bytes
             self.in_step = in_step
+            began = time.perf_counter()
             self.bound = tio.Bound(ctx, operation, descs, device=dev)
+            self.plan_us = (time.perf_counter() - began) * 1e6   # propose + prepare (plus the workspace allocation)
+            self.first_launch_us = None
+            self.variant = ""
             self.route = self.bound.prepared.route_name()
             self.sets = [make_set(i) for i in range(sets)]  # each: (inputs, outputs)
             self.addresses = [([t.data_ptr() for t in i], [t.data_ptr() for t in o]) for i, o in self.sets]
@@ -431,6 +435,9 @@ def main() -> int:
         ("ceiling_copy_67mb", "copy", F32, torch.float32, [4096, 2048], 10),
         ("ceiling_scan_38mb", "scan", F32, torch.float32, [9496, 1024], 16),
         ("ceiling_scan_67mb", "scan", F32, torch.float32, [16384, 1024], 10),
+        # the same read-only kernel far above the 256 MB memory-side cache: does a launch that only reads
+        # saturate where the small ones do, or higher?
+        ("ceiling_scan_1gib", "scan", F32, torch.float32, [262144, 1024], 2),
     )
     needed = {o.ceiling for o in ops if o.ceiling}
     for name, form, dtype, torch_dtype, dims, sets in ceiling_lines:
@@ -467,9 +474,16 @@ def main() -> int:
     # one launch call, so eager submission would measure the host, not the GPU.  The
     # reference replays captured graphs the same way (capture_compatible,
     # include/hyle/compute/provider.h:136-139).  One graph per rotation phase.
-    for op in ops:
-        op.launch(stream)
+    # The first launch of a kernel out of each source file of the library also loads that file's code
+    # object (the reference's contract: "kernel/configuration binding is cold",
+    # include/hyle/compute/providers/cuda.h:55-56): each op's first launch is timed to its completion.
     torch.cuda.synchronize()
+    for op in ops:
+        began = time.perf_counter()
+        op.launch(stream)
+        op.variant = hc.last_launch_variant()
+        torch.cuda.synchronize()
+        op.first_launch_us = (time.perf_counter() - began) * 1e6
     PHASES = 16
 
     def capture(members, launches_each=1):
@@ -529,7 +543,8 @@ def main() -> int:
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / reps
         gbps = op.credited / us / 1e3
-        entry = {"op": op.name, "in_step": op.in_step, "route": op.route, "dtype": op.dtype,
+        entry = {"op": op.name, "in_step": op.in_step, "route": op.route, "variant": op.variant, "dtype": op.dtype,
+                 "plan_us": round(op.plan_us, 1), "first_launch_us": round(op.first_launch_us, 1),
                  "bytes": op.bytes, "bytes_credited": op.credited,
                  "buffer_sets": len(op.sets), "launches": reps, "us": round(us, 3),
                  "gbps": round(gbps, 1), "frac": round(gbps / HBM_PEAK_GBPS, 4),
@@ -572,6 +587,22 @@ def main() -> int:
         del src, dst
 
     achieved = dominant.credited / dominant_us / 1e3
+    # every kernel of the step in short keys (us per launch, GB/s of credited bytes, fraction of the
+    # 8 TB/s peak, and against the plain kernel of the same traffic where one was timed)
+    per_config = {}
+    for op in step_ops:
+        entry = by_name[op.name]
+        line = {"us": entry["us"], "gbps": entry["gbps"], "frac": entry["frac"]}
+        if "ceiling" in entry:
+            line["ceiling"] = entry["ceiling"]
+            line["ceiling_gbps"] = entry["ceiling_gbps"]
+            line["frac_of_ceiling"] = entry["frac_of_ceiling"]
+        per_config[op.name] = line
+    ceilings = {entry["op"]: {"us": entry["us"], "gbps": entry["gbps"], "frac": entry["frac"]}
+                for entry in per_op if entry["op"].startswith("ceiling_")}
+    cold = {"first_launch_ms_max": round(max(o.first_launch_us for o in ops) / 1e3, 2),
+            "first_launch_ms": {o.name: round(o.first_launch_us / 1e3, 2) for o in step_ops},
+            "plan_create_us_max": round(max(o.plan_us for o in ops), 1)}
     result = {
         "metric": "achieved HBM GB/s and % of 8 TB/s peak per op (RMSNorm, SwiGLU, softmax)",
         "value": round(step_credited / (ms_per_step * 1e-3) / 1e9, 1),
@@ -590,7 +621,12 @@ def main() -> int:
         "roofline": {"bound": "hbm", "kernel": dominant.name, "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "us_per_launch": round(dominant_us, 2), "algorithmic_bytes": dominant.bytes,
-                     "credited_bytes": dominant.credited, "traffic": TRAFFIC.get(dominant.name)},
+                     "credited_bytes": dominant.credited, "traffic": TRAFFIC.get(dominant.name),
+                     "traffic_source": "profiles/hot_path_step_hbm_traffic_pmc.md (rocprofv3 --pmc FETCH_SIZE / "
+                                       "WRITE_SIZE of an earlier run of this script: a recorded figure, not a "
+                                       "counter read in this run)",
+                     "per_config": per_config, "ceilings": ceilings},
+        "cold": cold,
         "per_op": per_op,
     }
     result["device"] = device_state(torch)
@@ -705,7 +741,8 @@ def cpu_baseline(args, ops, np, torch, wl):
 
     lib = C.CDLL(os.path.join(ROOT, "oracle", "libhyle_oracle.so"))
     vp, sz = C.c_void_p, C.c_size_t
-    cores = min(len(os.sched_getaffinity(0)), 16)
+    THREAD_CAP = 16  # the CPU share of a one-GPU box, whatever the host shows
+    cores = min(len(os.sched_getaffinity(0)), THREAD_CAP)
     pool = ThreadPoolExecutor(max_workers=cores)
 
     def ptr(a):
@@ -804,6 +841,7 @@ def cpu_baseline(args, ops, np, torch, wl):
     pool.shutdown()
     step_bytes = sum(o.bytes for o in ops)
     return {"value": round(step_bytes / total_seconds_full / 1e9, 3), "unit": "GB/s", "cores": cores,
+            "thread_cap": THREAD_CAP, "host_cores_visible": len(os.sched_getaffinity(0)),
             "kind": "port",
             "build": "oracle/hyle_oracle.c, gcc -O3 -march=x86-64-v3 -ffp-contract=off (AVX2 + FMA, not "
                      "-march=native: the library is built before it travels to this host)",
