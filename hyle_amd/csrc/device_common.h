@@ -177,13 +177,13 @@ constexpr int kDppSwap2 = 0x4E;        // quad_perm [2,3,0,1]
 constexpr int kDppHalfMirror = 0x141;  // lane i <-> 7 - i within 8
 constexpr int kDppRowMirror = 0x140;   // lane i <-> 15 - i within 16
 
-// Combine across `kLanes` adjacent lanes (8, 16, 32 or 64) with `op`.
+// Combine across `kLanes` adjacent lanes (4, 8, 16, 32 or 64) with `op`.
 template <int kLanes, class V, class Op>
 __device__ __forceinline__ V group_reduce(V v, Op op) {
-  static_assert(kLanes == 8 || kLanes == 16 || kLanes == 32 || kLanes == 64, "group width");
+  static_assert(kLanes == 4 || kLanes == 8 || kLanes == 16 || kLanes == 32 || kLanes == 64, "group width");
   v = op(v, v.template moved<kDppSwap1>());
   v = op(v, v.template moved<kDppSwap2>());
-  v = op(v, v.template moved<kDppHalfMirror>());
+  if constexpr (kLanes >= 8) v = op(v, v.template moved<kDppHalfMirror>());
   if constexpr (kLanes >= 16) v = op(v, v.template moved<kDppRowMirror>());
   if constexpr (kLanes >= 32) v = op(v, v.shuffled_xor(16));
   if constexpr (kLanes >= 64) v = op(v, v.shuffled_xor(32));

@@ -699,20 +699,339 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_quads(const unsi
   }
 }
 
+inline const char *kind_word(int kind) { return kind == 0 ? "q4_k" : (kind == 1 ? "q6_k" : "q8_0"); }
+// gguf_matvec_q8_<form>/<format>[/<detail>]
+template <int kKind, int kSets, bool kRegisters> struct QuadsTag {
+  static std::string text() {
+    return std::string("gguf_matvec_q8_quads/") + kind_word(kKind) + "/" + std::to_string(4 * kSets) + "-tokens" + (kRegisters ? "/registers" : "/lds");
+  }
+};
+template <int kKind, int kM, bool kRegisters> struct LinesTag {
+  static std::string text() {
+    return std::string("gguf_matvec_q8_lines/") + kind_word(kKind) + "/" + std::to_string(kM) + "-tokens" + (kRegisters ? "/registers" : "/lds");
+  }
+};
+template <int kKind, int kSpans> struct SpansTag {
+  static std::string text() { return std::string("gguf_matvec_q8_spans/") + kind_word(kKind) + "/" + std::to_string(kSpans) + "-spans"; }
+};
+template <int kKind, int kM> struct BlocksTag {
+  static std::string text() { return std::string("gguf_matvec_q8_blocks/") + kind_word(kKind) + "/" + std::to_string(kM) + "-tokens"; }
+};
+
+// ---- any whole number of blocks per row, rows at any even byte stride ---------------------------
+// The kernels above want rows of 2048 n values made of whole 16-byte vectors.  The reference's own
+// projection shapes are wider than that (K = 128, 1024, 5120, 7168, 17408;
+// tests/compute_models/cpu_c5_gguf_inputs.h:231-314), and a GGUF row of Q6_K or Q8_0 blocks starts on a
+// 16-byte boundary only when K is a multiple of 2048 or 256.  Here every block first quantises the
+// activation rows into LDS in their natural order (int8 codes [m][K], one f32 scale per activation
+// block), then a wave walks its weight rows 1024 values at a time: the aligned 16-byte vectors that
+// cover the step's bytes go through a wave-private LDS slot (the next step's are in flight
+// meanwhile), sixteen lanes take each run of 256 values -- the pieces of the K-quant block, or eight
+// Q8_0 blocks, two lanes each -- from aligned LDS words and a funnel shift by the step's byte
+// offset, and meet the codes of the same positions with v_dot4c_i32_i8.  Same integer dots and f32
+// closing products as the span kernels; only the order of the f32 sums differs.
+template <int kWords> __device__ __forceinline__ void lds_words(const unsigned char *base, uint32_t offset, uint32_t (&out)[kWords]) {
+  const uint32_t *words = reinterpret_cast<const uint32_t *>(base + (offset & ~3u));
+  uint32_t w[kWords + 1];
+#pragma unroll
+  for (int i = 0; i <= kWords; ++i) w[i] = words[i];
+#pragma unroll
+  for (int i = 0; i < kWords; ++i) out[i] = __builtin_amdgcn_alignbyte(w[i + 1], w[i], offset & 3u);
+}
+
+template <int kKind> struct BlocksGeometry;
+template <> struct BlocksGeometry<0> {  // Q4_K
+  static constexpr uint32_t kRunBytes = 144, kActivationBlock = 256;
+};
+template <> struct BlocksGeometry<1> {  // Q6_K
+  static constexpr uint32_t kRunBytes = 210, kActivationBlock = 256;
+};
+template <> struct BlocksGeometry<2> {  // Q8_0: a run of 256 values is eight blocks of 34 bytes
+  static constexpr uint32_t kRunBytes = 272, kActivationBlock = 32;
+};
+template <int kKind> struct BlocksStep {
+  static constexpr uint32_t kBytes = 4 * BlocksGeometry<kKind>::kRunBytes;   // 1024 values of a row
+  static constexpr int kLoads = (int)((kBytes + 14 + 15) / 16 + kWaveLanes - 1) / kWaveLanes;
+  static constexpr uint32_t kSlotBytes = kLoads * kWaveLanes * 16;
+};
+
+// One lane's sixteen values of a run of 256 (run `at` bytes into the slot) against the codes of the
+// same positions of one activation row; `codes` points at the row's codes of this run.
+template <int kKind> struct RunDot;
+template <> struct RunDot<0> {  // lane u: chunk u / 4, quant bytes 8 (u % 4) .. + 7: low nibbles sub-block 2 c, high 2 c + 1
+  uint32_t low[2], high[2];
+  int sc_low, sc_high, m_low, m_high;
+  float d, dmin;
+  uint32_t first;  // position of the lane's low-nibble values inside the run
+  __device__ __forceinline__ void decode(const unsigned char *slot, uint32_t at, uint32_t u) {
+    const uint32_t chunk = u / 4;
+    uint32_t head[4], quants[2];
+    lds_words<4>(slot, at, head);
+    lds_words<2>(slot, at + 16 + 32 * chunk + 8 * (u % 4), quants);
+    d = f16_to_f32((uint16_t)head[0]);
+    dmin = f16_to_f32((uint16_t)(head[0] >> 16));
+    sc_low = q4k_six_bits(head[1], head[2], head[3], 2 * chunk, false);
+    sc_high = q4k_six_bits(head[1], head[2], head[3], 2 * chunk + 1, false);
+    m_low = q4k_six_bits(head[1], head[2], head[3], 2 * chunk, true);
+    m_high = q4k_six_bits(head[1], head[2], head[3], 2 * chunk + 1, true);
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      low[w] = quants[w] & 0x0F0F0F0Fu;
+      high[w] = (quants[w] >> 4) & 0x0F0F0F0Fu;
+    }
+    first = 64 * chunk + 8 * (u % 4);
+  }
+  __device__ __forceinline__ float against(const unsigned char *codes, float a_scale) const {
+    const uint32_t *lo = reinterpret_cast<const uint32_t *>(codes + first);
+    const uint32_t *hi = reinterpret_cast<const uint32_t *>(codes + first + 32);
+    const uint32_t c0 = lo[0], c1 = lo[1], c2 = hi[0], c3 = hi[1];
+    const int lows = dot4(low[0], c0, dot4(low[1], c1, 0)), highs = dot4(high[0], c2, dot4(high[1], c3, 0));
+    const int sum_low = dot4(0x01010101u, c0, dot4(0x01010101u, c1, 0)), sum_high = dot4(0x01010101u, c2, dot4(0x01010101u, c3, 0));
+    const int scaled = mad24(sc_low, lows, __mul24(sc_high, highs));
+    const int minima = mad24(m_low, sum_low, __mul24(m_high, sum_high));
+    return a_scale * (d * (float)scaled - dmin * (float)minima);
+  }
+};
+template <> struct RunDot<1> {  // lane u: half u / 8, positions 4 j .. 4 j + 3 (j = u % 8) of the half's four groups of 32
+  uint32_t q[4];
+  int scale[4];
+  float step;  // d / 4
+  uint32_t first;
+  __device__ __forceinline__ void decode(const unsigned char *slot, uint32_t at, uint32_t u) {
+    const uint32_t half = u / 8, j = u % 8;
+    uint32_t a[1], b[1], t[1], scales[2];
+    lds_words<1>(slot, at + 64 * half + 4 * j, a);
+    lds_words<1>(slot, at + 64 * half + 32 + 4 * j, b);
+    lds_words<1>(slot, at + 128 + 32 * half + 4 * j, t);
+    lds_words<2>(slot, at + 192 + 8 * half, scales);
+    step = f16_to_f32(*reinterpret_cast<const uint16_t *>(slot + at + 208)) * 0.25f;
+    const uint32_t top = t[0] ^ 0xAAAAAAAAu;  // q - 32 modulo 64: bytes of 4 (q - 32) as int8
+    q[0] = ((a[0] << 2) & 0x3C3C3C3Cu) | ((top << 6) & 0xC0C0C0C0u);
+    q[1] = ((b[0] << 2) & 0x3C3C3C3Cu) | ((top << 4) & 0xC0C0C0C0u);
+    q[2] = ((a[0] >> 2) & 0x3C3C3C3Cu) | ((top << 2) & 0xC0C0C0C0u);
+    q[3] = ((b[0] >> 2) & 0x3C3C3C3Cu) | (top & 0xC0C0C0C0u);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const uint32_t byte = 2 * g + j / 4;  // scales[8 half + 2 g + l / 16], l = 4 j
+      scale[g] = (int)(signed char)(scales[byte / 4] >> (8 * (byte % 4)));
+    }
+    first = 128 * half + 4 * j;
+  }
+  __device__ __forceinline__ float against(const unsigned char *codes, float a_scale) const {
+    int total = 0;
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      total = mad24(scale[g], dot4(q[g], *reinterpret_cast<const uint32_t *>(codes + first + 32 * g), 0), total);
+    return (step * a_scale) * (float)total;
+  }
+};
+template <> struct RunDot<2> {  // lane u: block u / 2 of the run's eight, quants 16 (u % 2) .. + 15
+  uint32_t q[4];
+  float d;
+  uint32_t first;
+  __device__ __forceinline__ void decode(const unsigned char *slot, uint32_t at, uint32_t u) {
+    const uint32_t block = at + 34 * (u / 2);
+    lds_words<4>(slot, block + 2 + 16 * (u % 2), q);
+    d = f16_to_f32(*reinterpret_cast<const uint16_t *>(slot + block));
+    first = 16 * u;
+  }
+  __device__ __forceinline__ float against(const unsigned char *codes, float a_scale) const {
+    const uint32_t *c = reinterpret_cast<const uint32_t *>(codes + first);
+    int total = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) total = dot4(q[i], c[i], total);
+    return (d * a_scale) * (float)total;
+  }
+};
+
+// staged: int8 codes [m][k], then f32 scales [m][k / activation block].  kM: activation rows
+// served at once (rows past m repeat the last one and are not stored).
+template <int kKind, class TX, int kM>
+__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_blocks(const unsigned char *weights, const void *x, void *y,
+                                                                       uint32_t rows, uint64_t row_stride, uint32_t k,
+                                                                       uint32_t m) {
+  using Geometry = BlocksGeometry<kKind>;
+  using Step = BlocksStep<kKind>;
+  constexpr uint32_t kActivationBlock = Geometry::kActivationBlock;
+  constexpr int kQuantiseLanes = kActivationBlock / 8;  // a lane quantises eight neighbouring values
+  __shared__ __align__(16) unsigned char slots[kWavesPerBlock][Step::kSlotBytes];
+  extern __shared__ __align__(16) uint32_t staged[];
+  unsigned char *codes = reinterpret_cast<unsigned char *>(staged);
+  float *scales = reinterpret_cast<float *>(codes + (size_t)m * k);  // k is a multiple of 32: aligned
+  const uint32_t activation_blocks = k / kActivationBlock;
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+
+  // ---- the activation rows, quantised once per block ------------------------------------------
+  for (uint32_t r = 0; r < m; ++r) {
+    for (uint32_t base = 0; base < k; base += kBlockThreads * 8) {
+      const uint32_t p = base + threadIdx.x * 8;
+      const bool inside = p < k;  // the same for all lanes that share an activation block
+      float values[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) values[e] = inside ? Traits<TX>::load(x, (size_t)r * k + p + e) : 0.0f;
+      LaneMax mine{0.0f, 0.0f, 0u};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {  // positions rise with e, so ">" keeps the first
+        const float magnitude = __builtin_fabsf(values[e]);
+        if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], p + e};
+      }
+      if (mine.magnitude == 0.0f) mine.position = 0xFFFFFFFFu;  // no candidate: any lane with one goes first
+      const LaneMax top = block_largest<kQuantiseLanes>(mine);
+      float factor = 0.0f, stored = 0.0f;
+      if (top.magnitude != 0.0f) {
+        if constexpr (kKind == 2) {
+          stored = f16_to_f32(f32_to_f16(top.magnitude / 127.0f));
+          factor = 127.0f / top.magnitude;
+        } else {
+          factor = -127.0f / top.value;
+          stored = 1.0f / factor;
+        }
+      }
+      uint32_t words[2] = {0u, 0u};
+      if (top.magnitude != 0.0f) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) words[e / 4] |= code_of(values[e] * factor) << (8 * (e % 4));
+      }
+      if (inside) {
+        uint32_t *to = reinterpret_cast<uint32_t *>(codes + (size_t)r * k + p);
+        to[0] = words[0];
+        to[1] = words[1];
+        if (p % kActivationBlock == 0) scales[r * activation_blocks + p / kActivationBlock] = stored;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- the weight rows ----------------------------------------------------------------------
+  const uint32_t stride = gridDim.x * kWavesPerBlock;
+  const uint32_t first = blockIdx.x * kWavesPerBlock + wave;
+  if (first >= rows) return;  // no barrier follows
+  unsigned char *slot = slots[wave];
+  const uint32_t runs = (k + 255) / 256;           // runs of 256 values in a row (the last one of a Q8_0 row may be short)
+  const uint32_t steps = (runs + 3) / 4;
+  const uint64_t row_bytes = (uint64_t)(k / kActivationBlock) * (kKind == 2 ? 34u : Geometry::kRunBytes);
+  const uint32_t run = lane / 16, u = lane % 16;
+  if (steps == 0) {  // K = 0: every product is an empty sum
+    for (uint32_t row = first; row < rows; row += stride)
+      if (lane < m) Traits<TX>::store(y, (size_t)lane * rows + row, 0.0f);
+    return;
+  }
+
+  // the aligned 16-byte vectors that cover step `step` of row `row`; lanes past them repeat the last one
+  auto load_step = [&](uint32_t row, uint32_t step, u32x4 (&into)[Step::kLoads], uint32_t *shift) {
+    const uint64_t begin = (uint64_t)row * row_stride + (uint64_t)step * Step::kBytes;
+    const uint64_t left = row_bytes - (uint64_t)step * Step::kBytes;
+    const uint32_t bytes = left < Step::kBytes ? (uint32_t)left : Step::kBytes;
+    const uintptr_t address = reinterpret_cast<uintptr_t>(weights) + begin;
+    const uint32_t off = (uint32_t)(address & 15u);
+    const u32x4 *vectors = reinterpret_cast<const u32x4 *>(address - off);
+    const uint32_t needed = (off + bytes + 15) / 16;
+#pragma unroll
+    for (int i = 0; i < Step::kLoads; ++i) {
+      const uint32_t wanted = lane + i * kWaveLanes;
+      into[i] = __builtin_nontemporal_load(vectors + (wanted < needed ? wanted : needed - 1));
+    }
+    *shift = off;
+  };
+
+  u32x4 ring[Step::kLoads];
+  uint32_t shift = 0;
+  load_step(first, 0, ring, &shift);
+  for (uint32_t row = first; row < rows; row += stride) {
+    float totals[kM] = {};
+    for (uint32_t step = 0; step < steps; ++step) {
+#pragma unroll
+      for (int i = 0; i < Step::kLoads; ++i) *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = ring[i];
+      const uint32_t at = shift + run * Geometry::kRunBytes;
+      {
+        // the next step of this row, the first of the wave's next row, or (at the very end) the
+        // wave's first row again: a valid address whose bytes go unused
+        const bool last = step + 1 == steps;
+        const uint32_t next_row = last ? (row + stride < rows ? row + stride : first) : row;
+        load_step(next_row, last ? 0u : step + 1, ring, &shift);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+      const uint32_t run_index = step * 4 + run;
+      const uint32_t position = run_index * 256 + (kKind == 2 ? 16 * u : 0u);  // of the lane's first value (K-quants: of its run)
+      const bool live = position < k;
+      RunDot<kKind> decoded;
+      decoded.decode(slot, at, u);
+      if (!live) decoded.first = 0;  // a lane past the row reads the row's first codes and adds nothing
+      const uint32_t run_codes = live ? run_index * 256 : 0u;
+      const uint32_t scale_index = live ? (kKind == 2 ? run_index * 8 + u / 2 : run_index) : 0u;
+#pragma unroll
+      for (int r = 0; r < kM; ++r) {
+        const uint32_t token = (uint32_t)r < m ? (uint32_t)r : m - 1;
+        const float part = decoded.against(codes + (size_t)token * k + run_codes, scales[token * activation_blocks + scale_index]);
+        totals[r] += live ? part : 0.0f;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+#pragma unroll
+    for (int r = 0; r < kM; ++r) {
+      const float whole = group_sum<kWaveLanes>(totals[r]);
+      if (lane == 0 && (uint32_t)r < m) Traits<TX>::store(y, (size_t)r * rows + row, whole);
+    }
+  }
+}
+
+// Bytes of LDS one activation row takes in gguf_matvec_q8_blocks.
+inline size_t blocks_row_bytes(int kind, uint32_t k) { return (size_t)k + (size_t)(k / (kind == 2 ? 32u : 256u)) * sizeof(float); }
+constexpr size_t kBlocksSharedBudget = 56 * 1024;  // beside the waves' row slots (at most 8 KiB) in a block's 64 KiB
+
+template <int kKind, class TX>
+hipError_t run_blocks(const MatVecParams &p, const void *w, const void *x, void *y, int compute_units, hipStream_t s) {
+  const size_t per_row = blocks_row_bytes(kKind, p.k);
+  uint32_t fit = per_row == 0 ? 8u : (uint32_t)(kBlocksSharedBudget / per_row);
+  if (fit == 0) return hipErrorInvalidValue;  // the plan declines such K
+  fit = fit >= 8 ? 8 : (fit >= 4 ? 4 : (fit >= 2 ? 2 : 1));
+  const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
+  const uint32_t machine = (uint32_t)(compute_units > 0 ? compute_units : 256) * 3u;  // three blocks per compute unit
+  const dim3 grid(wanted < machine ? wanted : machine);
+  const unsigned char *in = static_cast<const unsigned char *>(w);
+  // activation rows in groups that fit LDS together; every group walks the weight again
+  for (uint32_t done = 0; done < p.m; done += fit) {
+    const uint32_t m = p.m - done < fit ? p.m - done : fit;
+    const void *xs = static_cast<const char *>(x) + (size_t)done * p.k * Traits<TX>::kSize;
+    void *ys = static_cast<char *>(y) + (size_t)done * p.rows * Traits<TX>::kSize;
+    const size_t shared = m * per_row;
+#define HYLE_BLOCKS(M)                 \
+  note_variant<BlocksTag<kKind, M>>(); \
+  hipLaunchKernelGGL((gguf_matvec_q8_blocks<kKind, TX, M>), grid, dim3(kBlockThreads), shared, s, in, xs, ys, (uint32_t)p.rows, p.row_stride, p.k, m)
+    if (m == 1) { HYLE_BLOCKS(1); }
+    else if (m == 2) { HYLE_BLOCKS(2); }
+    else if (m <= 4) { HYLE_BLOCKS(4); }
+    else { HYLE_BLOCKS(8); }
+#undef HYLE_BLOCKS
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+  }
+  return hipSuccess;
+}
+
 template <int kKind, class TX>
 hipError_t run_quads(const MatVecParams &p, const void *w, const void *x, void *y, uint32_t spans, dim3 grid,
                      size_t shared, hipStream_t s) {
   const unsigned char *in = static_cast<const unsigned char *>(w);
 #define HYLE_QUADS(SETS, REGISTERS)                                                                             \
+  note_variant<QuadsTag<kKind, SETS, REGISTERS>>();                                                                 \
   hipLaunchKernelGGL((gguf_matvec_q8_quads<kKind, TX, SETS, REGISTERS>), grid, dim3(kBlockThreads), shared, s, in, x, \
                      y, (uint32_t)p.rows, p.row_stride, spans, p.m)
   const bool registers = spans == 1 && kKind != 0;  // Q4_K fetches its codes from LDS share by share
   if (p.m <= 4) {
-    if (registers) HYLE_QUADS(1, true);
-    else HYLE_QUADS(1, false);
+    if constexpr (kKind != 0) {
+      if (registers) { HYLE_QUADS(1, true); }
+    }
+    if (!registers) { HYLE_QUADS(1, false); }
   } else {
-    if (registers) HYLE_QUADS(2, true);
-    else HYLE_QUADS(2, false);
+    if constexpr (kKind != 0) {
+      if (registers) { HYLE_QUADS(2, true); }
+    }
+    if (!registers) { HYLE_QUADS(2, false); }
   }
 #undef HYLE_QUADS
   return hipGetLastError();
@@ -722,17 +1041,25 @@ template <int kKind, class TX, int kM>
 hipError_t run_registers(const MatVecParams &p, const void *w, const void *x, void *y, uint32_t spans, dim3 grid,
                          size_t shared, hipStream_t s) {
   const unsigned char *in = static_cast<const unsigned char *>(w);
-  if (spans == 1)
+  if (spans == 1) {
+    note_variant<LinesTag<kKind, kM, true>>();
     hipLaunchKernelGGL((gguf_matvec_q8_lines<kKind, TX, kM, true>), grid, dim3(kBlockThreads), shared, s, in, x, y,
                        (uint32_t)p.rows, p.row_stride, spans, p.m);
-  else
+  } else {
+    note_variant<LinesTag<kKind, kM, false>>();
     hipLaunchKernelGGL((gguf_matvec_q8_lines<kKind, TX, kM, false>), grid, dim3(kBlockThreads), shared, s, in, x, y,
                        (uint32_t)p.rows, p.row_stride, spans, p.m);
+  }
   return hipGetLastError();
 }
 
 template <int kKind, class TX>
 hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, int compute_units, hipStream_t s) {
+  // the span kernels: rows of 2048 n values made of whole 16-byte vectors, codes of every activation
+  // row in LDS beside the waves' row buffers (12 KiB); everything else walks block by block
+  if (p.k == 0 || p.k % 2048 != 0 || p.row_stride % 16 != 0 || (reinterpret_cast<uintptr_t>(w) & 15u) != 0 ||
+      gguf_matvec_q8_shared_bytes(p.m, p.k) + 12 * 1024 > 64 * 1024)
+    return run_blocks<kKind, TX>(p, w, x, y, compute_units, s);
   const uint32_t spans = p.k / 2048;
   const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
   const uint32_t machine = (uint32_t)(compute_units > 0 ? compute_units : 256) * 3u;  // three blocks per compute unit
@@ -755,12 +1082,12 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
     const unsigned char *in = static_cast<const unsigned char *>(w);
     const uint32_t rows = (uint32_t)p.rows;
     switch (spans) {
-      case 1: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 1>), blocks, dim3(1 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      case 2: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 2>), blocks, dim3(2 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      case 3: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 3>), blocks, dim3(3 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      case 4: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 4>), blocks, dim3(4 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      case 5: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 5>), blocks, dim3(5 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      default: hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 6>), blocks, dim3(6 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      case 1: note_variant<SpansTag<kKind, 1>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 1>), blocks, dim3(1 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      case 2: note_variant<SpansTag<kKind, 2>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 2>), blocks, dim3(2 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      case 3: note_variant<SpansTag<kKind, 3>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 3>), blocks, dim3(3 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      case 4: note_variant<SpansTag<kKind, 4>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 4>), blocks, dim3(4 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      case 5: note_variant<SpansTag<kKind, 5>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 5>), blocks, dim3(5 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+      default: note_variant<SpansTag<kKind, 6>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 6>), blocks, dim3(6 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
     }
     return hipGetLastError();
   }
@@ -785,8 +1112,18 @@ size_t gguf_matvec_q8_shared_bytes(uint32_t m, uint32_t k) {
   return (size_t)m * (k / 2048) * kCodeWords * kWaveLanes * sizeof(uint32_t);
 }
 
-// Needs K = 2048 n, rows made of whole 16-byte vectors at a 16-byte aligned address, M <= 8 and
-// gguf_matvec_q8_shared_bytes(m, k) + 12 KiB within a block's 64 KiB (the plan checks all four).
+bool gguf_matvec_q8_serves(int kind, uint32_t k) { return blocks_row_bytes(kind, k) <= kBlocksSharedBudget; }
+
+uint32_t gguf_matvec_q8_dispatches(int kind, uint32_t m, uint32_t k, uint64_t row_stride) {
+  if (m == 0 || k == 0) return 1;
+  if (k % 2048 == 0 && row_stride % 16 == 0 && gguf_matvec_q8_shared_bytes(m, k) + 12 * 1024 <= 64 * 1024) return 1;
+  uint32_t fit = (uint32_t)(kBlocksSharedBudget / blocks_row_bytes(kind, k));
+  fit = fit >= 8 ? 8 : (fit >= 4 ? 4 : (fit >= 2 ? 2 : 1));
+  return (m + fit - 1) / fit;
+}
+
+// K a whole number of blocks with one activation row's codes within LDS (gguf_matvec_q8_serves),
+// rows at an even address and stride, M <= 8 (the plan checks all three).
 hipError_t launch_gguf_matvec_q8(Elem x_type, const MatVecParams &p, const void *weights, const void *x, void *y,
                                  int compute_units, hipStream_t stream) {
   if (p.rows == 0 || p.m == 0) return hipSuccess;

@@ -213,8 +213,13 @@ struct MatVecParams {
   uint32_t compute_units = 256;  // of the plan's device: the grids are three blocks per unit
 };
 size_t gguf_matvec_shared_bytes(uint32_t m, uint32_t k);
-// The 8-bit activation route: K = 2048 n, rows of whole 16-byte vectors, M <= 8.
+// The 8-bit activation route: any whole number of blocks per row at even addresses, M <= 8.
+// Rows of 2048 n values made of whole 16-byte vectors take the span kernels (the codes of all M
+// rows in LDS: gguf_matvec_q8_shared_bytes); other shapes walk block by block, M in groups that
+// fit LDS (gguf_matvec_q8_dispatches launches).  gguf_matvec_q8_serves: one activation row fits.
 size_t gguf_matvec_q8_shared_bytes(uint32_t m, uint32_t k);
+bool gguf_matvec_q8_serves(int kind, uint32_t k);
+uint32_t gguf_matvec_q8_dispatches(int kind, uint32_t m, uint32_t k, uint64_t row_stride);
 hipError_t launch_gguf_matvec_q8(Elem x_type, const MatVecParams &p, const void *weights, const void *x, void *y,
                                  int compute_units, hipStream_t stream);
 hipError_t launch_gguf_matvec(Elem x_type, const MatVecParams &p, const void *weights, const void *x, void *y,

@@ -1118,15 +1118,15 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       if ((s = admit_gguf_rows(in[0])) != HYLE_HIP_OK) return s;
       const int64_t m = in[1].rank == 2 ? in[1].dims[0] : 1;
       if (m > 8) return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec serves at most 8 activation rows");
+      const uint8_t matvec_kind = per_block == 32 ? 2 : (block_bytes == 144 ? 0 : 1);
       if (r.kind2 == HYLE_HIP_ACTIVATIONS_GGML_Q8) {
-        // whole spans of 2048 values in rows of whole 16-byte vectors; the codes of every
-        // activation row sit in LDS beside the waves' row buffers (12 KiB)
-        if (k % 2048 != 0 || in[0].byte_strides[1] % 16 != 0)
-          return fail(HYLE_HIP_UNIMPLEMENTED,
-                      "GGUF matvec with 8-bit activation blocks serves K = 2048 n and 16-byte aligned rows");
-        if (gguf_matvec_q8_shared_bytes((uint32_t)m, (uint32_t)k) + 12 * 1024 > 64 * 1024)
-          return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec keeps the activation codes in LDS: M * K is too large");
-        p->input_alignment[0] = 16;
+        // any whole number of blocks per row; the blocks are read as 16-bit aligned pieces, so rows
+        // start at even addresses; one activation row's 8-bit codes must fit a block's LDS
+        if (in[0].byte_strides[1] % 2 != 0)
+          return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec with 8-bit activation blocks serves rows at even byte strides");
+        if (!gguf_matvec_q8_serves(matvec_kind, (uint32_t)k))
+          return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec keeps the activation codes in LDS: K is too large");
+        p->input_alignment[0] = 2;
       } else if (gguf_matvec_shared_bytes((uint32_t)m, (uint32_t)k) > 64 * 1024) {
         return fail(HYLE_HIP_UNIMPLEMENTED, "GGUF matvec keeps the activations in LDS: M * K is too large");
       }
@@ -1138,9 +1138,11 @@ hyle_hip_status admit(hyle_hip_plan *p) {
       p->matvec.k = (uint32_t)k;
       p->matvec.m = (uint32_t)m;
       p->matvec.row_stride = (uint64_t)in[0].byte_strides[1];
-      p->matvec.kind = per_block == 32 ? 2 : (block_bytes == 144 ? 0 : 1);
+      p->matvec.kind = matvec_kind;
       if (r.kind2 != HYLE_HIP_ACTIVATIONS_GGML_Q8) p->input_alignment[0] = 1;
-      p->dispatches = 1;
+      p->dispatches = r.kind2 == HYLE_HIP_ACTIVATIONS_GGML_Q8
+                          ? gguf_matvec_q8_dispatches(matvec_kind, (uint32_t)m, (uint32_t)k, (uint64_t)in[0].byte_strides[1])
+                          : 1;
       return HYLE_HIP_OK;
     }
     case HYLE_HIP_OP_FILL: {

@@ -44,14 +44,21 @@ def raw_bytes_for(tag, rng, rows, k):
     return raw.reshape(rows, -1)
 
 
-def check(tag, x_tag, raw, rows, k, x, row_stride=None):
+def check(tag, x_tag, raw, rows, k, x, row_stride=None, byte_offset=0, kernel=None):
+    """byte_offset: the weight starts that many bytes into its (256-byte aligned) allocation;
+    kernel: the launch shape the case is written for (a prefix of the label)."""
     kind, gguf = KINDS[tag]
     stored = host_values(x, x_tag)
     wide = stored if x_tag == "f32" else orc.to_f32(TYPES[x_tag][1], stored)
-    storage = torch.from_numpy(np.ascontiguousarray(raw).reshape(-1)).to(DEVICE)
+    flat = np.ascontiguousarray(raw).reshape(-1)
+    if byte_offset:
+        flat = np.concatenate([np.zeros(byte_offset, np.uint8), flat])
+    storage = torch.from_numpy(flat).to(DEVICE)[byte_offset:]
     descs = [hc.TensorDesc.gguf_weight(gguf, TYPES[x_tag][0], k, rows, row_stride),
              hc.TensorDesc.dense(TYPES[x_tag][0], list(x.shape))]
     (out,) = run(Q8, storage, to_device(stored, x_tag), descs=descs)
+    if kernel is not None:
+        assert hc.last_launch_variant().startswith(kernel), (hc.last_launch_variant(), kernel)
     assert list(out.shape) == ([rows] if x.ndim == 1 else [x.shape[0], rows])
     centre, bound = orc.gguf_matvec_q8(kind, raw.reshape(-1), rows, k, wide, row_stride)
     centre, bound = centre.reshape(out.shape), bound.reshape(out.shape)
@@ -115,13 +122,83 @@ def test_q8_route_vocabulary_sized_weight(tag, m):
     check(tag, "f32", raw, rows, k, x)
 
 
+def test_q8_route_the_reference_s_own_projection_shapes():
+    """The shapes of the reference's Q8_0 / Q4_K projection cases
+    (tests/compute_models/cpu_c5_gguf_inputs.h:231,237,259,287,314): none is a multiple of 2048 wide,
+    so every one takes the kernel that walks a row block by block."""
+    rng = np.random.default_rng(1803)
+    for tag, k, rows in (("q8_0", 1024, 32768), ("q4_k", 5120, 10240), ("q8_0", 7168, 3072), ("q8_0", 17408, 5120),
+                         ("q8_0", 128, 512)):
+        raw = weights_for(tag, rng, rows, k)
+        x = rng.normal(0, 1.5, (k,)).astype(np.float32)
+        note(f"q8 matvec {tag} [{k} -> {rows}], one activation row")
+        check(tag, "f32", raw, rows, k, x, kernel=f"gguf_matvec_q8_blocks/{tag}/1-tokens")
+
+
+@pytest.mark.parametrize("x_tag", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("tag", list(KINDS))
+def test_q8_route_any_whole_number_of_blocks_and_activation_rows(tag, x_tag):
+    """K from one block up, not a multiple of 2048 (Q8_0 also not of 256: the last run of 256 values is
+    short); 1 to 8 activation rows; more rows than waves, fewer rows than waves of a block."""
+    rng = np.random.default_rng(1804)
+    per = 32 if tag == "q8_0" else 256
+    widths = (32, 96, 128, 480, 1024, 5120) if tag == "q8_0" else (256, 768, 1024, 2304, 5120)
+    for k in widths:
+        for rows, m in ((1, 1), (3, 2), (70, 1), (33, 3), (257, 4), (19, 5), (40, 8)):
+            # uniformly random block bytes for the short rows (their products overflow f16: modest weights there)
+            raw = raw_bytes_for(tag, rng, rows, k) if k <= 1024 and x_tag != "f16" else weights_for(tag, rng, rows, k)
+            x = rng.normal(0, 1.5, (m, k) if m > 1 else (k,)).astype(np.float32)
+            note(f"q8 matvec {tag} x {x_tag} rows {rows} k {k} (blocks of {per}) m {m}")
+            label = {1: 1, 2: 2, 3: 4, 4: 4, 5: 8, 8: 8}[m]
+            check(tag, x_tag, raw, rows, k, x, kernel=f"gguf_matvec_q8_blocks/{tag}/{label}-tokens")
+
+
+@pytest.mark.parametrize("tag", list(KINDS))
+def test_q8_route_rows_at_even_addresses_and_strides(tag):
+    """Rows that start 2, 6 or 14 bytes off a 16-byte boundary (the weight inside its allocation, and a
+    row stride that is not a multiple of 16), for K = 2048 too: those leave the span kernels for the
+    block-walking one, and must give what the aligned launch gives."""
+    rng = np.random.default_rng(1805)
+    for k, rows, m in ((2048, 37, 1), (2048, 9, 4), (4096, 21, 2), (1280 if tag != "q8_0" else 1120, 50, 3)):
+        raw = raw_bytes_for(tag, rng, rows, k)
+        x = rng.normal(0, 2, (m, k) if m > 1 else (k,)).astype(np.float32)
+        row_bytes = raw.shape[1]
+        for byte_offset, pad in ((2, 0), (6, 2), (14, 10), (0, 6)):
+            padded = np.zeros((rows, row_bytes + pad), np.uint8)
+            padded[:, :row_bytes] = raw
+            note(f"q8 matvec {tag} k {k} rows {rows} m {m}: weight {byte_offset} bytes off, rows {pad} bytes apart")
+            check(tag, "f32", padded, rows, k, x, row_stride=row_bytes + pad, byte_offset=byte_offset,
+                  kernel="gguf_matvec_q8_blocks/")
+
+
+def test_q8_route_activation_rows_in_groups_when_their_codes_do_not_fit_together():
+    """Eight activation rows of 17408 values need 8 x 19.6 KB of codes: they are served two at a
+    time, four dispatches over the same weight."""
+    rng = np.random.default_rng(1806)
+    rows, k, m = 300, 17408, 8
+    raw = weights_for("q8_0", rng, rows, k)
+    x = rng.normal(0, 1.0, (m, k)).astype(np.float32)
+    weight = hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ8_0, hc.DataType.kFloat32, k, rows)
+    prepared = hc.prepare(context(), Q8, weight, hc.TensorDesc.dense(hc.DataType.kFloat32, [m, k]))
+    assert prepared.dispatch_count() == 4
+    note(f"q8 matvec q8_0 [{k} -> {rows}] x {m}: activation rows in groups of two")
+    check("q8_0", "f32", raw, rows, k, x, kernel="gguf_matvec_q8_blocks/q8_0/2-tokens + gguf_matvec_q8_blocks/q8_0/2-tokens")
+
+
 def test_q8_route_declines_what_it_does_not_serve():
     ctx = context()
+    # more than eight activation rows
     weight = hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ6K, hc.DataType.kFloat32, 1024, 16)
     with pytest.raises(hc.StatusError) as declined:
-        hc.prepare(ctx, Q8, weight, hc.TensorDesc.dense(hc.DataType.kFloat32, [1024]))
+        hc.prepare(ctx, Q8, weight, hc.TensorDesc.dense(hc.DataType.kFloat32, [9, 1024]))
     assert declined.value.is_unimplemented()
-    weight = hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ6K, hc.DataType.kFloat32, 8192, 16)
+    # one activation row's codes beyond a block's LDS
+    weight = hc.TensorDesc.gguf_weight(hc.GgufQuantizedType.kQ8_0, hc.DataType.kFloat32, 65536, 4)
     with pytest.raises(hc.StatusError) as declined:
-        hc.prepare(ctx, Q8, weight, hc.TensorDesc.dense(hc.DataType.kFloat32, [8, 8192]))
+        hc.prepare(ctx, Q8, weight, hc.TensorDesc.dense(hc.DataType.kFloat32, [65536]))
     assert declined.value.is_unimplemented()
+    # what it now serves: widths that are whole blocks but no multiple of 2048, eight rows of 8192
+    for gguf, k, m in ((hc.GgufQuantizedType.kQ6K, 1024, 1), (hc.GgufQuantizedType.kQ6K, 8192, 8),
+                       (hc.GgufQuantizedType.kQ8_0, 32, 1)):
+        weight = hc.TensorDesc.gguf_weight(gguf, hc.DataType.kFloat32, k, 16)
+        hc.prepare(ctx, Q8, weight, hc.TensorDesc.dense(hc.DataType.kFloat32, [m, k] if m > 1 else [k]))
