@@ -89,6 +89,31 @@ class MemoryResource:
             pass
 
 
+class TransferMode(enum.IntEnum):  # include/hyle/compute/transfer.h:19-22
+    kImmediate = 0
+    kQueuedDirect = 1
+
+
+@dataclass(frozen=True)
+class TransferProperties:  # include/hyle/compute/transfer.h:27-30
+    mode: TransferMode
+    peer: bool
+
+
+@dataclass(frozen=True)
+class CompletionEndpoint:  # who emits a queue's completions: (authority, identity) as addresses
+    authority: int = 0
+    identity: int = 0
+
+    def valid(self) -> bool:
+        return bool(self.authority) and bool(self.identity)
+
+
+def same_device(left: int, right: int) -> bool:
+    """BackendVTable::same_device over device indices."""
+    return bool(capi.load().hyle_hip_backend_same_device(left, right))
+
+
 def validate_resource(context: Context, resource: MemoryResource) -> None:
     _check(capi.load().hyle_hip_backend_validate_resource(context._handle, resource._handle))
 
@@ -144,6 +169,24 @@ class Queue:
 
     def wait_completion(self, completion: Completion) -> None:
         _check(capi.load().hyle_hip_queue_wait_completion(self._handle, completion._handle))
+
+    def transfer_properties(self, destination: "Optional[MemoryResource]", source: "Optional[MemoryResource]") -> "TransferProperties":
+        """transfer_properties(queue, destination, source) (include/hyle/compute/transfer.h:31-33): the
+        route a copy between the two resources takes on this queue; StatusError(Unimplemented) when none is offered."""
+        out = capi.TransferPropertiesC()
+        _check(capi.load().hyle_hip_queue_transfer_properties(
+            self._handle, destination._handle if destination else None, source._handle if source else None, C.byref(out)))
+        return TransferProperties(TransferMode(out.mode), bool(out.peer))
+
+    def completion_endpoint(self) -> "CompletionEndpoint":
+        out = capi.CompletionEndpointC()
+        _check(capi.load().hyle_hip_queue_completion_endpoint(self._handle, C.byref(out)))
+        return CompletionEndpoint(out.authority or 0, out.identity or 0)
+
+    def can_wait_endpoint(self, source: "CompletionEndpoint") -> bool:
+        """True commits wait_completion() on this queue to a pending completion emitted by `source`."""
+        return bool(capi.load().hyle_hip_queue_can_wait_endpoint(
+            self._handle, capi.CompletionEndpointC(source.authority or None, source.identity or None)))
 
     def copy_async(self, destination_resource: MemoryResource, destination: int, source_resource: MemoryResource,
                    source: int, size: int) -> None:

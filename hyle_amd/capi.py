@@ -76,6 +76,14 @@ class MemoryPropertiesC(C.Structure):
                 ("maximum_allocation", C.c_size_t)]
 
 
+class TransferPropertiesC(C.Structure):
+    _fields_ = [("mode", C.c_uint32), ("peer", C.c_uint32)]
+
+
+class CompletionEndpointC(C.Structure):
+    _fields_ = [("authority", C.c_void_p), ("identity", C.c_void_p)]
+
+
 class MemoryStatsC(C.Structure):
     _fields_ = [("used_bytes", C.c_size_t), ("peak_bytes", C.c_size_t), ("live_allocations", C.c_uint64),
                 ("total_allocations", C.c_uint64)]
@@ -146,6 +154,10 @@ EXPORTS = {
     "hyle_hip_completion_wait": (C.c_int, [C.c_void_p]),
     "hyle_hip_completion_release": (None, [C.c_void_p]),
     "hyle_hip_queue_wait_completion": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "hyle_hip_backend_same_device": (C.c_int, [C.c_size_t, C.c_size_t]),
+    "hyle_hip_queue_transfer_properties": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(TransferPropertiesC)]),
+    "hyle_hip_queue_completion_endpoint": (C.c_int, [C.c_void_p, C.POINTER(CompletionEndpointC)]),
+    "hyle_hip_queue_can_wait_endpoint": (C.c_int, [C.c_void_p, CompletionEndpointC]),
     "hyle_hip_queue_copy_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
     "hyle_hip_queue_fill_async": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint8, C.c_size_t]),
     "hyle_hip_queue_drain": (C.c_int, [C.c_void_p]),

@@ -4,6 +4,8 @@
 // queue-ordered copy and fill.  Host code, plus the one fill kernel.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -92,9 +94,11 @@ struct hyle_hip_memory_resource {
 struct hyle_hip_completion {
   hyle_hip_queue *owner = nullptr;
   hipEvent_t event = nullptr;
-  bool pending = false;    // the event was recorded and has not been seen finished
-  bool in_use = false;     // handed out by begin_sequence / finish_sequence, not yet released
-  hyle_hip_status terminal = HYLE_HIP_OK;
+  // A completion may be polled and waited for from any thread (the reference's Completion is
+  // pollable from any thread): its state moves through atomics, never through plain fields.
+  std::atomic<bool> pending{false};  // the event was recorded and has not been seen finished
+  bool in_use = false;               // handed out by begin_sequence / finish_sequence, not yet released (queue mutex)
+  std::atomic<int> terminal{HYLE_HIP_OK};
 };
 // A sequence is its completion slot, reserved by begin.
 struct hyle_hip_sequence {
@@ -129,7 +133,7 @@ hyle_hip_sequence *new_slot(hyle_hip_queue *queue, hyle_hip_status *status) {
 }
 
 hyle_hip_status settle(hyle_hip_completion *completion, bool wait, int *done) {
-  if (completion->pending) {
+  if (completion->pending.load(std::memory_order_acquire)) {
     DeviceScope scope(completion->owner->device);
     if (scope.error != hipSuccess) return hip_fail(scope.error, "hipSetDevice");
     const hipError_t err = wait ? hipEventSynchronize(completion->event) : hipEventQuery(completion->event);
@@ -138,15 +142,20 @@ hyle_hip_status settle(hyle_hip_completion *completion, bool wait, int *done) {
       if (done) *done = 0;
       return HYLE_HIP_OK;
     }
-    completion->pending = false;
-    if (err != hipSuccess && completion->terminal == HYLE_HIP_OK)
-      completion->terminal = hip_fail(err, wait ? "hipEventSynchronize" : "hipEventQuery");
+    if (err != hipSuccess) {  // the first failure seen stays the completion's status
+      int expected = HYLE_HIP_OK;
+      completion->terminal.compare_exchange_strong(expected, (int)hip_fail(err, wait ? "hipEventSynchronize" : "hipEventQuery"));
+    }
+    completion->pending.store(false, std::memory_order_release);
   }
   if (done) *done = 1;
-  if (completion->terminal != HYLE_HIP_OK)
-    return fail(completion->terminal, "the sequence ended with %s", hyle_hip_status_name(completion->terminal));
+  const hyle_hip_status terminal = (hyle_hip_status)completion->terminal.load(std::memory_order_acquire);
+  if (terminal != HYLE_HIP_OK) return fail(terminal, "the sequence ended with %s", hyle_hip_status_name(terminal));
   return HYLE_HIP_OK;
 }
+
+// What a CompletionEndpoint of this backend carries as its authority: one address per library.
+const char kCompletionAuthority = 0;
 
 }  // namespace
 
@@ -372,8 +381,8 @@ hyle_hip_status hyle_hip_queue_begin_sequence(hyle_hip_queue *queue, hyle_hip_se
     queue->slots.push_back(found);
   }
   found->slot.in_use = true;
-  found->slot.pending = false;
-  found->slot.terminal = HYLE_HIP_OK;
+  found->slot.pending.store(false, std::memory_order_relaxed);
+  found->slot.terminal.store(HYLE_HIP_OK, std::memory_order_relaxed);
   queue->active = found;
   *sequence = found;
   return HYLE_HIP_OK;
@@ -381,21 +390,27 @@ hyle_hip_status hyle_hip_queue_begin_sequence(hyle_hip_queue *queue, hyle_hip_se
 
 hyle_hip_completion *hyle_hip_queue_finish_sequence(hyle_hip_queue *queue, hyle_hip_sequence *sequence, int accepted,
                                                     hyle_hip_status terminal) {
-  if (queue == nullptr || sequence == nullptr || sequence->slot.owner != queue || queue->active != sequence) {
+  bool owned = queue != nullptr && sequence != nullptr && sequence->slot.owner == queue;
+  if (owned) {
+    std::lock_guard<std::mutex> lock(queue->mutex);
+    owned = queue->active == sequence;
+  }
+  if (!owned) {
     (void)fail(HYLE_HIP_INTERNAL, "sequence does not belong to the queue");
     return nullptr;
   }
   hyle_hip_completion *completion = &sequence->slot;
-  completion->terminal = terminal;
+  completion->terminal.store(terminal, std::memory_order_relaxed);
   if (accepted) {
     DeviceScope scope(queue->device);
     const hipError_t err = scope.error != hipSuccess ? scope.error : hipEventRecord(completion->event, queue->stream);
     if (err == hipSuccess) {
-      completion->pending = true;
+      completion->pending.store(true, std::memory_order_release);
     } else {
       // no event to wait on: fall back to draining the stream now, as the reference's stream fallback does
       (void)hipStreamSynchronize(queue->stream);
-      if (completion->terminal == HYLE_HIP_OK) completion->terminal = hip_fail(err, "hipEventRecord");
+      int expected = HYLE_HIP_OK;
+      completion->terminal.compare_exchange_strong(expected, (int)hip_fail(err, "hipEventRecord"));
     }
   }
   std::lock_guard<std::mutex> lock(queue->mutex);
@@ -424,12 +439,47 @@ hyle_hip_status hyle_hip_queue_wait_completion(hyle_hip_queue *queue, hyle_hip_c
   if (queue == nullptr || completion == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "null argument");
   if (completion->owner->device != queue->device)
     return fail(HYLE_HIP_UNIMPLEMENTED, "a queue waits for completions of its own device only");
-  if (!completion->pending) return HYLE_HIP_OK;  // already finished: nothing to order after
+  if (!completion->pending.load(std::memory_order_acquire)) return HYLE_HIP_OK;  // already finished: nothing to order after
   DeviceScope scope(queue->device);
   if (scope.error != hipSuccess) return hip_fail(scope.error, "hipSetDevice");
   const hipError_t err = hipStreamWaitEvent(queue->stream, completion->event, 0);
   if (err != hipSuccess) return hip_fail(err, "hipStreamWaitEvent");
   return HYLE_HIP_OK;
+}
+
+int hyle_hip_backend_same_device(size_t left, size_t right) {
+  size_t count = 0;
+  if (hyle_hip_backend_device_count(&count) != HYLE_HIP_OK || left >= count || right >= count) return 0;
+  return left == right ? 1 : 0;  // a device is its ordinal
+}
+
+hyle_hip_status hyle_hip_queue_transfer_properties(const hyle_hip_queue *queue,
+                                                   const hyle_hip_memory_resource *destination,
+                                                   const hyle_hip_memory_resource *source,
+                                                   hyle_hip_transfer_properties *properties) {
+  if (queue == nullptr || properties == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "null argument");
+  properties->mode = HYLE_HIP_TRANSFER_IMMEDIATE;
+  properties->peer = 0;
+  // the same admission as copy_async: storage of the queue's own device, device or pinned host on
+  // either side; nothing else is offered (no hidden staging, no host wait dressed up as a copy)
+  if (destination == nullptr || source == nullptr || destination->device != queue->device ||
+      source->device != queue->device)
+    return fail(HYLE_HIP_UNIMPLEMENTED, "HIP async transfer requires device or pinned storage of the queue's own device");
+  properties->mode = HYLE_HIP_TRANSFER_QUEUED_DIRECT;
+  return HYLE_HIP_OK;
+}
+
+hyle_hip_status hyle_hip_queue_completion_endpoint(const hyle_hip_queue *queue, hyle_hip_completion_endpoint *endpoint) {
+  if (endpoint == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "endpoint output is null");
+  endpoint->authority = queue != nullptr ? &kCompletionAuthority : nullptr;
+  endpoint->identity = queue;  // equality means one ordered endpoint: this queue
+  return HYLE_HIP_OK;
+}
+
+int hyle_hip_queue_can_wait_endpoint(const hyle_hip_queue *destination, hyle_hip_completion_endpoint source) {
+  if (destination == nullptr || source.authority != &kCompletionAuthority || source.identity == nullptr) return 0;
+  // what hyle_hip_queue_wait_completion accepts: completions of queues of the same device
+  return static_cast<const hyle_hip_queue *>(source.identity)->device == destination->device ? 1 : 0;
 }
 
 hyle_hip_status hyle_hip_queue_copy_async(hyle_hip_queue *queue, hyle_hip_memory_resource *destination_resource,

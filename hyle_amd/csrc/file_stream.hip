@@ -13,6 +13,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <thread>
 #include <type_traits>
@@ -51,14 +52,33 @@ struct Slot {
 
 }  // namespace
 
+struct hyle_hip_stream_ticket;
+
 struct hyle_hip_file_pipeline {
   int device = 0;
   uint32_t slot_count = 0;
   size_t slot_bytes = 0;
-  Slot slots[kMaxSlots];
+  Slot slots[kMaxSlots];  // touched by the thread of the running request only (or, idle, by the caller)
   uint32_t next_slot = 0;
   std::atomic<bool> busy{false};  // a request (on the caller's thread or behind a ticket) is running
+  std::mutex guard;                         // protects `live`
+  hyle_hip_stream_ticket *live = nullptr;   // the ticket whose thread may still use the slots
 };
+
+namespace {
+// Waits for every copy that still reads or writes a slot.  Only the thread that runs the
+// pipeline's request, or a caller of an idle pipeline, may call it.
+hyle_hip_status wait_slots(hyle_hip_file_pipeline *p) {
+  for (uint32_t s = 0; s < p->slot_count; ++s) {
+    if (!p->slots[s].in_flight) continue;
+    const hipError_t err = hipEventSynchronize(p->slots[s].drained);
+    if (err != hipSuccess) return hip_fail(err, "hipEventSynchronize");
+    p->slots[s].in_flight = false;
+  }
+  return HYLE_HIP_OK;
+}
+void end_live_ticket(hyle_hip_file_pipeline *p);
+}  // namespace
 
 extern "C" {
 
@@ -133,17 +153,17 @@ hyle_hip_status hyle_hip_file_pipeline_create(hyle_hip_context *context,
 
 hyle_hip_status hyle_hip_file_pipeline_wait(hyle_hip_file_pipeline *p) {
   if (p == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "pipeline is null");
-  for (uint32_t s = 0; s < p->slot_count; ++s) {
-    if (!p->slots[s].in_flight) continue;
-    const hipError_t err = hipEventSynchronize(p->slots[s].drained);
-    if (err != hipSuccess) return hip_fail(err, "hipEventSynchronize");
-    p->slots[s].in_flight = false;
-  }
-  return HYLE_HIP_OK;
+  // the slots belong to the running request's thread: wait for the ticket instead
+  if (p->busy.load(std::memory_order_acquire))
+    return fail(HYLE_HIP_FAILED_PRECONDITION, "the pipeline is running a request: wait for its ticket");
+  return wait_slots(p);
 }
 
 void hyle_hip_file_pipeline_destroy(hyle_hip_file_pipeline *p) {
   if (p == nullptr) return;
+  // a ticket's thread may still fill, copy from or wait for the slots: ask it to stop and let it
+  // end before anything is freed (its ticket stays valid and reports the progress it made)
+  end_live_ticket(p);
   (void)hipSetDevice(p->device);
   for (uint32_t s = 0; s < p->slot_count; ++s) {
     if (p->slots[s].in_flight) (void)hipEventSynchronize(p->slots[s].drained);
@@ -180,17 +200,33 @@ hyle_hip_status wait_slot(Slot &slot, hyle_hip_stream_result &out) {
 
 bool cancelled(const std::atomic<bool> *cancel) { return cancel != nullptr && cancel->load(std::memory_order_relaxed); }
 
+// What another thread may read of a running request: a copy of the counters, refreshed at
+// every slot boundary under a lock (the request's own counters are its thread's alone).
+struct Progress {
+  std::mutex lock;
+  hyle_hip_stream_result shown{};
+  void publish(const hyle_hip_stream_result &now) {
+    std::lock_guard<std::mutex> hold(lock);
+    shown = now;
+  }
+};
+void publish(Progress *progress, const hyle_hip_stream_result &now) {
+  if (progress != nullptr) progress->publish(now);
+}
+
 // file -> pinned slots -> device.  Ranges are packed into a slot back to back (several small
 // ranges share one, a large one takes many in turn); a slot goes to the device as soon as it is
 // full or the ranges end.  `out` is updated as the work proceeds, so another thread may read
 // the progress; a cancellation request is honoured before each slot is filled.
 hyle_hip_status run_read(hyle_hip_file_pipeline *p, int fd, const hyle_hip_read_range *ranges, uint32_t range_count,
-                         hipStream_t stream, hyle_hip_stream_result &out, const std::atomic<bool> *cancel) {
+                         hipStream_t stream, hyle_hip_stream_result &out, const std::atomic<bool> *cancel,
+                         Progress *progress) {
   hipError_t err = hipSetDevice(p->device);
   if (err != hipSuccess) return hip_fail(err, "hipSetDevice");
   uint32_t r = 0;
   size_t done_in_range = 0;
   while (r < range_count) {
+    publish(progress, out);
     if (cancelled(cancel)) return fail(HYLE_HIP_CANCELLED, "the read was cancelled");
     Slot &slot = p->slots[p->next_slot];
     hyle_hip_status status = wait_slot(slot, out);
@@ -247,7 +283,8 @@ hyle_hip_status run_read(hyle_hip_file_pipeline *p, int fd, const hyle_hip_read_
 // device -> pinned slots -> file.  Up to slot_count pieces are on their way from the device
 // while the oldest one is written to the file; pieces leave in range order.
 hyle_hip_status run_write(hyle_hip_file_pipeline *p, int fd, const hyle_hip_write_range *ranges, uint32_t range_count,
-                          hipStream_t stream, hyle_hip_stream_result &out, const std::atomic<bool> *cancel) {
+                          hipStream_t stream, hyle_hip_stream_result &out, const std::atomic<bool> *cancel,
+                          Progress *progress) {
   hipError_t err = hipSetDevice(p->device);
   if (err != hipSuccess) return hip_fail(err, "hipSetDevice");
   hyle_hip_status status = HYLE_HIP_OK;
@@ -291,6 +328,7 @@ hyle_hip_status run_write(hyle_hip_file_pipeline *p, int fd, const hyle_hip_writ
       if (p->slots[s].in_flight && hipEventSynchronize(p->slots[s].drained) == hipSuccess) p->slots[s].in_flight = false;
   };
   while (r < range_count || filled != 0) {
+    publish(progress, out);
     if (cancelled(cancel)) {
       drain_in_flight();
       return fail(HYLE_HIP_CANCELLED, "the write was cancelled");
@@ -355,14 +393,17 @@ bool claim(hyle_hip_file_pipeline *p) {
 
 }  // namespace
 
-// A request running on a thread of its own.  `result` is written by that thread only, in
-// whole fields; readers take a snapshot that may be a moment old.
+// A request running on a thread of its own.  `result` is that thread's alone until `ended`;
+// while it runs, readers get `progress.shown`, a copy refreshed at every slot boundary.
 struct hyle_hip_stream_ticket {
-  hyle_hip_file_pipeline *pipeline = nullptr;
+  // null once the pipeline has been destroyed or has taken a later request
+  std::atomic<hyle_hip_file_pipeline *> pipeline{nullptr};
   std::thread worker;
+  std::mutex join_lock;  // the worker is joined once, by whichever of wait / release / pipeline destroy comes first
   std::atomic<bool> cancel{false};
   std::atomic<bool> ended{false};
   hyle_hip_stream_result result{};
+  Progress progress;
   std::vector<hyle_hip_read_range> reads;
   std::vector<hyle_hip_write_range> writes;
   char error_text[320] = "";
@@ -373,18 +414,42 @@ struct hyle_hip_stream_ticket {
 
 namespace {
 
+void join_worker(hyle_hip_stream_ticket *t) {
+  std::lock_guard<std::mutex> hold(t->join_lock);
+  if (t->worker.joinable()) t->worker.join();
+}
+
 void ticket_main(hyle_hip_stream_ticket *t) {
+  hyle_hip_file_pipeline *p = t->pipeline.load();  // alive until this thread has been joined
   hyle_hip_status status;
   if (t->is_write)
-    status = run_write(t->pipeline, t->fd, t->writes.data(), (uint32_t)t->writes.size(), t->stream, t->result, &t->cancel);
+    status = run_write(p, t->fd, t->writes.data(), (uint32_t)t->writes.size(), t->stream, t->result, &t->cancel, &t->progress);
   else
-    status = run_read(t->pipeline, t->fd, t->reads.data(), (uint32_t)t->reads.size(), t->stream, t->result, &t->cancel);
-  if (status == HYLE_HIP_OK && !t->is_write) status = hyle_hip_file_pipeline_wait(t->pipeline);  // the copies too
+    status = run_read(p, t->fd, t->reads.data(), (uint32_t)t->reads.size(), t->stream, t->result, &t->cancel, &t->progress);
+  // the copies too; after a failure or a cancellation as well, so that no copy still touches a
+  // slot when the request reports its end
+  const hyle_hip_status drained = wait_slots(p);
+  if (status == HYLE_HIP_OK) status = drained;
   std::snprintf(t->error_text, sizeof t->error_text, "%s", hyle_hip_last_error());  // this thread's text
   t->result.status = status;
   t->result.complete = 1;
-  t->pipeline->busy.store(false);
+  // the ticket reports its end before the pipeline takes the next request
   t->ended.store(true, std::memory_order_release);
+  p->busy.store(false, std::memory_order_release);
+}
+
+// hyle_hip_file_pipeline_destroy: the live ticket's thread must be gone before the slots are.
+void end_live_ticket(hyle_hip_file_pipeline *p) {
+  hyle_hip_stream_ticket *t = nullptr;
+  {
+    std::lock_guard<std::mutex> hold(p->guard);
+    t = p->live;
+    p->live = nullptr;
+  }
+  if (t == nullptr) return;
+  t->cancel.store(true, std::memory_order_relaxed);
+  join_worker(t);
+  t->pipeline.store(nullptr);
 }
 
 template <class Range>
@@ -409,7 +474,12 @@ hyle_hip_status submit(hyle_hip_file_pipeline *p, int fd, const Range *ranges, u
   try {
     if constexpr (std::is_same<Range, hyle_hip_write_range>::value) t->writes.assign(ranges, ranges + range_count);
     else t->reads.assign(ranges, ranges + range_count);
+    std::lock_guard<std::mutex> hold(p->guard);
+    // an earlier ticket has ended (the pipeline was idle): it no longer needs the slots, and must
+    // not look for this pipeline when it is released after the pipeline is gone
+    if (p->live != nullptr) p->live->pipeline.store(nullptr);
     t->worker = std::thread(ticket_main, t);
+    p->live = t;
   } catch (...) {
     p->busy.store(false);
     delete t;
@@ -435,7 +505,7 @@ hyle_hip_status hyle_hip_file_pipeline_read(hyle_hip_file_pipeline *p, int fd, c
   if (status == HYLE_HIP_OK && !claim(p))
     status = fail(HYLE_HIP_FAILED_PRECONDITION, "the pipeline is running another request");
   else if (status == HYLE_HIP_OK) {
-    status = run_read(p, fd, ranges, range_count, static_cast<hipStream_t>(stream_handle), out, nullptr);
+    status = run_read(p, fd, ranges, range_count, static_cast<hipStream_t>(stream_handle), out, nullptr, nullptr);
     p->busy.store(false);
   }
   out.status = status;
@@ -455,7 +525,7 @@ hyle_hip_status hyle_hip_file_pipeline_write(hyle_hip_file_pipeline *p, int fd, 
   if (status == HYLE_HIP_OK && !claim(p))
     status = fail(HYLE_HIP_FAILED_PRECONDITION, "the pipeline is running another request");
   else if (status == HYLE_HIP_OK) {
-    status = run_write(p, fd, ranges, range_count, static_cast<hipStream_t>(stream_handle), out, nullptr);
+    status = run_write(p, fd, ranges, range_count, static_cast<hipStream_t>(stream_handle), out, nullptr, nullptr);
     p->busy.store(false);
   }
   out.status = status;
@@ -476,18 +546,23 @@ hyle_hip_status hyle_hip_file_pipeline_submit_write(hyle_hip_file_pipeline *p, i
 
 hyle_hip_status hyle_hip_stream_ticket_result(hyle_hip_stream_ticket *ticket, hyle_hip_stream_result *result) {
   if (ticket == nullptr || result == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "null argument");
-  const bool ended = ticket->ended.load(std::memory_order_acquire);
-  *result = ticket->result;
-  if (!ended) {  // a snapshot of a running request: its status is not known yet
-    result->status = HYLE_HIP_OK;
-    result->complete = 0;
+  if (ticket->ended.load(std::memory_order_acquire)) {
+    *result = ticket->result;
+    return HYLE_HIP_OK;
   }
+  {  // a running request: the progress it last published; its status is not known yet
+    std::lock_guard<std::mutex> hold(ticket->progress.lock);
+    *result = ticket->progress.shown;
+  }
+  result->total_ranges = (uint32_t)(ticket->is_write ? ticket->writes.size() : ticket->reads.size());
+  result->status = HYLE_HIP_OK;
+  result->complete = 0;
   return HYLE_HIP_OK;
 }
 
 hyle_hip_status hyle_hip_stream_ticket_wait(hyle_hip_stream_ticket *ticket, hyle_hip_stream_result *result) {
   if (ticket == nullptr) return fail(HYLE_HIP_INVALID_ARGUMENT, "ticket is null");
-  if (ticket->worker.joinable()) ticket->worker.join();
+  join_worker(ticket);
   if (result != nullptr) *result = ticket->result;
   if (ticket->result.status != HYLE_HIP_OK) return fail(ticket->result.status, "%s", ticket->error_text);
   return HYLE_HIP_OK;
@@ -500,7 +575,11 @@ void hyle_hip_stream_ticket_request_cancel(hyle_hip_stream_ticket *ticket) {
 void hyle_hip_stream_ticket_release(hyle_hip_stream_ticket *ticket) {
   if (ticket == nullptr) return;
   ticket->cancel.store(true, std::memory_order_relaxed);
-  if (ticket->worker.joinable()) ticket->worker.join();
+  join_worker(ticket);
+  if (hyle_hip_file_pipeline *p = ticket->pipeline.load()) {  // still there: it must forget this ticket
+    std::lock_guard<std::mutex> hold(p->guard);
+    if (p->live == ticket) p->live = nullptr;
+  }
   delete ticket;
 }
 

@@ -239,7 +239,7 @@ __global__ __launch_bounds__(kBlockThreads) void categorical_rows(const void *lo
   __shared__ float joint[kBlockThreads / kWaveLanes];
   __shared__ double wave_totals[kBlockThreads / kWaveLanes];
   __shared__ Crossing crossing;
-  __shared__ uint32_t found;
+  __shared__ uint32_t found, claim;
   constexpr float kInfinity = __builtin_huge_valf();
   const uint32_t row = blockIdx.x;
   const CategoricalTile *mine = parts + (size_t)row * tiles;
@@ -267,9 +267,19 @@ __global__ __launch_bounds__(kBlockThreads) void categorical_rows(const void *lo
   // the 52-bit midpoint is exact in double at both ends (sampling.cc:155-158)
   const double uniform = ((double)draw.x0 * 0x1p20 + (double)(draw.x1 >> 12) + 0.5) * 0x1p-52;
   const double threshold = total * uniform;
-  if (threadIdx.x == 0) crossing.tile = 0xFFFFFFFFu;
+  if (threadIdx.x == 0) {
+    crossing.tile = 0xFFFFFFFFu;
+    claim = 0xFFFFFFFFu;
+  }
   __syncthreads();
-  if (!(before > threshold) && through > threshold) {  // the first tile whose running mass exceeds the threshold is here
+  // The scan's running sums are associated differently from lane to lane, so they need not be
+  // monotone in their last bit: a thread without mass may see the threshold between its equal
+  // `before` and `through`, and two neighbours may both see it.  Only threads with mass of their
+  // own may hold the crossing, and the lowest of them answers.
+  const bool candidate = own > 0 && !(before > threshold) && through > threshold;
+  if (candidate) atomicMin(&claim, threadIdx.x);
+  __syncthreads();
+  if (candidate && claim == threadIdx.x) {  // the first tile whose running mass exceeds the threshold is here
     double running = before;
     uint32_t tile = 0xFFFFFFFFu, last_with_mass = 0xFFFFFFFFu;
     for (uint32_t t = begin; t < end; ++t) {
@@ -285,7 +295,9 @@ __global__ __launch_bounds__(kBlockThreads) void categorical_rows(const void *lo
       tile = last_with_mass;
       running = threshold;
     }
-    crossing = Crossing{threshold - running, tile, mine[tile].maximum, scale_of(tile)};
+    // (a run without mass cannot get here; if it did, the crossing stays unset and the row's last
+    // maximum answers below, never an index outside the tiles)
+    if (tile != 0xFFFFFFFFu) crossing = Crossing{threshold - running, tile, mine[tile].maximum, scale_of(tile)};
   }
   __syncthreads();
   if (crossing.tile == 0xFFFFFFFFu) {

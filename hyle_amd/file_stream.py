@@ -49,8 +49,10 @@ class StreamWriteRange:  # include/hyle/compute/file_stream.h:92-105 (StreamWrit
 class StreamTicket:
     """include/hyle/compute/file_stream.h:158-180: a request running on a thread of the pipeline."""
 
-    def __init__(self, handle: int):
+    def __init__(self, handle: int, pipeline: "Optional[FileResourcePipeline]" = None):
         self._handle: Optional[int] = handle
+        # the request's thread uses the pipeline's staging: the pipeline lives as long as its ticket
+        self._pipeline = pipeline
 
     @staticmethod
     def _snapshot(c_result) -> StreamResult:
@@ -78,6 +80,7 @@ class StreamTicket:
         if self._handle:
             capi.load().hyle_hip_stream_ticket_release(self._handle)
             self._handle = None
+        self._pipeline = None
 
     def __del__(self):
         try:
@@ -153,7 +156,7 @@ class FileResourcePipeline:
         handle = C.c_void_p()
         _check(capi.load().hyle_hip_file_pipeline_submit_read(self._handle, fd, c_ranges, len(ranges), stream,
                                                               C.byref(handle)))
-        return StreamTicket(handle.value)
+        return self._ticket(handle.value)
 
     def submit_write(self, fd: int, ranges: Sequence["StreamWriteRange"], stream: int) -> "StreamTicket":
         c_ranges = (capi.WriteRangeC * max(len(ranges), 1))(*[capi.WriteRangeC(r.source, r.file_offset, r.bytes)
@@ -161,12 +164,17 @@ class FileResourcePipeline:
         handle = C.c_void_p()
         _check(capi.load().hyle_hip_file_pipeline_submit_write(self._handle, fd, c_ranges, len(ranges), stream,
                                                                C.byref(handle)))
-        return StreamTicket(handle.value)
+        return self._ticket(handle.value)
+
+    def _ticket(self, handle: int) -> "StreamTicket":
+        return StreamTicket(handle, self)
 
     def wait(self) -> None:
         _check(capi.load().hyle_hip_file_pipeline_wait(self._handle))
 
     def close(self) -> None:
+        """Ends a request still running behind a ticket (it is cancelled; the ticket keeps its
+        progress and stays usable), then frees the staging."""
         if self._handle:
             capi.load().hyle_hip_file_pipeline_destroy(self._handle)
             self._handle = None

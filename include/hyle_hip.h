@@ -357,7 +357,10 @@ HYLE_HIP_API int hyle_hip_plan_device_status_offset(const hyle_hip_plan *plan, s
  * the array is refused with RESOURCE_EXHAUSTED.  All calls on one device share the one array:
  * calls that may overlap on a device (different streams, different threads) race, so serialise
  * them on one stream or use hyle_hip_plan_launch with separate workspaces.  Results are those of
- * hyle_hip_plan_launch bit for bit. */
+ * hyle_hip_plan_launch bit for bit.  The device verdict of a checked Gather or a Categorical
+ * launched this way lives in that shared array too: read it with
+ * hyle_hip_plan_device_status(plan, NULL, stream) before the next static launch on the device,
+ * which may overwrite it (the next launch of any plan with a workspace, even on the same stream). */
 HYLE_HIP_API hyle_hip_status hyle_hip_plan_launch_static(const hyle_hip_plan *plan,
                                                          const void *const *inputs, uint32_t input_count,
                                                          void *const *outputs, uint32_t output_count,

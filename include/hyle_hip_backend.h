@@ -36,6 +36,10 @@ HYLE_HIP_API hyle_hip_status hyle_hip_backend_device_count(size_t *count);
 HYLE_HIP_API hyle_hip_status hyle_hip_backend_device_properties(size_t index,
                                                                 hyle_hip_device_properties *properties);
 
+/* BackendVTable::same_device (src/compute_backend_cuda/cuda_backend.cc:803-806): 1 when both
+ * indices name an existing device and it is the same one (a device is its ordinal), else 0. */
+HYLE_HIP_API int hyle_hip_backend_same_device(size_t left, size_t right);
+
 /* ---- memory resources (include/hyle/mem/resource.h:108-151) ------------------------- */
 /* MemoryProperty bits (include/hyle/mem/resource.h:19-33). */
 enum {
@@ -126,6 +130,42 @@ HYLE_HIP_API void hyle_hip_completion_release(hyle_hip_completion *completion);
  * finished.  The host does not wait. */
 HYLE_HIP_API hyle_hip_status hyle_hip_queue_wait_completion(hyle_hip_queue *queue,
                                                             hyle_hip_completion *completion);
+
+/* TransferMode / TransferProperties (include/hyle/compute/transfer.h:19-30). */
+enum { HYLE_HIP_TRANSFER_IMMEDIATE = 0, HYLE_HIP_TRANSFER_QUEUED_DIRECT = 1 };
+typedef struct hyle_hip_transfer_properties {
+  uint32_t mode; /* HYLE_HIP_TRANSFER_* */
+  uint32_t peer; /* always 0: one device */
+} hyle_hip_transfer_properties;
+/* BackendVTable::transfer_properties (cuda_backend.cc:1100-1115): the route a copy between two
+ * resources would take on `queue`, asked cold before the copies are enqueued.  Storage of the
+ * queue's own device -- device memory or pinned host memory, on either side -- travels as one
+ * stream-ordered copy (QUEUED_DIRECT, no peer).  Anything else is UNIMPLEMENTED: no hidden
+ * staging and no host wait is passed off as an asynchronous copy.  The same admission as
+ * hyle_hip_queue_copy_async. */
+HYLE_HIP_API hyle_hip_status hyle_hip_queue_transfer_properties(const hyle_hip_queue *queue,
+                                                                const hyle_hip_memory_resource *destination,
+                                                                const hyle_hip_memory_resource *source,
+                                                                hyle_hip_transfer_properties *properties);
+
+/* CompletionEndpoint (include/hyle/compute/completion.h; src/compute/backend_internal.h:54-62):
+ * who emits a queue's completions.  `authority` is one address for every queue of this library,
+ * `identity` the queue: equal endpoints are one ordered queue, not merely queues whose events can
+ * meet. */
+typedef struct hyle_hip_completion_endpoint {
+  const void *authority;
+  const void *identity;
+} hyle_hip_completion_endpoint;
+/* BackendVTable::completion_endpoint (cuda_backend.cc:1214-1226): cold; a null queue gives the
+ * invalid endpoint {NULL, NULL}. */
+HYLE_HIP_API hyle_hip_status hyle_hip_queue_completion_endpoint(const hyle_hip_queue *queue,
+                                                                hyle_hip_completion_endpoint *endpoint);
+/* BackendVTable::can_wait_endpoint (cuda_backend.cc:1228-1239): 1 commits
+ * hyle_hip_queue_wait_completion on `destination` to accepting a pending completion emitted by
+ * `source` without a host wait (a queue of this library on the same device); 0 -- another
+ * library's endpoint, an invalid one, another device -- leaves the caller to wait on the host. */
+HYLE_HIP_API int hyle_hip_queue_can_wait_endpoint(const hyle_hip_queue *destination,
+                                                  hyle_hip_completion_endpoint source);
 
 /* BackendVTable::copy_async (cuda_backend.cc:1117-1135): `bytes` from `source` (inside an
  * allocation of `source_resource`) to `destination` (inside one of

@@ -104,7 +104,11 @@ typedef struct hyle_hip_stream_ticket hyle_hip_stream_ticket;
 HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_create(hyle_hip_context *context,
                                                            const hyle_hip_file_stream_options *options,
                                                            hyle_hip_file_pipeline **pipeline);
-/* Waits for the slots still in flight, then frees the staging. */
+/* Frees the staging.  A request still running behind a ticket is asked to cancel and its
+ * thread has ended (no copy touches a slot any more) before anything is freed; the ticket stays
+ * valid, reports CANCELLED (or what it had reached) with its progress, and must still be
+ * released.  Slots left in flight by a finished request are waited for.  Must not run
+ * concurrently with another call on this pipeline or with the release of its ticket. */
 HYLE_HIP_API void hyle_hip_file_pipeline_destroy(hyle_hip_file_pipeline *pipeline);
 
 /* Read every range from the open file `fd` (pread: the file position is not
@@ -119,7 +123,8 @@ HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_read(hyle_hip_file_pipeline 
                                                          uint32_t range_count, void *stream,
                                                          hyle_hip_stream_result *result);
 /* StreamTicket::wait (include/hyle/compute/file_stream.h:171): block until
- * every copy this pipeline enqueued has finished. */
+ * every copy this pipeline enqueued has finished.  While a request runs behind a ticket the
+ * slots belong to its thread: FAILED_PRECONDITION, wait for the ticket instead. */
 HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_wait(hyle_hip_file_pipeline *pipeline);
 
 /* The write direction (FileResourcePipeline::write, include/hyle/compute/file_stream.h:205-206;
@@ -138,7 +143,9 @@ HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_write(hyle_hip_file_pipeline
  * run on a thread of the pipeline; the call returns at once with a ticket.  One request
  * (with or without a ticket) runs on a pipeline at a time: a second one is
  * FAILED_PRECONDITION.  The ranges are copied; the file must stay open and the device
- * memory alive until the ticket has ended. */
+ * memory alive until the ticket has ended.  Order of teardown: release the ticket, then destroy
+ * the pipeline; a pipeline destroyed first ends the ticket's request itself (see
+ * hyle_hip_file_pipeline_destroy), and the ticket is then released afterwards. */
 HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_submit_read(hyle_hip_file_pipeline *pipeline, int fd,
                                                                 const hyle_hip_read_range *ranges,
                                                                 uint32_t range_count, void *stream,
@@ -148,7 +155,7 @@ HYLE_HIP_API hyle_hip_status hyle_hip_file_pipeline_submit_write(hyle_hip_file_p
                                                                  uint32_t range_count, void *stream,
                                                                  hyle_hip_stream_ticket **ticket);
 /* StreamTicket::result: the progress so far, without waiting (`complete` says whether the
- * request has ended). */
+ * request has ended).  Of a running request this is the state at its last slot boundary. */
 HYLE_HIP_API hyle_hip_status hyle_hip_stream_ticket_result(hyle_hip_stream_ticket *ticket,
                                                            hyle_hip_stream_result *result);
 /* StreamTicket::wait: block until the request has ended and, for a read, until its copies

@@ -149,6 +149,53 @@ def test_a_queue_waits_for_another_queues_completion():
     pinned.close()
 
 
+def test_endpoints_say_which_completions_a_queue_may_wait_for_and_which_copies_are_direct():
+    """BackendVTable::completion_endpoint / can_wait_endpoint / transfer_properties / same_device
+    (src/compute/backend_internal.h:22-23,45-47,57-62): Graph asks them cold, before it lets one
+    queue wait for another's completion without a host wait, or records a copy as queue-ordered."""
+    ctx = context()
+    device, pinned = hb.MemoryResource(ctx, hb.MemoryKind.kDevice), hb.MemoryResource(ctx, hb.MemoryKind.kPinnedHost)
+    producer, consumer = hb.Queue(ctx), hb.Queue(ctx)
+    note("backend: endpoints of two queues of one device")
+    own, other = consumer.completion_endpoint(), producer.completion_endpoint()
+    assert own.valid() and other.valid()
+    assert own.authority == other.authority and own.identity != other.identity   # one library, two ordered queues
+    assert consumer.completion_endpoint() == own                                  # stable
+    assert consumer.can_wait_endpoint(other) and consumer.can_wait_endpoint(own) and producer.can_wait_endpoint(own)
+    # a foreign endpoint (another authority), an invalid one, and one without identity are refused
+    assert not consumer.can_wait_endpoint(hb.CompletionEndpoint(other.authority + 8, other.identity))
+    assert not consumer.can_wait_endpoint(hb.CompletionEndpoint())
+    assert not consumer.can_wait_endpoint(hb.CompletionEndpoint(other.authority, 0))
+    # what can_wait_endpoint promised holds: the consumer accepts the producer's pending completion
+    size = 32 << 20
+    d_src, h_out = device.allocate(size), pinned.allocate(4096)
+    producer.begin_sequence()
+    for value in (9, 8, 7):
+        producer.fill_async(device, d_src, value, size)
+    filled = producer.finish_sequence()
+    consumer.wait_completion(filled)
+    consumer.copy_async(pinned, h_out, device, d_src + size - 4096, 4096)
+    consumer.drain()
+    assert np.all(host_view(h_out, 4096) == 7)
+    filled.release()
+    note("backend: transfer properties of every resource pair")
+    for destination, source in ((device, device), (device, pinned), (pinned, device), (pinned, pinned)):
+        route = consumer.transfer_properties(destination, source)
+        assert route.mode == hb.TransferMode.kQueuedDirect and not route.peer
+    for destination, source in ((device, None), (None, pinned)):
+        with pytest.raises(hc.StatusError) as unsupported:
+            consumer.transfer_properties(destination, source)
+        assert unsupported.value.is_unimplemented()
+    assert hb.same_device(0, 0)
+    assert not hb.same_device(0, hb.device_count())       # an index that names no device
+    device.deallocate(d_src)
+    pinned.deallocate(h_out)
+    for queue in (producer, consumer):
+        queue.close()
+    device.close()
+    pinned.close()
+
+
 def test_provider_launches_on_a_backend_queue():
     """The stream a provider enqueues on is the queue's (cuda::stream(sequence) in the reference)."""
     ctx = context()
@@ -229,13 +276,15 @@ def test_tickets_report_progress_and_cancellation_keeps_what_was_done():
         torch.cuda.synchronize()
         ticket = pipeline.submit_read(fd, [fs.StreamReadRange(0, target.data_ptr(), total)], stream_handle())
         ticket.request_cancel()
-        with pytest.raises(hc.StatusError) as stopped:
+        try:  # the request may also have finished before it saw the cancellation: both are valid ends
             ticket.wait()
+            assert ticket.last_result.copied_bytes == total and ticket.last_result.ready_ranges == 1
+        except hc.StatusError as stopped:
+            assert stopped.code == hc.StatusCode.kCancelled
+            assert ticket.last_result.complete == 1 and ticket.last_result.status == capi.CANCELLED
+            assert ticket.last_result.copied_bytes < total and ticket.last_result.copied_bytes % (64 * 1024) == 0
+            assert ticket.last_result.ready_ranges == 0
         progress = ticket.last_result
-        if stopped.value.code == hc.StatusCode.kCancelled:
-            assert progress.complete == 1 and progress.status == capi.CANCELLED
-            assert progress.copied_bytes < total and progress.copied_bytes % (64 * 1024) == 0
-            assert progress.ready_ranges == 0
         torch.cuda.synchronize()
         got = target.cpu().numpy()
         assert np.array_equal(got[:progress.copied_bytes], payload[:progress.copied_bytes])   # what was done stands
@@ -263,6 +312,58 @@ def test_tickets_report_progress_and_cancellation_keeps_what_was_done():
         pipeline.read(fd, [fs.StreamReadRange(total - 4096, small.data_ptr(), 4096)], stream_handle())
         pipeline.wait()
         pipeline.close()
+    finally:
+        os.close(fd)
+        os.unlink(path)
+
+
+def test_a_pipeline_closed_under_a_running_ticket_ends_the_request_first():
+    """Destroying the pipeline while a ticket's thread still fills and drains the pinned slots must
+    stop that thread before the slots are freed; the ticket stays valid, reports where it stopped,
+    and what it copied stands.  While the request runs, the pipeline's own wait is refused."""
+    rng = np.random.default_rng(1903)
+    total = 64 * 1024 * 1024
+    payload = rng.integers(0, 256, total, dtype=np.uint8)
+    with tempfile.NamedTemporaryFile(delete=False) as handle:
+        handle.write(payload.tobytes())
+        path = handle.name
+    fd = os.open(path, os.O_RDWR)
+    try:
+        for direction in ("read", "write"):
+            pipeline = fs.FileResourcePipeline.create(context(), fs.FileStreamOptions(2, 64 * 1024))
+            target = torch.zeros(total, dtype=torch.uint8, device=DEVICE)
+            torch.cuda.synchronize()
+            note(f"file pipeline: closed while a {direction} runs behind a ticket")
+            if direction == "read":
+                ticket = pipeline.submit_read(fd, [fs.StreamReadRange(0, target.data_ptr(), total)], stream_handle())
+            else:
+                ticket = pipeline.submit_write(fd, [fs.StreamWriteRange(target.data_ptr(), 0, total)], stream_handle())
+            try:
+                pipeline.wait()
+                assert ticket.result().complete == 1   # only an ended request leaves the pipeline to its caller
+            except hc.StatusError as refused:
+                assert refused.code == hc.StatusCode.kFailedPrecondition
+            pipeline.close()                            # the request's thread has ended when this returns
+            seen = ticket.result()
+            assert seen.complete == 1
+            try:
+                ticket.wait()
+            except hc.StatusError as stopped:
+                assert stopped.code == hc.StatusCode.kCancelled
+            done = ticket.last_result
+            assert done.complete == 1 and done.copied_bytes <= total
+            if direction == "read":
+                torch.cuda.synchronize()
+                got = target.cpu().numpy()
+                assert np.array_equal(got[:done.copied_bytes], payload[:done.copied_bytes])
+                assert not got[done.copied_bytes:].any()
+            ticket.close()                              # after its pipeline: must not look for it
+        # and the other order: the ticket released first, then the pipeline
+        pipeline = fs.FileResourcePipeline.create(context(), fs.FileStreamOptions(2, 64 * 1024))
+        ticket = pipeline.submit_read(fd, [fs.StreamReadRange(0, target.data_ptr(), total)], stream_handle())
+        ticket.close()
+        pipeline.close()
+        torch.cuda.synchronize()
     finally:
         os.close(fd)
         os.unlink(path)

@@ -522,3 +522,12 @@ def test_backend_and_stream_calls_reject_bad_arguments_without_a_device():
     lib.hyle_hip_stream_ticket_release(None)
     lib.hyle_hip_completion_release(None)
     assert lib.hyle_hip_status_name(capi.CANCELLED) == b"CANCELLED"
+    # endpoints and transfer routes: a null queue has the invalid endpoint, which nobody may wait for
+    endpoint = capi.CompletionEndpointC(1, 1)
+    assert lib.hyle_hip_queue_completion_endpoint(None, C.byref(endpoint)) == capi.OK
+    assert endpoint.authority is None and endpoint.identity is None
+    assert lib.hyle_hip_queue_completion_endpoint(None, None) == capi.INVALID_ARGUMENT
+    assert lib.hyle_hip_queue_can_wait_endpoint(None, endpoint) == 0
+    route = capi.TransferPropertiesC()
+    assert lib.hyle_hip_queue_transfer_properties(None, None, None, C.byref(route)) == capi.INVALID_ARGUMENT
+    assert lib.hyle_hip_backend_same_device(10 ** 6, 10 ** 6) == 0
