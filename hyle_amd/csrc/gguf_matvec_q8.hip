@@ -749,6 +749,7 @@ template <> struct BlocksGeometry<1> {  // Q6_K
 template <> struct BlocksGeometry<2> {  // Q8_0: a run of 256 values is eight blocks of 34 bytes
   static constexpr uint32_t kRunBytes = 272, kActivationBlock = 32;
 };
+constexpr int kBlocksDepth = 4;  // steps of a wave whose bytes are in flight
 template <int kKind> struct BlocksStep {
   static constexpr uint32_t kBytes = 4 * BlocksGeometry<kKind>::kRunBytes;   // 1024 values of a row
   static constexpr int kLoads = (int)((kBytes + 14 + 15) / 16 + kWaveLanes - 1) / kWaveLanes;
@@ -770,10 +771,22 @@ template <> struct RunDot<0> {  // lane u: chunk u / 4, quant bytes 8 (u % 4) ..
     lds_words<2>(slot, at + 16 + 32 * chunk + 8 * (u % 4), quants);
     d = f16_to_f32((uint16_t)head[0]);
     dmin = f16_to_f32((uint16_t)(head[0] >> 16));
-    sc_low = q4k_six_bits(head[1], head[2], head[3], 2 * chunk, false);
-    sc_high = q4k_six_bits(head[1], head[2], head[3], 2 * chunk + 1, false);
-    m_low = q4k_six_bits(head[1], head[2], head[3], 2 * chunk, true);
-    m_high = q4k_six_bits(head[1], head[2], head[3], 2 * chunk + 1, true);
+    // sub-blocks 2 c and 2 c + 1 sit in one half of the table (both below 4 or both from 4 on), in
+    // neighbouring bytes: one branch per lane, the same in every step
+    const uint32_t shift = 16 * (chunk % 2);
+    if (chunk < 2) {  // six bits whole: sc in scales[j], m in scales[j + 4]
+      const uint32_t sc = head[1] >> shift, mn = head[2] >> shift;
+      sc_low = (int)(sc & 63u);
+      sc_high = (int)((sc >> 8) & 63u);
+      m_low = (int)(mn & 63u);
+      m_high = (int)((mn >> 8) & 63u);
+    } else {  // four bits in a nibble of scales[j + 4], two more in the top of scales[j - 4] (sc) or scales[j] (m)
+      const uint32_t main = head[3] >> shift, sc_top = head[1] >> shift, m_top = head[2] >> shift;
+      sc_low = (int)((main & 15u) | ((sc_top >> 2) & 48u));
+      sc_high = (int)(((main >> 8) & 15u) | ((sc_top >> 10) & 48u));
+      m_low = (int)(((main >> 4) & 15u) | ((m_top >> 2) & 48u));
+      m_high = (int)(((main >> 12) & 15u) | ((m_top >> 10) & 48u));
+    }
 #pragma unroll
     for (int w = 0; w < 2; ++w) {
       low[w] = quants[w] & 0x0F0F0F0Fu;
@@ -845,8 +858,9 @@ template <> struct RunDot<2> {  // lane u: block u / 2 of the run's eight, quant
 };
 
 // staged: int8 codes [m][k], then f32 scales [m][k / activation block].  kM: activation rows
-// served at once (rows past m repeat the last one and are not stored).
-template <int kKind, class TX, int kM>
+// served at once (rows past m repeat the last one and are not stored).  kVectorX: x starts on a
+// 16-byte boundary, so its rows (K is a multiple of 32) are read as whole vectors.
+template <int kKind, class TX, int kM, bool kVectorX>
 __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_blocks(const unsigned char *weights, const void *x, void *y,
                                                                        uint32_t rows, uint64_t row_stride, uint32_t k,
                                                                        uint32_t m) {
@@ -862,64 +876,30 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_blocks(const uns
   const uint32_t lane = threadIdx.x % kWaveLanes;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
 
-  // ---- the activation rows, quantised once per block ------------------------------------------
-  for (uint32_t r = 0; r < m; ++r) {
-    for (uint32_t base = 0; base < k; base += kBlockThreads * 8) {
-      const uint32_t p = base + threadIdx.x * 8;
-      const bool inside = p < k;  // the same for all lanes that share an activation block
-      float values[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) values[e] = inside ? Traits<TX>::load(x, (size_t)r * k + p + e) : 0.0f;
-      LaneMax mine{0.0f, 0.0f, 0u};
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {  // positions rise with e, so ">" keeps the first
-        const float magnitude = __builtin_fabsf(values[e]);
-        if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], p + e};
-      }
-      if (mine.magnitude == 0.0f) mine.position = 0xFFFFFFFFu;  // no candidate: any lane with one goes first
-      const LaneMax top = block_largest<kQuantiseLanes>(mine);
-      float factor = 0.0f, stored = 0.0f;
-      if (top.magnitude != 0.0f) {
-        if constexpr (kKind == 2) {
-          stored = f16_to_f32(f32_to_f16(top.magnitude / 127.0f));
-          factor = 127.0f / top.magnitude;
-        } else {
-          factor = -127.0f / top.value;
-          stored = 1.0f / factor;
-        }
-      }
-      uint32_t words[2] = {0u, 0u};
-      if (top.magnitude != 0.0f) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) words[e / 4] |= code_of(values[e] * factor) << (8 * (e % 4));
-      }
-      if (inside) {
-        uint32_t *to = reinterpret_cast<uint32_t *>(codes + (size_t)r * k + p);
-        to[0] = words[0];
-        to[1] = words[1];
-        if (p % kActivationBlock == 0) scales[r * activation_blocks + p / kActivationBlock] = stored;
-      }
-    }
-  }
-  __syncthreads();
-
-  // ---- the weight rows ----------------------------------------------------------------------
+  // ---- what the wave walks: its rows, 1024 values (a step) at a time ---------------------------
   const uint32_t stride = gridDim.x * kWavesPerBlock;
   const uint32_t first = blockIdx.x * kWavesPerBlock + wave;
-  if (first >= rows) return;  // no barrier follows
   unsigned char *slot = slots[wave];
   const uint32_t runs = (k + 255) / 256;           // runs of 256 values in a row (the last one of a Q8_0 row may be short)
   const uint32_t steps = (runs + 3) / 4;
   const uint64_t row_bytes = (uint64_t)(k / kActivationBlock) * (kKind == 2 ? 34u : Geometry::kRunBytes);
   const uint32_t run = lane / 16, u = lane % 16;
-  if (steps == 0) {  // K = 0: every product is an empty sum
-    for (uint32_t row = first; row < rows; row += stride)
-      if (lane < m) Traits<TX>::store(y, (size_t)lane * rows + row, 0.0f);
-    return;
-  }
+  const uint32_t own_rows = first < rows ? (rows - first + stride - 1) / stride : 0u;
+  const uint64_t segments = (uint64_t)own_rows * steps;  // (row, step) pairs of this wave, in order
 
-  // the aligned 16-byte vectors that cover step `step` of row `row`; lanes past them repeat the last one
-  auto load_step = [&](uint32_t row, uint32_t step, u32x4 (&into)[Step::kLoads], uint32_t *shift) {
+  // The aligned 16-byte vectors that cover one step of one row; lanes past them repeat the last
+  // one.  The stream of loads runs kBlocksDepth steps ahead of the stream of decodes; past the
+  // wave's last step it reads the wave's first one again, a valid address whose bytes go unused.
+  uint32_t load_row = first, load_step = 0;
+  uint64_t loaded = 0;
+  auto next_load = [&](u32x4 (&into)[Step::kLoads], uint32_t *shift) {
+    const bool live = loaded < segments;
+    const uint32_t row = live ? load_row : first, step = live ? load_step : 0u;
+    ++loaded;
+    if (++load_step == steps) {
+      load_step = 0;
+      load_row += stride;
+    }
     const uint64_t begin = (uint64_t)row * row_stride + (uint64_t)step * Step::kBytes;
     const uint64_t left = row_bytes - (uint64_t)step * Step::kBytes;
     const uint32_t bytes = left < Step::kBytes ? (uint32_t)left : Step::kBytes;
@@ -934,23 +914,101 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_blocks(const uns
     }
     *shift = off;
   };
-
-  u32x4 ring[Step::kLoads];
-  uint32_t shift = 0;
-  load_step(first, 0, ring, &shift);
-  for (uint32_t row = first; row < rows; row += stride) {
-    float totals[kM] = {};
-    for (uint32_t step = 0; step < steps; ++step) {
+  u32x4 ring[kBlocksDepth][Step::kLoads];
+  uint32_t shifts[kBlocksDepth] = {};
+  if (segments != 0) {  // the wave's first steps are on their way while the block quantises the activations
 #pragma unroll
-      for (int i = 0; i < Step::kLoads; ++i) *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = ring[i];
-      const uint32_t at = shift + run * Geometry::kRunBytes;
-      {
-        // the next step of this row, the first of the wave's next row, or (at the very end) the
-        // wave's first row again: a valid address whose bytes go unused
-        const bool last = step + 1 == steps;
-        const uint32_t next_row = last ? (row + stride < rows ? row + stride : first) : row;
-        load_step(next_row, last ? 0u : step + 1, ring, &shift);
+    for (int d = 0; d < kBlocksDepth; ++d) next_load(ring[d], &shifts[d]);
+  }
+
+  // ---- the activation rows, quantised once per block ------------------------------------------
+  // A thread takes eight neighbouring values at a time (one 16-byte vector of a narrow type, two of
+  // f32, when x allows vector loads), the next eight already on their way.
+  auto fetch_values = [&](uint32_t r, uint32_t p, float (&values)[8]) {
+    const bool inside = p < k;
+    const size_t at = (size_t)r * k + (inside ? p : 0u);  // a thread past the row reads its start and keeps nothing
+    if constexpr (kVectorX) {
+      if constexpr (Traits<TX>::kVec == 8) {
+        Traits<TX>::unpack(load16(x, at / 8), values);
+      } else {
+        float half[4];
+        Traits<TX>::unpack(load16(x, at / 4), half);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) values[e] = half[e];
+        Traits<TX>::unpack(load16(x, at / 4 + 1), half);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) values[4 + e] = half[e];
       }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) values[e] = Traits<TX>::load(x, at + e);
+    }
+    if (!inside) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) values[e] = 0.0f;
+    }
+  };
+  const uint32_t pieces = (k + kBlockThreads * 8 - 1) / (kBlockThreads * 8);  // per activation row
+  const uint32_t turns = m * pieces;
+  float ahead[8];
+  if (turns != 0) fetch_values(0, threadIdx.x * 8, ahead);
+  for (uint32_t turn = 0; turn < turns; ++turn) {
+    const uint32_t r = turn / pieces, p = (turn % pieces) * (kBlockThreads * 8) + threadIdx.x * 8;
+    const bool inside = p < k;  // the same for all lanes that share an activation block
+    float values[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) values[e] = ahead[e];
+    if (turn + 1 < turns)
+      fetch_values((turn + 1) / pieces, ((turn + 1) % pieces) * (kBlockThreads * 8) + threadIdx.x * 8, ahead);
+    LaneMax mine{0.0f, 0.0f, 0u};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {  // positions rise with e, so ">" keeps the first
+      const float magnitude = __builtin_fabsf(values[e]);
+      if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], p + e};
+    }
+    if (mine.magnitude == 0.0f) mine.position = 0xFFFFFFFFu;  // no candidate: any lane with one goes first
+    const LaneMax top = block_largest<kQuantiseLanes>(mine);
+    float factor = 0.0f, stored = 0.0f;
+    if (top.magnitude != 0.0f) {
+      if constexpr (kKind == 2) {
+        stored = f16_to_f32(f32_to_f16(top.magnitude / 127.0f));
+        factor = 127.0f / top.magnitude;
+      } else {
+        factor = -127.0f / top.value;
+        stored = 1.0f / factor;
+      }
+    }
+    uint32_t words[2] = {0u, 0u};
+    if (top.magnitude != 0.0f) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) words[e / 4] |= code_of(values[e] * factor) << (8 * (e % 4));
+    }
+    if (inside) {
+      uint32_t *to = reinterpret_cast<uint32_t *>(codes + (size_t)r * k + p);
+      to[0] = words[0];
+      to[1] = words[1];
+      if (p % kActivationBlock == 0) scales[r * activation_blocks + p / kActivationBlock] = stored;
+    }
+  }
+  __syncthreads();
+  if (own_rows == 0) return;  // no barrier follows
+  if (steps == 0) {  // K = 0: every product is an empty sum
+    for (uint32_t row = first; row < rows; row += stride)
+      if (lane < m) Traits<TX>::store(y, (size_t)lane * rows + row, 0.0f);
+    return;
+  }
+
+  // ---- the weight rows ----------------------------------------------------------------------
+  uint32_t row = first, step = 0;
+  float totals[kM] = {};
+  for (uint64_t done = 0; done < segments; done += kBlocksDepth) {
+#pragma unroll
+    for (int d = 0; d < kBlocksDepth; ++d) {
+      if (done + d >= segments) break;
+#pragma unroll
+      for (int i = 0; i < Step::kLoads; ++i) *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = ring[d][i];
+      const uint32_t at = shifts[d] + run * Geometry::kRunBytes;
+      next_load(ring[d], &shifts[d]);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -970,11 +1028,16 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_blocks(const uns
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-    }
+      if (++step == steps) {  // the row is complete
 #pragma unroll
-    for (int r = 0; r < kM; ++r) {
-      const float whole = group_sum<kWaveLanes>(totals[r]);
-      if (lane == 0 && (uint32_t)r < m) Traits<TX>::store(y, (size_t)r * rows + row, whole);
+        for (int r = 0; r < kM; ++r) {
+          const float whole = group_sum<kWaveLanes>(totals[r]);
+          if (lane == 0 && (uint32_t)r < m) Traits<TX>::store(y, (size_t)r * rows + row, whole);
+          totals[r] = 0.0f;
+        }
+        step = 0;
+        row += stride;
+      }
     }
   }
 }
@@ -999,9 +1062,15 @@ hipError_t run_blocks(const MatVecParams &p, const void *w, const void *x, void 
     const void *xs = static_cast<const char *>(x) + (size_t)done * p.k * Traits<TX>::kSize;
     void *ys = static_cast<char *>(y) + (size_t)done * p.rows * Traits<TX>::kSize;
     const size_t shared = m * per_row;
-#define HYLE_BLOCKS(M)                 \
-  note_variant<BlocksTag<kKind, M>>(); \
-  hipLaunchKernelGGL((gguf_matvec_q8_blocks<kKind, TX, M>), grid, dim3(kBlockThreads), shared, s, in, xs, ys, (uint32_t)p.rows, p.row_stride, p.k, m)
+    const bool vector_x = (reinterpret_cast<uintptr_t>(xs) & 15u) == 0;
+#define HYLE_BLOCKS(M)                                                                                                          \
+  note_variant<BlocksTag<kKind, M>>();                                                                                          \
+  if (vector_x)                                                                                                                 \
+    hipLaunchKernelGGL((gguf_matvec_q8_blocks<kKind, TX, M, true>), grid, dim3(kBlockThreads), shared, s, in, xs, ys,          \
+                       (uint32_t)p.rows, p.row_stride, p.k, m);                                                                 \
+  else                                                                                                                          \
+    hipLaunchKernelGGL((gguf_matvec_q8_blocks<kKind, TX, M, false>), grid, dim3(kBlockThreads), shared, s, in, xs, ys,         \
+                       (uint32_t)p.rows, p.row_stride, p.k, m)
     if (m == 1) { HYLE_BLOCKS(1); }
     else if (m == 2) { HYLE_BLOCKS(2); }
     else if (m <= 4) { HYLE_BLOCKS(4); }

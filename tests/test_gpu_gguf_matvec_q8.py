@@ -44,8 +44,9 @@ def raw_bytes_for(tag, rng, rows, k):
     return raw.reshape(rows, -1)
 
 
-def check(tag, x_tag, raw, rows, k, x, row_stride=None, byte_offset=0, kernel=None):
+def check(tag, x_tag, raw, rows, k, x, row_stride=None, byte_offset=0, kernel=None, x_offset=0):
     """byte_offset: the weight starts that many bytes into its (256-byte aligned) allocation;
+    x_offset: the activations start that many elements into theirs;
     kernel: the launch shape the case is written for (a prefix of the label)."""
     kind, gguf = KINDS[tag]
     stored = host_values(x, x_tag)
@@ -56,7 +57,12 @@ def check(tag, x_tag, raw, rows, k, x, row_stride=None, byte_offset=0, kernel=No
     storage = torch.from_numpy(flat).to(DEVICE)[byte_offset:]
     descs = [hc.TensorDesc.gguf_weight(gguf, TYPES[x_tag][0], k, rows, row_stride),
              hc.TensorDesc.dense(TYPES[x_tag][0], list(x.shape))]
-    (out,) = run(Q8, storage, to_device(stored, x_tag), descs=descs)
+    activations = to_device(stored, x_tag)
+    if x_offset:
+        padded = torch.zeros(activations.numel() + x_offset, dtype=activations.dtype, device=DEVICE)
+        padded[x_offset:] = activations.reshape(-1)
+        activations = padded[x_offset:].view(activations.shape)
+    (out,) = run(Q8, storage, activations, descs=descs)
     if kernel is not None:
         assert hc.last_launch_variant().startswith(kernel), (hc.last_launch_variant(), kernel)
     assert list(out.shape) == ([rows] if x.ndim == 1 else [x.shape[0], rows])
@@ -169,6 +175,9 @@ def test_q8_route_rows_at_even_addresses_and_strides(tag):
             note(f"q8 matvec {tag} k {k} rows {rows} m {m}: weight {byte_offset} bytes off, rows {pad} bytes apart")
             check(tag, "f32", padded, rows, k, x, row_stride=row_bytes + pad, byte_offset=byte_offset,
                   kernel="gguf_matvec_q8_blocks/")
+        for x_tag, x_offset in (("f32", 1), ("bf16", 3), ("f16", 1)):
+            note(f"q8 matvec {tag} k {k} rows {rows} m {m}: {x_tag} activations {x_offset} elements off a 16-byte boundary")
+            check(tag, x_tag, weights_for(tag, rng, rows, k), rows, k, x, x_offset=x_offset)
 
 
 def test_q8_route_activation_rows_in_groups_when_their_codes_do_not_fit_together():
