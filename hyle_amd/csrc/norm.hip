@@ -50,7 +50,14 @@ __global__ __launch_bounds__(kBlockThreads) void norm_generic(const void *x, con
   }
 }
 
-template <class T, class W, bool kLayer, int kLanes, int kVpl, int kThreads = kBlockThreads, int kRows = 1>
+template <bool kLayer> struct GenericTag {
+  static std::string text() { return std::string("norm_generic/") + (kLayer ? "layer" : "rms"); }
+};
+
+// kExactElsewhere: whenever this shape would cover the tensor exactly, a shape of norm_exact.h has
+// already taken the launch (same width, a row count it divides), so no exact form is built here.
+template <class T, class W, bool kLayer, int kLanes, int kVpl, int kThreads = kBlockThreads, int kRows = 1,
+          bool kExactElsewhere = false>
 hipError_t run_rows(const NormParams &p, const Bound &io, int parameters, hipStream_t s) {
   constexpr int kRowsPerBlock = kThreads / kLanes * kRows;
   const uint32_t rows = (uint32_t)p.shape.rows, row_vectors = p.shape.width / Traits<T>::kVec;
@@ -66,9 +73,13 @@ hipError_t run_rows(const NormParams &p, const Bound &io, int parameters, hipStr
                        (float)p.shape.width, p.epsilon);
   };
   auto by_shape = [&](auto parameters_tag) {
-    if constexpr (kLayer) {
-      if (exact) return go(parameters_tag, std::true_type{});
+    if constexpr (kLayer && !kExactElsewhere) {
+      if (exact) {
+        note_variant<NormTag<kLayer, kLanes, kVpl, kThreads, kRows, 2>>();
+        return go(parameters_tag, std::true_type{});
+      }
     }
+    note_variant<NormTag<kLayer, kLanes, kVpl, kThreads, kRows, 1>>();
     go(parameters_tag, std::false_type{});
   };
   if (parameters == kPlain) by_shape(std::integral_constant<int, kPlain>{});
@@ -90,22 +101,23 @@ hipError_t run(const NormParams &p, const Bound &io, bool vectorised, hipStream_
     // Two vectors per lane, two rows per lane group and small blocks measured best on MI355X
     // for X[8192, 2048] bf16: 11.2 us, against 12.3-13.5 us for the same rows in blocks of
     // 256-1024 threads and 13.7-15.4 us for one vector per lane with four or eight rows.
-    if (vectors <= 128) return run_rows<T, W, kLayer, 64, 2, 256, 2>(p, io, parameters, s);
+    if (vectors <= 128) return run_rows<T, W, kLayer, 64, 2, 256, 2, true>(p, io, parameters, s);
     if (vectors <= 256) {
       // One wave per row (no barrier), two rows one after the other: the second row's loads are
       // in flight while the first is reduced, scaled and stored.  [8192, 2048] bf16 on MI355X:
       // LayerNorm 11.3 us in blocks of one wave (11.5-11.8 us in blocks of 2-8 waves, 12.2 us
       // with four rows per wave, 13.5 us with one, 14.3 us for two waves per row); RMSNorm
       // 11.2 us in blocks of four waves (11.6-11.9 us for two waves per row).
-      if constexpr (kLayer) return run_rows<T, W, kLayer, 64, 4, 64, 2>(p, io, parameters, s);
-      return run_rows<T, W, kLayer, 64, 4, 256, 2>(p, io, parameters, s);
+      if constexpr (kLayer) return run_rows<T, W, kLayer, 64, 4, 64, 2, true>(p, io, parameters, s);
+      else return run_rows<T, W, kLayer, 64, 4, 256, 2>(p, io, parameters, s);
     }
-    if (vectors <= 512) return run_rows<T, W, kLayer, 256, 2, 256, 2>(p, io, parameters, s);
+    if (vectors <= 512) return run_rows<T, W, kLayer, 256, 2, 256, 2, true>(p, io, parameters, s);
     if (vectors <= 1024) return run_rows<T, W, kLayer, 256, 4>(p, io, parameters, s);
     if (vectors <= 2048) return run_rows<T, W, kLayer, 256, 8>(p, io, parameters, s);
     if (vectors <= 4096) return run_rows<T, W, kLayer, 1024, 4, 1024>(p, io, parameters, s);
     return run_rows<T, W, kLayer, 1024, 8, 1024>(p, io, parameters, s);
   }
+  note_variant<GenericTag<kLayer>>();
   hipLaunchKernelGGL((norm_generic<T, W, kLayer>), dim3((uint32_t)p.shape.rows), dim3(kBlockThreads), 0, s,
                      io.x, io.w, io.b, io.y, p.shape.width, p.epsilon, parameters);
   return hipGetLastError();

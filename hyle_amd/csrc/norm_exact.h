@@ -27,10 +27,12 @@ template <class T, class W, bool kLayer, int kLanes>
 bool run_exact_lanes(uint32_t per_lane, const NormParams &p, const Bound &io, int parameters, hipStream_t s) {
   switch (per_lane) {
     case 3: if constexpr (kLanes == 64) return run_exact<T, W, kLayer, kLanes, 3, kLanes, 2>(p, io, parameters, s); break;
-    case 4: if constexpr (kLanes == 64) return run_exact<T, W, kLayer, kLanes, 4, kLanes, 2>(p, io, parameters, s); break;
-    // with more lanes only the counts that 64 lanes cannot hold in eight vectors arrive here
-    case 5: return run_exact<T, W, kLayer, kLanes, 5, kLanes, 2>(p, io, parameters, s);
-    case 6: return run_exact<T, W, kLayer, kLanes, 6, kLanes, 2>(p, io, parameters, s);
+    // RMSNorm rows of 256 vectors keep norm.hip's shape (run_exact_shape)
+    case 4: if constexpr (kLanes == 64 && kLayer) return run_exact<T, W, kLayer, kLanes, 4, kLanes, 2>(p, io, parameters, s); break;
+    // with more lanes only the counts that fewer lanes do not take arrive here: 128 lanes get 7 and
+    // 8 vectors each (896 and 1024 per row), 256 lanes 5 to 8
+    case 5: if constexpr (kLanes != 128) return run_exact<T, W, kLayer, kLanes, 5, kLanes, 2>(p, io, parameters, s); break;
+    case 6: if constexpr (kLanes != 128) return run_exact<T, W, kLayer, kLanes, 6, kLanes, 2>(p, io, parameters, s); break;
     case 7: return run_exact<T, W, kLayer, kLanes, 7, kLanes, 2>(p, io, parameters, s);
     case 8: return run_exact<T, W, kLayer, kLanes, 8, kLanes, 2>(p, io, parameters, s);
     // one wave per row still pays with 9, 10 or 12 vectors per lane (about 240 registers for two rows)

@@ -139,12 +139,22 @@ struct Bound {
   void *y;
 };
 
+// <family>/<rms|layer>/<lanes>x<vectors per lane>/<threads per block>/<rows per lane group>[/<ragged|exact>]
+template <bool kLayer, int kLanes, int kVpl, int kThreads, int kRows, int kForm> struct NormTag {  // kForm: 0 exact-only shape, 1 ragged, 2 exact
+  static std::string text() {
+    return std::string(kForm == 0 ? "norm_rows_exact/" : "norm_rows/") + (kLayer ? "layer/" : "rms/") + std::to_string(kLanes) + "x" +
+           std::to_string(kVpl) + "/" + std::to_string(kThreads) + "/" + std::to_string(kRows) +
+           (kForm == 1 ? "/ragged" : (kForm == 2 ? "/exact" : ""));
+  }
+};
+
 // A launch shape used only when it covers the tensor exactly (no masked variant is built for it).
 template <class T, class W, bool kLayer, int kLanes, int kVpl, int kThreads, int kRows>
 bool run_exact(const NormParams &p, const Bound &io, int parameters, hipStream_t s) {
   constexpr int kRowsPerBlock = kThreads / kLanes * kRows;
   const uint32_t rows = (uint32_t)p.shape.rows, row_vectors = p.shape.width / Traits<T>::kVec;
   if (rows % kRowsPerBlock != 0 || row_vectors != (uint32_t)(kLanes * kVpl)) return false;
+  note_variant<NormTag<kLayer, kLanes, kVpl, kThreads, kRows, 0>>();
   const dim3 grid(rows / kRowsPerBlock), block(kThreads);
   const float width = (float)p.shape.width;
   if (parameters == kPlain)

@@ -38,10 +38,11 @@ def test_library_exports_every_declared_symbol():
     assert lib.hyle_hip_abi_version() == capi.ABI_VERSION
 
 
-def test_launch_shape_labels_are_listed_and_the_softmax_table_names_each_of_them():
+def test_launch_shape_labels_are_listed_and_the_softmax_and_norm_tables_name_each_of_them():
     """The labels register themselves when the library loads (no device needed).  Every Softmax
-    launch shape compiled in must be a row of the table the GPU cases walk
-    (tests/test_gpu_softmax_variants.py), and the table must name nothing the library lacks."""
+    and norm launch shape compiled in must be a row of the table the GPU cases walk
+    (tests/test_gpu_softmax_variants.py, tests/test_gpu_norm_variants.py), and the tables must name
+    nothing the library lacks."""
     labels = hc.launch_variants()
     assert labels and len(set(labels)) == len(labels)
     assert capi.load().hyle_hip_variant_label(len(labels)) == b""
@@ -49,6 +50,10 @@ def test_launch_shape_labels_are_listed_and_the_softmax_table_names_each_of_them
     import test_gpu_softmax_variants as table
     compiled = {label for label in labels if label.startswith("softmax")}
     tabled = {case[5] for case in table.CASES}
+    assert compiled == tabled, (sorted(compiled - tabled), sorted(tabled - compiled))
+    import test_gpu_norm_variants as norm_table
+    compiled = {label for label in labels if label.startswith("norm")}
+    tabled = {case[4] for case in norm_table.CASES}
     assert compiled == tabled, (sorted(compiled - tabled), sorted(tabled - compiled))
 
 
