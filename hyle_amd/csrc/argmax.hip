@@ -148,12 +148,21 @@ __global__ __launch_bounds__(kBlockThreads) void argmax_finish(const void *x, co
   }
 }
 
+template <bool kVector> struct TilesTag {
+  static std::string text() { return kVector ? "argmax_tiles/vector" : "argmax_tiles/scalar"; }
+};
+template <int kLanes> struct FinishTag {
+  static std::string text() { return "argmax_finish/" + std::to_string(kLanes) + "-lanes"; }
+};
+
 template <class T>
 hipError_t run(const ArgmaxParams &p, const void *x, void *values, int32_t *indices, void *workspace,
                bool vectorised, hipStream_t s) {
   const uint32_t rows = (uint32_t)p.shape.rows, width = p.shape.width;
   auto *partial = static_cast<Candidate *>(workspace);
   const bool vec = vectorised && width % Traits<T>::kVec == 0 && p.tile_elems % Traits<T>::kVec == 0;
+  if (vec) note_variant<TilesTag<true>>();
+  else note_variant<TilesTag<false>>();
   if (vec)
     hipLaunchKernelGGL((argmax_tiles<T, true>), dim3(rows * p.tiles), dim3(kBlockThreads), 0, s, x,
                        partial, width, p.tiles, p.tile_elems);
@@ -164,10 +173,12 @@ hipError_t run(const ArgmaxParams &p, const void *x, void *values, int32_t *indi
   if (err != hipSuccess) return err;
   if (p.tiles <= 16) {
     constexpr int kRowsPerBlock = kBlockThreads / 16;
+    note_variant<FinishTag<16>>();
     hipLaunchKernelGGL((argmax_finish<T, 16>), dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock),
                        dim3(kBlockThreads), 0, s, x, partial, values, indices, rows, width, p.tiles);
   } else {
     constexpr int kRowsPerBlock = kBlockThreads / kWaveLanes;
+    note_variant<FinishTag<kWaveLanes>>();
     hipLaunchKernelGGL((argmax_finish<T, kWaveLanes>), dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock),
                        dim3(kBlockThreads), 0, s, x, partial, values, indices, rows, width, p.tiles);
   }

@@ -188,12 +188,22 @@ __global__ __launch_bounds__(kBlockThreads) void cast_general(const char *in, vo
   store_element<D::kSize>(out, e, convert_bits<S, D>(load_element<S::kSize>(in + offset)));
 }
 
+template <int kUnroll, int kThreads, bool kSerial> struct FlatTag {
+  static std::string text() {
+    return "cast_flat/" + std::to_string(kUnroll) + "x" + std::to_string(kThreads) + (kSerial ? "/serial" : "/batched");
+  }
+};
+struct GeneralTag {
+  static std::string text() { return "cast_general"; }
+};
+
 template <class S, class D, int kUnroll, int kThreads, bool kSerial>
 hipError_t run_flat_as(const void *in, void *out, uint64_t elements, hipStream_t s) {
   const uint64_t groups = elements / group_elements<S, D>();
   const uint64_t per_block = (uint64_t)kUnroll * kThreads;
   uint64_t blocks = (groups + per_block - 1) / per_block;
   if (blocks == 0) blocks = 1;  // the tail still needs block 0
+  note_variant<FlatTag<kUnroll, kThreads, kSerial>>();
   hipLaunchKernelGGL((cast_flat<S, D, kUnroll, kThreads, kSerial>), dim3((uint32_t)blocks), dim3(kThreads), 0, s,
                      in, out, (uint32_t)groups, (uint32_t)elements);
   return hipGetLastError();
@@ -219,6 +229,7 @@ hipError_t run_pair(const CastParams &p, const void *in, void *out, bool vectori
     layout.strides[i] = p.strides[i];
   }
   const uint64_t blocks = (p.elements + kBlockThreads - 1) / kBlockThreads;
+  note_variant<GeneralTag>();
   hipLaunchKernelGGL((cast_general<S, D>), dim3((uint32_t)blocks), dim3(kBlockThreads), 0, s,
                      static_cast<const char *>(in), out, p.elements, layout);
   return hipGetLastError();

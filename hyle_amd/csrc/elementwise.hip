@@ -459,6 +459,24 @@ Operand make_operand(const void *base, uint32_t period, int vec) {
   return op;
 }
 
+// ew_full: every operand as long as the output; ew_flat: some operand periodic (a dense broadcast
+// suffix) or a scalar.  <vectors per lane>x<threads per block>[/serial: one vector after another]
+template <int kUnroll, int kThreads, int kForm> struct EwTag {  // kForm: 0 flat, 1 full with the vectors in flight at once, 2 full serial
+  static std::string text() {
+    return std::string(kForm == 0 ? "ew_flat/" : "ew_full/") + std::to_string(kUnroll) + "x" + std::to_string(kThreads) +
+           (kForm == 2 ? "/serial" : (kForm == 1 ? "/batched" : ""));
+  }
+};
+struct EwScalarTag {
+  static std::string text() { return "ew_flat_scalar"; }
+};
+struct EwGeneralTag {
+  static std::string text() { return "ew_general"; }
+};
+template <bool kVector> struct PackedTag {
+  static std::string text() { return kVector ? "gated_packed/vector" : "gated_packed/scalar"; }
+};
+
 template <class T, class Fn, int kUnroll, int kThreads, bool kSerial>
 hipError_t run_full_as(const EwFlat &p, Operand a, Operand b, Operand c, void *out, hipStream_t s) {
   constexpr int kVec = Traits<T>::kVec;
@@ -466,6 +484,7 @@ hipError_t run_full_as(const EwFlat &p, Operand a, Operand b, Operand c, void *o
   const uint64_t per_block = (uint64_t)kUnroll * kThreads;
   uint64_t blocks = (vectors + per_block - 1) / per_block;
   if (blocks == 0) blocks = 1;  // the tail still needs block 0
+  note_variant<EwTag<kUnroll, kThreads, kSerial ? 2 : 1>>();
   hipLaunchKernelGGL((ew_full_vec<T, Fn, kUnroll, kThreads, kSerial>), dim3((uint32_t)blocks),
                      dim3(kThreads), 0, s, a.base, b.base, c.base, out, (uint32_t)vectors,
                      (uint32_t)p.elements, Fn{});
@@ -479,6 +498,7 @@ hipError_t run_flat_as(const EwFlat &p, Operand a, Operand b, Operand c, void *o
   const uint64_t per_block = (uint64_t)kUnroll * kThreads;
   uint64_t blocks = (vectors + per_block - 1) / per_block;
   if (blocks == 0) blocks = 1;  // the tail still needs block 0
+  note_variant<EwTag<kUnroll, kThreads, 0>>();
   hipLaunchKernelGGL((ew_flat_vec<T, Fn, kUnroll, kThreads>), dim3((uint32_t)blocks), dim3(kThreads), 0, s,
                      a, b, c, out, (uint32_t)vectors, (uint32_t)p.elements, Fn{});
   return hipGetLastError();
@@ -533,6 +553,7 @@ hipError_t run_flat(const EwFlat &p, const void *a, const void *b, const void *c
     whole_vectors = whole_vectors && (p.period[i] <= 1 || p.period[i] % kVec == 0);
   if (!vectorised || !chain_fast || !whole_vectors) {
     const uint64_t blocks = (p.elements + kBlockThreads - 1) / kBlockThreads;
+    note_variant<EwScalarTag>();
     hipLaunchKernelGGL((ew_flat_scalar<T>), dim3((uint32_t)blocks), dim3(kBlockThreads), 0, s, oa,
                        ob, oc, out, (uint32_t)p.elements, (int)p.inputs,
                        RuntimeFn{p.op, (int)p.kind0, (int)p.kind1});
@@ -592,6 +613,7 @@ hipError_t run_general(const EwGeneral &p, const void *a, const void *b, const v
     for (int k = 0; k < 3; ++k) layout.strides[k][i] = p.strides[k][i];
   }
   const uint64_t blocks = (p.elements + kBlockThreads - 1) / kBlockThreads;
+  note_variant<EwGeneralTag>();
   hipLaunchKernelGGL((ew_general<T>), dim3((uint32_t)blocks), dim3(kBlockThreads), 0, s,
                      static_cast<const char *>(a), static_cast<const char *>(b),
                      static_cast<const char *>(c), out, p.elements, (int)p.inputs, layout,
@@ -607,9 +629,11 @@ hipError_t run_packed(const EwPacked &p, const void *packed, void *out, bool vec
   if (vectorised && p.hidden % kVec == 0) {
     const uint64_t vectors = elements / kVec;
     const uint64_t per_block = (uint64_t)kUnroll * kBlockThreads;
+    note_variant<PackedTag<true>>();
     hipLaunchKernelGGL((swiglu_packed_vec<T>), dim3((uint32_t)((vectors + per_block - 1) / per_block)),
                        dim3(kBlockThreads), 0, s, packed, out, p.hidden / kVec, vectors, (int)p.activation);
   } else {
+    note_variant<PackedTag<false>>();
     hipLaunchKernelGGL((swiglu_packed_scalar<T>),
                        dim3((uint32_t)((elements + kBlockThreads - 1) / kBlockThreads)),
                        dim3(kBlockThreads), 0, s, packed, out, p.hidden, elements, (int)p.activation);

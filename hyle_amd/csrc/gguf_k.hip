@@ -150,6 +150,12 @@ __global__ __launch_bounds__(kBlockThreads) void k_quant_lines(const unsigned ch
 
 }  // namespace
 
+namespace {
+template <int kKind, bool kLines> struct KQuantTag {
+  static std::string text() { return std::string(kLines ? "k_quant_lines/" : "k_quant_rows/") + (kKind == 0 ? "q4_k" : "q6_k"); }
+};
+}  // namespace
+
 hipError_t launch_k_quant_dequant(const KQuantParams &p, const void *blocks, void *out, float *sumsq,
                                   hipStream_t stream) {
   if (p.rows == 0) return hipSuccess;
@@ -158,6 +164,8 @@ hipError_t launch_k_quant_dequant(const KQuantParams &p, const void *blocks, voi
   if (lines) {
     constexpr int kWaves = kBlockThreads / kWaveLanes;
     const dim3 grid(((uint32_t)p.rows + kWaves - 1) / kWaves), block(kBlockThreads);
+    if (p.kind == 0) note_variant<KQuantTag<0, true>>();
+    else note_variant<KQuantTag<1, true>>();
     if (p.kind == 0)
       hipLaunchKernelGGL((k_quant_lines<0>), grid, block, 0, stream, in, out, sumsq, (uint32_t)p.rows, p.k,
                          p.row_stride);
@@ -168,6 +176,8 @@ hipError_t launch_k_quant_dequant(const KQuantParams &p, const void *blocks, voi
   }
   constexpr int kRows = 4;
   const dim3 grid(((uint32_t)p.rows + kRows - 1) / kRows), block(kBlockThreads);
+  if (p.kind == 0) note_variant<KQuantTag<0, false>>();
+  else note_variant<KQuantTag<1, false>>();
   if (p.kind == 0)
     hipLaunchKernelGGL((k_quant_rows<0, kRows>), grid, block, 0, stream, in, out, sumsq, (uint32_t)p.rows, p.k,
                        p.row_stride);

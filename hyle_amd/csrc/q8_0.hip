@@ -169,11 +169,22 @@ __global__ __launch_bounds__(kBlockThreads) void q8_0_rows_bytes(const uint8_t *
   if (row_ok && lane == 0) sumsq[row] = squares;
 }
 
+struct LinesTag {
+  static std::string text() { return "q8_0_lines"; }
+};
+struct RowsTag {
+  static std::string text() { return "q8_0_rows"; }
+};
+struct BytesTag {
+  static std::string text() { return "q8_0_rows_bytes"; }
+};
+
 template <int kWaves, int kRows>
 hipError_t run_rows(const Q8Params &p, const void *blocks, void *out, float *sumsq,
                     uint32_t row_bytes, hipStream_t stream) {
   const uint32_t rows = (uint32_t)p.rows;
   constexpr int kRowsPerBlock = kWaves * kRows;
+  note_variant<RowsTag>();
   hipLaunchKernelGGL((q8_0_rows<kWaves, kRows>), dim3((rows + kRowsPerBlock - 1) / kRowsPerBlock),
                      dim3(kWaves * kWaveLanes), (size_t)kRowsPerBlock * row_bytes, stream,
                      static_cast<const char *>(blocks), static_cast<uint16_t *>(out), sumsq, rows, p.k,
@@ -196,6 +207,7 @@ hipError_t launch_q8_0_dequant(const Q8Params &p, const void *blocks, void *out,
     // plain stores; a wave that walks several rows with the next row in flight 7.3 - 9.3 us; the
     // block-staged kernel below 7.1 us.
     constexpr int kWaves = 4;
+    note_variant<LinesTag>();
     hipLaunchKernelGGL((q8_0_lines<kWaves>), dim3((rows + kWaves - 1) / kWaves), dim3(kWaves * kWaveLanes), 0, stream,
                        static_cast<const unsigned char *>(blocks), out, sumsq, rows, p.k, p.row_stride);
     return hipGetLastError();
@@ -206,6 +218,7 @@ hipError_t launch_q8_0_dequant(const Q8Params &p, const void *blocks, void *out,
     return run_rows<4, 1>(p, blocks, out, sumsq, row_bytes, stream);
   }
   constexpr int kWaves = kBlockThreads / kWaveLanes;
+  note_variant<BytesTag>();
   hipLaunchKernelGGL(q8_0_rows_bytes, dim3((rows + kWaves - 1) / kWaves), dim3(kBlockThreads), 0,
                      stream, static_cast<const uint8_t *>(blocks), static_cast<uint16_t *>(out),
                      sumsq, rows, p.k, p.row_stride);

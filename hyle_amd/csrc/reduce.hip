@@ -226,11 +226,26 @@ __global__ __launch_bounds__(kBlockThreads) void reduce_general(const char *x, v
 // ---- host side --------------------------------------------------------------------------------
 uint32_t ceil_div(uint64_t a, uint64_t b) { return (uint32_t)((a + b - 1) / b); }
 
+// reduce_rows/<block|wave per unit>/<vector|scalar>, reduce_columns/<vector|scalar>, reduce_general[/bytes]
+template <bool kBlock, bool kVector> struct RowsTag {
+  static std::string text() { return std::string("reduce_rows/") + (kBlock ? "block" : "wave") + (kVector ? "/vector" : "/scalar"); }
+};
+template <bool kVector> struct ColumnsTag {
+  static std::string text() { return std::string("reduce_columns/") + (kVector ? "vector" : "scalar"); }
+};
+template <bool kBytewise> struct GeneralTag {
+  static std::string text() { return kBytewise ? "reduce_general/bytes" : "reduce_general"; }
+};
+
 template <class TIn, class TOut, int kKind>
 void rows_launch(const void *x, void *y, uint32_t rows, uint32_t width, uint32_t tiles,
                  uint32_t tile_width, float divisor, bool vector, hipStream_t s) {
   const uint32_t units = rows * tiles;
   const bool wide = (size_t)std::min(width, tile_width) * Traits<TIn>::kSize >= 8192;
+  if (wide && vector) note_variant<RowsTag<true, true>>();
+  else if (wide) note_variant<RowsTag<true, false>>();
+  else if (vector) note_variant<RowsTag<false, true>>();
+  else note_variant<RowsTag<false, false>>();
   if (wide) {
     if (vector)
       hipLaunchKernelGGL((reduce_rows<TIn, TOut, kKind, kBlockThreads, true>), dim3(units),
@@ -268,6 +283,8 @@ void columns_launch(const void *x, void *y, uint32_t outer, uint32_t reduced, ui
   const uint32_t log2 = lanes_x_log2_for(units, outer);
   const uint32_t x_tiles = ceil_div(units, 1u << log2);
   const dim3 grid(x_tiles * outer, segments, 1);
+  if (vector) note_variant<ColumnsTag<true>>();
+  else note_variant<ColumnsTag<false>>();
   if (vector)
     hipLaunchKernelGGL((reduce_columns<TIn, TOut, kKind, true>), grid, dim3(kBlockThreads), 0, s, x, y,
                        outer, reduced, inner, log2, x_tiles, segment_rows, divisor);
@@ -317,6 +334,8 @@ hipError_t run_kind(const ReduceParams &p, const void *x, void *y, void *workspa
         g.strides[a] = p.strides[a];
       }
       const uint32_t blocks = ceil_div(p.rows, kBlockThreads / kWaveLanes);
+      if (p.bytewise) note_variant<GeneralTag<true>>();
+      else note_variant<GeneralTag<false>>();
       if (p.bytewise)
         hipLaunchKernelGGL((reduce_general<T, kKind, true>), dim3(blocks), dim3(kBlockThreads), 0, s,
                            static_cast<const char *>(x), y, g, p.divisor);

@@ -55,8 +55,18 @@ def host_values(array: np.ndarray, tag: str) -> np.ndarray:
     return array if tag == "f32" else orc.from_f32(TYPES[tag][1], array)
 
 
+# Labels of the kernel launch shapes the tests of this session launched through run()
+# (hyle_hip_last_launch_variant): tests/test_zy_launch_shape_coverage.py holds them against the list
+# of shapes compiled into the library.
+LAUNCHED = set()
+
+
 def run(operation, *tensors, descs=None, outputs=None):
-    return tio.run(context(), operation, *tensors, descs=descs, outputs=outputs)
+    result = tio.run(context(), operation, *tensors, descs=descs, outputs=outputs)
+    chosen = hc.last_launch_variant()
+    if chosen:
+        LAUNCHED.update(chosen.split(" + "))
+    return result
 
 
 # ---- comparisons ----------------------------------------------------------------------------
