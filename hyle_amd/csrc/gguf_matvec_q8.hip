@@ -1090,17 +1090,23 @@ hipError_t run_quads(const MatVecParams &p, const void *w, const void *x, void *
   note_variant<QuadsTag<kKind, SETS, REGISTERS>>();                                                                 \
   hipLaunchKernelGGL((gguf_matvec_q8_quads<kKind, TX, SETS, REGISTERS>), grid, dim3(kBlockThreads), shared, s, in, x, \
                      y, (uint32_t)p.rows, p.row_stride, spans, p.m)
-  const bool registers = spans == 1 && kKind != 0;  // Q4_K fetches its codes from LDS share by share
+  // Which forms a shape can reach follows from what fits a block's LDS beside the four row slots per
+  // wave (run_m): one set of four tokens for every format, with the codes in registers when K = 2048
+  // (Q4_K fetches its codes from LDS share by share); two sets only for Q4_K (codes in LDS) and for
+  // Q6_K at K = 2048 (codes in registers); Q8_0's wider slots leave no room for a second set.
+  const bool registers = spans == 1 && kKind != 0;
   if (p.m <= 4) {
     if constexpr (kKind != 0) {
       if (registers) { HYLE_QUADS(1, true); }
     }
     if (!registers) { HYLE_QUADS(1, false); }
+  } else if constexpr (kKind == 0) {
+    HYLE_QUADS(2, false);
+  } else if constexpr (kKind == 1) {
+    if (!registers) return hipErrorInvalidValue;
+    HYLE_QUADS(2, true);
   } else {
-    if constexpr (kKind != 0) {
-      if (registers) { HYLE_QUADS(2, true); }
-    }
-    if (!registers) { HYLE_QUADS(2, false); }
+    return hipErrorInvalidValue;
   }
 #undef HYLE_QUADS
   return hipGetLastError();
@@ -1110,15 +1116,20 @@ template <int kKind, class TX, int kM>
 hipError_t run_registers(const MatVecParams &p, const void *w, const void *x, void *y, uint32_t spans, dim3 grid,
                          size_t shared, hipStream_t s) {
   const unsigned char *in = static_cast<const unsigned char *>(w);
-  if (spans == 1) {
-    note_variant<LinesTag<kKind, kM, true>>();
-    hipLaunchKernelGGL((gguf_matvec_q8_lines<kKind, TX, kM, true>), grid, dim3(kBlockThreads), shared, s, in, x, y,
-                       (uint32_t)p.rows, p.row_stride, spans, p.m);
-  } else {
-    note_variant<LinesTag<kKind, kM, false>>();
-    hipLaunchKernelGGL((gguf_matvec_q8_lines<kKind, TX, kM, false>), grid, dim3(kBlockThreads), shared, s, in, x, y,
-                       (uint32_t)p.rows, p.row_stride, spans, p.m);
+  // One span per row with the codes in registers is reached by Q8_0 with 5 to 8 tokens only (every
+  // other K = 2048 shape takes the span or the quad kernel); the form that fetches the codes from
+  // LDS serves any number of spans.
+  if constexpr (kKind == 2 && kM == 8) {
+    if (spans == 1) {
+      note_variant<LinesTag<kKind, kM, true>>();
+      hipLaunchKernelGGL((gguf_matvec_q8_lines<kKind, TX, kM, true>), grid, dim3(kBlockThreads), shared, s, in, x, y,
+                         (uint32_t)p.rows, p.row_stride, spans, p.m);
+      return hipGetLastError();
+    }
   }
+  note_variant<LinesTag<kKind, kM, false>>();
+  hipLaunchKernelGGL((gguf_matvec_q8_lines<kKind, TX, kM, false>), grid, dim3(kBlockThreads), shared, s, in, x, y,
+                     (uint32_t)p.rows, p.row_stride, spans, p.m);
   return hipGetLastError();
 }
 

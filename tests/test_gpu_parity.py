@@ -75,6 +75,18 @@ def test_config1_broadcast_add_then_scale_f32_bit_exact():
     assert_bits_equal(to_host(fused)[:rows], orc.binary_chain(orc.ADD, orc.MULTIPLY, orc.F32, a[:rows], b, s))
 
 
+def test_binary_broadcast_row_over_a_large_launch_bit_exact():
+    """A[6000, 2048] + b[2048] f32: 98 MB of traffic with a periodic operand, above the size where
+    the launcher changes from fat blocks to one vector per lane."""
+    note("binary f32 [6000,2048] + [2048]")
+    rng = np.random.default_rng(101)
+    a = rng.normal(0, 1, (6000, 2048)).astype(np.float32)
+    b = rng.uniform(-1, 1, 2048).astype(np.float32)
+    (out,) = run(hc.Binary(BK.kAdd), to_device(a, "f32"), to_device(b, "f32"))
+    assert hc.last_launch_variant() == "ew_flat/1x256"
+    assert_bits_equal(to_host(out), a + b[None, :])
+
+
 @pytest.mark.parametrize("tag", ["f32", "bf16"])
 def test_binary_chain_rounds_intermediate_to_storage(tag):
     oid = TYPES[tag][1]
