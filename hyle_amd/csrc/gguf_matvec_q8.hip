@@ -86,9 +86,27 @@ struct LaneCodes {
 template <int kKind, class TX>
 __device__ __forceinline__ LaneCodes quantise_span(const void *x, size_t row_offset, uint32_t span, uint32_t lane) {
   using Kind = Lines<kKind>;
+  // the lane's positions come in runs of eight neighbours (Lines<kind>::position), each a whole
+  // 16-byte vector of a narrow type or two of f32: x starts on a 16-byte boundary (run_m)
   float values[32];
 #pragma unroll
-  for (int e = 0; e < 32; ++e) values[e] = Traits<TX>::load(x, row_offset + Kind::position(span, lane, e));
+  for (int g = 0; g < 4; ++g) {
+    const size_t at = row_offset + Kind::position(span, lane, 8 * g);
+    if constexpr (Traits<TX>::kVec == 8) {
+      float piece[8];
+      Traits<TX>::unpack(load16(x, at / 8), piece);
+#pragma unroll
+      for (int t = 0; t < 8; ++t) values[8 * g + t] = piece[t];
+    } else {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        float piece[4];
+        Traits<TX>::unpack(load16(x, at / 4 + h), piece);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) values[8 * g + 4 * h + t] = piece[t];
+      }
+    }
+  }
   LaneCodes out;
   // Q8_0: the lane's 32 values are one block.  Q6_K: eight lanes share a block of 256.
   // Q4_K: the lane's values 0..15 and 16..31 belong to two blocks of 256, sixteen lanes each.
@@ -1135,9 +1153,11 @@ hipError_t run_registers(const MatVecParams &p, const void *w, const void *x, vo
 
 template <int kKind, class TX>
 hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, int compute_units, hipStream_t s) {
-  // the span kernels: rows of 2048 n values made of whole 16-byte vectors, codes of every activation
-  // row in LDS beside the waves' row buffers (12 KiB); everything else walks block by block
-  if (p.k == 0 || p.k % 2048 != 0 || p.row_stride % 16 != 0 || (reinterpret_cast<uintptr_t>(w) & 15u) != 0 ||
+  // the span kernels: rows of 2048 n values made of whole 16-byte vectors, activations on a 16-byte
+  // boundary, codes of every activation row in LDS beside the waves' row buffers (12 KiB); everything
+  // else walks block by block
+  if (p.k == 0 || p.k % 2048 != 0 || p.row_stride % 16 != 0 ||
+      ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(x)) & 15u) != 0 ||
       gguf_matvec_q8_shared_bytes(p.m, p.k) + 12 * 1024 > 64 * 1024)
     return run_blocks<kKind, TX>(p, w, x, y, compute_units, s);
   const uint32_t spans = p.k / 2048;

@@ -440,6 +440,38 @@ DEVICE_TEST(Q8_0DequantBitExactWithRowSumSquares) {
   EXPECT(close);  // summation order differs from the index-order oracle: 1e-5 relative
 }
 
+// MatMul over a GGUF weight as the reference's ggml CPU route computes it, on one of the reference's own
+// projection widths (1024: tests/compute_models/cpu_c5_gguf_inputs.h:231), held to the bound its tests
+// accept of that route (tests/compute_models/dspark_original_shared_reference.h:219-262).
+DEVICE_TEST(GgufMatMulInTheGgmlRouteArithmeticOverAReferenceWidth) {
+  constexpr std::int64_t n = 200, k = 1024, blocks = k / 32, m = 3;
+  std::mt19937 rng(21);
+  std::vector<std::uint8_t> weight(n * blocks * 34);
+  for (std::int64_t b = 0; b < n * blocks; ++b) {
+    const std::uint16_t d = hyle_oracle_f32_to_f16(std::ldexp(static_cast<float>(rng() % 2048) / 2048.0F + 0.5F, -static_cast<int>(4 + rng() % 8)));
+    std::memcpy(&weight[b * 34], &d, 2);
+    for (int j = 0; j < 32; ++j) weight[b * 34 + 2 + j] = static_cast<std::uint8_t>(rng());
+  }
+  const std::vector<float> x = normal(m * k, 22, 1.5F);
+  const TensorDesc dw = *TensorDesc::gguf_q8_0_weight(DataType::kFloat32, k, n);
+  const TensorDesc dx = *TensorDesc::dense(DataType::kFloat32, {m, k});
+  auto prepared = prepare(fixture().context, GgufMatVec{ActivationArithmetic::kGgmlQ8}, dw, dx);
+  REQUIRE(prepared.has_value());
+  DeviceBuffer bw = upload(weight), bx = upload(x), out = DeviceBuffer::create(m * n * 4).value();
+  auto completion = prepared->create_invocation()->submit(fixture().queue,
+                                                          {*ConstTensorView::create(dw, bw), *ConstTensorView::create(dx, bx)},
+                                                          {*TensorView::create(*prepared->output_description(0), out)});
+  REQUIRE(completion.has_value());
+  EXPECT(completion->wait().ok());
+  EXPECT(std::string(hyle_hip_last_launch_variant()) == "gguf_matvec_q8_blocks/q8_0/4-tokens");
+  std::vector<double> centre(m * n), bound(m * n);
+  hyle_oracle_gguf_matvec_q8(2, weight.data(), n, k, blocks * 34, x.data(), m, centre.data(), bound.data());
+  const auto got = download<float>(out, m * n);
+  bool inside = true;
+  for (std::int64_t i = 0; i < m * n; ++i) inside = inside && std::fabs(static_cast<double>(got[i]) - centre[i]) <= bound[i];
+  EXPECT(inside);
+}
+
 DEVICE_TEST(CastNarrowsWidensAndMaterialisesStridedInputBitExactly) {
   constexpr std::int64_t rows = 257, cols = 2048;
   auto values = normal(rows * cols, 12, 2.0F);
