@@ -725,14 +725,14 @@ def file_stream_rate(mib, ctx, torch, dev):
 # (profiles/hot_path_step_hbm_traffic_pmc.md: FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors
 # the same counters need to read a plain 1 GiB copy correctly).
 TRAFFIC = {
-    "cfg4_softmax_f32_causal": 3256479642,
-    "cfg4_softmax_f32_causal_additive": 4362172313,
-    "cfg3_swiglu_bf16": 302043955,
-    "cfg3_residual_add_bf16": 100731801,
-    "cfg1_broadcast_add_mul_f32": 67302297,
-    "cfg2_rmsnorm_bf16": 67215667,
+    "cfg4_softmax_f32_causal": 3256527872,
+    "cfg4_softmax_f32_causal_additive": 4362134118,
+    "cfg3_swiglu_bf16": 302044160,
+    "cfg3_residual_add_bf16": 100732518,
+    "cfg1_broadcast_add_mul_f32": 67312742,
+    "cfg2_rmsnorm_bf16": 67252838,
     "cfg4_argmax_f32": 39140659,
-    "cfg5_q8_0_dequant_sumsq": 38638592,
+    "cfg5_q8_0_dequant_sumsq": 38641869,
 }
 
 
