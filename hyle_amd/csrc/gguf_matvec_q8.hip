@@ -717,6 +717,150 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_quads(const unsi
   }
 }
 
+// ---- Q4_K, one activation row of 2048 values: the sub-block dots on the matrix unit ---------------
+// v_mfma_i32_16x16x64_i8: lane (c, p) = c + 16 p gives sixteen int8 of row c of A and of column c of
+// B at k-slots 16 p .. 16 p + 15, and gets D[4 p .. 4 p + 3][c] back.  Here a column is a weight row
+// (sixteen per wave) and the sixteen rows of A are sixteen 32-value sub-blocks: row m carries the
+// activation codes of its sub-block at the k-slots whose weights belong to it and zeros elsewhere,
+// so that D[m][c] is the integer dot of sub-block m of weight row c.  A lane loads its operands
+// straight from global memory, 16 quant bytes at a time (a Q4_K block is nine 16-byte vectors: the
+// header, then eight chunks): lane (c, p) takes chunk 4 i + p of block b of row c, whose low nibbles
+// are sixteen values of sub-block 4 i + 2 (p / 2) and whose high nibbles are sixteen of the next
+// one.  The instruction (b, i, nibble) therefore feeds rows 4 b + 2 (p / 2) + nibble of the
+// accumulator of half i, and after four blocks lane (c, p) holds the eight sub-block dots of block
+// p of its row: it alone extracts that block's sixteen six-bit factors, multiplies them in as
+// integers and closes the block in f32.  What the vector unit does per 32 weights is three
+// instructions of nibble masking and a sixteenth of a block's closing arithmetic.
+//
+// A is the same for every weight row, so the block builds the 32 operands of a row of 2048 values
+// once in LDS (32 KiB, one sixteenth of it codes) while its weight bytes are on their way, and
+// every instruction reads its operand at a fixed offset.
+constexpr uint32_t kTileRows = 16;    // weight rows of a wave
+constexpr uint64_t kTileMinimumRows = 16;  // fewer rows: the span kernel
+constexpr uint32_t kTileSlices = 32;  // matrix instructions per 2048 values: (group of four blocks, block, half, nibble)
+
+struct TileShared {
+  u32x4 operand[kTileSlices][kWaveLanes];
+  int sums[8][8];   // [activation block][sub-block]: sum of the 32 codes
+  float scale[8];   // of the activation blocks
+};
+
+// Block barrier that orders LDS accesses only: the weight loads issued before it stay in flight.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Thread t of the block quantises values 8 t .. 8 t + 7 of the activation row (Q8_K: a block of 256
+// is 32 adjacent lanes) and files the codes where the instructions expect them.
+template <class TX>
+__device__ __forceinline__ void tile_operands(TileShared &shared, const void *x, uint32_t t) {
+  float values[8];
+  if constexpr (Traits<TX>::kVec == 8) {
+    Traits<TX>::unpack(load16(x, t), values);
+  } else {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      float piece[4];
+      Traits<TX>::unpack(load16(x, 2 * (size_t)t + h), piece);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) values[4 * h + e] = piece[e];
+    }
+  }
+  u32x4 *flat = &shared.operand[0][0];
+#pragma unroll
+  for (uint32_t j = 0; j < kTileSlices * kWaveLanes / kBlockThreads; ++j) flat[t + j * kBlockThreads] = u32x4{0u, 0u, 0u, 0u};
+  LaneMax mine{0.0f, 0.0f, 0u};
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {  // positions rise with e, so ">" keeps the first
+    const float magnitude = __builtin_fabsf(values[e]);
+    if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], 8 * t + (uint32_t)e};
+  }
+  if (mine.magnitude == 0.0f) mine.position = 0xFFFFFFFFu;
+  const LaneMax top = block_largest<32>(mine);
+  float factor = 0.0f, stored = 0.0f;
+  if (top.magnitude != 0.0f) {
+    factor = -127.0f / top.value;
+    stored = 1.0f / factor;
+  }
+  uint32_t words[2];
+#pragma unroll
+  for (int w = 0; w < 2; ++w) {
+    uint32_t word = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) word |= code_of(values[4 * w + e] * factor) << (8 * e);
+    words[w] = top.magnitude != 0.0f ? word : 0u;
+  }
+  int sum = dot4(0x01010101u, words[0], dot4(0x01010101u, words[1], 0));
+  sum += dpp_move<kDppSwap1>(sum);
+  sum += dpp_move<kDppSwap2>(sum);  // the four lanes of a 32-value sub-block
+  lds_barrier();  // the zeros are in place
+  // position 8 u of block B: 64-value group j, nibble, half h of the chunk pair, bytes 8 (u % 2) .. + 7
+  const uint32_t block = t / 32, u = t % 32;
+  const uint32_t j = u / 8, nibble = (u / 4) % 2, h = (u / 2) % 2;
+  const uint32_t part = 2 * (j % 2) + h, row = 4 * (block % 4) + 2 * (j % 2) + nibble;
+  const uint32_t slice = (((block / 4) * 4 + block % 4) * 2 + j / 2) * 2 + nibble;
+  uint32_t *at = reinterpret_cast<uint32_t *>(&shared.operand[slice][row + 16 * part]) + 2 * (u % 2);
+  at[0] = words[0];
+  at[1] = words[1];
+  if (u % 4 == 0) shared.sums[block][u / 4] = sum;
+  if (u == 0) shared.scale[block] = stored;
+  lds_barrier();
+}
+
+template <class TX>
+__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_tiles(const unsigned char *weights, const void *x, void *y,
+                                                                      uint32_t rows, uint64_t row_stride) {
+  __shared__ TileShared shared;
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  const uint32_t column = lane % 16, part = lane / 16;
+  const uint32_t row = (blockIdx.x * kWavesPerBlock + wave) * kTileRows + column;
+  // rows past the last repeat it (valid addresses) and are not stored
+  const unsigned char *mine = weights + (size_t)(row < rows ? row : rows - 1) * row_stride;
+  u32x4 head[2], quants[2][4][2];
+#pragma unroll
+  for (uint32_t g = 0; g < 2; ++g) {
+    head[g] = load16(mine, (4 * g + part) * 9);
+#pragma unroll
+    for (uint32_t b = 0; b < 4; ++b)
+#pragma unroll
+      for (uint32_t i = 0; i < 2; ++i) quants[g][b][i] = load16(mine, (4 * g + b) * 9 + 1 + 4 * i + part);
+  }
+  tile_operands<TX>(shared, x, threadIdx.x);
+  float total = 0.0f;
+#pragma unroll
+  for (uint32_t g = 0; g < 2; ++g) {
+    i32x4 dots[2] = {i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}};
+#pragma unroll
+    for (uint32_t b = 0; b < 4; ++b) {
+#pragma unroll
+      for (uint32_t i = 0; i < 2; ++i) {
+        const u32x4 q = quants[g][b][i];
+        const u32x4 low = q & 0x0F0F0F0Fu, high = (q >> 4) & 0x0F0F0F0Fu;
+        const uint32_t slice = ((g * 4 + b) * 2 + i) * 2;
+        dots[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8((i32x4)shared.operand[slice][lane], (i32x4)low, dots[i], 0, 0, 0);
+        dots[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8((i32x4)shared.operand[slice + 1][lane], (i32x4)high, dots[i], 0, 0, 0);
+      }
+    }
+    // block 4 g + part of the lane's row
+    const u32x4 h = head[g];
+    const int *sums = shared.sums[4 * g + part];
+    int scaled = 0, minima = 0;
+#pragma unroll
+    for (uint32_t s = 0; s < 8; ++s) {
+      scaled = mad24(q4k_six_bits(h.y, h.z, h.w, s, false), dots[s / 4][s % 4], scaled);
+      minima = mad24(q4k_six_bits(h.y, h.z, h.w, s, true), sums[s], minima);
+    }
+    const float d = f16_to_f32((uint16_t)h.x), dmin = f16_to_f32((uint16_t)(h.x >> 16));
+    total += shared.scale[4 * g + part] * (d * (float)scaled - dmin * (float)minima);
+  }
+  total += __shfl_xor(total, 16, kWaveLanes);
+  total += __shfl_xor(total, 32, kWaveLanes);
+  if (part == 0 && row < rows) Traits<TX>::store(y, (size_t)row, total);
+}
+
 inline const char *kind_word(int kind) { return kind == 0 ? "q4_k" : (kind == 1 ? "q6_k" : "q8_0"); }
 // gguf_matvec_q8_<form>/<format>[/<detail>]
 template <int kKind, int kSets, bool kRegisters> struct QuadsTag {
@@ -731,6 +875,9 @@ template <int kKind, int kM, bool kRegisters> struct LinesTag {
 };
 template <int kKind, int kSpans> struct SpansTag {
   static std::string text() { return std::string("gguf_matvec_q8_spans/") + kind_word(kKind) + "/" + std::to_string(kSpans) + "-spans"; }
+};
+struct TilesTag {
+  static std::string text() { return "gguf_matvec_q8_tiles/q4_k"; }
 };
 template <int kKind, int kM> struct BlocksTag {
   static std::string text() { return std::string("gguf_matvec_q8_blocks/") + kind_word(kKind) + "/" + std::to_string(kM) + "-tokens"; }
@@ -1169,6 +1316,16 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
     // several activation rows: the quad form, if its four row slots per wave fit beside the codes
     const size_t slots = (size_t)kWavesPerBlock * 4 * (LinesRow<kKind, 1>::kSlotBytes + 32);
     if (p.m >= 2 && slots + shared <= 64 * 1024) return run_quads<kKind, TX>(p, w, x, y, spans, grid, shared, s);
+  }
+  if constexpr (kKind == 0) {
+    // Q4_K, one activation row of 2048 values: sixteen weight rows per wave on the matrix unit
+    if (p.m == 1 && spans == 1 && p.rows >= kTileMinimumRows) {
+      const uint32_t tiles = (uint32_t)((p.rows + kTileRows - 1) / kTileRows);
+      note_variant<TilesTag>();
+      hipLaunchKernelGGL((gguf_matvec_q8_tiles<TX>), dim3((tiles + kWavesPerBlock - 1) / kWavesPerBlock), dim3(kBlockThreads), 0, s,
+                         static_cast<const unsigned char *>(w), x, y, (uint32_t)p.rows, p.row_stride);
+      return hipGetLastError();
+    }
   }
   if (p.m == 1 && spans <= 6) {
     // One activation row: a wave per span.  Eight waves per compute unit measured best or equal in

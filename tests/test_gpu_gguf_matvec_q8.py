@@ -214,3 +214,32 @@ def test_q8_route_declines_what_it_does_not_serve():
                        (hc.GgufQuantizedType.kQ8_0, 32, 1)):
         weight = hc.TensorDesc.gguf_weight(gguf, hc.DataType.kFloat32, k, 16)
         hc.prepare(ctx, Q8, weight, hc.TensorDesc.dense(hc.DataType.kFloat32, [m, k] if m > 1 else [k]))
+
+
+@pytest.mark.parametrize("x_tag", ["f32", "bf16", "f16"])
+def test_q8_route_q4_k_sub_block_dots_on_the_matrix_unit(x_tag):
+    """Q4_K, one activation row of 2048 values: sixteen weight rows per wave, every 32-value sub-block
+    dot from a 16 x 16 x 64 int8 matrix instruction.  Row counts around the wave's sixteen and the
+    block's sixty-four, every scale slot and nibble pattern (raw bytes), activation blocks of zeros
+    and of equal magnitudes, rows further apart than their blocks."""
+    rng = np.random.default_rng(1810)
+    k = 2048
+    for rows in (16, 17, 31, 63, 64, 65, 200, 1037):
+        raw = raw_bytes_for("q4_k", rng, rows, k)
+        x = rng.normal(0, 2, k).astype(np.float32)
+        if rows % 2:
+            x[256:512] = 0.0
+            x[512:768] = np.where(np.arange(256) % 2 == 0, 1.25, -1.25)
+            x[1999] = 40.0
+        note(f"q8 matvec q4_k tiles x {x_tag} rows {rows}")
+        check("q4_k", x_tag, raw, rows, k, x, kernel="gguf_matvec_q8_tiles/q4_k")
+    rows = 70
+    raw = raw_bytes_for("q4_k", rng, rows, k)
+    padded = np.zeros((rows, raw.shape[1] + 48), np.uint8)
+    padded[:, :raw.shape[1]] = raw
+    note(f"q8 matvec q4_k tiles x {x_tag}: rows 48 bytes further apart than their blocks")
+    check("q4_k", x_tag, padded, rows, k, rng.normal(0, 1, k).astype(np.float32), row_stride=raw.shape[1] + 48,
+          kernel="gguf_matvec_q8_tiles/q4_k")
+    note(f"q8 matvec q4_k x {x_tag}: fewer than sixteen rows keep the span kernel")
+    check("q4_k", x_tag, raw_bytes_for("q4_k", rng, 15, k), 15, k, rng.normal(0, 1, k).astype(np.float32),
+          kernel="gguf_matvec_q8_spans/q4_k/1-spans")
