@@ -26,6 +26,8 @@
 //   Q4_K  nibbles are already bytes 0..15; sc * dot and m * (sum of activation codes) stay
 //         integers; d * a.scale and dmin * a.scale close the sub-blocks
 //   Q8_0  the bytes are the int8 quants; d * a.scale closes the block
+#include <type_traits>
+
 #include "device_common.h"
 #include "gguf_decode.h"
 #include "gguf_lines.h"
@@ -717,33 +719,45 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_quads(const unsi
   }
 }
 
-// ---- Q4_K, one activation row of 2048 values: the sub-block dots on the matrix unit ---------------
+// ---- Q4_K: the sub-block dots on the matrix unit --------------------------------------------------
 // v_mfma_i32_16x16x64_i8: lane (c, p) = c + 16 p gives sixteen int8 of row c of A and of column c of
 // B at k-slots 16 p .. 16 p + 15, and gets D[4 p .. 4 p + 3][c] back.  Here a column is a weight row
-// (sixteen per wave) and the sixteen rows of A are sixteen 32-value sub-blocks: row m carries the
-// activation codes of its sub-block at the k-slots whose weights belong to it and zeros elsewhere,
-// so that D[m][c] is the integer dot of sub-block m of weight row c.  A lane loads its operands
-// straight from global memory, 16 quant bytes at a time (a Q4_K block is nine 16-byte vectors: the
-// header, then eight chunks): lane (c, p) takes chunk 4 i + p of block b of row c, whose low nibbles
+// (sixteen per wave) and B is its nibbles: a lane loads its operands straight from global memory,
+// 16 quant bytes at a time (a Q4_K block is nine 16-byte vectors: the header, then eight chunks).
+// In a group of four blocks lane (c, p) takes chunk 4 i + p of block b of row c, whose low nibbles
 // are sixteen values of sub-block 4 i + 2 (p / 2) and whose high nibbles are sixteen of the next
-// one.  The instruction (b, i, nibble) therefore feeds rows 4 b + 2 (p / 2) + nibble of the
-// accumulator of half i, and after four blocks lane (c, p) holds the eight sub-block dots of block
-// p of its row: it alone extracts that block's sixteen six-bit factors, multiplies them in as
-// integers and closes the block in f32.  What the vector unit does per 32 weights is three
-// instructions of nibble masking and a sixteenth of a block's closing arithmetic.
+// one.  What the vector unit does per 32 weights is three instructions of nibble masking.
 //
-// A is the same for every weight row, so the block builds the 32 operands of a row of 2048 values
-// once in LDS (32 KiB, one sixteenth of it codes) while its weight bytes are on their way, and
-// every instruction reads its operand at a fixed offset.
-constexpr uint32_t kTileRows = 16;    // weight rows of a wave
-constexpr uint64_t kTileMinimumRows = 16;  // fewer rows: the span kernel
-constexpr uint32_t kTileSlices = 32;  // matrix instructions per 2048 values: (group of four blocks, block, half, nibble)
+// The rows of A keep the 32-value sub-blocks apart: a row carries activation codes at the k-slots
+// whose weights belong to its sub-block and zeros elsewhere, so that D[row][c] is one integer
+// sub-block dot of weight row c.
+//   One activation row: the sixteen rows are four sub-blocks of each of the group's four blocks;
+//   instruction (b, i, nibble) feeds rows 4 b + 2 (p / 2) + nibble of the accumulator of half i, and
+//   after the four blocks lane (c, p) holds the eight sub-block dots of block p of its row.
+//   Four activation rows (eight: two sets): the sixteen rows are four sub-blocks of four activation
+//   rows; instruction (i, nibble) of a block feeds rows 4 t + 2 (p / 2) + nibble, and after the
+//   block lane (c, p) holds its eight sub-block dots against activation row p.
+// Either way one lane per (weight row, block, activation row) extracts the block's six-bit factors,
+// multiplies them in as integers and closes the block in f32.
+//
+// A lane's share of an A operand is nonzero for one instruction in eight (in two): its sixteen
+// codes sit in LDS in their natural order behind a row of zeros, and the lane reads every operand
+// at "its base for this instruction + what the instruction adds for all lanes", where the base is
+// its codes' for the instruction that wants them and the row of zeros' for the others.  The block
+// quantises the activation rows once while its first weight bytes are on their way.
+constexpr uint32_t kTileRows = 16;  // weight rows of a wave
 
-struct TileShared {
-  u32x4 operand[kTileSlices][kWaveLanes];
-  int sums[8][8];   // [activation block][sub-block]: sum of the 32 codes
-  float scale[8];   // of the activation blocks
+struct TileGroup {  // what a lane holds of four blocks of its weight row
+  u32x4 head;          // of block `part` of the group
+  u32x4 quants[4][2];  // chunk 4 i + part of block b
 };
+
+// Shared memory of a block: zeros [K] | codes [tokens][K] | sums [tokens][blocks][8] | scales [tokens][blocks] |
+// shares [waves][64][tokens / 4 or 1]
+__host__ __device__ inline size_t tile_shared_bytes(uint32_t tokens, uint32_t blocks) {
+  return (size_t)(1 + tokens) * blocks * 256 + (size_t)tokens * blocks * (32 + 4) +
+         (size_t)kWavesPerBlock * kWaveLanes * (tokens >= 4 ? tokens / 4 : 1) * 4;
+}
 
 // Block barrier that orders LDS accesses only: the weight loads issued before it stay in flight.
 __device__ __forceinline__ void lds_barrier() {
@@ -752,30 +766,41 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
-// Thread t of the block quantises values 8 t .. 8 t + 7 of the activation row (Q8_K: a block of 256
-// is 32 adjacent lanes) and files the codes where the instructions expect them.
+// Half a wave quantises an activation block of 256 values (Q8_K), eight values per lane.
+struct TileValues {
+  u32x4 raw[2];
+};
+template <class TX> __device__ __forceinline__ TileValues tile_fetch(const void *x, size_t first, uint32_t u) {
+  TileValues out;
+  if constexpr (Traits<TX>::kVec == 8) {
+    out.raw[0] = load16(x, first / 8 + u);
+    out.raw[1] = out.raw[0];
+  } else {
+    out.raw[0] = load16(x, first / 4 + 2 * (size_t)u);
+    out.raw[1] = load16(x, first / 4 + 2 * (size_t)u + 1);
+  }
+  return out;
+}
 template <class TX>
-__device__ __forceinline__ void tile_operands(TileShared &shared, const void *x, uint32_t t) {
+__device__ __forceinline__ void tile_quantise(const TileValues &fetched, uint32_t u, unsigned char *codes, int *sums,
+                                              float *scale) {
   float values[8];
   if constexpr (Traits<TX>::kVec == 8) {
-    Traits<TX>::unpack(load16(x, t), values);
+    Traits<TX>::unpack(fetched.raw[0], values);
   } else {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       float piece[4];
-      Traits<TX>::unpack(load16(x, 2 * (size_t)t + h), piece);
+      Traits<TX>::unpack(fetched.raw[h], piece);
 #pragma unroll
       for (int e = 0; e < 4; ++e) values[4 * h + e] = piece[e];
     }
   }
-  u32x4 *flat = &shared.operand[0][0];
-#pragma unroll
-  for (uint32_t j = 0; j < kTileSlices * kWaveLanes / kBlockThreads; ++j) flat[t + j * kBlockThreads] = u32x4{0u, 0u, 0u, 0u};
   LaneMax mine{0.0f, 0.0f, 0u};
 #pragma unroll
   for (int e = 0; e < 8; ++e) {  // positions rise with e, so ">" keeps the first
     const float magnitude = __builtin_fabsf(values[e]);
-    if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], 8 * t + (uint32_t)e};
+    if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], 8 * u + (uint32_t)e};
   }
   if (mine.magnitude == 0.0f) mine.position = 0xFFFFFFFFu;
   const LaneMax top = block_largest<32>(mine);
@@ -795,70 +820,254 @@ __device__ __forceinline__ void tile_operands(TileShared &shared, const void *x,
   int sum = dot4(0x01010101u, words[0], dot4(0x01010101u, words[1], 0));
   sum += dpp_move<kDppSwap1>(sum);
   sum += dpp_move<kDppSwap2>(sum);  // the four lanes of a 32-value sub-block
-  lds_barrier();  // the zeros are in place
-  // position 8 u of block B: 64-value group j, nibble, half h of the chunk pair, bytes 8 (u % 2) .. + 7
-  const uint32_t block = t / 32, u = t % 32;
-  const uint32_t j = u / 8, nibble = (u / 4) % 2, h = (u / 2) % 2;
-  const uint32_t part = 2 * (j % 2) + h, row = 4 * (block % 4) + 2 * (j % 2) + nibble;
-  const uint32_t slice = (((block / 4) * 4 + block % 4) * 2 + j / 2) * 2 + nibble;
-  uint32_t *at = reinterpret_cast<uint32_t *>(&shared.operand[slice][row + 16 * part]) + 2 * (u % 2);
+  uint32_t *at = reinterpret_cast<uint32_t *>(codes) + 2 * u;
   at[0] = words[0];
   at[1] = words[1];
-  if (u % 4 == 0) shared.sums[block][u / 4] = sum;
-  if (u == 0) shared.scale[block] = stored;
-  lds_barrier();
+  if (u % 4 == 0) sums[u / 4] = sum;
+  if (u == 0) *scale = stored;
 }
 
-template <class TX>
-__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_tiles(const unsigned char *weights, const void *x, void *y,
-                                                                      uint32_t rows, uint64_t row_stride) {
-  __shared__ TileShared shared;
-  const uint32_t lane = threadIdx.x % kWaveLanes;
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
-  const uint32_t column = lane % 16, part = lane / 16;
-  const uint32_t row = (blockIdx.x * kWavesPerBlock + wave) * kTileRows + column;
-  // rows past the last repeat it (valid addresses) and are not stored
-  const unsigned char *mine = weights + (size_t)(row < rows ? row : rows - 1) * row_stride;
-  u32x4 head[2], quants[2][4][2];
+// The sixteen six-bit factors of a block: sc[s] and mn[s] of sub-block s.
+struct TileFactors {
+  int sc[8], mn[8];
+  float d, dmin;
+  __device__ __forceinline__ explicit TileFactors(const u32x4 &h) {
 #pragma unroll
-  for (uint32_t g = 0; g < 2; ++g) {
-    head[g] = load16(mine, (4 * g + part) * 9);
-#pragma unroll
-    for (uint32_t b = 0; b < 4; ++b)
-#pragma unroll
-      for (uint32_t i = 0; i < 2; ++i) quants[g][b][i] = load16(mine, (4 * g + b) * 9 + 1 + 4 * i + part);
-  }
-  tile_operands<TX>(shared, x, threadIdx.x);
-  float total = 0.0f;
-#pragma unroll
-  for (uint32_t g = 0; g < 2; ++g) {
-    i32x4 dots[2] = {i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}};
-#pragma unroll
-    for (uint32_t b = 0; b < 4; ++b) {
-#pragma unroll
-      for (uint32_t i = 0; i < 2; ++i) {
-        const u32x4 q = quants[g][b][i];
-        const u32x4 low = q & 0x0F0F0F0Fu, high = (q >> 4) & 0x0F0F0F0Fu;
-        const uint32_t slice = ((g * 4 + b) * 2 + i) * 2;
-        dots[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8((i32x4)shared.operand[slice][lane], (i32x4)low, dots[i], 0, 0, 0);
-        dots[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8((i32x4)shared.operand[slice + 1][lane], (i32x4)high, dots[i], 0, 0, 0);
-      }
+    for (uint32_t s = 0; s < 8; ++s) {
+      sc[s] = q4k_six_bits(h.y, h.z, h.w, s, false);
+      mn[s] = q4k_six_bits(h.y, h.z, h.w, s, true);
     }
-    // block 4 g + part of the lane's row
-    const u32x4 h = head[g];
-    const int *sums = shared.sums[4 * g + part];
+    d = f16_to_f32((uint16_t)h.x);
+    dmin = f16_to_f32((uint16_t)(h.x >> 16));
+  }
+  // dots[i][r]: sub-block 4 i + r against the activation block whose sub-block sums are `sum`
+  __device__ __forceinline__ float close(const i32x4 (&dots)[2], const int *sum, float scale) const {
     int scaled = 0, minima = 0;
 #pragma unroll
     for (uint32_t s = 0; s < 8; ++s) {
-      scaled = mad24(q4k_six_bits(h.y, h.z, h.w, s, false), dots[s / 4][s % 4], scaled);
-      minima = mad24(q4k_six_bits(h.y, h.z, h.w, s, true), sums[s], minima);
+      scaled = mad24(sc[s], dots[s / 4][s % 4], scaled);
+      minima = mad24(mn[s], sum[s], minima);
     }
-    const float d = f16_to_f32((uint16_t)h.x), dmin = f16_to_f32((uint16_t)(h.x >> 16));
-    total += shared.scale[4 * g + part] * (d * (float)scaled - dmin * (float)minima);
+    return scale * (d * (float)scaled - dmin * (float)minima);
   }
-  total += __shfl_xor(total, 16, kWaveLanes);
-  total += __shfl_xor(total, 32, kWaveLanes);
-  if (part == 0 && row < rows) Traits<TX>::store(y, (size_t)row, total);
+};
+
+// `blocks` >= 4 Q4_K blocks per row.  kSets == 0: one activation row; kSets == 1, 2: four or eight
+// (rows past m repeat the last one and are not stored).  1 << split_log2 waves share a tile of
+// sixteen weight rows: wave w of them walks the groups w, w + split, ... and the first adds the
+// shares in wave order.
+template <class TX, int kSets, bool kOneBatch>
+__global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_tiles(const unsigned char *weights, const void *x, void *y,
+                                                                      uint32_t rows, uint64_t row_stride, uint32_t blocks,
+                                                                      uint32_t m, uint32_t split_log2) {
+  constexpr uint32_t kTokens = kSets == 0 ? 1 : 4 * kSets;
+  constexpr int kTotals = kSets == 0 ? 1 : kSets;
+  extern __shared__ __align__(16) unsigned char shared[];
+  const uint32_t k = blocks * 256;
+  unsigned char *codes = shared + k;  // behind the row of zeros
+  int *sums = reinterpret_cast<int *>(shared + (size_t)(1 + kTokens) * k);
+  float *scales = reinterpret_cast<float *>(sums + (size_t)kTokens * blocks * 8);
+  float *shares = scales + (size_t)kTokens * blocks;
+  const uint32_t lane = threadIdx.x % kWaveLanes;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWaveLanes);
+  const uint32_t column = lane % 16, part = lane / 16;
+  const uint32_t split = 1u << split_log2, member = wave & (split - 1);
+  const uint32_t row = ((blockIdx.x * kWavesPerBlock + wave) >> split_log2) * kTileRows + column;
+  // rows past the last repeat it (valid addresses) and are not stored
+  const unsigned char *mine = weights + (size_t)(row < rows ? row : rows - 1) * row_stride;
+  const uint32_t groups = (blocks + 3) / 4;
+  // A row's last group starts at its fourth block from the end: when the row is not a whole number
+  // of groups it overlaps the one before, and the blocks they share are skipped.
+  auto start_of = [&](uint32_t g) { return 4 * g + 4 <= blocks ? 4 * g : blocks - 4; };
+  const unsigned char *heads = mine + part * 144, *chunks = mine + 16 + part * 16;
+  auto load_group = [&](uint32_t g) {
+    TileGroup out;
+    const size_t start = (size_t)start_of(g) * 144;
+    out.head = load16(heads + start, 0);
+#pragma unroll
+    for (uint32_t b = 0; b < 4; ++b)
+#pragma unroll
+      for (uint32_t i = 0; i < 2; ++i) out.quants[b][i] = load16(chunks + start, b * 9 + 4 * i);
+    return out;
+  };
+  auto clamped = [&](uint32_t g) { return g < groups ? g : groups - 1; };
+  // activation blocks go round the block's eight half waves, four of a half wave's loads in flight; the
+  // first four are asked for before the weights: loads return in order
+  constexpr uint32_t kHalves = kBlockThreads / 32, kBatch = 4;
+  const uint32_t half = threadIdx.x / 32, u = threadIdx.x % 32;
+  const uint32_t units = kTokens * blocks;
+  auto fetch_batch = [&](uint32_t first, TileValues (&fetched)[kBatch]) {
+#pragma unroll
+    for (uint32_t j = 0; j < kBatch; ++j) {
+      const uint32_t unit = first + j * kHalves < units ? first + j * kHalves : units - 1;
+      const uint32_t token = unit / blocks, block = unit - token * blocks;
+      fetched[j] = tile_fetch<TX>(x, (size_t)(token < m ? token : m - 1) * k + (size_t)block * 256, u);
+    }
+  };
+  auto quantise_batch = [&](uint32_t first, const TileValues (&fetched)[kBatch]) {
+#pragma unroll
+    for (uint32_t j = 0; j < kBatch; ++j) {
+      const uint32_t unit = first + j * kHalves;
+      if (unit < units) tile_quantise<TX>(fetched[j], u, codes + (size_t)unit * 256, sums + (size_t)unit * 8, scales + unit);
+    }
+  };
+  TileValues fetched[kBatch];
+  fetch_batch(half, fetched);
+  TileGroup ring[2];
+  ring[0] = load_group(clamped(member));
+  ring[1] = load_group(clamped(member + split));
+  for (uint32_t at = threadIdx.x * 16; at < k; at += kBlockThreads * 16) *reinterpret_cast<u32x4 *>(shared + at) = u32x4{0u, 0u, 0u, 0u};
+  quantise_batch(half, fetched);
+  if constexpr (!kOneBatch) {  // more than 32 activation blocks: the rest wait for the weights before them
+    for (uint32_t first = half + kHalves * kBatch; first < units; first += kHalves * kBatch) {
+      fetch_batch(first, fetched);
+      quantise_batch(first, fetched);
+    }
+  }
+  lds_barrier();
+  float totals[kTotals] = {};
+  if constexpr (kSets == 0) {
+    // rows of A: 4 b + 2 (part / 2) + nibble.  The lane's codes (block column / 4 of the group, nibble
+    // column % 2, if column / 2 and part / 2 agree in their low bit) go to instruction (b, nibble).
+    uint32_t base[4][2];
+    {
+      const bool faces = ((column >> 1) & 1u) == (part >> 1);
+      const uint32_t own = k + (column / 4) * 256 + (part >> 1) * 64 + (column & 1u) * 32 + (part & 1u) * 16;
+#pragma unroll
+      for (uint32_t b = 0; b < 4; ++b)
+#pragma unroll
+        for (uint32_t nibble = 0; nibble < 2; ++nibble) base[b][nibble] = faces && column / 4 == b && (column & 1u) == nibble ? own : 0u;
+    }
+    auto work = [&](const TileGroup &held, uint32_t g, auto whole) {
+      constexpr bool kWhole = decltype(whole)::value;  // the usual group, none of its blocks skipped: no branch in it
+      const uint32_t start = start_of(g), skipped = kWhole ? 0u : 4 * g - start;
+      i32x4 dots[2] = {i32x4{0, 0, 0, 0}, i32x4{0, 0, 0, 0}};
+#pragma unroll
+      for (uint32_t b = 0; b < 4; ++b) {
+        if (!kWhole && b < skipped) continue;  // the same for the whole wave
+#pragma unroll
+        for (uint32_t i = 0; i < 2; ++i) {
+          const u32x4 q = held.quants[b][i];
+          const u32x4 nibbles[2] = {q & 0x0F0F0F0Fu, (q >> 4) & 0x0F0F0F0Fu};
+#pragma unroll
+          for (uint32_t nibble = 0; nibble < 2; ++nibble) {
+            const u32x4 operand = *reinterpret_cast<const u32x4 *>(shared + base[b][nibble] + start * 256 + i * 128);
+            dots[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8((i32x4)operand, (i32x4)nibbles[nibble], dots[i], 0, 0, 0);
+          }
+        }
+      }
+      if (kWhole || part >= skipped) {  // block start + part of the lane's row
+        const uint32_t block = start + part;
+        totals[0] += TileFactors(held.head).close(dots, sums + (size_t)block * 8, scales[block]);
+      }
+    };
+    auto step = [&](const TileGroup &held, uint32_t g) {
+      if (4 * g + 4 <= blocks) work(held, g, std::true_type{});
+      else work(held, g, std::false_type{});
+    };
+    if (member + 2 * split >= groups) {
+      // at most two groups, both in flight: straight-line code, every block starts as soon as its bytes are there
+      step(ring[0], member);
+      if (member + split < groups) step(ring[1], member + split);
+    } else {
+      for (uint32_t g = member; g < groups; g += 2 * split) {
+#pragma unroll
+        for (uint32_t slot = 0; slot < 2; ++slot) {
+          const uint32_t now = g + slot * split;
+          if (now >= groups) break;
+          step(ring[slot], now);
+          if (now + 2 * split < groups) ring[slot] = load_group(now + 2 * split);  // the other slot's bytes are in flight
+        }
+      }
+    }
+    totals[0] += __shfl_xor(totals[0], 16, kWaveLanes);
+    totals[0] += __shfl_xor(totals[0], 32, kWaveLanes);
+  } else {
+    // rows of A: 4 t + 2 (part / 2) + nibble for activation row t of a set.  The lane's codes
+    // (activation row column / 4, nibble column % 2, if column / 2 and part / 2 agree in their low
+    // bit) go to the instructions of that nibble.
+    uint32_t base[kSets][2];
+    {
+      const bool faces = ((column >> 1) & 1u) == (part >> 1);
+#pragma unroll
+      for (uint32_t set = 0; set < (uint32_t)kSets; ++set) {
+        const uint32_t own = k * (1 + 4 * set + column / 4) + (part >> 1) * 64 + (column & 1u) * 32 + (part & 1u) * 16;
+#pragma unroll
+        for (uint32_t nibble = 0; nibble < 2; ++nibble) base[set][nibble] = faces && (column & 1u) == nibble ? own : 0u;
+      }
+    }
+    auto work = [&](const TileGroup &held, uint32_t g, auto whole) {
+      constexpr bool kWhole = decltype(whole)::value;
+      const uint32_t start = start_of(g), skipped = kWhole ? 0u : 4 * g - start;
+#pragma unroll
+      for (uint32_t b = 0; b < 4; ++b) {
+        if (!kWhole && b < skipped) continue;  // the same for the whole wave
+        const uint32_t block = start + b;
+        i32x4 dots[kSets][2];
+#pragma unroll
+        for (int set = 0; set < kSets; ++set) dots[set][0] = dots[set][1] = i32x4{0, 0, 0, 0};
+#pragma unroll
+        for (uint32_t i = 0; i < 2; ++i) {
+          const u32x4 q = held.quants[b][i];
+          const u32x4 nibbles[2] = {q & 0x0F0F0F0Fu, (q >> 4) & 0x0F0F0F0Fu};
+#pragma unroll
+          for (uint32_t nibble = 0; nibble < 2; ++nibble) {
+#pragma unroll
+            for (int set = 0; set < kSets; ++set) {
+              const u32x4 operand = *reinterpret_cast<const u32x4 *>(shared + base[set][nibble] + block * 256 + i * 128);
+              dots[set][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8((i32x4)operand, (i32x4)nibbles[nibble], dots[set][i], 0, 0, 0);
+            }
+          }
+        }
+        // the header of block b is with lane (column, b); the lane closes the block against activation row part of every set
+        const int from = (int)(column + 16 * b);
+        const TileFactors factors(u32x4{(uint32_t)__shfl((int)held.head.x, from, kWaveLanes), (uint32_t)__shfl((int)held.head.y, from, kWaveLanes),
+                                        (uint32_t)__shfl((int)held.head.z, from, kWaveLanes), (uint32_t)__shfl((int)held.head.w, from, kWaveLanes)});
+#pragma unroll
+        for (int set = 0; set < kSets; ++set) {
+          const uint32_t unit = (4 * (uint32_t)set + part) * blocks + block;
+          totals[set] += factors.close(dots[set], sums + (size_t)unit * 8, scales[unit]);
+        }
+      }
+    };
+    auto step = [&](const TileGroup &held, uint32_t g) {
+      if (4 * g + 4 <= blocks) work(held, g, std::true_type{});
+      else work(held, g, std::false_type{});
+    };
+    if (member + 2 * split >= groups) {
+      // at most two groups, both in flight: straight-line code, every block starts as soon as its bytes are there
+      step(ring[0], member);
+      if (member + split < groups) step(ring[1], member + split);
+    } else {
+      for (uint32_t g = member; g < groups; g += 2 * split) {
+#pragma unroll
+        for (uint32_t slot = 0; slot < 2; ++slot) {
+          const uint32_t now = g + slot * split;
+          if (now >= groups) break;
+          step(ring[slot], now);
+          if (now + 2 * split < groups) ring[slot] = load_group(now + 2 * split);  // the other slot's bytes are in flight
+        }
+      }
+    }
+  }
+  if (split_log2 != 0) {
+#pragma unroll
+    for (int t = 0; t < kTotals; ++t) shares[((size_t)wave * kWaveLanes + lane) * kTotals + t] = totals[t];
+    lds_barrier();
+    if (member != 0) return;
+#pragma unroll
+    for (int t = 0; t < kTotals; ++t)
+      for (uint32_t other = 1; other < split; ++other) totals[t] += shares[((size_t)(wave + other) * kWaveLanes + lane) * kTotals + t];
+  }
+  if (row < rows) {
+    if constexpr (kSets == 0) {
+      if (part == 0) Traits<TX>::store(y, (size_t)row, totals[0]);
+    } else {
+#pragma unroll
+      for (uint32_t set = 0; set < (uint32_t)kSets; ++set)
+        if (4 * set + part < m) Traits<TX>::store(y, (size_t)(4 * set + part) * rows + row, totals[set]);
+    }
+  }
 }
 
 inline const char *kind_word(int kind) { return kind == 0 ? "q4_k" : (kind == 1 ? "q6_k" : "q8_0"); }
@@ -876,8 +1085,10 @@ template <int kKind, int kM, bool kRegisters> struct LinesTag {
 template <int kKind, int kSpans> struct SpansTag {
   static std::string text() { return std::string("gguf_matvec_q8_spans/") + kind_word(kKind) + "/" + std::to_string(kSpans) + "-spans"; }
 };
-struct TilesTag {
-  static std::string text() { return "gguf_matvec_q8_tiles/q4_k"; }
+template <int kSets, bool kOneBatch> struct TilesTag {
+  static std::string text() {
+    return "gguf_matvec_q8_tiles/q4_k/" + std::to_string(kSets == 0 ? 1 : 4 * kSets) + "-tokens" + (kOneBatch ? "" : "/long");
+  }
 };
 template <int kKind, int kM> struct BlocksTag {
   static std::string text() { return std::string("gguf_matvec_q8_blocks/") + kind_word(kKind) + "/" + std::to_string(kM) + "-tokens"; }
@@ -1298,8 +1509,51 @@ hipError_t run_registers(const MatVecParams &p, const void *w, const void *x, vo
   return hipGetLastError();
 }
 
+// Q4_K on the matrix unit: K a whole number of blocks, rows and activations made of whole 16-byte
+// vectors, the codes of every activation row within a block's 64 KiB of LDS.
+inline uint32_t tile_tokens(uint32_t m) { return m <= 1 ? 1 : (m <= 4 ? 4 : 8); }
+inline bool tiles_serve(const MatVecParams &p, const void *w, const void *x) {
+  return p.k >= 1024 && p.k % 256 == 0 && p.m <= 8 && p.row_stride % 16 == 0 &&
+         ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(x)) & 15u) == 0 &&
+         tile_shared_bytes(tile_tokens(p.m), p.k / 256) <= 64 * 1024;
+}
+template <class TX, int kSets>
+hipError_t run_tiles_m(const MatVecParams &p, const void *w, const void *x, void *y, int compute_units, hipStream_t s) {
+  const uint32_t blocks = p.k / 256, groups = (blocks + 3) / 4;
+  const uint32_t tiles = (uint32_t)((p.rows + kTileRows - 1) / kTileRows);
+  // few rows: up to four waves share a tile, each walking every second or fourth group of four blocks,
+  // until there are eight waves per compute unit
+  const uint64_t wanted = 8ull * (uint64_t)(compute_units > 0 ? compute_units : 256);
+  uint32_t split_log2 = 0;
+  while (split_log2 < 2 && (2u << split_log2) <= groups && ((uint64_t)tiles << split_log2) < wanted) ++split_log2;
+  const uint32_t waves = tiles << split_log2;
+  const size_t shared = tile_shared_bytes(kSets == 0 ? 1 : 4 * kSets, blocks);
+  const dim3 grid((waves + kWavesPerBlock - 1) / kWavesPerBlock);
+  const unsigned char *in = static_cast<const unsigned char *>(w);
+  // at most 32 activation blocks in all: one round of the block's half waves, no loop around it
+  if ((kSets == 0 ? 1u : 4u * kSets) * blocks <= 32) {
+    note_variant<TilesTag<kSets, true>>();
+    hipLaunchKernelGGL((gguf_matvec_q8_tiles<TX, kSets, true>), grid, dim3(kBlockThreads), shared, s, in, x, y, (uint32_t)p.rows,
+                       p.row_stride, blocks, p.m, split_log2);
+  } else {
+    note_variant<TilesTag<kSets, false>>();
+    hipLaunchKernelGGL((gguf_matvec_q8_tiles<TX, kSets, false>), grid, dim3(kBlockThreads), shared, s, in, x, y, (uint32_t)p.rows,
+                       p.row_stride, blocks, p.m, split_log2);
+  }
+  return hipGetLastError();
+}
+template <class TX>
+hipError_t run_tiles(const MatVecParams &p, const void *w, const void *x, void *y, int compute_units, hipStream_t s) {
+  if (p.m <= 1) return run_tiles_m<TX, 0>(p, w, x, y, compute_units, s);
+  if (p.m <= 4) return run_tiles_m<TX, 1>(p, w, x, y, compute_units, s);
+  return run_tiles_m<TX, 2>(p, w, x, y, compute_units, s);
+}
+
 template <int kKind, class TX>
 hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, int compute_units, hipStream_t s) {
+  if constexpr (kKind == 0) {
+    if (tiles_serve(p, w, x)) return run_tiles<TX>(p, w, x, y, compute_units, s);
+  }
   // the span kernels: rows of 2048 n values made of whole 16-byte vectors, activations on a 16-byte
   // boundary, codes of every activation row in LDS beside the waves' row buffers (12 KiB); everything
   // else walks block by block
@@ -1316,16 +1570,6 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
     // several activation rows: the quad form, if its four row slots per wave fit beside the codes
     const size_t slots = (size_t)kWavesPerBlock * 4 * (LinesRow<kKind, 1>::kSlotBytes + 32);
     if (p.m >= 2 && slots + shared <= 64 * 1024) return run_quads<kKind, TX>(p, w, x, y, spans, grid, shared, s);
-  }
-  if constexpr (kKind == 0) {
-    // Q4_K, one activation row of 2048 values: sixteen weight rows per wave on the matrix unit
-    if (p.m == 1 && spans == 1 && p.rows >= kTileMinimumRows) {
-      const uint32_t tiles = (uint32_t)((p.rows + kTileRows - 1) / kTileRows);
-      note_variant<TilesTag>();
-      hipLaunchKernelGGL((gguf_matvec_q8_tiles<TX>), dim3((tiles + kWavesPerBlock - 1) / kWavesPerBlock), dim3(kBlockThreads), 0, s,
-                         static_cast<const unsigned char *>(w), x, y, (uint32_t)p.rows, p.row_stride);
-      return hipGetLastError();
-    }
   }
   if (p.m == 1 && spans <= 6) {
     // One activation row: a wave per span.  Eight waves per compute unit measured best or equal in

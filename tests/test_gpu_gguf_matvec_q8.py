@@ -133,15 +133,16 @@ def test_q8_route_vocabulary_sized_weight(tag, m):
 
 def test_q8_route_the_reference_s_own_projection_shapes():
     """The shapes of the reference's Q8_0 / Q4_K projection cases
-    (tests/compute_models/cpu_c5_gguf_inputs.h:231,237,259,287,314): none is a multiple of 2048 wide,
-    so every one takes the kernel that walks a row block by block."""
+    (tests/compute_models/cpu_c5_gguf_inputs.h:231,237,259,287,314): none is a multiple of 2048 wide.
+    The Q8_0 ones take the kernel that walks a row block by block, the Q4_K one the matrix-unit kernel."""
     rng = np.random.default_rng(1803)
     for tag, k, rows in (("q8_0", 1024, 32768), ("q4_k", 5120, 10240), ("q8_0", 7168, 3072), ("q8_0", 17408, 5120),
                          ("q8_0", 128, 512)):
         raw = weights_for(tag, rng, rows, k)
         x = rng.normal(0, 1.5, (k,)).astype(np.float32)
         note(f"q8 matvec {tag} [{k} -> {rows}], one activation row")
-        check(tag, "f32", raw, rows, k, x, kernel=f"gguf_matvec_q8_blocks/{tag}/1-tokens")
+        check(tag, "f32", raw, rows, k, x,
+              kernel="gguf_matvec_q8_tiles/q4_k/1-tokens" if tag == "q4_k" else f"gguf_matvec_q8_blocks/{tag}/1-tokens")
 
 
 @pytest.mark.parametrize("x_tag", ["f32", "bf16", "f16"])
@@ -159,7 +160,10 @@ def test_q8_route_any_whole_number_of_blocks_and_activation_rows(tag, x_tag):
             x = rng.normal(0, 1.5, (m, k) if m > 1 else (k,)).astype(np.float32)
             note(f"q8 matvec {tag} x {x_tag} rows {rows} k {k} (blocks of {per}) m {m}")
             label = {1: 1, 2: 2, 3: 4, 4: 4, 5: 8, 8: 8}[m]
-            check(tag, x_tag, raw, rows, k, x, kernel=f"gguf_matvec_q8_blocks/{tag}/{label}-tokens")
+            if tag == "q4_k" and k >= 1024:   # Q4_K rows of four blocks or more: the matrix unit, four activation rows a set
+                check(tag, x_tag, raw, rows, k, x, kernel=f"gguf_matvec_q8_tiles/q4_k/{1 if m == 1 else (4 if m <= 4 else 8)}-tokens")
+            else:
+                check(tag, x_tag, raw, rows, k, x, kernel=f"gguf_matvec_q8_blocks/{tag}/{label}-tokens")
 
 
 @pytest.mark.parametrize("tag", list(KINDS))
@@ -218,13 +222,13 @@ def test_q8_route_declines_what_it_does_not_serve():
 
 @pytest.mark.parametrize("x_tag", ["f32", "bf16", "f16"])
 def test_q8_route_q4_k_sub_block_dots_on_the_matrix_unit(x_tag):
-    """Q4_K, one activation row of 2048 values: sixteen weight rows per wave, every 32-value sub-block
+    """Q4_K with rows of whole 16-byte vectors: sixteen weight rows per wave, every 32-value sub-block
     dot from a 16 x 16 x 64 int8 matrix instruction.  Row counts around the wave's sixteen and the
     block's sixty-four, every scale slot and nibble pattern (raw bytes), activation blocks of zeros
     and of equal magnitudes, rows further apart than their blocks."""
     rng = np.random.default_rng(1810)
     k = 2048
-    for rows in (16, 17, 31, 63, 64, 65, 200, 1037):
+    for rows in (1, 15, 16, 17, 31, 63, 64, 65, 200, 1037):
         raw = raw_bytes_for("q4_k", rng, rows, k)
         x = rng.normal(0, 2, k).astype(np.float32)
         if rows % 2:
@@ -232,14 +236,39 @@ def test_q8_route_q4_k_sub_block_dots_on_the_matrix_unit(x_tag):
             x[512:768] = np.where(np.arange(256) % 2 == 0, 1.25, -1.25)
             x[1999] = 40.0
         note(f"q8 matvec q4_k tiles x {x_tag} rows {rows}")
-        check("q4_k", x_tag, raw, rows, k, x, kernel="gguf_matvec_q8_tiles/q4_k")
+        check("q4_k", x_tag, raw, rows, k, x, kernel="gguf_matvec_q8_tiles/q4_k/1-tokens")
     rows = 70
     raw = raw_bytes_for("q4_k", rng, rows, k)
     padded = np.zeros((rows, raw.shape[1] + 48), np.uint8)
     padded[:, :raw.shape[1]] = raw
     note(f"q8 matvec q4_k tiles x {x_tag}: rows 48 bytes further apart than their blocks")
     check("q4_k", x_tag, padded, rows, k, rng.normal(0, 1, k).astype(np.float32), row_stride=raw.shape[1] + 48,
-          kernel="gguf_matvec_q8_tiles/q4_k")
-    note(f"q8 matvec q4_k x {x_tag}: fewer than sixteen rows keep the span kernel")
-    check("q4_k", x_tag, raw_bytes_for("q4_k", rng, 15, k), 15, k, rng.normal(0, 1, k).astype(np.float32),
-          kernel="gguf_matvec_q8_spans/q4_k/1-spans")
+          kernel="gguf_matvec_q8_tiles/q4_k/1-tokens")
+
+
+@pytest.mark.parametrize("x_tag", ["f32", "bf16"])
+def test_q8_route_q4_k_matrix_unit_widths_tokens_and_shared_tiles(x_tag):
+    """Any whole number of blocks from four up (a last group of four that overlaps the one before),
+    one to eight activation rows (one, or one or two sets of four), and few rows of many blocks,
+    where two or four waves share a tile and add their shares."""
+    rng = np.random.default_rng(1811)
+    for rows, k, m in ((40, 1024, 1), (33, 1280, 1), (50, 1536, 2), (21, 1792, 3), (70, 2304, 1), (19, 3328, 4),
+                       (48, 5120, 1), (130, 5120, 4), (35, 5120, 5), (20, 4096, 8), (600, 2048, 2), (90, 6144, 7),
+                       (10240, 5120, 1), (2100, 7680, 1), (64, 16384, 1), (17, 9984, 2)):
+        raw = raw_bytes_for("q4_k", rng, rows, k)
+        x = rng.normal(0, 1.5, (m, k) if m > 1 else (k,)).astype(np.float32)
+        if m > 1:
+            x[m - 1, 256:512] = 0.0
+        tokens = 1 if m == 1 else (4 if m <= 4 else 8)
+        note(f"q8 matvec q4_k tiles x {x_tag} rows {rows} k {k} m {m}")
+        check("q4_k", x_tag, raw, rows, k, x, kernel=f"gguf_matvec_q8_tiles/q4_k/{tokens}-tokens")
+    note("q8 matvec q4_k: fewer than four blocks per row, an odd row stride and unaligned activations keep the block-walking kernel")
+    raw = raw_bytes_for("q4_k", rng, 20, 768)
+    check("q4_k", x_tag, raw, 20, 768, rng.normal(0, 1, 768).astype(np.float32), kernel="gguf_matvec_q8_blocks/q4_k/1-tokens")
+    raw = raw_bytes_for("q4_k", rng, 20, 2048)
+    padded = np.zeros((20, raw.shape[1] + 2), np.uint8)
+    padded[:, :raw.shape[1]] = raw
+    check("q4_k", x_tag, padded, 20, 2048, rng.normal(0, 1, 2048).astype(np.float32), row_stride=raw.shape[1] + 2,
+          kernel="gguf_matvec_q8_blocks/q4_k/1-tokens")
+    check("q4_k", x_tag, raw, 20, 2048, rng.normal(0, 1, 2048).astype(np.float32), x_offset=1,
+          kernel="gguf_matvec_q8_blocks/q4_k/1-tokens")
