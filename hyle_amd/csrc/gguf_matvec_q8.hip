@@ -16,16 +16,18 @@
 // The integer parts are exact here; the f32 products and sums differ from ggml's only in their
 // order, which the reference's tests allow for with gamma(K / 4 + 65, 2^-24) * sum |terms|.
 //
-// Rows are read exactly as in gguf_matvec.hip (whole 16-byte vectors through wave-private LDS,
-// four spans of 2048 values in flight per wave, gguf_lines.h).  The activation codes of a lane's
-// 32 positions are eight 32-bit words per activation row, so a weight word of four quants meets
-// them in one v_dot4c_i32_i8, and decoding a span once serves every activation row:
+// Q6_K and Q8_0 rows are read exactly as in gguf_matvec.hip (whole 16-byte vectors through
+// wave-private LDS, four spans of 2048 values in flight per wave, gguf_lines.h).  The activation
+// codes of a lane's 32 positions are eight 32-bit words per activation row, so a weight word of four
+// quants meets them in one v_dot4c_i32_i8, and decoding a span once serves every activation row:
 //   Q6_K  four quants are assembled per word as int8 bytes 4 (q - 32); a 16-value group's dot is
 //         multiplied by its int8 scale as an integer; one conversion and (d / 4) * a.scale close
 //         the half block
-//   Q4_K  nibbles are already bytes 0..15; sc * dot and m * (sum of activation codes) stay
-//         integers; d * a.scale and dmin * a.scale close the sub-blocks
 //   Q8_0  the bytes are the int8 quants; d * a.scale closes the block
+// Q4_K blocks are whole 16-byte vectors, so its rows go from global memory straight into the
+// operands of 16 x 16 x 64 int8 matrix instructions, sixteen weight rows per wave
+// (gguf_matvec_q8_tiles): nibbles are already bytes 0..15; sc * dot and m * (sum of activation
+// codes) stay integers; d * a.scale and dmin * a.scale close the block.
 #include <type_traits>
 
 #include "device_common.h"
@@ -74,12 +76,10 @@ __device__ __forceinline__ uint32_t code_of(float scaled) {
 }
 
 // What a lane holds of one activation row for one span of 2048 values: the codes of its 32
-// positions (word e / 4, byte e % 4), the scale of the activation block(s) they belong to and,
-// for Q4_K, the sums of the codes of its four runs of eight.
+// positions (word e / 4, byte e % 4) and the scale of the activation block they belong to.
 struct LaneCodes {
   uint32_t codes[8];
-  float scale[2];
-  int sums[4];
+  float scale;
 };
 
 // Quantises the lane's share of span `span` of the activation row at `x` (k values of type TX).
@@ -111,44 +111,33 @@ __device__ __forceinline__ LaneCodes quantise_span(const void *x, size_t row_off
   }
   LaneCodes out;
   // Q8_0: the lane's 32 values are one block.  Q6_K: eight lanes share a block of 256.
-  // Q4_K: the lane's values 0..15 and 16..31 belong to two blocks of 256, sixteen lanes each.
-  constexpr int kParts = kKind == 0 ? 2 : 1;
-  constexpr int kPartValues = 32 / kParts;
-  constexpr int kLanesPerBlock = kKind == 0 ? 16 : (kKind == 1 ? 8 : 1);
+  constexpr int kLanesPerBlock = kKind == 1 ? 8 : 1;
+  LaneMax mine{0.0f, 0.0f, 0u};
 #pragma unroll
-  for (int part = 0; part < kParts; ++part) {
-    LaneMax mine{0.0f, 0.0f, 0u};
-#pragma unroll
-    for (int t = 0; t < kPartValues; ++t) {  // positions rise with e, so ">" keeps the first
-      const int e = part * kPartValues + t;
-      const float magnitude = __builtin_fabsf(values[e]);
-      if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], Kind::position(span, lane, e)};
-    }
-    if (mine.magnitude == 0.0f) mine.position = 0xFFFFFFFFu;  // no candidate: any lane with one goes first
-    const LaneMax top = block_largest<kLanesPerBlock>(mine);
-    float factor = 0.0f, stored = 0.0f;
-    if (top.magnitude != 0.0f) {
-      if constexpr (kKind == 2) {
-        stored = f16_to_f32(f32_to_f16(top.magnitude / 127.0f));
-        factor = 127.0f / top.magnitude;
-      } else {
-        factor = -127.0f / top.value;
-        stored = 1.0f / factor;
-      }
-    }
-    out.scale[part] = stored;
-#pragma unroll
-    for (int w = 0; w < kPartValues / 4; ++w) {
-      uint32_t word = 0;
-#pragma unroll
-      for (int t = 0; t < 4; ++t) word |= code_of(values[part * kPartValues + 4 * w + t] * factor) << (8 * t);
-      out.codes[part * (kPartValues / 4) + w] = top.magnitude != 0.0f ? word : 0u;
+  for (int e = 0; e < 32; ++e) {  // positions rise with e, so ">" keeps the first
+    const float magnitude = __builtin_fabsf(values[e]);
+    if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], Kind::position(span, lane, e)};
+  }
+  if (mine.magnitude == 0.0f) mine.position = 0xFFFFFFFFu;  // no candidate: any lane with one goes first
+  const LaneMax top = block_largest<kLanesPerBlock>(mine);
+  float factor = 0.0f, stored = 0.0f;
+  if (top.magnitude != 0.0f) {
+    if constexpr (kKind == 2) {
+      stored = f16_to_f32(f32_to_f16(top.magnitude / 127.0f));
+      factor = 127.0f / top.magnitude;
+    } else {
+      factor = -127.0f / top.value;
+      stored = 1.0f / factor;
     }
   }
-  if constexpr (kParts == 1) out.scale[1] = out.scale[0];
+  out.scale = stored;
 #pragma unroll
-  for (int run = 0; run < 4; ++run)
-    out.sums[run] = dot4(0x01010101u, out.codes[2 * run], dot4(0x01010101u, out.codes[2 * run + 1], 0));
+  for (int w = 0; w < 8; ++w) {
+    uint32_t word = 0;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) word |= code_of(values[4 * w + t] * factor) << (8 * t);
+    out.codes[w] = top.magnitude != 0.0f ? word : 0u;
+  }
   return out;
 }
 
@@ -182,7 +171,7 @@ template <> struct SpanDot<1> {  // Q6_K
     int total = 0;
 #pragma unroll
     for (int g = 0; g < 4; ++g) total = mad24(scale[g], dot4(q[g][0], a.codes[2 * g], dot4(q[g][1], a.codes[2 * g + 1], 0)), total);
-    return (step * a.scale[0]) * (float)total;
+    return (step * a.scale) * (float)total;
   }
 };
 
@@ -217,73 +206,6 @@ __device__ __forceinline__ int q4k_six_bits(uint32_t s0, uint32_t s1, uint32_t s
   return (int)(((s2 >> (shift + (minimum ? 4u : 0u))) & 15u) | (((own >> (shift + 6)) & 3u) << 4));
 }
 
-template <> struct SpanDot<0> {  // Q4_K
-  uint32_t low[2][2], high[2][2];
-  int sc_low[2], sc_high[2], m_low[2], m_high[2];
-  float d[2], dmin[2];
-  // The same without the block's other lanes (in the quad layout they hold other weight rows):
-  // the lane works out the four factors of its two sub-blocks, 2 chunk and 2 chunk + 1, itself.
-  // They are the same for the four shares a quad lane walks, so they are taken once per span.
-  __device__ __forceinline__ void scales_alone(const unsigned char *slot, const Lines<0>::Lane &at, uint32_t chunk) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const u32x4 head = *reinterpret_cast<const u32x4 *>(slot + at.header[i]);
-      d[i] = f16_to_f32((uint16_t)head.x);
-      dmin[i] = f16_to_f32((uint16_t)(head.x >> 16));
-      sc_low[i] = q4k_six_bits(head.y, head.z, head.w, 2 * chunk, false);
-      sc_high[i] = q4k_six_bits(head.y, head.z, head.w, 2 * chunk + 1, false);
-      m_low[i] = q4k_six_bits(head.y, head.z, head.w, 2 * chunk, true);
-      m_high[i] = q4k_six_bits(head.y, head.z, head.w, 2 * chunk + 1, true);
-    }
-  }
-  __device__ __forceinline__ void quants_alone(const unsigned char *slot, const Lines<0>::Lane &at) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint32_t *words = reinterpret_cast<const uint32_t *>(slot + at.quants[i]);
-#pragma unroll
-      for (int w = 0; w < 2; ++w) {
-        low[i][w] = words[w] & 0x0F0F0F0Fu;
-        high[i][w] = (words[w] >> 4) & 0x0F0F0F0Fu;
-      }
-    }
-  }
-  __device__ __forceinline__ void decode(const unsigned char *slot, const Lines<0>::Lane &at) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const u32x4 head = *reinterpret_cast<const u32x4 *>(slot + at.header[i]);
-      const uint32_t s0 = head.y, s1 = head.z, s2 = head.w;
-      d[i] = f16_to_f32((uint16_t)head.x);
-      dmin[i] = f16_to_f32((uint16_t)(head.x >> 16));
-      // lane u of the block's sixteen works out sc (u < 8) or m (u >= 8) of sub-block u % 8
-      const uint32_t own = at.minimum ? s1 : s0;
-      const int bits = (int)((((at.main_in_s2 ? s2 : own) >> at.main_shift) & at.main_mask) |
-                             (((own >> at.top_shift) & at.top_mask) << 4));
-      sc_low[i] = __shfl(bits, at.source);
-      sc_high[i] = __shfl(bits, at.source + 1);
-      m_low[i] = __shfl(bits, at.source + 8);
-      m_high[i] = __shfl(bits, at.source + 9);
-      const uint32_t *words = reinterpret_cast<const uint32_t *>(slot + at.quants[i]);
-#pragma unroll
-      for (int w = 0; w < 2; ++w) {
-        low[i][w] = words[w] & 0x0F0F0F0Fu;
-        high[i][w] = (words[w] >> 4) & 0x0F0F0F0Fu;
-      }
-    }
-  }
-  __device__ __forceinline__ float against(const LaneCodes &a) const {
-    float total = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int lows = dot4(low[i][0], a.codes[4 * i], dot4(low[i][1], a.codes[4 * i + 1], 0));
-      const int highs = dot4(high[i][0], a.codes[4 * i + 2], dot4(high[i][1], a.codes[4 * i + 3], 0));
-      const int scaled = mad24(sc_low[i], lows, __mul24(sc_high[i], highs));
-      const int minima = mad24(m_low[i], a.sums[2 * i], __mul24(m_high[i], a.sums[2 * i + 1]));
-      total += a.scale[i] * (d[i] * (float)scaled - dmin[i] * (float)minima);
-    }
-    return total;
-  }
-};
-
 template <> struct SpanDot<2> {  // Q8_0
   uint32_t q[8];
   float d;
@@ -300,31 +222,25 @@ template <> struct SpanDot<2> {  // Q8_0
     int total = 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) total = dot4(q[i], a.codes[i], total);
-    return (d * a.scale[0]) * (float)total;
+    return (d * a.scale) * (float)total;
   }
 };
 
 // LDS of a block: for every (activation row, span) the 64 lanes' LaneCodes, stored as
 // [word][lane] so that a wave reads each word of its lanes from consecutive banks.
-constexpr uint32_t kCodeWords = 8 + 2 + 4;  // codes, scales, sums
+constexpr uint32_t kCodeWords = 8 + 1;  // codes, scale
 __device__ __forceinline__ void park(uint32_t *staged, uint32_t pair, uint32_t lane, const LaneCodes &c) {
   uint32_t *at = staged + (size_t)pair * kCodeWords * kWaveLanes + lane;
 #pragma unroll
   for (int w = 0; w < 8; ++w) at[w * kWaveLanes] = c.codes[w];
-  at[8 * kWaveLanes] = f32_bits(c.scale[0]);
-  at[9 * kWaveLanes] = f32_bits(c.scale[1]);
-#pragma unroll
-  for (int w = 0; w < 4; ++w) at[(10 + w) * kWaveLanes] = (uint32_t)c.sums[w];
+  at[8 * kWaveLanes] = f32_bits(c.scale);
 }
 __device__ __forceinline__ LaneCodes fetch(const uint32_t *staged, uint32_t pair, uint32_t lane) {
   const uint32_t *at = staged + (size_t)pair * kCodeWords * kWaveLanes + lane;
   LaneCodes c;
 #pragma unroll
   for (int w = 0; w < 8; ++w) c.codes[w] = at[w * kWaveLanes];
-  c.scale[0] = bits_f32(at[8 * kWaveLanes]);
-  c.scale[1] = bits_f32(at[9 * kWaveLanes]);
-#pragma unroll
-  for (int w = 0; w < 4; ++w) c.sums[w] = (int)at[(10 + w) * kWaveLanes];
+  c.scale = bits_f32(at[8 * kWaveLanes]);
   return c;
 }
 
@@ -540,50 +456,10 @@ template <> struct QuadDot<1> {  // Q6_K
 #pragma unroll
       for (int i = 0; i < 4; ++i) total[i] = mad24(w.scale[g], dots[i], total[i]);
     }
-    sums[0] += (w.step * quad_lane<0>(a.scale[0])) * (float)total[0];
-    sums[1] += (w.step * quad_lane<1>(a.scale[0])) * (float)total[1];
-    sums[2] += (w.step * quad_lane<2>(a.scale[0])) * (float)total[2];
-    sums[3] += (w.step * quad_lane<3>(a.scale[0])) * (float)total[3];
-  }
-};
-// Q4_K.  The four shares a quad lane walks in a span lie in the same two weight blocks and the
-// same two activation blocks, so their integer dots are accumulated in the matrix unit across the
-// shares -- codes . low nibbles, codes . high nibbles and, for the minima, codes . m with m as four
-// equal bytes -- and the scales are applied once per span.
-template <> struct QuadDot<0> {
-  struct Sums {
-    i32x4 lows[2], highs[2], minima[2];
-  };
-  static __device__ __forceinline__ void clear(Sums &acc) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) acc.lows[i] = acc.highs[i] = acc.minima[i] = i32x4{0, 0, 0, 0};
-  }
-  static __device__ __forceinline__ void add(const SpanDot<0> &w, const LaneCodes &a, Sums &acc) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint32_t m_low = (uint32_t)w.m_low[i] * 0x01010101u, m_high = (uint32_t)w.m_high[i] * 0x01010101u;
-      acc.lows[i] = quad_dots(a.codes[4 * i + 1], w.low[i][1], quad_dots(a.codes[4 * i], w.low[i][0], acc.lows[i]));
-      acc.highs[i] = quad_dots(a.codes[4 * i + 3], w.high[i][1], quad_dots(a.codes[4 * i + 2], w.high[i][0], acc.highs[i]));
-      acc.minima[i] = quad_dots(a.codes[4 * i + 1], m_low, quad_dots(a.codes[4 * i], m_low, acc.minima[i]));
-      acc.minima[i] = quad_dots(a.codes[4 * i + 3], m_high, quad_dots(a.codes[4 * i + 2], m_high, acc.minima[i]));
-    }
-  }
-  template <int kRow>
-  static __device__ __forceinline__ float row(const SpanDot<0> &w, const float (&scale)[2], const Sums &acc) {
-    float total = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int scaled = mad24(w.sc_low[i], acc.lows[i][kRow], __mul24(w.sc_high[i], acc.highs[i][kRow]));
-      total += quad_lane<kRow>(scale[i]) * (w.d[i] * (float)scaled - w.dmin[i] * (float)acc.minima[i][kRow]);
-    }
-    return total;
-  }
-  // scale: the activation blocks' scales of this lane's activation row (the same for the four shares)
-  static __device__ __forceinline__ void close(const SpanDot<0> &w, const float (&scale)[2], const Sums &acc, float (&sums)[4]) {
-    sums[0] += row<0>(w, scale, acc);
-    sums[1] += row<1>(w, scale, acc);
-    sums[2] += row<2>(w, scale, acc);
-    sums[3] += row<3>(w, scale, acc);
+    sums[0] += (w.step * quad_lane<0>(a.scale)) * (float)total[0];
+    sums[1] += (w.step * quad_lane<1>(a.scale)) * (float)total[1];
+    sums[2] += (w.step * quad_lane<2>(a.scale)) * (float)total[2];
+    sums[3] += (w.step * quad_lane<3>(a.scale)) * (float)total[3];
   }
 };
 template <> struct QuadDot<2> {  // Q8_0
@@ -591,10 +467,10 @@ template <> struct QuadDot<2> {  // Q8_0
     i32x4 dots = {0, 0, 0, 0};
 #pragma unroll
     for (int i = 0; i < 8; ++i) dots = quad_dots(a.codes[i], w.q[i], dots);
-    sums[0] += (w.d * quad_lane<0>(a.scale[0])) * (float)dots[0];
-    sums[1] += (w.d * quad_lane<1>(a.scale[0])) * (float)dots[1];
-    sums[2] += (w.d * quad_lane<2>(a.scale[0])) * (float)dots[2];
-    sums[3] += (w.d * quad_lane<3>(a.scale[0])) * (float)dots[3];
+    sums[0] += (w.d * quad_lane<0>(a.scale)) * (float)dots[0];
+    sums[1] += (w.d * quad_lane<1>(a.scale)) * (float)dots[1];
+    sums[2] += (w.d * quad_lane<2>(a.scale)) * (float)dots[2];
+    sums[3] += (w.d * quad_lane<3>(a.scale)) * (float)dots[3];
   }
 };
 
@@ -668,39 +544,14 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_quads(const unsi
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      if constexpr (kKind == 0) {
-        // Q4_K: the four shares one after another in a loop that is not unrolled (unrolled, their
-        // decodes are all hoisted to the front and the kernel needs every register there is: 256
-        // + 67 against 90), the codes fetched from LDS share by share
-        SpanDot<0> decoded;
-        decoded.scales_alone(own_slot, Kind::lane_of(0, 4 * quad), quad % 4);  // chunk = (4 quad + t) % 16 / 4
-        typename QuadDot<0>::Sums acc[kSets];
-        float scale[kSets][2];
 #pragma unroll
-        for (int set = 0; set < kSets; ++set) QuadDot<0>::clear(acc[set]);
-#pragma unroll 1
-        for (int t = 0; t < 4; ++t) {
-          decoded.quants_alone(own_slot, Kind::lane_of(0, 4 * quad + t));
+      for (int t = 0; t < 4; ++t) {
+        SpanDot<kKind> decoded;
+        decoded.decode(own_slot, at[t]);
 #pragma unroll
-          for (int set = 0; set < kSets; ++set) {
-            const LaneCodes a = fetch(staged, token[set] * spans + span, 4 * quad + t);
-            scale[set][0] = a.scale[0];
-            scale[set][1] = a.scale[1];
-            QuadDot<0>::add(decoded, a, acc[set]);
-          }
-        }
-#pragma unroll
-        for (int set = 0; set < kSets; ++set) QuadDot<0>::close(decoded, scale[set], acc[set], sums[set]);
-      } else {
-#pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          SpanDot<kKind> decoded;
-          decoded.decode(own_slot, at[t]);
-#pragma unroll
-          for (int set = 0; set < kSets; ++set) {
-            if constexpr (kRegisters) QuadDot<kKind>::add(decoded, held[set * 4 + t], sums[set]);
-            else QuadDot<kKind>::add(decoded, fetch(staged, token[set] * spans + span, 4 * quad + t), sums[set]);
-          }
+        for (int set = 0; set < kSets; ++set) {
+          if constexpr (kRegisters) QuadDot<kKind>::add(decoded, held[set * 4 + t], sums[set]);
+          else QuadDot<kKind>::add(decoded, fetch(staged, token[set] * spans + span, 4 * quad + t), sums[set]);
         }
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -1468,16 +1319,12 @@ hipError_t run_quads(const MatVecParams &p, const void *w, const void *x, void *
                      y, (uint32_t)p.rows, p.row_stride, spans, p.m)
   // Which forms a shape can reach follows from what fits a block's LDS beside the four row slots per
   // wave (run_m): one set of four tokens for every format, with the codes in registers when K = 2048
-  // (Q4_K fetches its codes from LDS share by share); two sets only for Q4_K (codes in LDS) and for
-  // Q6_K at K = 2048 (codes in registers); Q8_0's wider slots leave no room for a second set.
-  const bool registers = spans == 1 && kKind != 0;
+  // two sets only for Q6_K at K = 2048 (codes in registers); Q8_0's wider slots leave no room for a
+  // second set.  (Q4_K takes the tile kernel.)
+  const bool registers = spans == 1;
   if (p.m <= 4) {
-    if constexpr (kKind != 0) {
-      if (registers) { HYLE_QUADS(1, true); }
-    }
-    if (!registers) { HYLE_QUADS(1, false); }
-  } else if constexpr (kKind == 0) {
-    HYLE_QUADS(2, false);
+    if (registers) { HYLE_QUADS(1, true); }
+    else { HYLE_QUADS(1, false); }
   } else if constexpr (kKind == 1) {
     if (!registers) return hipErrorInvalidValue;
     HYLE_QUADS(2, true);
@@ -1552,8 +1399,10 @@ hipError_t run_tiles(const MatVecParams &p, const void *w, const void *x, void *
 template <int kKind, class TX>
 hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, int compute_units, hipStream_t s) {
   if constexpr (kKind == 0) {
+    // Q4_K: the matrix unit, or block by block
     if (tiles_serve(p, w, x)) return run_tiles<TX>(p, w, x, y, compute_units, s);
-  }
+    return run_blocks<kKind, TX>(p, w, x, y, compute_units, s);
+  } else {
   // the span kernels: rows of 2048 n values made of whole 16-byte vectors, activations on a 16-byte
   // boundary, codes of every activation row in LDS beside the waves' row buffers (12 KiB); everything
   // else walks block by block
@@ -1569,16 +1418,16 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
   {
     // several activation rows: the quad form, if its four row slots per wave fit beside the codes
     const size_t slots = (size_t)kWavesPerBlock * 4 * (LinesRow<kKind, 1>::kSlotBytes + 32);
-    if (p.m >= 2 && slots + shared <= 64 * 1024) return run_quads<kKind, TX>(p, w, x, y, spans, grid, shared, s);
+    // (a second set of four rows only for Q6_K with its codes in registers, K = 2048)
+    const bool sets = p.m <= 4 || (kKind == 1 && spans == 1);
+    if (p.m >= 2 && sets && slots + shared <= 64 * 1024) return run_quads<kKind, TX>(p, w, x, y, spans, grid, shared, s);
   }
   if (p.m == 1 && spans <= 6) {
     // One activation row: a wave per span.  Eight waves per compute unit measured best or equal in
     // 25 of 27 shapes (three formats, K = 2048 ... 12288, 1024 ... 151936 rows: 0-30 % below the
-    // kernel that parks the codes in LDS first); Q4_K over many rows wants twelve
-    // ([4096 -> 151936]: 79 us with 12, 90 us with 8, 93 us parked).
+    // kernel that parks the codes in LDS first).
     const uint32_t units = (uint32_t)(compute_units > 0 ? compute_units : 256);
-    const uint32_t waves = kKind == 0 && p.rows * spans >= 65536 ? 12u : 8u;
-    const uint32_t most = units * (waves / spans);
+    const uint32_t most = units * (8u / spans);
     const dim3 blocks((uint32_t)p.rows < most ? (uint32_t)p.rows : most);
     const unsigned char *in = static_cast<const unsigned char *>(w);
     const uint32_t rows = (uint32_t)p.rows;
@@ -1596,6 +1445,7 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
   if (p.m == 2) return run_registers<kKind, TX, 2>(p, w, x, y, spans, grid, shared, s);
   if (p.m <= 4) return run_registers<kKind, TX, 4>(p, w, x, y, spans, grid, shared, s);
   return run_registers<kKind, TX, 8>(p, w, x, y, spans, grid, shared, s);
+  }
 }
 
 template <class TX>
@@ -1617,7 +1467,11 @@ bool gguf_matvec_q8_serves(int kind, uint32_t k) { return blocks_row_bytes(kind,
 
 uint32_t gguf_matvec_q8_dispatches(int kind, uint32_t m, uint32_t k, uint64_t row_stride) {
   if (m == 0 || k == 0) return 1;
-  if (k % 2048 == 0 && row_stride % 16 == 0 && gguf_matvec_q8_shared_bytes(m, k) + 12 * 1024 <= 64 * 1024) return 1;
+  if (kind == 0) {
+    if (k >= 1024 && k % 256 == 0 && m <= 8 && row_stride % 16 == 0 && tile_shared_bytes(tile_tokens(m), k / 256) <= 64 * 1024) return 1;
+  } else if (k % 2048 == 0 && row_stride % 16 == 0 && gguf_matvec_q8_shared_bytes(m, k) + 12 * 1024 <= 64 * 1024) {
+    return 1;
+  }
   uint32_t fit = (uint32_t)(kBlocksSharedBudget / blocks_row_bytes(kind, k));
   fit = fit >= 8 ? 8 : (fit >= 4 ? 4 : (fit >= 2 ? 2 : 1));
   return (m + fit - 1) / fit;

@@ -91,7 +91,7 @@ def test_q8_route_shapes_and_batches(tag, x_tag):
                        (9000, 2048, 1), (5000, 4096, 1), (1030, 6144, 1), (600, 10240, 1), (5, 14336, 1),
                        # several tokens whose codes leave no room for the quad kernel's row slots: the kernel that
                        # fetches the codes from LDS span by span, for two, four and eight tokens
-                       (11, 10240, 2), (7, 6144, 2), (9, 8192, 3), (10, 4096, 5), (6, 4096, 7)):
+                       (11, 18432, 2), (7, 20480, 2), (9, 12288, 3), (10, 8192, 5), (6, 6144, 7)):
         raw = weights_for(tag, rng, rows, k)
         x = rng.normal(0, 1.5, (m, k) if m > 1 else (k,)).astype(np.float32)
         note(f"q8 matvec {tag} x {x_tag} rows {rows} k {k} m {m}")
