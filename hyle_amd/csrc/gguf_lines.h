@@ -199,12 +199,13 @@ template <int kKind, int kPasses> struct LinesRow {
   static constexpr int kLoads = (kVectors + kWaveLanes - 1) / kWaveLanes;
   static constexpr int kSlotBytes = kLoads * kWaveLanes * 16;            // LDS bytes of one wave
   u32x4 v[kLoads];
-  static __device__ __forceinline__ LinesRow load(const unsigned char *row, uint32_t lane) {
+  // `vectors`: how many of the row's vectors exist (fewer than kVectors for a last, shorter span)
+  static __device__ __forceinline__ LinesRow load(const unsigned char *row, uint32_t lane, uint32_t vectors = kVectors) {
     LinesRow r;
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
       const uint32_t wanted = lane + i * kWaveLanes;  // past the row: its last vector again (parked in LDS, never read)
-      r.v[i] = load16_stream(row, wanted < (uint32_t)kVectors ? wanted : (uint32_t)kVectors - 1);
+      r.v[i] = load16_stream(row, wanted < vectors ? wanted : vectors - 1);
     }
     return r;
   }

@@ -85,15 +85,17 @@ struct LaneCodes {
 // Quantises the lane's share of span `span` of the activation row at `x` (k values of type TX).
 // Every lane of a wave calls it; lanes that share an activation block agree on its scale through
 // a cross-lane maximum.
+// `live`: the lane's positions exist (a Q8_0 row's last span may be short: lanes past it read the
+// row's first values and come back with zero codes and a zero scale).
 template <int kKind, class TX>
-__device__ __forceinline__ LaneCodes quantise_span(const void *x, size_t row_offset, uint32_t span, uint32_t lane) {
+__device__ __forceinline__ LaneCodes quantise_span(const void *x, size_t row_offset, uint32_t span, uint32_t lane, bool live = true) {
   using Kind = Lines<kKind>;
   // the lane's positions come in runs of eight neighbours (Lines<kind>::position), each a whole
   // 16-byte vector of a narrow type or two of f32: x starts on a 16-byte boundary (run_m)
   float values[32];
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
-    const size_t at = row_offset + Kind::position(span, lane, 8 * g);
+    const size_t at = row_offset + (live ? Kind::position(span, lane, 8 * g) : (uint32_t)(8 * g));
     if constexpr (Traits<TX>::kVec == 8) {
       float piece[8];
       Traits<TX>::unpack(load16(x, at / 8), piece);
@@ -119,7 +121,8 @@ __device__ __forceinline__ LaneCodes quantise_span(const void *x, size_t row_off
     if (magnitude > mine.magnitude) mine = LaneMax{magnitude, values[e], Kind::position(span, lane, e)};
   }
   if (mine.magnitude == 0.0f) mine.position = 0xFFFFFFFFu;  // no candidate: any lane with one goes first
-  const LaneMax top = block_largest<kLanesPerBlock>(mine);
+  LaneMax top = block_largest<kLanesPerBlock>(mine);
+  if (!live) top.magnitude = 0.0f;
   float factor = 0.0f, stored = 0.0f;
   if (top.magnitude != 0.0f) {
     if constexpr (kKind == 2) {
@@ -353,9 +356,14 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_lines(const unsi
 // span of x straight into registers (nothing is parked in LDS and no barrier precedes the first
 // row), walks the block's rows at its span and leaves its share of each row in LDS, where the
 // first wave adds the spans' shares in span order.
-template <int kKind, class TX, int kSpans>
+//
+// tail_lanes: how many lanes of the last span's wave have a block of the row (64 unless the row is
+// a Q8_0 row whose width is a multiple of 256 but not of 2048: a lane is a block of 32 values
+// there, and the last span then holds 8, 16, ... 56 blocks in 17, 34, ... 119 whole vectors).
+template <int kKind, class TX, int kSpans, bool kShort>
 __global__ __launch_bounds__(kSpans * kWaveLanes) void gguf_matvec_q8_spans(const unsigned char *weights, const void *x, void *y,
-                                                                          uint32_t rows, uint64_t row_stride) {
+                                                                          uint32_t rows, uint64_t row_stride, uint32_t tail_lanes) {
+  static_assert(!kShort || kKind == 2, "only Q8_0 rows have short last spans");
   using Row = LinesRow<kKind, 1>;
   using Kind = Lines<kKind>;
   constexpr uint32_t kSpanBytes = Kind::kPassVectors * 16;
@@ -367,13 +375,17 @@ __global__ __launch_bounds__(kSpans * kWaveLanes) void gguf_matvec_q8_spans(cons
   const typename Kind::Lane at = Kind::lane_of(0, lane);
   const uint32_t stride = gridDim.x, first = blockIdx.x;  // first < rows: the grid has at most `rows` blocks
   const unsigned char *mine = weights + (size_t)span * kSpanBytes;
+  // (whole spans: constants, and the compiler drops what depends on them)
+  const uint32_t live_lanes = kShort && span == (uint32_t)kSpans - 1 ? tail_lanes : (uint32_t)kWaveLanes;
+  const bool live = !kShort || lane < live_lanes;
+  const uint32_t vectors = kShort ? (live_lanes * 34u + 15u) / 16u : (uint32_t)Kind::kPassVectors;
   Row ring[kLinesDepth];
 #pragma unroll
   for (int d = 0; d < kLinesDepth; ++d) {
     const uint64_t wanted = (uint64_t)first + (uint64_t)d * stride;
-    ring[d] = Row::load(mine + (size_t)(wanted < rows ? (uint32_t)wanted : first) * row_stride, lane);
+    ring[d] = Row::load(mine + (size_t)(wanted < rows ? (uint32_t)wanted : first) * row_stride, lane, vectors);
   }
-  const LaneCodes held = quantise_span<kKind, TX>(x, 0, span, lane);  // while the first rows are on their way
+  const LaneCodes held = quantise_span<kKind, TX>(x, 0, span, lane, live);  // while the first rows are on their way
   for (uint64_t base = first; base < rows; base += (uint64_t)kLinesDepth * stride) {
     float totals[kLinesDepth] = {};
 #pragma unroll
@@ -384,13 +396,14 @@ __global__ __launch_bounds__(kSpans * kWaveLanes) void gguf_matvec_q8_spans(cons
       for (int i = 0; i < Row::kLoads; ++i)
         *reinterpret_cast<u32x4 *>(slot + (size_t)(lane + i * kWaveLanes) * 16) = ring[d].v[i];
       const uint64_t wanted = row + (uint64_t)kLinesDepth * stride;
-      ring[d] = Row::load(mine + (size_t)(wanted < rows ? (uint32_t)wanted : first) * row_stride, lane);
+      ring[d] = Row::load(mine + (size_t)(wanted < rows ? (uint32_t)wanted : first) * row_stride, lane, vectors);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
       SpanDot<kKind> decoded;
       decoded.decode(slot, at);
-      totals[d] = decoded.against(held);
+      const float mine_of_row = decoded.against(held);
+      totals[d] = live ? mine_of_row : 0.0f;  // a lane past a short last span decoded bytes that are not the row's
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
     }
@@ -933,8 +946,10 @@ template <int kKind, int kM, bool kRegisters> struct LinesTag {
     return std::string("gguf_matvec_q8_lines/") + kind_word(kKind) + "/" + std::to_string(kM) + "-tokens" + (kRegisters ? "/registers" : "/lds");
   }
 };
-template <int kKind, int kSpans> struct SpansTag {
-  static std::string text() { return std::string("gguf_matvec_q8_spans/") + kind_word(kKind) + "/" + std::to_string(kSpans) + "-spans"; }
+template <int kKind, int kSpans, bool kShort> struct SpansTag {
+  static std::string text() {
+    return std::string("gguf_matvec_q8_spans/") + kind_word(kKind) + "/" + std::to_string(kSpans) + "-spans" + (kShort ? "/short" : "");
+  }
 };
 template <int kSets, bool kOneBatch> struct TilesTag {
   static std::string text() {
@@ -1356,6 +1371,51 @@ hipError_t run_registers(const MatVecParams &p, const void *w, const void *x, vo
   return hipGetLastError();
 }
 
+// One activation row: a wave per span.  Eight waves per compute unit measured best or equal in
+// 25 of 27 shapes (three formats, K = 2048 ... 12288, 1024 ... 151936 rows: 0-30 % below the
+// kernel that parks the codes in LDS first).
+template <int kKind, class TX>
+hipError_t run_spans(const MatVecParams &p, const void *w, const void *x, void *y, uint32_t spans, uint32_t tail_lanes,
+                     int compute_units, hipStream_t s) {
+  const uint32_t units = (uint32_t)(compute_units > 0 ? compute_units : 256);
+  const uint32_t most = units * (spans <= 8 ? 8u / spans : 1u);
+  const dim3 blocks((uint32_t)p.rows < most ? (uint32_t)p.rows : most);
+  const unsigned char *in = static_cast<const unsigned char *>(w);
+  const uint32_t rows = (uint32_t)p.rows;
+#define HYLE_SPANS(N, SHORT)                                                                                             \
+  note_variant<SpansTag<kKind, N, SHORT>>();                                                                             \
+  hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, N, SHORT>), blocks, dim3(N * kWaveLanes), 0, s, in, x, y, rows,      \
+                     p.row_stride, tail_lanes)
+  if (tail_lanes == kWaveLanes) {
+    switch (spans) {
+      case 1: HYLE_SPANS(1, false); break;
+      case 2: HYLE_SPANS(2, false); break;
+      case 3: HYLE_SPANS(3, false); break;
+      case 4: HYLE_SPANS(4, false); break;
+      case 5: HYLE_SPANS(5, false); break;
+      case 6: HYLE_SPANS(6, false); break;
+      default: return hipErrorInvalidValue;  // whole rows of more spans take the kernel that parks the codes
+    }
+  } else if constexpr (kKind == 2) {
+    switch (spans) {
+      case 1: HYLE_SPANS(1, true); break;
+      case 2: HYLE_SPANS(2, true); break;
+      case 3: HYLE_SPANS(3, true); break;
+      case 4: HYLE_SPANS(4, true); break;
+      case 5: HYLE_SPANS(5, true); break;
+      case 6: HYLE_SPANS(6, true); break;
+      case 7: HYLE_SPANS(7, true); break;
+      case 8: HYLE_SPANS(8, true); break;
+      case 9: HYLE_SPANS(9, true); break;
+      default: return hipErrorInvalidValue;
+    }
+  } else {
+    return hipErrorInvalidValue;
+  }
+#undef HYLE_SPANS
+  return hipGetLastError();
+}
+
 // Q4_K on the matrix unit: K a whole number of blocks, rows and activations made of whole 16-byte
 // vectors, the codes of every activation row within a block's 64 KiB of LDS.
 inline uint32_t tile_tokens(uint32_t m) { return m <= 1 ? 1 : (m <= 4 ? 4 : 8); }
@@ -1403,6 +1463,14 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
     if (tiles_serve(p, w, x)) return run_tiles<TX>(p, w, x, y, compute_units, s);
     return run_blocks<kKind, TX>(p, w, x, y, compute_units, s);
   } else {
+  if constexpr (kKind == 2) {
+    // Q8_0, one activation row, a width of 256 n that is no multiple of 2048 (8 blocks are 17 whole
+    // vectors): the span kernel with a short last span, up to nine spans
+    const uint32_t whole = (p.k + 2047) / 2048;
+    if (p.m == 1 && p.k >= 1024 && p.k % 256 == 0 && p.k % 2048 != 0 && whole <= 9 && p.row_stride % 16 == 0 &&
+        ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(x)) & 15u) == 0)
+      return run_spans<kKind, TX>(p, w, x, y, whole, (p.k % 2048) / 32, compute_units, s);
+  }
   // the span kernels: rows of 2048 n values made of whole 16-byte vectors, activations on a 16-byte
   // boundary, codes of every activation row in LDS beside the waves' row buffers (12 KiB); everything
   // else walks block by block
@@ -1422,25 +1490,7 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, i
     const bool sets = p.m <= 4 || (kKind == 1 && spans == 1);
     if (p.m >= 2 && sets && slots + shared <= 64 * 1024) return run_quads<kKind, TX>(p, w, x, y, spans, grid, shared, s);
   }
-  if (p.m == 1 && spans <= 6) {
-    // One activation row: a wave per span.  Eight waves per compute unit measured best or equal in
-    // 25 of 27 shapes (three formats, K = 2048 ... 12288, 1024 ... 151936 rows: 0-30 % below the
-    // kernel that parks the codes in LDS first).
-    const uint32_t units = (uint32_t)(compute_units > 0 ? compute_units : 256);
-    const uint32_t most = units * (8u / spans);
-    const dim3 blocks((uint32_t)p.rows < most ? (uint32_t)p.rows : most);
-    const unsigned char *in = static_cast<const unsigned char *>(w);
-    const uint32_t rows = (uint32_t)p.rows;
-    switch (spans) {
-      case 1: note_variant<SpansTag<kKind, 1>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 1>), blocks, dim3(1 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      case 2: note_variant<SpansTag<kKind, 2>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 2>), blocks, dim3(2 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      case 3: note_variant<SpansTag<kKind, 3>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 3>), blocks, dim3(3 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      case 4: note_variant<SpansTag<kKind, 4>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 4>), blocks, dim3(4 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      case 5: note_variant<SpansTag<kKind, 5>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 5>), blocks, dim3(5 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-      default: note_variant<SpansTag<kKind, 6>>(); hipLaunchKernelGGL((gguf_matvec_q8_spans<kKind, TX, 6>), blocks, dim3(6 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-    }
-    return hipGetLastError();
-  }
+  if (p.m == 1 && spans <= 6) return run_spans<kKind, TX>(p, w, x, y, spans, kWaveLanes, compute_units, s);
   if (p.m == 1) return run_registers<kKind, TX, 1>(p, w, x, y, spans, grid, shared, s);
   if (p.m == 2) return run_registers<kKind, TX, 2>(p, w, x, y, spans, grid, shared, s);
   if (p.m <= 4) return run_registers<kKind, TX, 4>(p, w, x, y, spans, grid, shared, s);

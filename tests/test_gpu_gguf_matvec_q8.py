@@ -134,15 +134,18 @@ def test_q8_route_vocabulary_sized_weight(tag, m):
 def test_q8_route_the_reference_s_own_projection_shapes():
     """The shapes of the reference's Q8_0 / Q4_K projection cases
     (tests/compute_models/cpu_c5_gguf_inputs.h:231,237,259,287,314): none is a multiple of 2048 wide.
-    The Q8_0 ones take the kernel that walks a row block by block, the Q4_K one the matrix-unit kernel."""
+    The Q8_0 ones of 256 n values take the span kernel with a short last span (128 values: the kernel
+    that walks a row block by block), the Q4_K one the matrix-unit kernel."""
     rng = np.random.default_rng(1803)
     for tag, k, rows in (("q8_0", 1024, 32768), ("q4_k", 5120, 10240), ("q8_0", 7168, 3072), ("q8_0", 17408, 5120),
                          ("q8_0", 128, 512)):
         raw = weights_for(tag, rng, rows, k)
         x = rng.normal(0, 1.5, (k,)).astype(np.float32)
         note(f"q8 matvec {tag} [{k} -> {rows}], one activation row")
-        check(tag, "f32", raw, rows, k, x,
-              kernel="gguf_matvec_q8_tiles/q4_k/1-tokens" if tag == "q4_k" else f"gguf_matvec_q8_blocks/{tag}/1-tokens")
+        kernel = {1024: "gguf_matvec_q8_spans/q8_0/1-spans/short", 5120: "gguf_matvec_q8_tiles/q4_k/1-tokens",
+                  7168: "gguf_matvec_q8_spans/q8_0/4-spans/short", 17408: "gguf_matvec_q8_spans/q8_0/9-spans/short",
+                  128: "gguf_matvec_q8_blocks/q8_0/1-tokens"}[k]
+        check(tag, "f32", raw, rows, k, x, kernel=kernel)
 
 
 @pytest.mark.parametrize("x_tag", ["f32", "bf16", "f16"])
@@ -162,6 +165,8 @@ def test_q8_route_any_whole_number_of_blocks_and_activation_rows(tag, x_tag):
             label = {1: 1, 2: 2, 3: 4, 4: 4, 5: 8, 8: 8}[m]
             if tag == "q4_k" and k >= 1024:   # Q4_K rows of four blocks or more: the matrix unit, four activation rows a set
                 check(tag, x_tag, raw, rows, k, x, kernel=f"gguf_matvec_q8_tiles/q4_k/{1 if m == 1 else (4 if m <= 4 else 8)}-tokens")
+            elif tag == "q8_0" and k >= 1024 and m == 1:   # Q8_0 rows of 256 n values, one activation row: a short last span
+                check(tag, x_tag, raw, rows, k, x, kernel=f"gguf_matvec_q8_spans/q8_0/{-(-k // 2048)}-spans/short")
             else:
                 check(tag, x_tag, raw, rows, k, x, kernel=f"gguf_matvec_q8_blocks/{tag}/{label}-tokens")
 
@@ -272,3 +277,27 @@ def test_q8_route_q4_k_matrix_unit_widths_tokens_and_shared_tiles(x_tag):
           kernel="gguf_matvec_q8_blocks/q4_k/1-tokens")
     check("q4_k", x_tag, raw, 20, 2048, rng.normal(0, 1, 2048).astype(np.float32), x_offset=1,
           kernel="gguf_matvec_q8_blocks/q4_k/1-tokens")
+
+
+@pytest.mark.parametrize("x_tag", ["f32", "bf16", "f16"])
+def test_q8_route_q8_0_rows_with_a_short_last_span(x_tag):
+    """Q8_0 rows of 256 n values (8 blocks are 17 whole vectors) take the span kernel, whose last wave
+    then has 8 to 56 blocks: one to nine spans, the lanes past the row's end neither read past it nor
+    add to it, every quant and scale pattern."""
+    rng = np.random.default_rng(1812)
+    for k in (1024, 1280, 2304, 3840, 5120, 7168, 9216, 10496, 12544, 14592, 17408, 18176):
+        for rows in (1, 5, 70) if k != 7168 else (1, 5, 70, 3072):
+            raw = raw_bytes_for("q8_0", rng, rows, k) if x_tag != "f16" else weights_for("q8_0", rng, rows, k)
+            x = rng.normal(0, 1.5, k).astype(np.float32)
+            if rows == 5:
+                x[k - 256:] = 0.0            # the last activation blocks are zeros
+                x[32:64] = -2.5              # a block whose every value is the (negative) maximum
+            note(f"q8 matvec q8_0 short last span x {x_tag} rows {rows} k {k}")
+            check("q8_0", x_tag, raw, rows, k, x, kernel=f"gguf_matvec_q8_spans/q8_0/{-(-k // 2048)}-spans/short")
+    note("q8 matvec q8_0: more than nine spans, several activation rows and misplaced rows keep the block-walking kernel")
+    raw = raw_bytes_for("q8_0", rng, 20, 18688)
+    check("q8_0", x_tag, raw if x_tag != "f16" else weights_for("q8_0", rng, 20, 18688), 20, 18688,
+          rng.normal(0, 1, 18688).astype(np.float32), kernel="gguf_matvec_q8_blocks/q8_0/1-tokens")
+    raw = weights_for("q8_0", rng, 20, 5120)
+    check("q8_0", x_tag, raw, 20, 5120, rng.normal(0, 1, (2, 5120)).astype(np.float32), kernel="gguf_matvec_q8_blocks/q8_0/2-tokens")
+    check("q8_0", x_tag, raw, 20, 5120, rng.normal(0, 1, 5120).astype(np.float32), byte_offset=2, kernel="gguf_matvec_q8_blocks/q8_0/1-tokens")
