@@ -475,6 +475,21 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec(const unsigned char
   }
 }
 
+// Launch-shape labels: gguf_matvec_<form>/<format>/<detail>
+inline const char *matvec_kind_word(int kind) { return kind == 0 ? "q4_k" : (kind == 1 ? "q6_k" : "q8_0"); }
+template <int kKind> struct ExactLinesTag {
+  static std::string text() { return std::string("gguf_matvec_lines/") + matvec_kind_word(kKind); }
+};
+template <int kKind, int kSpans> struct ExactSpansTag {
+  static std::string text() { return std::string("gguf_matvec_spans/") + matvec_kind_word(kKind) + "/" + std::to_string(kSpans) + "-spans"; }
+};
+template <int kKind, int kM> struct ExactLongTag {
+  static std::string text() { return std::string("gguf_matvec_lines_long/") + matvec_kind_word(kKind) + "/" + std::to_string(kM) + "-tokens"; }
+};
+template <int kKind, int kM> struct ExactGeneralTag {
+  static std::string text() { return std::string("gguf_matvec_general/") + matvec_kind_word(kKind) + "/" + std::to_string(kM) + "-tokens"; }
+};
+
 template <int kKind, class TX>
 hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, hipStream_t s) {
   // Rows per wave: one when there are few rows (every wave in flight at once), up to eight for
@@ -495,6 +510,7 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
       // 45.9 us, against 6.4 and 47.7 us with five; counts that are not a multiple of the
       // compute units leave some of them a block short and are slower)
       const dim3 machine(wanted < units * 3u ? wanted : units * 3u);
+      note_variant<ExactLinesTag<kKind>>();
       hipLaunchKernelGGL((gguf_matvec_lines<kKind, TX, 1>), machine, block, 0, s, in, x, y, (uint32_t)p.rows,
                          p.row_stride);
       return hipGetLastError();
@@ -514,11 +530,11 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
       const dim3 machine((uint32_t)p.rows < most ? (uint32_t)p.rows : most);
       const uint32_t rows = (uint32_t)p.rows;
       switch (spans) {
-        case 2: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 2>), machine, dim3(2 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-        case 3: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 3>), machine, dim3(3 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-        case 4: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 4>), machine, dim3(4 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-        case 5: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 5>), machine, dim3(5 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
-        default: hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 6>), machine, dim3(6 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+        case 2: note_variant<ExactSpansTag<kKind, 2>>(); hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 2>), machine, dim3(2 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+        case 3: note_variant<ExactSpansTag<kKind, 3>>(); hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 3>), machine, dim3(3 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+        case 4: note_variant<ExactSpansTag<kKind, 4>>(); hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 4>), machine, dim3(4 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+        case 5: note_variant<ExactSpansTag<kKind, 5>>(); hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 5>), machine, dim3(5 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
+        default: note_variant<ExactSpansTag<kKind, 6>>(); hipLaunchKernelGGL((gguf_matvec_spans<kKind, TX, 6>), machine, dim3(6 * kWaveLanes), 0, s, in, x, y, rows, p.row_stride); break;
       }
       return hipGetLastError();
     }
@@ -526,30 +542,49 @@ hipError_t run_m(const MatVecParams &p, const void *w, const void *x, void *y, h
       const uint32_t spans = p.k / 2048;
       const uint32_t wanted = (uint32_t)((p.rows + kWavesPerBlock - 1) / kWavesPerBlock);
       const dim3 machine(wanted < units * 3u ? wanted : units * 3u);
-      if (p.m == 1)
-        hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 1>), machine, block, staged, s, in, x, y,
-                           (uint32_t)p.rows, p.row_stride, spans, p.m);
-      else if (p.m == 2)
+      if (p.m == 1) {
+        // one activation row arrives here with seven spans or more: only Q6_K's then fit beside its row buffers
+        if constexpr (kKind == 1) {
+          note_variant<ExactLongTag<kKind, 1>>();
+          hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 1>), machine, block, staged, s, in, x, y,
+                             (uint32_t)p.rows, p.row_stride, spans, p.m);
+        } else {
+          return hipErrorInvalidValue;
+        }
+      }
+      else if (p.m == 2) {
+        note_variant<ExactLongTag<kKind, 2>>();
         hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 2>), machine, block, staged, s, in, x, y,
                            (uint32_t)p.rows, p.row_stride, spans, p.m);
-      else if (p.m <= 4)
+      }
+      else if (p.m <= 4) {
+        note_variant<ExactLongTag<kKind, 4>>();
         hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 4>), machine, block, staged, s, in, x, y,
                            (uint32_t)p.rows, p.row_stride, spans, p.m);
-      else
+      }
+      else {
+        note_variant<ExactLongTag<kKind, 8>>();
         hipLaunchKernelGGL((gguf_matvec_lines_long<kKind, TX, 8>), machine, block, staged, s, in, x, y,
                            (uint32_t)p.rows, p.row_stride, spans, p.m);
+      }
       return hipGetLastError();
     }
   }
-  if (p.m == 1)
+  if (p.m == 1) {
+    note_variant<ExactGeneralTag<kKind, 1>>();
     hipLaunchKernelGGL((gguf_matvec<kKind, 1, TX>), grid, block, shared, s, in, x, y, (uint32_t)p.rows, p.k,
                        p.row_stride, p.m, rows_per_wave);
-  else if (p.m <= 4)
+  }
+  else if (p.m <= 4) {
+    note_variant<ExactGeneralTag<kKind, 4>>();
     hipLaunchKernelGGL((gguf_matvec<kKind, 4, TX>), grid, block, shared, s, in, x, y, (uint32_t)p.rows, p.k,
                        p.row_stride, p.m, rows_per_wave);
-  else
+  }
+  else {
+    note_variant<ExactGeneralTag<kKind, 8>>();
     hipLaunchKernelGGL((gguf_matvec<kKind, 8, TX>), grid, block, shared, s, in, x, y, (uint32_t)p.rows, p.k,
                        p.row_stride, p.m, rows_per_wave);
+  }
   return hipGetLastError();
 }
 

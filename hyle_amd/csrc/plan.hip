@@ -1463,6 +1463,8 @@ const char *add(const std::string &label) {
   return list.labels.back()->c_str();
 }
 void note(const char *label) {
+  // a loop of dispatches of one shape (merge rounds) is one entry
+  if (g_noted_count != 0 && g_noted[g_noted_count - 1] == label) return;
   if (g_noted_count < kNotedVariants) g_noted[g_noted_count++] = label;
 }
 }  // namespace variants

@@ -797,6 +797,29 @@ __global__ __launch_bounds__(kMergeThreads) void topk_rank_lists(const char *x, 
   emit<T, kBytewise, kFinal>(ranked, a, row, x, values, indices, list);
 }
 
+// Launch-shape labels: topk_<kernel>/<form>...
+inline std::string access_word(bool vector, bool bytewise) { return vector ? "vector" : (bytewise ? "bytes" : "scalar"); }
+template <int kE, bool kVector, bool kBytewise, bool kFinal> struct SelectTag {
+  static std::string text() {
+    return "topk_select/" + std::to_string(kE) + "x256/" + access_word(kVector, kBytewise) + (kFinal ? "/final" : "/lists");
+  }
+};
+template <bool kBytewise, bool kFinal> struct RankListsTag {
+  static std::string text() { return std::string("topk_rank_lists") + (kBytewise ? "/bytes" : "") + (kFinal ? "/final" : "/lists"); }
+};
+template <bool kVector, bool kBytewise, bool kFinal> struct TilesTag {
+  static std::string text() { return "topk_tiles/" + access_word(kVector, kBytewise) + (kFinal ? "/final" : "/lists"); }
+};
+template <bool kBytewise, bool kFinal> struct MergeTag {
+  static std::string text() { return std::string("topk_merge") + (kBytewise ? "/bytes" : "") + (kFinal ? "/final" : "/lists"); }
+};
+struct MergeRunsTag {
+  static std::string text() { return "topk_merge_runs"; }
+};
+template <bool kBytewise> struct EmitRunTag {
+  static std::string text() { return std::string("topk_emit_run") + (kBytewise ? "/bytes" : ""); }
+};
+
 template <class T, int kE, bool kBytewise>
 void select_tiles_launch(const TopKParams &p, const Addressing &a, const char *in, void *values,
                          int32_t *indices, uint64_t *lists, bool vector, hipStream_t s) {
@@ -804,14 +827,16 @@ void select_tiles_launch(const TopKParams &p, const Addressing &a, const char *i
   const uint32_t largest = p.largest ? 1u : 0u;
   const bool final = p.tiles == 1;
 #define HYLE_SELECT(VEC, BYTES, FINAL)                                                                   \
+  note_variant<SelectTag<kE, VEC, BYTES, FINAL>>();                                                         \
   hipLaunchKernelGGL((topk_select<T, kE, VEC, BYTES, FINAL>), grid, block, 0, s, in, values, indices, lists, a, \
                      p.tiles, largest)
+  // tiles of 2048 elements are chosen only for rows that one of them covers (topk_plan): no lists there
   if (vector) {
-    if (final) HYLE_SELECT(true, false, true);
-    else HYLE_SELECT(true, false, false);
+    if (final) { HYLE_SELECT(true, false, true); }
+    else if constexpr (kE != 8) { HYLE_SELECT(true, false, false); }
   } else {
-    if (final) HYLE_SELECT(false, kBytewise, true);
-    else HYLE_SELECT(false, kBytewise, false);
+    if (final) { HYLE_SELECT(false, kBytewise, true); }
+    else if constexpr (kE != 8) { HYLE_SELECT(false, kBytewise, false); }
   }
 #undef HYLE_SELECT
 }
@@ -822,12 +847,15 @@ void rank_lists_launch(const TopKParams &p, const Addressing &a, const char *in,
                        hipStream_t s) {
   const dim3 grid(p.rows * out), block(kMergeThreads);
   const size_t shared = (size_t)fan * p.count * sizeof(uint64_t);
-  if (out == 1)
+  if (out == 1) {
+    note_variant<RankListsTag<kBytewise, true>>();
     hipLaunchKernelGGL((topk_rank_lists<T, kBytewise, true>), grid, block, shared, s, in, values, indices, from, to,
                        a, lists, fan, out);
-  else
+  } else {
+    note_variant<RankListsTag<kBytewise, false>>();
     hipLaunchKernelGGL((topk_rank_lists<T, kBytewise, false>), grid, block, shared, s, in, values, indices, from,
                        to, a, lists, fan, out);
+  }
 }
 
 uint32_t pow2_at_least(uint32_t n, uint32_t floor) {
@@ -878,16 +906,20 @@ hipError_t run(const TopKParams &p, const void *x, void *values, int32_t *indice
     Addressing whole = a;
     whole.count = kTile;
     uint64_t *from = lists_a, *to = lists_a + (size_t)p.rows * p.tiles * kTile;
-    if (vector)
+    if (vector) {
+      note_variant<TilesTag<true, false, false>>();
       hipLaunchKernelGGL((topk_tiles<T, true, false, false>), dim3(p.rows * p.tiles), block, 0, s, in, values, indices,
                          from, whole, p.tiles, kTile, largest);
-    else
+    } else {
+      note_variant<TilesTag<false, kBytewise, false>>();
       hipLaunchKernelGGL((topk_tiles<T, false, kBytewise, false>), dim3(p.rows * p.tiles), block, 0, s, in, values,
                          indices, from, whole, p.tiles, kTile, largest);
+    }
     const uint32_t limit = (p.count + kTile - 1) / kTile * kTile;  // no run needs more keys than this
     uint32_t runs = p.tiles, run_keys = kTile;
     while (runs > 1) {
       const uint32_t runs_out = (runs + 1) / 2, out_keys = std::min(2 * run_keys, limit);
+      note_variant<MergeRunsTag>();
       hipLaunchKernelGGL(topk_merge_runs, dim3(p.rows * runs_out * (out_keys / kTile)), block, 0, s, from, to, runs,
                          run_keys, runs_out, out_keys);
       std::swap(from, to);
@@ -895,36 +927,46 @@ hipError_t run(const TopKParams &p, const void *x, void *values, int32_t *indice
       run_keys = out_keys;
     }
     const uint32_t blocks_per_row = (p.count + kBlockThreads - 1) / kBlockThreads;
+    note_variant<EmitRunTag<kBytewise>>();
     hipLaunchKernelGGL((topk_emit_run<T, kBytewise>), dim3(p.rows * blocks_per_row), block, 0, s, in, values, indices,
                        from, a, run_keys, blocks_per_row);
     return hipGetLastError();
   }
   if (p.tiles == 1) {
-    if (vector)
+    if (vector) {
+      note_variant<TilesTag<true, false, true>>();
       hipLaunchKernelGGL((topk_tiles<T, true, false, true>), dim3(p.rows), block, 0, s, in, values, indices,
                          lists_a, a, 1u, tile_n, largest);
-    else
+    } else {
+      note_variant<TilesTag<false, kBytewise, true>>();
       hipLaunchKernelGGL((topk_tiles<T, false, kBytewise, true>), dim3(p.rows), block, 0, s, in, values,
                          indices, lists_a, a, 1u, tile_n, largest);
+    }
     return hipGetLastError();
   }
-  if (vector)
+  if (vector) {
+    note_variant<TilesTag<true, false, false>>();
     hipLaunchKernelGGL((topk_tiles<T, true, false, false>), dim3(p.rows * p.tiles), block, 0, s, in, values,
                        indices, lists_a, a, p.tiles, kTile, largest);
-  else
+  } else {
+    note_variant<TilesTag<false, kBytewise, false>>();
     hipLaunchKernelGGL((topk_tiles<T, false, kBytewise, false>), dim3(p.rows * p.tiles), block, 0, s, in,
                        values, indices, lists_a, a, p.tiles, kTile, largest);
+  }
   uint32_t lists = p.tiles;
   uint64_t *from = lists_a, *to = lists_b;
   while (lists > 1) {
     const uint32_t out = (lists + p.fan - 1) / p.fan;
     const uint32_t sort_n = pow2_at_least(std::min(lists, p.fan) * p.count, 64);
-    if (out == 1)
+    if (out == 1) {
+      note_variant<MergeTag<kBytewise, true>>();
       hipLaunchKernelGGL((topk_merge<T, kBytewise, true>), dim3(p.rows), block, 0, s, in, values, indices, from,
                          to, a, lists, p.fan, 1u, sort_n);
-    else
+    } else {
+      note_variant<MergeTag<kBytewise, false>>();
       hipLaunchKernelGGL((topk_merge<T, kBytewise, false>), dim3(p.rows * out), block, 0, s, in, values,
                          indices, from, to, a, lists, p.fan, out, sort_n);
+    }
     std::swap(from, to);
     lists = out;
   }

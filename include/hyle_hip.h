@@ -314,8 +314,9 @@ HYLE_HIP_API const char *hyle_hip_plan_route_name(const hyle_hip_plan *plan);
  * shape compiled into the library has a label ("softmax_rows/512x2/additive/exact/steered");
  * hyle_hip_variant_count / hyle_hip_variant_label list them, and hyle_hip_last_launch_variant
  * returns the label(s) of the dispatches the calling thread's last hyle_hip_plan_launch or
- * hyle_hip_plan_launch_static enqueued, joined by " + " (empty when it enqueued nothing).  The
- * text stays valid until the thread's next call of the same function. */
+ * hyle_hip_plan_launch_static enqueued, joined by " + " (empty when it enqueued nothing; consecutive
+ * dispatches of one shape are one entry; at most four entries).  The text stays valid until the
+ * thread's next call of the same function. */
 HYLE_HIP_API uint32_t hyle_hip_variant_count(void);
 HYLE_HIP_API const char *hyle_hip_variant_label(uint32_t index);
 HYLE_HIP_API const char *hyle_hip_last_launch_variant(void);

@@ -230,3 +230,24 @@ def test_topk_int32_keys():
                 assert np.array_equal(to_host(values), want_values)
                 order = np.argsort(-x.astype(np.int64) if largest else x.astype(np.int64), axis=axis, kind="stable")
                 assert np.array_equal(np.take(order, range(count), axis=axis), want_indices)   # the oracle against numpy
+
+
+@pytest.mark.parametrize("tag", ["f32", "bf16"])
+def test_topk_rows_at_odd_addresses_on_every_route(tag):
+    """Byte strides that leave elements unaligned (src/compute_provider_native/cast.cc:113-116 allows
+    them) are read byte by byte: the select route with one tile, with lists, and with two rounds of
+    list merges; the sorting route with one tile, with merged lists (one and two rounds), and with
+    whole sorted runs."""
+    rng = np.random.default_rng(1190)
+    size = 4 if tag == "f32" else 2
+    for dims, count in (([3, 5000], 17), ([2, 20000], 40), ([2, 140000], 256), ([5, 300], 280), ([2, 5000], 300),
+                        ([2, 5000], 1000), ([2, 5000], 1500)):
+        values = tied_values(rng, dims, tag)
+        row_bytes = dims[1] * size + 3
+        raw = np.zeros(dims[0] * row_bytes + 8, np.uint8)
+        for r in range(dims[0]):
+            raw[r * row_bytes:r * row_bytes + dims[1] * size] = values[r].view(np.uint8)
+        desc = hc.TensorDesc.strided_bytes(TYPES[tag][0], dims, [row_bytes, size])
+        note(f"topk {tag} {dims} rows {row_bytes} bytes apart, count {count}")
+        outputs = run(hc.TopK(count=count), torch.from_numpy(raw).to(DEVICE), descs=[desc])
+        check(tag, raw, dims, count, 1, True, outputs, [row_bytes, size])
