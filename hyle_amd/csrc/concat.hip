@@ -85,6 +85,11 @@ uint32_t blocks_for(uint64_t units) {
 
 }  // namespace
 
+// Launch-shape labels
+template <int kUnit, bool kRuns> struct ConcatTag {
+  static std::string text() { return std::string(kRuns ? "concat_runs/" : "concat_general/") + std::to_string(kUnit) + "-bytes"; }
+};
+
 hipError_t launch_concat(const ConcatParams &p, const void *const *inputs, void *out, hipStream_t stream) {
   if (p.elements == 0) return hipSuccess;
   unsigned char *o = static_cast<unsigned char *>(out);
@@ -111,11 +116,11 @@ hipError_t launch_concat(const ConcatParams &p, const void *const *inputs, void 
     }
     const dim3 grid((uint32_t)blocks, p.inputs), block(kBlockThreads);
     switch (unit) {
-      case 16: hipLaunchKernelGGL((concat_runs<16>), grid, block, 0, stream, c, o); break;
-      case 8: hipLaunchKernelGGL((concat_runs<8>), grid, block, 0, stream, c, o); break;
-      case 4: hipLaunchKernelGGL((concat_runs<4>), grid, block, 0, stream, c, o); break;
-      case 2: hipLaunchKernelGGL((concat_runs<2>), grid, block, 0, stream, c, o); break;
-      default: hipLaunchKernelGGL((concat_runs<1>), grid, block, 0, stream, c, o); break;
+      case 16: note_variant<ConcatTag<16, true>>(); hipLaunchKernelGGL((concat_runs<16>), grid, block, 0, stream, c, o); break;
+      case 8: note_variant<ConcatTag<8, true>>(); hipLaunchKernelGGL((concat_runs<8>), grid, block, 0, stream, c, o); break;
+      case 4: note_variant<ConcatTag<4, true>>(); hipLaunchKernelGGL((concat_runs<4>), grid, block, 0, stream, c, o); break;
+      case 2: note_variant<ConcatTag<2, true>>(); hipLaunchKernelGGL((concat_runs<2>), grid, block, 0, stream, c, o); break;
+      default: note_variant<ConcatTag<1, true>>(); hipLaunchKernelGGL((concat_runs<1>), grid, block, 0, stream, c, o); break;
     }
     return hipGetLastError();
   }
@@ -132,10 +137,10 @@ hipError_t launch_concat(const ConcatParams &p, const void *const *inputs, void 
   }
   const dim3 grid(blocks_for(most), p.inputs), block(kBlockThreads);
   switch (p.size) {
-    case 8: hipLaunchKernelGGL((concat_general<8>), grid, block, 0, stream, l, o); break;
-    case 4: hipLaunchKernelGGL((concat_general<4>), grid, block, 0, stream, l, o); break;
-    case 2: hipLaunchKernelGGL((concat_general<2>), grid, block, 0, stream, l, o); break;
-    default: hipLaunchKernelGGL((concat_general<1>), grid, block, 0, stream, l, o); break;
+    case 8: note_variant<ConcatTag<8, false>>(); hipLaunchKernelGGL((concat_general<8>), grid, block, 0, stream, l, o); break;
+    case 4: note_variant<ConcatTag<4, false>>(); hipLaunchKernelGGL((concat_general<4>), grid, block, 0, stream, l, o); break;
+    case 2: note_variant<ConcatTag<2, false>>(); hipLaunchKernelGGL((concat_general<2>), grid, block, 0, stream, l, o); break;
+    default: note_variant<ConcatTag<1, false>>(); hipLaunchKernelGGL((concat_general<1>), grid, block, 0, stream, l, o); break;
   }
   return hipGetLastError();
 }

@@ -174,6 +174,10 @@ __global__ __launch_bounds__(kRowThreads) void gather_rows_fat(GatherRows p, Gat
   if (threadIdx.x < kFatChunks) {
     const uint32_t chunk = blockIdx.x * kFatChunks + threadIdx.x;
     uint32_t units = 0;
+    // a chunk past the last one (the last block's, when the chunks are no multiple of sixteen) has no
+    // units, but every lane still reads "its first unit": give it an address that exists
+    from_of[threadIdx.x] = p.source;
+    to_of[threadIdx.x] = out;
     if (chunk < chunks) {
       const uint32_t row = chunk / chunks_per_row, piece = chunk - row * chunks_per_row;
       const uint32_t outer = row / p.index_count, item = row - outer * p.index_count;
@@ -259,6 +263,20 @@ __global__ __launch_bounds__(kBlockThreads) void gather_general(GatherLayout l, 
   for (int b = 0; b < kSize; ++b) out[e * kSize + b] = source[b];
 }
 
+// Launch-shape labels: gather_<form>/<unit bytes>/<index width>/<dense|strided indices>
+inline std::string index_words(bool wide, bool dense) { return std::string(wide ? "i64" : "i32") + (dense ? "/dense" : "/strided"); }
+template <int kForm, int kUnit, bool kWide, bool kDense> struct GatherRowsTag {  // 0 fat rows, 1 rows, 2 units
+  static std::string text() {
+    return std::string(kForm == 0 ? "gather_rows_fat/" : (kForm == 1 ? "gather_rows/" : "gather_units/")) + std::to_string(kUnit) + "-bytes/" + index_words(kWide, kDense);
+  }
+};
+template <int kSize, bool kWide> struct GatherGeneralTag {
+  static std::string text() { return "gather_general/" + std::to_string(kSize) + "-bytes/" + (kWide ? "i64" : "i32"); }
+};
+template <bool kWide, bool kDense> struct GatherCheckTag {
+  static std::string text() { return "gather_check/" + index_words(kWide, kDense); }
+};
+
 template <int kUnit, bool kWide, bool kDense>
 void run_rows(const GatherRows &rows, const GatherIndexView &view, const GatherVerdict &verdict, unsigned char *out,
               hipStream_t stream) {
@@ -269,14 +287,18 @@ void run_rows(const GatherRows &rows, const GatherIndexView &view, const GatherV
     const uint32_t per_block = kRowThreads / kBlockThreads;
     // Enough chunks to give every compute unit a fat block: sixteen chunks per block, resolved
     // first and then streamed (11.8 us against 12.6 us for 8192 rows of 4 KiB picked at random).
-    if (chunks >= 4096)
+    if (chunks >= 4096) {
+      note_variant<GatherRowsTag<0, kUnit, kWide, kDense>>();
       hipLaunchKernelGGL((gather_rows_fat<kUnit, kWide, kDense>), dim3((uint32_t)((chunks + kFatChunks - 1) / kFatChunks)),
                          dim3(kRowThreads), 0, stream, rows, view, verdict, out, per_row, (uint32_t)chunks);
-    else
+    } else {
+      note_variant<GatherRowsTag<1, kUnit, kWide, kDense>>();
       hipLaunchKernelGGL((gather_rows<kUnit, kWide, kDense>), dim3((uint32_t)((chunks + per_block - 1) / per_block)),
                          dim3(kRowThreads), 0, stream, rows, view, verdict, out, per_row, (uint32_t)chunks);
+    }
   } else {
     const uint64_t units = (uint64_t)rows.rows * rows.row_units;
+    note_variant<GatherRowsTag<2, kUnit, kWide, kDense>>();
     hipLaunchKernelGGL((gather_units<kUnit, kWide, kDense>), dim3((uint32_t)((units + kBlockThreads - 1) / kBlockThreads)),
                        block, 0, stream, rows, view, verdict, out, (uint32_t)units);
   }
@@ -298,8 +320,13 @@ template <int kSize>
 void run_general(bool wide, const GatherLayout &l, const GatherVerdict &verdict, unsigned char *out, uint64_t elements,
                  hipStream_t stream) {
   const dim3 grid((uint32_t)((elements + kBlockThreads - 1) / kBlockThreads)), block(kBlockThreads);
-  if (wide) hipLaunchKernelGGL((gather_general<kSize, true>), grid, block, 0, stream, l, verdict, out, elements);
-  else hipLaunchKernelGGL((gather_general<kSize, false>), grid, block, 0, stream, l, verdict, out, elements);
+  if (wide) {
+    note_variant<GatherGeneralTag<kSize, true>>();
+    hipLaunchKernelGGL((gather_general<kSize, true>), grid, block, 0, stream, l, verdict, out, elements);
+  } else {
+    note_variant<GatherGeneralTag<kSize, false>>();
+    hipLaunchKernelGGL((gather_general<kSize, false>), grid, block, 0, stream, l, verdict, out, elements);
+  }
 }
 
 }  // namespace
@@ -326,11 +353,11 @@ hipError_t launch_gather(const GatherParams &p, const void *source, const void *
     verdict = GatherVerdict{words, blocks, words + kGatherStatusWord, p.extent};
     const dim3 grid(blocks), block(kBlockThreads);
     if (p.wide_indices) {
-      if (dense_indices) hipLaunchKernelGGL((gather_check<true, true>), grid, block, 0, stream, view, p.extent, words);
-      else hipLaunchKernelGGL((gather_check<true, false>), grid, block, 0, stream, view, p.extent, words);
+      if (dense_indices) { note_variant<GatherCheckTag<true, true>>(); hipLaunchKernelGGL((gather_check<true, true>), grid, block, 0, stream, view, p.extent, words); }
+      else { note_variant<GatherCheckTag<true, false>>(); hipLaunchKernelGGL((gather_check<true, false>), grid, block, 0, stream, view, p.extent, words); }
     } else {
-      if (dense_indices) hipLaunchKernelGGL((gather_check<false, true>), grid, block, 0, stream, view, p.extent, words);
-      else hipLaunchKernelGGL((gather_check<false, false>), grid, block, 0, stream, view, p.extent, words);
+      if (dense_indices) { note_variant<GatherCheckTag<false, true>>(); hipLaunchKernelGGL((gather_check<false, true>), grid, block, 0, stream, view, p.extent, words); }
+      else { note_variant<GatherCheckTag<false, false>>(); hipLaunchKernelGGL((gather_check<false, false>), grid, block, 0, stream, view, p.extent, words); }
     }
     const hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;

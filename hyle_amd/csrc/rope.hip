@@ -219,6 +219,14 @@ __global__ __launch_bounds__(kBlockThreads) void rope_elements(RopeOperands p, c
   Traits<T>::store(out, second, b);
 }
 
+// Launch-shape labels
+template <int kForm, bool kHalfSplit> struct RopeTag {  // 0 steps, 1 vectors
+  static std::string text() { return std::string(kForm == 0 ? "rope_steps/" : "rope_vectors/") + (kHalfSplit ? "half-split" : "interleaved"); }
+};
+struct RopeElementsTag {
+  static std::string text() { return "rope_elements"; }
+};
+
 template <class T>
 hipError_t run_rope(const RopeParams &p, const void *in, const void *positions, const void *frequencies, void *out,
                     bool vector_aligned, hipStream_t stream) {
@@ -244,21 +252,28 @@ hipError_t run_rope(const RopeParams &p, const void *in, const void *positions, 
       while (per_block > 1 && (size_t)per_block * p.rotary * sizeof(float) > 32768) --per_block;
       const size_t lds = (size_t)per_block * p.rotary * sizeof(float);
       const dim3 grid((uint32_t)((steps + per_block - 1) / per_block));
-      if (p.half_split)
+      if (p.half_split) {
+        note_variant<RopeTag<0, true>>();
         hipLaunchKernelGGL((rope_steps<T, true>), grid, block, lds, stream, o, in, out, per_row, places, per_block, (uint32_t)steps);
-      else
+      } else {
+        note_variant<RopeTag<0, false>>();
         hipLaunchKernelGGL((rope_steps<T, false>), grid, block, lds, stream, o, in, out, per_row, places, per_block, (uint32_t)steps);
+      }
       return hipGetLastError();
     }
     const dim3 grid((uint32_t)((units + kBlockThreads - 1) / kBlockThreads));
-    if (p.half_split)
+    if (p.half_split) {
+      note_variant<RopeTag<1, true>>();
       hipLaunchKernelGGL((rope_vectors<T, true>), grid, block, 0, stream, o, in, out, per_row, places, groups, (uint32_t)units);
-    else
+    } else {
+      note_variant<RopeTag<1, false>>();
       hipLaunchKernelGGL((rope_vectors<T, false>), grid, block, 0, stream, o, in, out, per_row, places, groups, (uint32_t)units);
+    }
     return hipGetLastError();
   }
   const uint32_t per_row = p.rotary / 2 + (p.depth - p.rotary);
   const uint64_t units = p.rows * per_row;
+  note_variant<RopeElementsTag>();
   hipLaunchKernelGGL((rope_elements<T>), dim3((uint32_t)((units + kBlockThreads - 1) / kBlockThreads)), block, 0, stream, o, in,
                      out, p.half_split, per_row, units);
   return hipGetLastError();

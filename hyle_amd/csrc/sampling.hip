@@ -356,22 +356,37 @@ __global__ __launch_bounds__(kBlockThreads) void categorical_rows(const void *lo
   }
 }
 
+// Launch-shape labels
+template <bool kVector> struct CategoricalTilesTag {
+  static std::string text() { return std::string("categorical_tiles/") + (kVector ? "vector" : "scalar"); }
+};
+template <bool kVector, bool kScored> struct CategoricalRowsTag {
+  static std::string text() { return std::string("categorical_rows/") + (kVector ? "vector" : "scalar") + (kScored ? "/scored" : ""); }
+};
+template <int kForm> struct RandomBitsTag {  // 0 rows of blocks, 1 flat
+  static std::string text() { return kForm == 0 ? "random_bits_rows" : "random_bits"; }
+};
+
 template <class T, bool kVector>
 hipError_t run_categorical(const CategoricalParams &p, const void *logits, const uint32_t *identities, int32_t *indices,
                            float *scores, void *workspace, hipStream_t stream) {
   CategoricalTile *parts = static_cast<CategoricalTile *>(workspace);
   uint32_t *status = reinterpret_cast<uint32_t *>(static_cast<unsigned char *>(workspace) + p.status_offset);
   const dim3 block(kBlockThreads);
+  note_variant<CategoricalTilesTag<kVector>>();
   hipLaunchKernelGGL((categorical_tiles<T, kVector>), dim3(p.rows * p.tiles), block, 0, stream, logits, p.width, p.tiles, parts,
                      status);
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return err;
-  if (p.scored)
+  if (p.scored) {
+    note_variant<CategoricalRowsTag<kVector, true>>();
     hipLaunchKernelGGL((categorical_rows<T, kVector, true>), dim3(p.rows), block, 0, stream, logits, identities, p.width,
                        p.tiles, parts, indices, scores, status);
-  else
+  } else {
+    note_variant<CategoricalRowsTag<kVector, false>>();
     hipLaunchKernelGGL((categorical_rows<T, kVector, false>), dim3(p.rows), block, 0, stream, logits, identities, p.width,
                        p.tiles, parts, indices, scores, status);
+  }
   return hipGetLastError();
 }
 
@@ -396,10 +411,12 @@ hipError_t launch_random_bits(const RandomBitsParams &p, const void *identities,
   if (vector && blocks_per_row >= kBlockThreads) {
     const uint32_t per_block = kBlockThreads * kBitsPerThread;
     const dim3 grid((blocks_per_row + per_block - 1) / per_block, p.rows < 65535u ? p.rows : 65535u);
+    note_variant<RandomBitsTag<0>>();
     hipLaunchKernelGGL(random_bits_rows, grid, dim3(kBlockThreads), 0, stream, static_cast<const uint32_t *>(identities),
                        static_cast<uint32_t *>(out), p.rows, p.word_count, blocks_per_row);
     return hipGetLastError();
   }
+  note_variant<RandomBitsTag<1>>();
   hipLaunchKernelGGL(random_bits, dim3((uint32_t)blocks), dim3(kBlockThreads), 0, stream, static_cast<const uint32_t *>(identities),
                      static_cast<uint32_t *>(out), p.rows, p.word_count, blocks_per_row, vector);
   return hipGetLastError();

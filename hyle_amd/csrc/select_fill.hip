@@ -146,6 +146,14 @@ __global__ __launch_bounds__(kBlockThreads) void select_general(const unsigned c
 
 }  // namespace
 
+// Launch-shape labels
+struct FillTag {
+  static std::string text() { return "fill_pattern"; }
+};
+template <int kSize, bool kFlat> struct SelectTag {
+  static std::string text() { return std::string(kFlat ? "select_flat/" : "select_general/") + std::to_string(kSize) + "-bytes"; }
+};
+
 hipError_t launch_fill(const FillParams &p, void *out, hipStream_t stream) {
   if (p.elements == 0) return hipSuccess;
   uint64_t pattern = p.bits;
@@ -155,6 +163,7 @@ hipError_t launch_fill(const FillParams &p, void *out, hipStream_t stream) {
   const uint64_t bytes = p.elements * p.size;
   uint64_t blocks = (bytes / 16 + kBlockThreads) / kBlockThreads;
   blocks = blocks > 2048 ? 2048 : blocks;
+  note_variant<FillTag>();
   hipLaunchKernelGGL(fill_pattern, dim3((uint32_t)blocks), dim3(kBlockThreads), 0, stream,
                      static_cast<unsigned char *>(out), bytes, pattern);
   return hipGetLastError();
@@ -173,10 +182,10 @@ hipError_t launch_select(const SelectParams &p, const void *condition, const voi
     blocks = blocks < 1 ? 1 : (blocks > 8192 ? 8192 : blocks);
     const dim3 grid((uint32_t)blocks), block(kBlockThreads);
     switch (p.size) {
-      case 1: hipLaunchKernelGGL((select_flat<1>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
-      case 2: hipLaunchKernelGGL((select_flat<2>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
-      case 8: hipLaunchKernelGGL((select_flat<8>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
-      default: hipLaunchKernelGGL((select_flat<4>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
+      case 1: note_variant<SelectTag<1, true>>(); hipLaunchKernelGGL((select_flat<1>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
+      case 2: note_variant<SelectTag<2, true>>(); hipLaunchKernelGGL((select_flat<2>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
+      case 8: note_variant<SelectTag<8, true>>(); hipLaunchKernelGGL((select_flat<8>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
+      default: note_variant<SelectTag<4, true>>(); hipLaunchKernelGGL((select_flat<4>), grid, block, 0, stream, flat, o, vectors, (uint32_t)p.elements); break;
     }
     return hipGetLastError();
   }
@@ -188,10 +197,10 @@ hipError_t launch_select(const SelectParams &p, const void *condition, const voi
   }
   const dim3 grid((uint32_t)((p.elements + kBlockThreads - 1) / kBlockThreads)), block(kBlockThreads);
   switch (p.size) {
-    case 1: hipLaunchKernelGGL((select_general<1>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
-    case 2: hipLaunchKernelGGL((select_general<2>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
-    case 8: hipLaunchKernelGGL((select_general<8>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
-    default: hipLaunchKernelGGL((select_general<4>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
+    case 1: note_variant<SelectTag<1, false>>(); hipLaunchKernelGGL((select_general<1>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
+    case 2: note_variant<SelectTag<2, false>>(); hipLaunchKernelGGL((select_general<2>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
+    case 8: note_variant<SelectTag<8, false>>(); hipLaunchKernelGGL((select_general<8>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
+    default: note_variant<SelectTag<4, false>>(); hipLaunchKernelGGL((select_general<4>), grid, block, 0, stream, c, a, b, o, p.elements, layout); break;
   }
   return hipGetLastError();
 }

@@ -55,18 +55,29 @@ def host_values(array: np.ndarray, tag: str) -> np.ndarray:
     return array if tag == "f32" else orc.from_f32(TYPES[tag][1], array)
 
 
-# Labels of the kernel launch shapes the tests of this session launched through run()
-# (hyle_hip_last_launch_variant): tests/test_zy_launch_shape_coverage.py holds them against the list
-# of shapes compiled into the library.
+# Labels of the kernel launch shapes the tests of this session launched (hyle_hip_last_launch_variant
+# after every submit): tests/test_zy_launch_shape_coverage.py holds them against the list of shapes
+# compiled into the library.
 LAUNCHED = set()
 
 
+def _noting(submit):
+    @functools.wraps(submit)
+    def noted(self, *args, **kwargs):
+        submit(self, *args, **kwargs)
+        chosen = hc.last_launch_variant()
+        if chosen:
+            LAUNCHED.update(chosen.split(" + "))
+    return noted
+
+
+# every launch a GPU test makes goes through one of these two, whichever helper it uses
+hc.OperationInvocation.submit = _noting(hc.OperationInvocation.submit)
+hc.OperationInvocation.submit_without_workspace = _noting(hc.OperationInvocation.submit_without_workspace)
+
+
 def run(operation, *tensors, descs=None, outputs=None):
-    result = tio.run(context(), operation, *tensors, descs=descs, outputs=outputs)
-    chosen = hc.last_launch_variant()
-    if chosen:
-        LAUNCHED.update(chosen.split(" + "))
-    return result
+    return tio.run(context(), operation, *tensors, descs=descs, outputs=outputs)
 
 
 # ---- comparisons ----------------------------------------------------------------------------

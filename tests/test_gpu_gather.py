@@ -292,3 +292,29 @@ def test_embedding_sized_lookup():
     assert status == 0 and np.array_equal(out[:64].cpu().numpy().view(np.uint16), want)
     assert torch.equal(out, table[ids.long()])
     assert host_ids.min() >= 0
+
+
+@pytest.mark.parametrize("unit", [1, 2, 4, 8, 16])
+def test_whole_rows_in_every_unit_form_and_index_layout(unit):
+    """Rows moved whole take the widest unit (1 to 16 bytes) that divides the row and both addresses,
+    in one of three forms: short rows unit by unit, long rows chunk by chunk, and many chunks in fat
+    blocks that resolve their lookups first; each with 32- and 64-bit indices, dense and strided."""
+    size = min(unit, 8)
+    kind = {1: DT.kUInt8, 2: DT.kUInt16, 4: DT.kUInt32, 8: DT.kUInt64}[size]
+    per_unit = unit // size
+    for form, units_per_row, picks in (("units", 9, 50), ("rows", 257, 100), ("rows_fat", 257, 2100)):
+        shape = [37, units_per_row * per_unit]       # an odd number of units: no wider unit divides the row
+        strides = byte_strides(shape, size, 0, 0)
+        storage, values = lay_out(reference_values(shape, size), strides, lead=unit)   # the source starts `unit` bytes in
+        for wide in (False, True):
+            for index_mode in (0, 1):
+                width = 8 if wide else 4
+                index_strides = byte_strides([picks], width, 0, index_mode)
+                index_storage, ids = lay_out(reference_indices([picks], shape[0], wide), index_strides, lead=width)
+                note(f"gather whole rows: unit {unit} form {form} wide={wide} index_mode={index_mode}")
+                status, got = gather_on_device(kind, size, storage, unit, shape, strides, True, 0, index_storage, width, [picks],
+                                               index_strides, index_mode == 0, wide, checked=index_mode == 0)
+                assert status == 0
+                assert np.array_equal(got, np.take(values, ids.astype(np.int64), axis=0))
+                label = f"gather_{form}/{unit}-bytes/{'i64' if wide else 'i32'}/{'dense' if index_mode == 0 else 'strided'}"
+                assert label in hc.last_launch_variant().split(" + "), (hc.last_launch_variant(), label)
