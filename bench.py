@@ -239,12 +239,13 @@ def main() -> int:
             ("next_matvec_ggml_q8_q4_k_ffn_down", hc.GgufQuantizedType.kQ4K, 144, 6144, 2048, 80, 1, GGML_Q8),
             ("next_matvec_ggml_q8_q4_k_vocab", hc.GgufQuantizedType.kQ4K, 144, 2048, 151936, 4, 1, GGML_Q8),
             ("next_matvec_ggml_q8_q4_k_vocab_4_tokens", hc.GgufQuantizedType.kQ4K, 144, 2048, 151936, 4, 4, GGML_Q8),
+            ("next_matvec_ggml_q8_q4_k_vocab_8_tokens", hc.GgufQuantizedType.kQ4K, 144, 2048, 151936, 4, 8, GGML_Q8),
             ("next_matvec_ggml_q8_q6_k_vocab", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 1, GGML_Q8),
             ("next_matvec_ggml_q8_q6_k_vocab_4_tokens", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 4, GGML_Q8),
             ("next_matvec_ggml_q8_q6_k_vocab_8_tokens", hc.GgufQuantizedType.kQ6K, 210, 2048, 151936, 3, 8, GGML_Q8),
             ("next_matvec_ggml_q8_q8_0_vocab", hc.GgufQuantizedType.kQ8_0, 34, 2048, 151936, 3, 1, GGML_Q8),
             # the reference's own projection shapes (tests/compute_models/cpu_c5_gguf_inputs.h:231-314): widths that
-            # are no multiple of 2048 take the kernel that walks a row block by block
+            # are no multiple of 2048 (Q8_0: the span kernel with a short last span; Q4_K: the matrix-unit kernel)
             ("next_matvec_ggml_q8_q8_0_1024_to_32768", hc.GgufQuantizedType.kQ8_0, 34, 1024, 32768, 16, 1, GGML_Q8),
             ("next_matvec_ggml_q8_q4_k_5120_to_10240", hc.GgufQuantizedType.kQ4K, 144, 5120, 10240, 18, 1, GGML_Q8),
             ("next_matvec_ggml_q8_q8_0_7168_to_3072", hc.GgufQuantizedType.kQ8_0, 34, 7168, 3072, 24, 1, GGML_Q8),

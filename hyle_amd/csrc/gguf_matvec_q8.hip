@@ -755,9 +755,9 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_tiles(const unsi
     return out;
   };
   auto clamped = [&](uint32_t g) { return g < groups ? g : groups - 1; };
-  // activation blocks go round the block's eight half waves, four of a half wave's loads in flight; the
-  // first four are asked for before the weights: loads return in order
-  constexpr uint32_t kHalves = kBlockThreads / 32, kBatch = 4;
+  // activation blocks go round the block's eight half waves, four (eight) of a half wave's loads in flight;
+  // the first round is asked for before the weights: loads return in order
+  constexpr uint32_t kHalves = kBlockThreads / 32, kBatch = kSets == 2 ? 8 : 4;  // (eight activation rows of 2048 values are 64 blocks)
   const uint32_t half = threadIdx.x / 32, u = threadIdx.x % 32;
   const uint32_t units = kTokens * blocks;
   auto fetch_batch = [&](uint32_t first, TileValues (&fetched)[kBatch]) {
@@ -782,7 +782,7 @@ __global__ __launch_bounds__(kBlockThreads) void gguf_matvec_q8_tiles(const unsi
   ring[1] = load_group(clamped(member + split));
   for (uint32_t at = threadIdx.x * 16; at < k; at += kBlockThreads * 16) *reinterpret_cast<u32x4 *>(shared + at) = u32x4{0u, 0u, 0u, 0u};
   quantise_batch(half, fetched);
-  if constexpr (!kOneBatch) {  // more than 32 activation blocks: the rest wait for the weights before them
+  if constexpr (!kOneBatch) {  // more activation blocks than one round takes: the rest wait for the weights before them
     for (uint32_t first = half + kHalves * kBatch; first < units; first += kHalves * kBatch) {
       fetch_batch(first, fetched);
       quantise_batch(first, fetched);
@@ -1437,8 +1437,8 @@ hipError_t run_tiles_m(const MatVecParams &p, const void *w, const void *x, void
   const size_t shared = tile_shared_bytes(kSets == 0 ? 1 : 4 * kSets, blocks);
   const dim3 grid((waves + kWavesPerBlock - 1) / kWavesPerBlock);
   const unsigned char *in = static_cast<const unsigned char *>(w);
-  // at most 32 activation blocks in all: one round of the block's half waves, no loop around it
-  if ((kSets == 0 ? 1u : 4u * kSets) * blocks <= 32) {
+  // at most 32 activation blocks in all (64 with eight rows): one round of the block's half waves, no loop around it
+  if ((kSets == 0 ? 1u : 4u * kSets) * blocks <= (kSets == 2 ? 64u : 32u)) {
     note_variant<TilesTag<kSets, true>>();
     hipLaunchKernelGGL((gguf_matvec_q8_tiles<TX, kSets, true>), grid, dim3(kBlockThreads), shared, s, in, x, y, (uint32_t)p.rows,
                        p.row_stride, blocks, p.m, split_log2);
