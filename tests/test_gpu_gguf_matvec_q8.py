@@ -301,3 +301,26 @@ def test_q8_route_q8_0_rows_with_a_short_last_span(x_tag):
     raw = weights_for("q8_0", rng, 20, 5120)
     check("q8_0", x_tag, raw, 20, 5120, rng.normal(0, 1, (2, 5120)).astype(np.float32), kernel="gguf_matvec_q8_blocks/q8_0/2-tokens")
     check("q8_0", x_tag, raw, 20, 5120, rng.normal(0, 1, 5120).astype(np.float32), byte_offset=2, kernel="gguf_matvec_q8_blocks/q8_0/1-tokens")
+
+
+def test_q8_route_q4_k_matrix_unit_seeded_random_shapes():
+    """Forty seeded draws of (rows, blocks per row, activation rows, activation type, row padding):
+    whatever combination of tile sharing, overlapped last group, token sets and quantising rounds they
+    hit must agree with the oracle like the hand-picked cases."""
+    rng = np.random.default_rng(1813)
+    for case in range(40):
+        blocks = int(rng.integers(4, 41))
+        k = 256 * blocks
+        m = int(rng.integers(1, 9))
+        tokens = 1 if m == 1 else (4 if m <= 4 else 8)
+        if (1 + tokens) * k + tokens * blocks * 36 + 1024 * max(tokens // 4, 1) > 65536:
+            m, tokens = 1, 1                                   # the codes of more rows would not fit a block's LDS
+        rows = int(rng.choice([1, 7, 16, 33, 64, 100, 257, 1000, 3000]))
+        x_tag = ("f32", "bf16", "f16")[case % 3]
+        pad = int(rng.choice([0, 16, 48]))
+        raw = raw_bytes_for("q4_k", rng, rows, k) if x_tag != "f16" else weights_for("q4_k", rng, rows, k)
+        padded = np.zeros((rows, raw.shape[1] + pad), np.uint8)
+        padded[:, :raw.shape[1]] = raw
+        x = rng.normal(0, 1.5, (m, k) if m > 1 else (k,)).astype(np.float32)
+        note(f"q8 matvec q4_k tiles draw {case}: rows {rows} k {k} m {m} x {x_tag} pad {pad}")
+        check("q4_k", x_tag, padded, rows, k, x, row_stride=raw.shape[1] + pad, kernel=f"gguf_matvec_q8_tiles/q4_k/{tokens}-tokens")
